@@ -1,0 +1,253 @@
+"""Tensor-level wrappers over the C ABI (include/axon_amd.h).
+
+Each function validates on the host, allocates outputs/workspace with torch,
+passes raw device pointers and the current stream to ``libaxon_amd.so`` and
+raises on a non-zero status.  Nothing here computes on the CPU.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import MASK_F32, MASK_I64, check, ptr, require_device, stream_ptr
+
+
+@dataclass
+class Rows:
+    """How a flat array of ``n_slots`` values splits into rows (sequences)."""
+
+    n_rows: int
+    n_slots: int
+    uniform_len: int  # T for a padded [B, T] layout, 0 for packed
+    cu: torch.Tensor | None  # int32 [n_rows + 1] on device for packed
+    shape: tuple
+
+    @property
+    def cu_ptr(self):
+        return ptr(self.cu)
+
+
+def rows_of(t: torch.Tensor, cu_seqlens: torch.Tensor | None = None) -> Rows:
+    """Row layout of ``t``: [B, T] padded, or packed [N] (also [1, N]) with ``cu_seqlens``."""
+    if cu_seqlens is not None:
+        if cu_seqlens.dtype != torch.int32:
+            cu_seqlens = cu_seqlens.to(torch.int32)
+        cu = cu_seqlens.to(t.device).contiguous()
+        return Rows(int(cu.numel()) - 1, int(t.numel()), 0, cu, tuple(t.shape))
+    if t.dim() != 2:
+        raise ValueError(f"expected a [batch, seq] tensor or packed data with cu_seqlens, got shape {tuple(t.shape)}")
+    b, s = t.shape
+    return Rows(int(b), int(b * s), int(s), None, tuple(t.shape))
+
+
+def f32(t: torch.Tensor) -> torch.Tensor:
+    return t.detach().to(torch.float32).contiguous()
+
+
+def mask_arg(mask: torch.Tensor):
+    """Normalise a response mask once: fp32 and int64 are read natively by the kernels."""
+    mask = mask.detach()
+    if mask.dtype == torch.int64:
+        return mask.contiguous(), MASK_I64
+    if mask.dtype != torch.float32:
+        mask = mask.to(torch.float32)
+    return mask.contiguous(), MASK_F32
+
+
+def _zeros(n, device, dtype=torch.float32):
+    return torch.zeros(n, device=device, dtype=dtype)
+
+
+def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=True, want_sum=True):
+    """Per-row (count, sum of (a-b)*mask, any-flag); see axon_row_stats."""
+    lib = _lib.load()
+    require_device(a, "row_stats")
+    dev = a.device
+    a = f32(a)
+    b = f32(b) if b is not None else None
+    mk = (None, MASK_F32) if mask is None else mask_arg(mask)
+    cnt = _zeros(rows.n_rows, dev) if want_cnt else None
+    ssum = _zeros(rows.n_rows, dev) if want_sum else None
+    flag = _zeros(rows.n_rows, dev, torch.int32) if flag_mode else None
+    check(
+        lib.axon_row_stats(ptr(a), ptr(b), ptr(mk[0]), mk[1], rows.cu_ptr, rows.n_rows, rows.n_slots,
+                           rows.uniform_len, flag_mode, float(threshold), ptr(cnt), ptr(ssum), ptr(flag),
+                           stream_ptr()),
+        "axon_row_stats",
+    )
+    return cnt, ssum, flag
+
+
+def group_stats(scores, gidx, n_groups, eps, norm_by_std=True, want_scalar=True):
+    lib = _lib.load()
+    require_device(scores, "group_stats")
+    dev = scores.device
+    scores = f32(scores).reshape(-1)
+    gidx = gidx.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
+    n = int(scores.numel())
+    stats = _zeros(3 * max(n_groups, 1), dev).view(3, -1)
+    scalar = torch.empty(n, device=dev, dtype=torch.float32) if want_scalar else None
+    check(
+        lib.axon_group_stats(ptr(scores), ptr(gidx), n, int(n_groups), float(eps), int(bool(norm_by_std)),
+                             ptr(stats[0]), ptr(stats[1]), ptr(stats[2]), ptr(scalar), stream_ptr()),
+        "axon_group_stats",
+    )
+    return stats[0][:n_groups], stats[1][:n_groups], stats[2][:n_groups], scalar
+
+
+def row_broadcast_mask(row_scalar, mask, rows: Rows, clamp_abs=0.0):
+    lib = _lib.load()
+    require_device(row_scalar, "row_broadcast_mask")
+    mk, kind = mask_arg(mask)
+    out = torch.empty(rows.shape, device=row_scalar.device, dtype=torch.float32)
+    check(
+        lib.axon_row_broadcast_mask(ptr(f32(row_scalar)), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                                    rows.uniform_len, float(clamp_abs), ptr(out), stream_ptr()),
+        "axon_row_broadcast_mask",
+    )
+    return out
+
+
+IS_MODES = {None: 0, "token": 1, "sequence": 2}
+RS_MODES = {None: 0, "token": 1, "sequence": 2, "geometric": 3}
+
+
+def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_threshold, rs_mode, rs_lr_lo, rs_lr_hi,
+                       log_veto):
+    """One row-stats pass (when a row-level quantity is needed) + one elementwise pass.
+
+    Returns (is_weights | None, new_mask fp32, acc[8] device tensor).
+    """
+    lib = _lib.load()
+    require_device(old_lp, "sampler_correction")
+    dev = old_lp.device
+    old_lp, samp_lp = f32(old_lp), f32(samp_lp)
+    mk, kind = mask_arg(mask)
+    has_veto = log_veto is not None
+    need_row = is_mode == 2 or rs_mode >= 2 or has_veto
+    cnt = ssum = flag = None
+    if need_row:
+        cnt, ssum, flag = row_stats(old_lp, samp_lp, mk, rows, flag_mode=1 if has_veto else 0,
+                                    threshold=log_veto if has_veto else 0.0)
+    isw = torch.empty(rows.shape, device=dev, dtype=torch.float32) if is_mode else None
+    new_mask = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    acc = _zeros(8, dev)
+    check(
+        lib.axon_sampler_correction(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                                    rows.uniform_len, is_mode, float(is_threshold), rs_mode, float(rs_lr_lo),
+                                    float(rs_lr_hi), int(has_veto), float(log_veto if has_veto else 0.0), ptr(cnt),
+                                    ptr(ssum), ptr(flag), ptr(isw), ptr(new_mask), ptr(acc), stream_ptr()),
+        "axon_sampler_correction",
+    )
+    return isw, new_mask, acc
+
+
+TOKEN_REDUCE = {"sum": 0, "mean": 1, "mean-norm": 2, "mean-program": 3}
+BATCH_REDUCE = {"token-mean": 0, "step-mean": 1, "program-mean": 2}
+
+
+def _i64_dev(x, dev):
+    if x is None:
+        return None
+    t = torch.as_tensor(x)
+    return t.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
+
+
+def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows, *, token_reduce,
+                batch_reduce, ratio_lo, ratio_hi, clip_c, per_row_token_count=None, num_program_tokens=None,
+                num_program_steps=None, valid_count=None):
+    """Forward + gradient of the clipped policy loss.  Returns (acc[8], grad like log_probs).
+
+    acc[0] is the loss; acc[1:5] are the metric sums (see axon_policy_loss).
+    """
+    lib = _lib.load()
+    require_device(log_probs, "policy_loss")
+    dev = log_probs.device
+    lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
+    mk, mkind = mask_arg(mask)
+    isw = f32(is_weights) if is_weights is not None else None
+    tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
+
+    cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
+    row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
+    row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
+    prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
+    npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
+    nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+    valid = _i64_dev(valid_count, dev)
+    check(
+        lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
+                                ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
+                                stream_ptr()),
+        "axon_loss_row_scale",
+    )
+    grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    acc = _zeros(8, dev)
+    check(
+        lib.axon_policy_loss(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
+                             rows.n_slots, rows.uniform_len, ptr(row_scale), ptr(row_mean), 0.0, float(ratio_lo),
+                             float(ratio_hi), float(clip_c), ptr(grad), ptr(acc), stream_ptr()),
+        "axon_policy_loss",
+    )
+    return acc, grad
+
+
+def lmhead_forward(hidden, weight, labels, inv_temperature):
+    """Returns logprobs, entropy, lse, entropy_b (all fp32 [N])."""
+    lib = _lib.load()
+    require_device(hidden, "lmhead_forward")
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    out = torch.empty(4, max(n, 1), device=dev, dtype=torch.float32)
+    ws_bytes = lib.axon_lmhead_fwd_workspace_bytes(n, h, v)
+    if ws_bytes < 0:
+        raise _lib.AxonAmdError(f"axon_lmhead_fwd: unsupported shape tokens={n} hidden={h} vocab={v} (hidden % 32 != 0?)")
+    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    check(
+        lib.axon_lmhead_fwd(ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), n, h, v,
+                            float(inv_temperature), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws),
+                            ws_bytes, stream_ptr()),
+        "axon_lmhead_fwd",
+    )
+    return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
+
+
+def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0):
+    """Returns d_hidden [N,H], d_weight [V,H] in bf16."""
+    lib = _lib.load()
+    require_device(hidden, "lmhead_backward")
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    d_hidden = torch.empty_like(hidden)
+    d_weight = torch.empty_like(weight)
+    ws_bytes = lib.axon_lmhead_bwd_workspace_bytes(n, h, v, int(vocab_chunk))
+    if ws_bytes < 0:
+        raise _lib.AxonAmdError(f"axon_lmhead_bwd: unsupported shape/chunk tokens={n} hidden={h} vocab={v}")
+    ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    g_lp = f32(dlogprobs)  # keep the converted copies alive until the launch is enqueued
+    g_en = f32(dentropy) if dentropy is not None else None
+    check(
+        lib.axon_lmhead_bwd(ptr(g_lp), ptr(g_en), ptr(hidden),
+                            ptr(weight), ptr(labels), int(labels.dtype == torch.int64), ptr(lse), ptr(entropy_b), n,
+                            h, v, float(inv_temperature), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
+                            ws_bytes, stream_ptr()),
+        "axon_lmhead_bwd",
+    )
+    return d_hidden, d_weight
+
+
+def gemm_nt(a, b):
+    """out[n][m] = sum_k a[m][k] * b[n][k]; bf16 in, fp32 out.  Test/benchmark helper."""
+    lib = _lib.load()
+    require_device(a, "gemm_nt")
+    m, k = a.shape
+    n = b.shape[0]
+    out = torch.empty(n, m, device=a.device, dtype=torch.float32)
+    check(lib.axon_gemm_nt_bf16(ptr(a), a.stride(0), ptr(b), b.stride(0), ptr(out), m, m, n, k, stream_ptr()),
+          "axon_gemm_nt_bf16")
+    return out

@@ -1,0 +1,138 @@
+// Shared device helpers for the stage-2/3 kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/axon_amd.h"
+
+namespace axon {
+
+constexpr int kWave = 64;
+constexpr int kBlock = 256;           // threads per workgroup for streaming kernels
+constexpr int kVec = 4;               // tokens per thread per step (one 16-byte load)
+constexpr int kIter = 4;              // steps per thread
+constexpr int kChunk = kBlock * kVec * kIter;  // tokens per workgroup
+constexpr int kLdsRows = 2048;        // cu_seqlens window cached in LDS per workgroup
+
+#define AXON_CHECK_LAUNCH()                                   \
+  do {                                                        \
+    if (hipGetLastError() != hipSuccess) return AXON_ERR_LAUNCH; \
+  } while (0)
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+  return v;
+}
+
+// Sum NV values over the workgroup; the total lands in thread 0.
+template <int NV>
+__device__ __forceinline__ void block_sum(float (&v)[NV], float* lds /* [NV * 4] */) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = wave_sum(v[i]);
+  if (lane == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) lds[wave * NV + i] = v[i];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      float s = 0.f;
+      for (int w = 0; w < kBlock / kWave; ++w) s += lds[w * NV + i];
+      v[i] = s;
+    }
+  }
+}
+
+// Mask loads: four consecutive slots as floats.
+template <int KIND>
+__device__ __forceinline__ void load_mask4(const void* mask, int64_t i, float (&m)[4]) {
+  if (mask == nullptr) {
+    m[0] = m[1] = m[2] = m[3] = 1.f;
+  } else if (KIND == AXON_MASK_F32) {
+    const float4 v = *reinterpret_cast<const float4*>(static_cast<const float*>(mask) + i);
+    m[0] = v.x; m[1] = v.y; m[2] = v.z; m[3] = v.w;
+  } else {
+    const longlong2* p = reinterpret_cast<const longlong2*>(static_cast<const int64_t*>(mask) + i);
+    const longlong2 a = p[0], b = p[1];
+    m[0] = (float)a.x; m[1] = (float)a.y; m[2] = (float)b.x; m[3] = (float)b.y;
+  }
+}
+template <int KIND>
+__device__ __forceinline__ float load_mask1(const void* mask, int64_t i) {
+  if (mask == nullptr) return 1.f;
+  if (KIND == AXON_MASK_F32) return static_cast<const float*>(mask)[i];
+  return (float)static_cast<const int64_t*>(mask)[i];
+}
+
+__device__ __forceinline__ void load4(const float* p, int64_t i, float (&v)[4]) {
+  const float4 x = *reinterpret_cast<const float4*>(p + i);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+__device__ __forceinline__ void store4(float* p, int64_t i, const float (&v)[4]) {
+  *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// Row lookup.  row(pos) = number of s in [1, n_rows] with cu[s] <= pos, i.e. the
+// row whose half-open range contains pos; empty rows are skipped.  A workgroup
+// owns the contiguous slots [c0, c1); it caches the cu_seqlens entries covering
+// that range in LDS when they fit.
+struct RowFinder {
+  const int32_t* cu;   // global
+  const int32_t* win;  // LDS window or nullptr
+  int lo;              // first row overlapping the chunk
+  int hi;              // last row overlapping the chunk
+  int64_t uniform;
+
+  // count of s in (lo_excl, hi_incl] with p[s] <= pos, searching global memory
+  __device__ static int upper(const int32_t* cu, int lo, int hi, int64_t pos) {
+    // invariant: cu[lo] <= pos (or lo == 0), answer in [lo, hi]
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if ((int64_t)cu[mid] <= pos) lo = mid; else hi = mid - 1;
+    }
+    return lo;
+  }
+
+  __device__ void init(const int32_t* cu_, int64_t n_rows, int64_t uniform_len, int64_t c0,
+                       int64_t c1, int32_t* lds) {
+    cu = cu_;
+    uniform = uniform_len;
+    win = nullptr;
+    if (uniform_len > 0) return;
+    lo = upper(cu, 0, (int)n_rows, c0);
+    hi = upper(cu, lo, (int)n_rows, c1 - 1);
+    if (lo >= n_rows) lo = (int)n_rows - 1;  // slots past cu[n_rows] (caller error) stay in range
+    if (hi >= n_rows) hi = (int)n_rows - 1;
+    const int n = hi - lo + 2;
+    if (n <= kLdsRows) {
+      for (int i = threadIdx.x; i < n; i += blockDim.x) lds[i] = cu[lo + i];
+      win = lds;
+    }
+    __syncthreads();
+  }
+
+  __device__ __forceinline__ int row(int64_t pos) const {
+    if (uniform > 0) return (int)(pos / uniform);
+    if (win != nullptr) {
+      int a = 0, b = hi - lo;
+      while (a < b) {
+        const int mid = (a + b + 1) >> 1;
+        if ((int64_t)win[mid] <= pos) a = mid; else b = mid - 1;
+      }
+      return lo + a;
+    }
+    return upper(cu, lo, hi, pos);
+  }
+  // first slot of the row after `r` (to test whether a 4-vector stays in one row)
+  __device__ __forceinline__ int64_t row_end(int r) const {
+    if (uniform > 0) return (int64_t)(r + 1) * uniform;
+    if (win != nullptr) return win[r - lo + 1];
+    return cu[r + 1];
+  }
+};
+
+}  // namespace axon

@@ -1,0 +1,604 @@
+// (a) Fused LM head: per-token log-prob and entropy, and its backward, without
+// materialising the [tokens x vocab] logits.
+//
+// Forward    logits^T tile = W[vocab tile] . hidden[token tile]^T on MFMA; the
+//            epilogue folds each tile into per-token (max, sum exp, sum logit*exp)
+//            partials; a small kernel merges partials and adds the label logit.
+// Backward   per vocab chunk:
+//   B1  recompute the logits tile, form dlogit in registers, write it as bf16
+//       twice: dl[token][vocab] and dlT[vocab][token];
+//   B2  dHidden[token][h] (+)= sum_v dl[token][v]  * WT[h][v]
+//   B3  dWeight[v][h]      =  sum_t dlT[v][t]      * hiddenT[h][t]
+// WT and hiddenT are bf16 transposes made once per call, so that all four GEMMs
+// run on the same K-contiguous main loop (gemm_nt.h).
+#include "common.h"
+#include "gemm_nt.h"
+
+namespace axon {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kMaskedLogit = -1.0e30f;  // finite stand-in for "row beyond the vocabulary"
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  // round-to-nearest-even; the values here are finite
+  uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
+  a += 0x7fffu + ((a >> 16) & 1u);
+  b += 0x7fffu + ((b >> 16) & 1u);
+  return (a >> 16) | (b & 0xffff0000u);
+}
+
+// ----------------------------------------------------------------------------
+// Forward: tile epilogue -> partial statistics
+// ----------------------------------------------------------------------------
+struct FwdParams {
+  float* pm;   // [parts][n_tokens] running max, in log2 units of the scaled logit
+  float* ps;   // sum 2^(x*c - max)
+  float* pe;   // sum raw_acc * 2^(x*c - max)
+  int n_tokens, vocab;
+  float c;     // inv_temperature * log2(e)
+};
+
+template <int BK>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
+                                                                  int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) char smem[];
+  int tm, tn;
+  tile_coords(tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kTile, n0 = tn * kTile;
+  f32x16 acc[4][4];
+  gemm_mainloop<BK>(g, m0, n0, acc, smem);
+
+  const LanePos lp;
+  const bool tail = (m0 + kTile > p.vocab);
+  const int part = tm * 2 + lp.wm;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (tail) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+          if (m0 + lp.m(i, q) >= p.vocab) acc[i][j][q] = kMaskedLogit;
+    }
+    float mx = acc[0][j][0];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) mx = fmaxf(mx, acc[i][j][q]);
+    const float M = mx * p.c;
+    float s = 0.f, e = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const float x = acc[i][j][q];
+        const float w = fast_exp2(fmaf(x, p.c, -M));
+        s += w;
+        e = fmaf(w, x, e);
+      }
+    // merge the two lanes that hold the same token (lane and lane^32)
+    const float M2 = __shfl_xor(M, 32, 64);
+    const float s2 = __shfl_xor(s, 32, 64);
+    const float e2 = __shfl_xor(e, 32, 64);
+    const float Mn = fmaxf(M, M2);
+    const float f1 = fast_exp2(M - Mn), f2 = fast_exp2(M2 - Mn);
+    s = s * f1 + s2 * f2;
+    e = e * f1 + e2 * f2;
+    const int n = n0 + lp.n(j);
+    if (lp.lhi == 0 && n < p.n_tokens) {
+      const int64_t o = (int64_t)part * p.n_tokens + n;
+      p.pm[o] = Mn;
+      p.ps[o] = s;
+      p.pe[o] = e;
+    }
+  }
+}
+
+// Merge partials: lse, entropy_b, entropy.  One thread per token.
+__global__ __launch_bounds__(256) void lmhead_merge_kernel(const float* __restrict__ pm,
+                                                           const float* __restrict__ ps,
+                                                           const float* __restrict__ pe, int parts,
+                                                           int n_tokens, float inv_temp,
+                                                           float* __restrict__ lse,
+                                                           float* __restrict__ entropy_b,
+                                                           float* __restrict__ entropy) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= n_tokens) return;
+  float M = pm[n], s = ps[n], e = pe[n];
+  for (int q = 1; q < parts; ++q) {
+    const int64_t o = (int64_t)q * n_tokens + n;
+    const float M2 = pm[o], s2 = ps[o], e2 = pe[o];
+    const float Mn = fmaxf(M, M2);
+    const float f1 = fast_exp2(M - Mn), f2 = fast_exp2(M2 - Mn);
+    s = s * f1 + s2 * f2;
+    e = e * f1 + e2 * f2;
+    M = Mn;
+  }
+  const float l = (M + __log2f(s)) * kLn2;   // logsumexp of logits / T
+  const float eb = (e / s) * inv_temp;       // sum softmax * logits / T
+  lse[n] = l;
+  entropy_b[n] = eb;
+  entropy[n] = l - eb;
+}
+
+// logprob[n] = hidden[n] . W[label[n]] / T - lse[n].  One wave per token.
+template <typename LabelT>
+__global__ __launch_bounds__(256) void lmhead_label_kernel(
+    const __bf16* __restrict__ hidden, const __bf16* __restrict__ weight,
+    const LabelT* __restrict__ labels, int n_tokens, int hidden_sz, int vocab, float inv_temp,
+    const float* __restrict__ lse, float* __restrict__ logprobs) {
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= n_tokens) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t lab = (int64_t)labels[n];
+  float dot = 0.f;
+  if (lab >= 0 && lab < vocab) {
+    const uint4* h = reinterpret_cast<const uint4*>(hidden + (int64_t)n * hidden_sz);
+    const uint4* w = reinterpret_cast<const uint4*>(weight + lab * hidden_sz);
+    for (int c = lane; c < hidden_sz / 8; c += 64) {
+      const uint4 hv = h[c], wv = w[c];
+      const uint32_t hs[4] = {hv.x, hv.y, hv.z, hv.w}, ws[4] = {wv.x, wv.y, wv.z, wv.w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        dot = fmaf(__uint_as_float(hs[k] << 16), __uint_as_float(ws[k] << 16), dot);
+        dot = fmaf(__uint_as_float(hs[k] & 0xffff0000u), __uint_as_float(ws[k] & 0xffff0000u), dot);
+      }
+    }
+  }
+  dot = wave_sum(dot);
+  if (lane == 0) logprobs[n] = dot * inv_temp - lse[n];
+}
+
+// ----------------------------------------------------------------------------
+// Backward B1: recompute logits, write dlogit (bf16) in both orientations
+// ----------------------------------------------------------------------------
+struct DlogitParams {
+  const float* lse;
+  const float* entropy_b;
+  const float* dlogprobs;
+  const float* dentropy;  // may be null
+  const void* labels;
+  int labels_i64;
+  __bf16* dl;    // [n_pad][chunk_cols]   token-major
+  __bf16* dlT;   // [chunk_cols][n_pad]   vocab-major
+  int64_t ld_dl, ld_dlT;
+  int n_tokens, vocab, v_begin;  // v_begin: first vocab row of this chunk
+  float inv_temp;
+};
+
+constexpr int kStagePitch = kTile + 4;  // bf16 elements per staged row (8-byte aligned rows)
+
+template <int BK>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperands g, DlogitParams p,
+                                                                     int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) char smem[];
+  int tm, tn;
+  tile_coords(tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kTile, n0 = tn * kTile;  // m0 relative to the chunk
+  f32x16 acc[4][4];
+  gemm_mainloop<BK>(g, m0, n0, acc, smem);
+  // all waves are past their last LDS read (the main loop ends with a barrier)
+
+  const LanePos lp;
+  const float c = p.inv_temp * kLog2e;
+  uint16_t* stage = reinterpret_cast<uint16_t*>(smem);  // [256 n][kStagePitch] bf16
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int nrel = lp.n(j);
+    const int n = n0 + nrel;
+    const bool n_ok = n < p.n_tokens;
+    const int nn = n_ok ? n : 0;
+    const float g_lp = n_ok ? p.dlogprobs[nn] : 0.f;
+    const float g_en = (n_ok && p.dentropy) ? p.dentropy[nn] : 0.f;
+    const float lse2 = p.lse[nn] * kLog2e;
+    const float eb = p.entropy_b[nn];
+    // dlogit = p * (a + b * x) + onehot * g / T,  x = logit / T
+    const float ca = (-g_lp + g_en * eb) * p.inv_temp;
+    const float cb = -g_en * p.inv_temp;
+    const float gl = g_lp * p.inv_temp;
+    int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[nn]
+                               : (int64_t) static_cast<const int32_t*>(p.labels)[nn];
+    // label position relative to this lane's first row in the wave tile
+    const int64_t lab_rel = lab - (int64_t)(p.v_begin + m0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float d[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int q = 4 * r + e;
+          const int mrel = lp.m(i, q);
+          const float raw = acc[i][j][q];
+          const float pr = fast_exp2(fmaf(raw, c, -lse2));
+          const float x = raw * p.inv_temp;
+          float v = pr * fmaf(cb, x, ca);
+          if ((int64_t)mrel == lab_rel) v += gl;
+          const bool ok = n_ok && (p.v_begin + m0 + mrel < p.vocab);
+          d[e] = ok ? v : 0.f;
+        }
+        const int mq = lp.m(i, 4 * r);  // first of four consecutive m
+        uint2 w;
+        w.x = pack_bf16(d[0], d[1]);
+        w.y = pack_bf16(d[2], d[3]);
+        *reinterpret_cast<uint2*>(stage + nrel * kStagePitch + mq) = w;
+      }
+    }
+  }
+  __syncthreads();
+  // token-major copy: row n, 256 m = 32 chunks of 16 bytes... rows are 8-byte aligned in
+  // LDS, so move 8 bytes per lane: 64 lanes cover one 512-byte row.
+  {
+    const int col = (threadIdx.x & 63) * 4;
+    for (int row = threadIdx.x >> 6; row < kTile; row += 4) {
+      const uint2 v = *reinterpret_cast<const uint2*>(stage + row * kStagePitch + col);
+      *reinterpret_cast<uint2*>(p.dl + (int64_t)(n0 + row) * p.ld_dl + m0 + col) = v;
+    }
+  }
+  // vocab-major copy: 4x4 blocks transposed in registers
+  {
+    const int nq = threadIdx.x & 63;  // token quad
+    for (int mq = threadIdx.x >> 6; mq < kTile / 4; mq += 4) {
+      uint2 rws[4];
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+        rws[f] = *reinterpret_cast<const uint2*>(stage + (nq * 4 + f) * kStagePitch + mq * 4);
+      uint2 o[4];
+      o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
+      o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
+      o[1].x = (rws[0].x >> 16) | (rws[1].x & 0xffff0000u);
+      o[1].y = (rws[2].x >> 16) | (rws[3].x & 0xffff0000u);
+      o[2].x = (rws[0].y & 0xffffu) | (rws[1].y << 16);
+      o[2].y = (rws[2].y & 0xffffu) | (rws[3].y << 16);
+      o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
+      o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        *reinterpret_cast<uint2*>(p.dlT + (int64_t)(m0 + mq * 4 + e) * p.ld_dlT + n0 + nq * 4) = o[e];
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// Backward B2/B3 and the plain GEMM: store the tile as out[n][m]
+// ----------------------------------------------------------------------------
+struct StoreParams {
+  float* out_f32;     // [n][ld_f32] fp32 accumulator / output (may be null)
+  __bf16* out_bf16;   // [n][ld_bf16] (may be null)
+  int64_t ld_f32, ld_bf16;
+  int m_valid, n_valid;
+  int accumulate;     // add the previous contents of out_f32 first
+};
+
+template <int BK>
+__global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g, StoreParams p,
+                                                                  int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) char smem[];
+  int tm, tn;
+  tile_coords(tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * kTile, n0 = tn * kTile;
+  f32x16 acc[4][4];
+  gemm_mainloop<BK>(g, m0, n0, acc, smem);
+  const LanePos lp;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + lp.n(j);
+    if (n >= p.n_valid) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + lp.m(i, 4 * r);
+        if (m >= p.m_valid) continue;  // m_valid % 4 == 0: a quad is all in or all out
+        float4 v = make_float4(acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2],
+                               acc[i][j][4 * r + 3]);
+        if (p.out_f32) {
+          float4* dst = reinterpret_cast<float4*>(p.out_f32 + (int64_t)n * p.ld_f32 + m);
+          if (p.accumulate) {
+            const float4 old = *dst;
+            v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
+          }
+          *dst = v;
+        }
+        if (p.out_bf16) {
+          uint2 w;
+          w.x = pack_bf16(v.x, v.y);
+          w.y = pack_bf16(v.z, v.w);
+          *reinterpret_cast<uint2*>(p.out_bf16 + (int64_t)n * p.ld_bf16 + m) = w;
+        }
+      }
+  }
+}
+
+// out[c][r] = in[r][c] for r < rows, c < cols; zero elsewhere in the padded
+// output [cols_pad][ld_out] for r in [rows, rows_pad).  32x32 tiles through LDS.
+__global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ in,
+                                                             int64_t ld_in, int rows, int cols,
+                                                             uint16_t* __restrict__ out,
+                                                             int64_t ld_out, int rows_pad) {
+  __shared__ uint16_t t[64][66];
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int r = i >> 6, c = i & 63;
+    uint16_t v = 0;
+    if (r0 + r < rows && c0 + c < cols) v = in[(int64_t)(r0 + r) * ld_in + c0 + c];
+    t[r][c] = v;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+    const int c = i >> 6, r = i & 63;
+    if (c0 + c < cols && r0 + r < rows_pad) out[(int64_t)(c0 + c) * ld_out + r0 + r] = t[r][c];
+  }
+}
+
+}  // namespace axon
+
+using namespace axon;
+
+namespace {
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+constexpr int64_t kDefaultVocabChunk = 16384;
+constexpr int64_t kAlign = 256;
+
+template <int BK>
+constexpr int lds_bytes() { return TileLds<BK>::kBytes; }
+// B1 re-uses the stage buffers to hold the bf16 tile it writes out
+template <int BK>
+constexpr int dlogit_lds_bytes() {
+  return TileLds<BK>::kBytes > kTile * kStagePitch * 2 ? TileLds<BK>::kBytes
+                                                       : kTile * kStagePitch * 2;
+}
+
+template <typename K>
+int set_lds(K kernel, int bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess
+             ? AXON_OK
+             : AXON_ERR_LAUNCH;
+}
+
+struct FwdWs {
+  float *pm, *ps, *pe;
+  int parts;
+  int64_t bytes;
+};
+FwdWs fwd_ws(int64_t n, int64_t vocab, void* base) {
+  FwdWs w;
+  w.parts = (int)(round_up(vocab, kTile) / kTile) * 2;
+  const int64_t one = round_up((int64_t)w.parts * n * 4, kAlign);
+  char* p = static_cast<char*>(base);
+  w.pm = reinterpret_cast<float*>(p);
+  w.ps = reinterpret_cast<float*>(p + one);
+  w.pe = reinterpret_cast<float*>(p + 2 * one);
+  w.bytes = 3 * one;
+  return w;
+}
+
+struct BwdWs {
+  __bf16 *wT, *hT, *dl, *dlT;
+  float* dh_acc;
+  int64_t v_pad, n_pad, chunk, bytes;
+  int chunks;
+};
+BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
+  BwdWs w;
+  w.v_pad = round_up(vocab, kTile);
+  w.n_pad = round_up(n, kTile);
+  w.chunk = (chunk <= 0) ? kDefaultVocabChunk : chunk;
+  if (w.chunk > w.v_pad) w.chunk = w.v_pad;
+  w.chunks = (int)((vocab + w.chunk - 1) / w.chunk);
+  char* p = static_cast<char*>(base);
+  int64_t off = 0;
+  w.wT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.v_pad * 2, kAlign);
+  w.hT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.n_pad * 2, kAlign);
+  w.dl = reinterpret_cast<__bf16*>(p + off);  off += round_up(w.n_pad * w.chunk * 2, kAlign);
+  w.dlT = reinterpret_cast<__bf16*>(p + off); off += round_up(w.chunk * w.n_pad * 2, kAlign);
+  w.dh_acc = reinterpret_cast<float*>(p + off);
+  if (w.chunks > 1) off += round_up(n * h * 4, kAlign);
+  w.bytes = off;
+  return w;
+}
+
+int check_head_shape(int64_t n, int64_t h, int64_t v) {
+  if (n < 0 || h <= 0 || v <= 0) return AXON_ERR_ARG;
+  if (h % 32 != 0) return AXON_ERR_SHAPE;
+  if (n >= (1 << 30) || v >= (1 << 30) || h >= (1 << 24)) return AXON_ERR_SHAPE;
+  return AXON_OK;
+}
+
+template <int BK>
+int launch_store(const GemmOperands& g, const StoreParams& sp, hipStream_t st) {
+  const int tiles_m = (g.m_rows + kTile - 1) / kTile, tiles_n = (g.n_rows + kTile - 1) / kTile;
+  int rc = set_lds(gemm_store_kernel<BK>, lds_bytes<BK>());
+  if (rc != AXON_OK) return rc;
+  hipLaunchKernelGGL(gemm_store_kernel<BK>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
+                     lds_bytes<BK>(), st, g, sp, tiles_m, tiles_n);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+int launch_transpose(const void* in, int64_t ld_in, int rows, int cols, void* out, int64_t ld_out,
+                     int rows_pad, hipStream_t st) {
+  const dim3 grid((rows_pad + 63) / 64, (cols + 63) / 64);
+  hipLaunchKernelGGL(transpose_bf16_kernel, grid, dim3(256), 0, st,
+                     static_cast<const uint16_t*>(in), ld_in, rows, cols,
+                     static_cast<uint16_t*>(out), ld_out, rows_pad);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t v) {
+  if (check_head_shape(n, h, v) != AXON_OK) return -1;
+  return fwd_ws(n, v, nullptr).bytes + kAlign;
+}
+
+extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
+                               int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
+                               float* logprobs, float* entropy, float* lse, float* entropy_b,
+                               void* workspace, int64_t ws_bytes, void* stream) {
+  int rc = check_head_shape(n, h, v);
+  if (rc != AXON_OK) return rc;
+  if (n == 0) return AXON_OK;
+  if (!hidden || !weight || !labels || !logprobs || !entropy || !lse || !entropy_b || !workspace)
+    return AXON_ERR_ARG;
+  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight)) & 15)
+    return AXON_ERR_ARG;
+  char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
+  const FwdWs w = fwd_ws(n, v, base);
+  if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
+  const hipStream_t st = (hipStream_t)stream;
+
+  GemmOperands g;
+  g.a = static_cast<const __bf16*>(weight);  g.lda = h;  g.m_rows = (int)v;
+  g.b = static_cast<const __bf16*>(hidden);  g.ldb = h;  g.n_rows = (int)n;
+  g.k = (int)h;
+  FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e};
+  const int tiles_m = (int)((v + kTile - 1) / kTile), tiles_n = (int)((n + kTile - 1) / kTile);
+  if (h % 64 == 0) {
+    rc = set_lds(lmhead_fwd_kernel<64>, lds_bytes<64>());
+    if (rc != AXON_OK) return rc;
+    hipLaunchKernelGGL(lmhead_fwd_kernel<64>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
+                       lds_bytes<64>(), st, g, p, tiles_m, tiles_n);
+  } else {
+    rc = set_lds(lmhead_fwd_kernel<32>, lds_bytes<32>());
+    if (rc != AXON_OK) return rc;
+    hipLaunchKernelGGL(lmhead_fwd_kernel<32>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
+                       lds_bytes<32>(), st, g, p, tiles_m, tiles_n);
+  }
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.pm,
+                     w.ps, w.pe, w.parts, (int)n, inv_temp, lse, entropy_b, entropy);
+  AXON_CHECK_LAUNCH();
+  const dim3 lg((unsigned)((n + 3) / 4));
+  if (labels_i64)
+    hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
+                       static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
+                       static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp, lse,
+                       logprobs);
+  else
+    hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
+                       static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
+                       static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp, lse,
+                       logprobs);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t v,
+                                                   int64_t chunk) {
+  if (check_head_shape(n, h, v) != AXON_OK) return -1;
+  if (chunk < 0 || chunk % kTile != 0) return -1;
+  return bwd_ws(n, h, v, chunk, nullptr).bytes + kAlign;
+}
+
+extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
+                               const void* weight, const void* labels, int labels_i64,
+                               const float* lse, const float* entropy_b, int64_t n, int64_t h,
+                               int64_t v, float inv_temp, void* d_hidden, void* d_weight,
+                               int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
+  int rc = check_head_shape(n, h, v);
+  if (rc != AXON_OK) return rc;
+  if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
+  if (!d_weight || !weight) return AXON_ERR_ARG;
+  const hipStream_t st = (hipStream_t)stream;
+  if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
+  if (!dlogprobs || !hidden || !labels || !lse || !entropy_b || !d_hidden || !workspace)
+    return AXON_ERR_ARG;
+  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
+       reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_weight)) & 15)
+    return AXON_ERR_ARG;
+  char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
+  const BwdWs w = bwd_ws(n, h, v, chunk, base);
+  if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
+
+  // K-contiguous copies for the two output GEMMs
+  rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.v_pad, (int)w.v_pad, st);
+  if (rc != AXON_OK) return rc;
+  rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.n_pad, (int)w.n_pad, st);
+  if (rc != AXON_OK) return rc;
+
+  for (int ci = 0; ci < w.chunks; ++ci) {
+    const int64_t v0 = (int64_t)ci * w.chunk;
+    const int64_t vc = (v - v0 < w.chunk) ? (v - v0) : w.chunk;  // valid vocab rows in this chunk
+    // B1: dlogit for vocab rows [v0, v0 + vc)
+    {
+      GemmOperands g;
+      g.a = static_cast<const __bf16*>(weight) + v0 * h;  g.lda = h;  g.m_rows = (int)vc;
+      g.b = static_cast<const __bf16*>(hidden);            g.ldb = h;  g.n_rows = (int)n;
+      g.k = (int)h;
+      DlogitParams p;
+      p.lse = lse; p.entropy_b = entropy_b; p.dlogprobs = dlogprobs; p.dentropy = dentropy;
+      p.labels = labels; p.labels_i64 = labels_i64;
+      p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.chunk; p.ld_dlT = w.n_pad;
+      p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
+      const int tiles_m = (int)((vc + kTile - 1) / kTile), tiles_n = (int)(w.n_pad / kTile);
+      if (h % 64 == 0) {
+        rc = set_lds(lmhead_dlogit_kernel<64>, dlogit_lds_bytes<64>());
+        if (rc != AXON_OK) return rc;
+        hipLaunchKernelGGL(lmhead_dlogit_kernel<64>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
+                           dlogit_lds_bytes<64>(), st, g, p, tiles_m, tiles_n);
+      } else {
+        rc = set_lds(lmhead_dlogit_kernel<32>, dlogit_lds_bytes<32>());
+        if (rc != AXON_OK) return rc;
+        hipLaunchKernelGGL(lmhead_dlogit_kernel<32>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
+                           dlogit_lds_bytes<32>(), st, g, p, tiles_m, tiles_n);
+      }
+      AXON_CHECK_LAUNCH();
+    }
+    const int64_t vc_red = round_up(vc, 64);  // columns [vc, vc_red) of dl were written as zeros
+    // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
+    {
+      GemmOperands g;
+      g.a = w.wT + v0;  g.lda = w.v_pad;  g.m_rows = (int)h;
+      g.b = w.dl;       g.ldb = w.chunk;  g.n_rows = (int)n;
+      g.k = (int)vc_red;
+      StoreParams sp;
+      const bool last = (ci == w.chunks - 1);
+      sp.out_f32 = (w.chunks > 1) ? w.dh_acc : nullptr;  sp.ld_f32 = h;
+      sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
+      sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0);
+      rc = launch_store<64>(g, sp, st);
+      if (rc != AXON_OK) return rc;
+    }
+    // B3: dWeight[v0 + v][h] = sum_t dlT[v][t] * hT[h][t]
+    {
+      GemmOperands g;
+      g.a = w.hT;   g.lda = w.n_pad;  g.m_rows = (int)h;
+      g.b = w.dlT;  g.ldb = w.n_pad;  g.n_rows = (int)vc;
+      g.k = (int)round_up(n, 64);
+      StoreParams sp;
+      sp.out_f32 = nullptr; sp.ld_f32 = 0;
+      sp.out_bf16 = static_cast<__bf16*>(d_weight) + v0 * h;  sp.ld_bf16 = h;
+      sp.m_valid = (int)h; sp.n_valid = (int)vc; sp.accumulate = 0;
+      rc = launch_store<64>(g, sp, st);
+      if (rc != AXON_OK) return rc;
+    }
+  }
+  return AXON_OK;
+}
+
+extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, float* out,
+                                 int64_t ldo, int64_t m, int64_t n, int64_t k, void* stream) {
+  if (!a || !b || !out) return AXON_ERR_ARG;
+  if (m <= 0 || n <= 0 || k <= 0) return AXON_ERR_ARG;
+  if (k % 32 != 0 || lda % 8 != 0 || ldb % 8 != 0 || m % 4 != 0 || ldo % 4 != 0)
+    return AXON_ERR_SHAPE;
+  if (m >= (1 << 30) || n >= (1 << 30)) return AXON_ERR_SHAPE;
+  GemmOperands g;
+  g.a = static_cast<const __bf16*>(a);  g.lda = lda;  g.m_rows = (int)m;
+  g.b = static_cast<const __bf16*>(b);  g.ldb = ldb;  g.n_rows = (int)n;
+  g.k = (int)k;
+  StoreParams sp;
+  sp.out_f32 = out; sp.ld_f32 = ldo; sp.out_bf16 = nullptr; sp.ld_bf16 = 0;
+  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0;
+  if (k % 64 == 0) return launch_store<64>(g, sp, (hipStream_t)stream);
+  return launch_store<32>(g, sp, (hipStream_t)stream);
+}

@@ -1,0 +1,347 @@
+// (c) Elementwise stage-2/3 kernels: sampler correction and the clipped policy
+// loss with its gradient.  One read of every input, one write of every output;
+// scalar sums leave through one atomic per workgroup per accumulator.
+#include "common.h"
+
+namespace axon {
+
+constexpr float kSafetyBound = 20.0f;  // axon/utils/rl/sampler.py:27, loss.py:77
+
+__device__ __forceinline__ float clampf(float x, float lo, float hi) {
+  // torch.clamp semantics: NaN propagates
+  return (x != x) ? x : fminf(fmaxf(x, lo), hi);
+}
+
+template <int MK>
+__global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
+    const float* __restrict__ oldp, const float* __restrict__ samp, const void* __restrict__ mask,
+    const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
+    int is_mode, float is_thr, int rs_mode, float rs_lo, float rs_hi, int has_veto, float log_veto,
+    const float* __restrict__ row_cnt, const float* __restrict__ row_sum,
+    const int32_t* __restrict__ row_flag, float* __restrict__ isw, float* __restrict__ new_mask,
+    float* acc) {
+  __shared__ int32_t lds_cu[kLdsRows];
+  __shared__ float lds_red[6 * (kBlock / kWave)];
+  const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+  const bool need_row = (is_mode == 2) || (rs_mode >= 2) || has_veto;
+  RowFinder rf;
+  if (need_row) rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+
+  float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int it = 0; it < kIter; ++it) {
+    const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+    if (i >= c1) continue;
+    float ov[4], sv[4], mv[4], wv[4], nm[4];
+    const bool full = (i + kVec <= n_slots);
+    if (full) {
+      load4(oldp, i, ov);
+      load4(samp, i, sv);
+      load_mask4<MK>(mask, i, mv);
+    } else {
+      for (int j = 0; j < 4; ++j) {
+        const bool ok = i + j < n_slots;
+        ov[j] = ok ? oldp[i + j] : 0.f;
+        sv[j] = ok ? samp[i + j] : 0.f;
+        mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+      }
+    }
+    int r = -1;
+    int64_t rend = -1;
+    float row_w = 0.f, row_keep = 1.f, row_veto_keep = 1.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t p = i + j;
+      if (p >= n_slots) { wv[j] = 0.f; nm[j] = 0.f; continue; }
+      if (need_row && p >= rend) {
+        r = rf.row(p);
+        rend = rf.row_end(r);
+        const float rsum = row_sum ? row_sum[r] : 0.f;
+        const float rcnt = row_cnt ? row_cnt[r] : 0.f;
+        if (is_mode == 2) row_w = expf(clampf(rsum, -kSafetyBound, kSafetyBound));
+        row_keep = 1.f;
+        if (rs_mode == 2) row_keep = (rsum >= rs_lo && rsum <= rs_hi) ? 1.f : 0.f;
+        if (rs_mode == 3) {
+          const float g = rsum / (rcnt + 1e-8f);
+          row_keep = (g >= rs_lo && g <= rs_hi) ? 1.f : 0.f;
+        }
+        row_veto_keep = (has_veto && row_flag[r]) ? 0.f : 1.f;
+      }
+      const float lr = ov[j] - sv[j];
+      const float m = mv[j];
+      const bool on = (m != 0.f);
+      // importance weight
+      float w = 0.f;
+      if (is_mode == 1) w = expf(clampf(lr, -kSafetyBound, kSafetyBound)) * m;
+      if (is_mode == 2) w = row_w * m;
+      a[1] += on ? w * m : 0.f;
+      w = (w != w) ? w : fminf(w, is_thr);  // clamp(max=thr), NaN propagates
+      wv[j] = w;
+      a[5] += on ? w * m : 0.f;
+      // rejection
+      float keep = 1.f;
+      if (rs_mode == 1) keep = (lr >= rs_lo && lr <= rs_hi) ? 1.f : 0.f;
+      if (rs_mode >= 2) keep = row_keep;
+      const float veto_keep = row_veto_keep;
+      a[2] += on ? (1.f - keep) * m : 0.f;
+      const bool cat = has_veto && on && (lr < log_veto);
+      a[3] += cat ? m : 0.f;
+      a[0] += m;
+      nm[j] = m * keep * veto_keep;
+    }
+    if (full) {
+      if (isw) store4(isw, i, wv);
+      store4(new_mask, i, nm);
+    } else {
+      for (int j = 0; j < 4 && i + j < n_slots; ++j) {
+        if (isw) isw[i + j] = wv[j];
+        new_mask[i + j] = nm[j];
+      }
+    }
+  }
+  if (blockIdx.x == 0 && has_veto) {
+    for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) a[4] += row_flag[r] ? 1.f : 0.f;
+  }
+  block_sum<6>(a, lds_red);
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < 6; ++k)
+      if (a[k] != 0.f) atomicAdd(acc + k, a[k]);
+  }
+}
+
+__global__ __launch_bounds__(1024) void loss_row_scale_kernel(
+    const float* __restrict__ row_cnt, const float* __restrict__ row_sum, int64_t n_rows,
+    int64_t row_len, int token_reduce, int batch_reduce, const int64_t* __restrict__ prtc,
+    const int64_t* __restrict__ npt, const int64_t* __restrict__ nps,
+    const int64_t* __restrict__ valid, float* __restrict__ row_scale,
+    float* __restrict__ row_mean) {
+  __shared__ float red[2 * 16];
+  __shared__ float tot[2];
+  float t[2] = {0.f, 0.f};
+  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+    const float c = row_cnt[r];
+    t[0] += c;
+    t[1] += (c > 0.f) ? 1.f : 0.f;
+  }
+  t[0] = wave_sum(t[0]);
+  t[1] = wave_sum(t[1]);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { red[wave * 2] = t[0]; red[wave * 2 + 1] = t[1]; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float s0 = 0.f, s1 = 0.f;
+    for (int w = 0; w < (int)(blockDim.x >> 6); ++w) { s0 += red[w * 2]; s1 += red[w * 2 + 1]; }
+    tot[0] = s0; tot[1] = s1;
+  }
+  __syncthreads();
+  float bden;
+  if (valid != nullptr) bden = fmaxf((float)valid[0], 1.f);
+  else if (batch_reduce == 0) bden = fmaxf(tot[0], 1.f);
+  else bden = fmaxf(tot[1], 1.f);
+  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+    const float c = row_cnt[r];
+    float td = 1.f;
+    if (token_reduce == 1) td = fmaxf(prtc ? (float)prtc[r] : c, 1.f);
+    if (token_reduce == 2) td = (float)row_len;
+    if (token_reduce == 3) td = fmaxf((float)npt[r], 1.f);
+    if (batch_reduce == 2) td *= fmaxf((float)nps[r], 1.f);
+    row_scale[r] = 1.f / (td * bden);
+    if (row_mean) row_mean[r] = (row_sum ? row_sum[r] : 0.f) / fmaxf(c, 1.f);
+  }
+}
+
+// max/min with PyTorch's gradient convention: ties split the gradient evenly.
+struct ValGrad { float v, g; };
+__device__ __forceinline__ ValGrad vg_max(ValGrad a, ValGrad b) {
+  if (a.v > b.v) return a;
+  if (a.v < b.v) return b;
+  if (a.v == b.v) return ValGrad{a.v, 0.5f * (a.g + b.g)};
+  return ValGrad{a.v + b.v, 0.f};  // NaN operand: propagate
+}
+
+template <int MK, int KIND>
+__global__ __launch_bounds__(kBlock) void policy_loss_kernel(
+    const float* __restrict__ logp, const float* __restrict__ oldp, const float* __restrict__ adv,
+    const void* __restrict__ mask, const float* __restrict__ isw, const int32_t* __restrict__ cu,
+    int64_t n_rows, int64_t n_slots, int64_t uniform_len, const float* __restrict__ row_scale,
+    const float* __restrict__ row_mean, float uniform_scale, float lo, float hi,
+    float clip_c, float* __restrict__ grad, float* acc) {
+  __shared__ int32_t lds_cu[kLdsRows];
+  __shared__ float lds_red[5 * (kBlock / kWave)];
+  const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+  const bool need_row = (row_scale != nullptr) || (KIND == 1);
+  RowFinder rf;
+  if (need_row) rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+
+  float a[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int it = 0; it < kIter; ++it) {
+    const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+    if (i >= c1) continue;
+    float lv[4], ov[4], av[4], mv[4], wv[4] = {1.f, 1.f, 1.f, 1.f}, gv[4];
+    const bool full = (i + kVec <= n_slots);
+    if (full) {
+      load4(logp, i, lv);
+      load4(oldp, i, ov);
+      load4(adv, i, av);
+      load_mask4<MK>(mask, i, mv);
+      if (isw) load4(isw, i, wv);
+    } else {
+      for (int j = 0; j < 4; ++j) {
+        const bool ok = i + j < n_slots;
+        lv[j] = ok ? logp[i + j] : 0.f;
+        ov[j] = ok ? oldp[i + j] : 0.f;
+        av[j] = ok ? adv[i + j] : 0.f;
+        mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+        wv[j] = (ok && isw) ? isw[i + j] : 1.f;
+      }
+    }
+    int64_t rend = -1;
+    float scale = uniform_scale, sbar = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t p = i + j;
+      if (p >= n_slots) { gv[j] = 0.f; continue; }
+      if (need_row && p >= rend) {
+        const int r = rf.row(p);
+        rend = rf.row_end(r);
+        if (row_scale) scale = row_scale[r];
+        if (KIND == 1) sbar = row_mean[r];
+      }
+      const float A = av[j], m = mv[j];
+      const float d = lv[j] - ov[j];
+      float x;  // exponent before the +-20 clamp
+      if (KIND == 0) x = d;
+      else x = (lv[j] - lv[j]) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
+      const bool pass = (x >= -kSafetyBound && x <= kSafetyBound);  // clamp passes grad inclusively
+      const float xc = clampf(x, -kSafetyBound, kSafetyBound);
+      const float r_ = expf(xc);
+      const ValGrad p1{-A * r_, -A * r_};
+      const float rc = clampf(r_, lo, hi);
+      const bool rin = (r_ >= lo && r_ <= hi);
+      const ValGrad p2{-A * rc, rin ? -A * r_ : 0.f};
+      ValGrad c = vg_max(p1, p2);
+      a[1] += (p2.v > p1.v) ? m : 0.f;
+      a[2] += (KIND == 0 ? -xc : -d) * m;  // ppo_kl: clamped for PPO (loss.py:77-79), raw for GSPO (loss.py:173)
+      if (KIND == 0) {
+        const float pg3 = -A * clip_c;
+        a[3] += (c.v > pg3 && A < 0.f) ? m : 0.f;
+        if (A < 0.f) {  // torch.min(pg3, c1), pg3 carries no gradient
+          if (pg3 < c.v) c = ValGrad{pg3, 0.f};
+          else if (pg3 == c.v) c = ValGrad{c.v, 0.5f * c.g};
+          else if (!(pg3 > c.v)) c = ValGrad{pg3 + c.v, 0.f};
+        }
+      }
+      a[4] += m;
+      const float w = wv[j];
+      a[0] += (c.v * w) * m * scale;
+      gv[j] = (pass ? c.g : 0.f) * w * m * scale;
+    }
+    if (full) store4(grad, i, gv);
+    else
+      for (int j = 0; j < 4 && i + j < n_slots; ++j) grad[i + j] = gv[j];
+  }
+  block_sum<5>(a, lds_red);
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int k = 0; k < 5; ++k)
+      if (a[k] != 0.f) atomicAdd(acc + k, a[k]);
+  }
+}
+
+}  // namespace axon
+
+using namespace axon;
+
+static int check_rows2(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
+                       bool need_row) {
+  if (n_rows < 0 || n_slots < 0 || uniform_len < 0) return AXON_ERR_ARG;
+  if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (need_row && uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
+  if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
+  return AXON_OK;
+}
+
+extern "C" int axon_sampler_correction(
+    const float* oldp, const float* samp, const void* mask, int mask_kind, const int32_t* cu,
+    int64_t n_rows, int64_t n_slots, int64_t uniform_len, int is_mode, float is_thr, int rs_mode,
+    float rs_lo, float rs_hi, int has_veto, float log_veto, const float* row_cnt,
+    const float* row_sum, const int32_t* row_flag, float* isw, float* new_mask, float* acc,
+    void* stream) {
+  const bool need_row = (is_mode == 2) || (rs_mode >= 2) || has_veto;
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0) return AXON_OK;
+  if (!oldp || !samp || !mask || !new_mask || !acc) return AXON_ERR_ARG;
+  if (is_mode < 0 || is_mode > 2 || rs_mode < 0 || rs_mode > 3) return AXON_ERR_ARG;
+  if (is_mode != 0 && isw == nullptr) return AXON_ERR_ARG;
+  if ((is_mode == 2 || rs_mode >= 2) && (!row_sum || !row_cnt)) return AXON_ERR_ARG;
+  if (has_veto && !row_flag) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  const dim3 g((unsigned)((n_slots + kChunk - 1) / kChunk)), blk(kBlock);
+  if (mask_kind == AXON_MASK_F32)
+    hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_F32>, g, blk, 0, (hipStream_t)stream,
+                       oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
+                       rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
+                       acc);
+  else
+    hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_I64>, g, blk, 0, (hipStream_t)stream,
+                       oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
+                       rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
+                       acc);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_rows,
+                                   int64_t row_len, int token_reduce, int batch_reduce,
+                                   const int64_t* prtc, const int64_t* npt, const int64_t* nps,
+                                   const int64_t* valid, float* row_scale, float* row_mean,
+                                   void* stream) {
+  if (n_rows < 0) return AXON_ERR_ARG;
+  if (n_rows == 0) return AXON_OK;
+  if (!row_cnt || !row_scale) return AXON_ERR_ARG;
+  if (token_reduce < 0 || token_reduce > 3 || batch_reduce < 0 || batch_reduce > 2)
+    return AXON_ERR_ARG;
+  if (token_reduce == 3 && !npt) return AXON_ERR_ARG;
+  if (token_reduce == 2 && row_len <= 0) return AXON_ERR_ARG;
+  if (batch_reduce == 2 && (!nps || !valid)) return AXON_ERR_ARG;
+  hipLaunchKernelGGL(loss_row_scale_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, row_cnt,
+                     row_sum, n_rows, row_len, token_reduce, batch_reduce, prtc, npt, nps, valid,
+                     row_scale, row_mean);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, const float* adv,
+                                const void* mask, int mask_kind, const float* isw,
+                                const int32_t* cu, int64_t n_rows, int64_t n_slots,
+                                int64_t uniform_len, const float* row_scale, const float* row_mean,
+                                float uniform_scale, float ratio_lo, float ratio_hi, float clip_c,
+                                float* grad, float* acc, void* stream) {
+  const bool need_row = (row_scale != nullptr) || (kind == 1);
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0) return AXON_OK;
+  if (kind != 0 && kind != 1) return AXON_ERR_ARG;
+  if (!logp || !oldp || !adv || !mask || !grad || !acc) return AXON_ERR_ARG;
+  if (kind == 1 && !row_mean) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  const dim3 g((unsigned)((n_slots + kChunk - 1) / kChunk)), blk(kBlock);
+  const hipStream_t st = (hipStream_t)stream;
+#define AXON_LAUNCH_PL(MK, KD)                                                                   \
+  hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
+                     n_rows, n_slots, uniform_len, row_scale, row_mean, uniform_scale, ratio_lo, \
+                     ratio_hi, clip_c, grad, acc)
+  if (mask_kind == AXON_MASK_F32) {
+    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0); else AXON_LAUNCH_PL(AXON_MASK_F32, 1);
+  } else {
+    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_I64, 0); else AXON_LAUNCH_PL(AXON_MASK_I64, 1);
+  }
+#undef AXON_LAUNCH_PL
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}

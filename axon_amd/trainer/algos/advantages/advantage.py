@@ -1,0 +1,47 @@
+"""Group-normalised GRPO advantage on the HIP path.
+
+``grpo_advantage_fn`` follows axon/trainer/algos/advantages/advantage.py:78-109:
+score = sum_t token_level_rewards, per-uid mean/std (Bessel, std floored at
+sqrt(eps), then +eps again in the divide), singleton groups -> 0, broadcast over
+``response_mask``.  Three launches: ragged row sum, one-workgroup group
+statistics, masked broadcast.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from axon_amd import _ops
+from axon_amd.trainer.algos.advantages.registry import AdvantageFn, register_advantage
+from axon_amd.utils.rl.advantage import as_torch_index
+
+
+def _stage(t: torch.Tensor):
+    """Tensors produced on the driver live on the CPU; the kernels need them in HBM."""
+    if t.is_cuda:
+        return t, None
+    if not torch.cuda.is_available():
+        _ops.require_device(t, "grpo_advantage_fn")
+    return t.cuda(), t.device
+
+
+@register_advantage(AdvantageFn.GRPO)
+def grpo_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
+    rewards, home = _stage(data.batch["token_level_rewards"])
+    mask, _ = _stage(data.batch["response_mask"])
+    uid = data.non_tensor_batch["uid"]
+    eps = config.get("epsilon", 1e-6)
+    norm = config.get("norm_adv_by_std", True)
+
+    cu = data.meta_info.get("cu_seqlens", None) if data.meta_info else None
+    rows = _ops.rows_of(rewards, cu)
+    gidx = as_torch_index(uid, device=rewards.device)
+    if gidx.numel() != rows.n_rows:
+        raise ValueError(f"uid has {gidx.numel()} entries, batch has {rows.n_rows} rows")
+    n_groups = int(gidx.max().item()) + 1 if gidx.numel() else 0
+    _, scores, _ = _ops.row_stats(rewards, None, None, rows, want_cnt=False)
+    _, _, _, scalar = _ops.group_stats(scores, gidx, n_groups, eps, norm)
+    adv = _ops.row_broadcast_mask(scalar, mask, rows, clamp_abs=clamp_abs)
+    if home is not None:
+        adv = adv.to(home)
+    return adv, adv

@@ -1,0 +1,111 @@
+"""PPO / DAPO and GSPO clipped policy losses on the HIP path.
+
+Same registry names, batch keys, config keys and metric names as
+axon/trainer/algos/loss/loss.py (``ppo_loss_fn`` :47-111, ``gspo_loss_fn``
+:114-180).  DAPO's clip-higher is ``clip_ratio_low`` / ``clip_ratio_high`` of the
+PPO loss.  One fused kernel evaluates ratio, clip, dual clip, importance
+weights, mask, the two-axis aggregation of ``agg_loss`` and the gradient with
+respect to ``log_probs``; the metric sums come back in a single readback.
+
+Layouts: the reference's padded ``[B, T]`` tensors, or packed ``[N]`` tensors with
+``data.meta_info["cu_seqlens"]`` (int32 ``[S+1]``).
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+from axon_amd import _lib, _ops
+from axon_amd.trainer.algos.constants import VALID_BATCH_REDUCE, VALID_TOKEN_REDUCE
+from axon_amd.trainer.algos.loss.registry import LossFn, register_loss
+
+_KIND_PPO, _KIND_GSPO = 0, 1
+
+
+class _ClippedPolicyLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, kind, batch, rows, hp):
+        acc, grad = _ops.policy_loss(
+            kind, log_probs, batch["old_log_probs"], batch["advantages"], batch["response_mask"],
+            batch["sampler_is_weights"], rows, **hp,
+        )
+        ctx.save_for_backward(grad)
+        ctx.in_dtype = log_probs.dtype
+        ctx.acc = acc
+        ctx.mark_non_differentiable(acc)
+        return acc[0].clone(), acc
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_acc):
+        (grad,) = ctx.saved_tensors
+        return (grad * g_loss).to(ctx.in_dtype), None, None, None, None
+
+
+def _run(kind: int, data, config, default_token_reduce: str):
+    b = data.batch
+    log_probs = b["log_probs"]
+    clip = config.get("clip_ratio", 0.2)
+    lo = config.get("clip_ratio_low", None)
+    hi = config.get("clip_ratio_high", None)
+    lo = clip if lo is None else lo
+    hi = clip if hi is None else hi
+    clip_c = config.get("clip_ratio_c", 3.0)
+    if kind == _KIND_PPO:
+        assert clip_c > 1.0, f"clip_ratio_c must be > 1.0, got {clip_c}"
+    token_reduce = config.get("token_reduce", default_token_reduce)
+    batch_reduce = config.get("batch_reduce", "token-mean")
+    if token_reduce not in VALID_TOKEN_REDUCE:
+        raise ValueError(f"Invalid token_reduce: {token_reduce!r}. Choose from: {sorted(VALID_TOKEN_REDUCE)}")
+    if batch_reduce not in VALID_BATCH_REDUCE:
+        raise ValueError(f"Invalid batch_reduce: {batch_reduce!r}. Choose from: {sorted(VALID_BATCH_REDUCE)}")
+    valid = {
+        "token-mean": b.get("valid_token_count", None),
+        "step-mean": b.get("valid_batch_size", None),
+        "program-mean": b.get("valid_program_count", None),
+    }[batch_reduce]
+    npt = b.get("num_program_tokens", None)
+    nps = b.get("num_program_steps", None)
+    if token_reduce == "mean-program":
+        assert npt is not None, "num_program_tokens required for token_reduce='mean-program'"
+    if batch_reduce == "program-mean":
+        assert nps is not None, f"num_program_steps required for batch_reduce='{batch_reduce}'"
+        assert valid is not None, "valid_program_count required for batch_reduce='program-mean'"
+
+    _lib.require_device(log_probs, "policy loss")
+    rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
+    tensors = {
+        "old_log_probs": b["old_log_probs"],
+        "advantages": b["advantages"],
+        "response_mask": b["response_mask"],
+        "sampler_is_weights": b.get("sampler_is_weights", None),
+    }
+    hp = dict(
+        token_reduce=token_reduce, batch_reduce=batch_reduce,
+        # bounds evaluated in double and rounded once, as torch.clamp does with Python scalars
+        ratio_lo=1 - lo, ratio_hi=1 + hi, clip_c=clip_c,
+        per_row_token_count=b.get("per_row_token_count", None), num_program_tokens=npt, num_program_steps=nps,
+        valid_count=valid,
+    )
+    loss, acc = _ClippedPolicyLoss.apply(log_probs, kind, tensors, rows, hp)
+    sums = acc.tolist()  # the only host sync of the loss
+    denom = max(sums[4], 1.0)
+    metrics: dict[str, Any] = {
+        "pg_clipfrac": sums[1] / denom,
+        "ppo_kl": sums[2] / denom,
+        "pg_clipfrac_lower": (sums[3] / denom) if kind == _KIND_PPO else 0.0,
+    }
+    return loss, metrics
+
+
+@register_loss(LossFn.PPO)
+def ppo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """Clipped PPO surrogate with dual clip (loss.py:47-111); defaults sum / token-mean."""
+    return _run(_KIND_PPO, data, config, "sum")
+
+
+@register_loss(LossFn.GSPO)
+def gspo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """GSPO sequence-level ratio loss (loss.py:114-180); code defaults mean / token-mean (:165-166)."""
+    return _run(_KIND_GSPO, data, config, "mean")

@@ -1,0 +1,63 @@
+"""Packed-batch layout helpers around the fused LM head.
+
+Index arithmetic of axon/utils/fsdp/forward_utils.py:88-182 (``unpad_inputs``,
+``prepare_rmpad_inputs``, ``rmpad_postprocess``) and ``get_unpad_data``
+(axon/utils/torch/ops.py:339-348), restated with torch index ops (the reference
+uses flash_attn.bert_padding for the same gathers).  These are tiny gathers over
+[B, T] integers and run on whatever device the inputs live on.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+
+def get_unpad_data(attention_mask: torch.Tensor):
+    """``(indices, cu_seqlens int32 [B+1], max_seqlen)`` of the valid positions."""
+    seqlens = attention_mask.sum(dim=-1, dtype=torch.int32)
+    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    max_len = int(seqlens.max().item()) if seqlens.numel() else 0
+    cu_seqlens = F.pad(torch.cumsum(seqlens, dim=0, dtype=torch.int32), (1, 0))
+    return indices, cu_seqlens, max_len
+
+
+def unpad_input_ids(input_ids: torch.Tensor, attention_mask: torch.Tensor):
+    """[B, T] ids -> packed ``(1, N)`` ids, flat ``indices`` [N], ``cu_seqlens``."""
+    indices, cu_seqlens, _ = get_unpad_data(attention_mask)
+    packed = input_ids.flatten()[indices].unsqueeze(0)
+    return packed, indices, cu_seqlens
+
+
+def rolled_labels(packed_ids: torch.Tensor) -> torch.Tensor:
+    """Next-token labels over the whole packed stream (forward_utils.py:131).  The label of
+    a sequence's last token is the next sequence's first token; it lands where
+    ``response_mask`` is 0 after ``shift_to_token_positions``."""
+    return torch.roll(packed_ids, shifts=-1, dims=-1)
+
+
+def pad_packed(values: torch.Tensor, indices: torch.Tensor, batch: int, seqlen: int) -> torch.Tensor:
+    """Scatter packed per-token values [N] back to [B, T] (zeros elsewhere)."""
+    out = torch.zeros(batch * seqlen, device=values.device, dtype=values.dtype)
+    out[indices] = values.reshape(-1)
+    return out.view(batch, seqlen)
+
+
+def shift_to_token_positions(full: torch.Tensor) -> torch.Tensor:
+    """``full[b, t]`` predicts token t+1; return ``r`` with ``r[b, t]`` = value for token t and
+    ``r[b, 0] = 0`` (forward_utils.py:180-182)."""
+    return F.pad(full[:, :-1], (1, 0), value=0.0)
+
+
+def rmpad_postprocess(t: torch.Tensor, *, indices: torch.Tensor, batch_size: int, seqlen: int) -> torch.Tensor:
+    """Packed head output -> [B, T] aligned to token positions."""
+    return shift_to_token_positions(pad_packed(t, indices, batch_size, seqlen))
+
+
+def shift_packed(values: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor:
+    """The same re-alignment without leaving the packed layout: ``out[p] = values[p-1]`` for a
+    token that is not first in its sequence, ``0`` for a first token."""
+    out = torch.roll(values, shifts=1, dims=0)
+    starts = cu_seqlens[:-1].long()
+    out[starts[starts < values.numel()]] = 0
+    return out

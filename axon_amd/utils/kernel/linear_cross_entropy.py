@@ -1,0 +1,77 @@
+"""``linear_cross_entropy`` — fused LM-head log-prob + entropy on MI355X.
+
+Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntropy``
+/ ``linear_cross_entropy = LinearCrossEntropy.apply``), the op called from
+``forward_with_triton_backend`` (axon/models/transformers/dense_common.py:221-227):
+
+    logprobs, entropy = linear_cross_entropy(hidden, weight, labels, temperature, "none")
+
+* ``hidden`` ``[N, H]`` or ``[1, N, H]`` bf16, ``weight`` ``[V, H]`` bf16, ``labels`` int32/int64;
+* outputs are flat fp32 ``[N]`` (never reshaped back, like the reference);
+* differentiable w.r.t. ``hidden`` and ``weight``; gradients come back in the input dtype;
+* ``reduction`` "sum"/"mean" reduce the log-probs as the reference's epilogue does
+  (kernels.py:369-378); the trainer path uses "none";
+* a ``dist_process_group`` (vocab-parallel head) is refused: one GPU only.
+
+The [tokens x vocab] logits are never written to memory, forward or backward.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from axon_amd import _lib, _ops
+
+_REDUCTIONS = ("none", "sum", "mean")
+
+
+class LinearCrossEntropy(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+        assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
+        assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
+        reduction = reduction.lower()
+        if reduction not in _REDUCTIONS:
+            raise ValueError(f"Invalid reduction: {reduction}")
+        if dist_process_group is not None:
+            raise NotImplementedError("vocab-parallel LM head (dist_process_group) is not part of the one-GPU path")
+        _lib.require_device(hidden, "linear_cross_entropy")
+        assert weight.device == hidden.device and labels.device == hidden.device
+        assert hidden.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "hidden and weight must be bf16"
+        assert labels.dtype in (torch.int32, torch.int64), "labels must be int32 or int64"
+
+        shape = hidden.shape
+        hidden2 = hidden.reshape(-1, shape[-1])
+        labels1 = labels.reshape(-1)
+        assert weight.dim() == 2 and hidden2.shape[1] == weight.shape[1]
+        assert hidden2.shape[0] == labels1.shape[0]
+        assert hidden2.is_contiguous() and weight.is_contiguous() and labels1.is_contiguous()
+
+        inv_t = 1.0 / temperature
+        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t)
+        ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b)
+        ctx.shape, ctx.inv_t, ctx.reduction = shape, inv_t, reduction
+        if reduction == "sum":
+            logprobs = logprobs.sum()
+        elif reduction == "mean":
+            logprobs = logprobs.mean()
+        return logprobs, entropy
+
+    @staticmethod
+    def backward(ctx, dlogprobs, dentropy):
+        hidden2, weight, labels1, lse, entropy_b = ctx.saved_tensors
+        n = hidden2.shape[0]
+        if dlogprobs is None:
+            dlogprobs = torch.zeros(n, device=hidden2.device, dtype=torch.float32)
+        elif ctx.reduction == "sum":
+            dlogprobs = dlogprobs.expand(n)
+        elif ctx.reduction == "mean":
+            dlogprobs = (dlogprobs / n).expand(n)
+        d_hidden, d_weight = _ops.lmhead_backward(
+            dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
+            entropy_b, ctx.inv_t,
+        )
+        return d_hidden.view(ctx.shape), d_weight, None, None, None, None
+
+
+linear_cross_entropy = LinearCrossEntropy.apply

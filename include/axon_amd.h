@@ -1,0 +1,201 @@
+/*
+ * axon_amd.h — C ABI of libaxon_amd.so (gfx950 / MI355X).
+ *
+ * The reference (modelcorp/axon) is pure Python and has no FFI; its plugin
+ * points for this path are Python callables.  Every entry point below is the
+ * device-side body of one of those callables and cites the reference function
+ * it stands behind.  The Python mirror in axon_amd/ binds them with ctypes.
+ *
+ * Conventions
+ *  - plain pointers to DEVICE memory, int64 sizes, scalars by value, an opaque
+ *    hipStream_t passed as void*;
+ *  - return 0 on success, a negative AXON_ERR_* code otherwise; never throws,
+ *    never exits, never synchronises, never allocates (the one exception is
+ *    documented at the function);
+ *  - workspace is caller-provided; *_workspace_bytes() gives the size;
+ *  - all launches go to `stream`; results are valid once that stream reaches
+ *    the point after the call.
+ *  - "rows": stage-2/3 kernels address a flat array of n_slots values split
+ *    into n_rows rows by int32 offsets cu_seqlens[n_rows+1].  The reference's
+ *    padded [B,T] layout is the special case cu_seqlens = {0,T,2T,...}; pass
+ *    uniform_len=T then (cu_seqlens may be NULL), else uniform_len=0.
+ */
+#ifndef AXON_AMD_H
+#define AXON_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AXON_AMD_ABI_VERSION 1
+
+enum {
+  AXON_OK = 0,
+  AXON_ERR_ARG = -1,       /* null pointer / bad enum / bad scalar            */
+  AXON_ERR_SHAPE = -2,     /* size constraint violated (see each function)    */
+  AXON_ERR_WORKSPACE = -3, /* workspace too small or misaligned               */
+  AXON_ERR_LAUNCH = -4,    /* hipGetLastError() after a launch was not success */
+  AXON_ERR_DEVICE = -5     /* not a gfx950 device                             */
+};
+
+/* mask element types accepted by stage-2/3 kernels (response_mask is int64 in
+ * the reference's production pipeline, float in its unit tests). */
+enum { AXON_MASK_F32 = 0, AXON_MASK_I64 = 1 };
+
+int axon_amd_abi_version(void);
+const char* axon_amd_error_string(int code);
+
+/* ------------------------------------------------------------------------- *
+ * (a) LM head: log-prob + entropy without materialising [tokens x vocab]
+ * ------------------------------------------------------------------------- */
+
+/* Forward.  Replaces efficient_entropy_forward
+ * (axon/utils/kernel/kernels.py:506-695) as called by LinearCrossEntropy.forward
+ * (axon/utils/kernel/linear_cross_entropy.py:50-99) with reduction "none", and
+ * _fused_linear_for_ppo_fwd (axon/utils/torch/fused_linear.py:26-46) evaluated
+ * with fp32 accumulation.
+ *   hidden  [n_tokens, hidden] bf16 row-major, 16-byte aligned rows
+ *   weight  [vocab, hidden]    bf16 row-major
+ *   labels  [n_tokens] int32 or int64; ids outside [0,vocab) contribute logit 0
+ *   out: logprobs, entropy [n_tokens] fp32;
+ *        lse = logsumexp(logits/T), entropy_b = sum softmax*logits/T  [n_tokens]
+ *        fp32, the statistics the backward needs (the reference saves
+ *        maximum/accumulate/entropy_b, linear_cross_entropy.py:93).
+ * Constraints: hidden % 32 == 0, hidden >= 32, vocab >= 1, n_tokens >= 0. */
+int64_t axon_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab);
+int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void* labels,
+                    int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
+                    float inv_temperature, float* logprobs, float* entropy, float* lse,
+                    float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Backward.  Replaces efficient_entropy_backward
+ * (axon/utils/kernel/kernels.py:1377-1585, default _Split_Dlogits_N) and
+ * _fused_linear_for_ppo_bwd (axon/utils/torch/fused_linear.py:49-89):
+ *   dlogit = [g*(onehot - p) - gH*p*(logit/T - entropy_b)] / T, rounded to bf16,
+ *   d_hidden = dlogit @ W, d_weight = dlogit^T @ hidden, both written as bf16.
+ * dentropy may be NULL (treated as zeros).  vocab_chunk (multiple of 256, or 0
+ * for the library default) bounds the bf16 dlogit scratch to
+ * 2 * n_tokens_padded * vocab_chunk * 2 bytes. */
+int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab,
+                                        int64_t vocab_chunk);
+int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
+                    const void* weight_bf16, const void* labels, int labels_are_i64,
+                    const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
+                    int64_t vocab, float inv_temperature, void* d_hidden_bf16,
+                    void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+
+/* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
+ * (fp32 accumulate, fp32 output).  No reference counterpart: it exists so tests
+ * and the benchmark can measure the main loop in isolation.
+ * Constraints: k % 32 == 0, lda/ldb multiples of 8 elements. */
+int axon_gemm_nt_bf16(const void* a_bf16, int64_t lda, const void* b_bf16, int64_t ldb,
+                      float* out, int64_t ldo, int64_t m, int64_t n, int64_t k, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * (b) ragged segmented reductions over cu_seqlens
+ * ------------------------------------------------------------------------- */
+
+/* Per-row statistics in one pass over the tokens:
+ *   cnt[r]  = sum_t mask                      (mask NULL -> 1)
+ *   sum[r]  = sum_t (a - b) * mask            (b NULL -> 0)
+ *   flag[r] = any_t  mask != 0 && cond(a-b)   cond: flag_mode 1: (a-b) <  flag_threshold
+ *                                                   flag_mode 2: |a-b| > flag_threshold
+ *                                                   flag_mode 0: no flag (flag may be NULL)
+ * Any of cnt/sum/flag may be NULL.  Outputs must be zero-filled by the caller
+ * (axon_fill_zero).  Serves masked row sums in
+ * compute_sampler_rejection_mask (axon/utils/rl/sampler.py:70-79), the veto
+ * any() (sampler.py:418-420), GSPO's sequence mean (axon/trainer/algos/loss/loss.py:143-145),
+ * agg_loss row counts (axon/trainer/algos/loss/utils.py:236-251), GRPO's score sum
+ * (axon/trainer/algos/advantages/advantage.py:98) and the zero-advantage row test
+ * (axon/utils/rl/utils.py:35-36). */
+int axon_row_stats(const float* a, const float* b, const void* mask, int mask_kind,
+                   const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
+                   int flag_mode, float flag_threshold, float* cnt, float* sum, int32_t* flag,
+                   void* stream);
+
+/* group_mean_std (axon/utils/rl/advantage.py:106-150) + the GRPO scalar
+ * (axon/trainer/algos/advantages/advantage.py:98-107):
+ *   count/s1/s2 by group, mean, var with Bessel, std = sqrt(max(var, eps)),
+ *   count<=1 -> mean 0, std 1;
+ *   scalar[i] = (score[i]-mean[g])/(std[g]+eps) or score-mean; * (count[g] > 1).
+ * mean/std/count [n_groups] are outputs AND scratch: zero-fill them first.
+ * scalar may be NULL (plain group_mean_std).  Single workgroup; n_rows < 2^31. */
+int axon_group_stats(const float* scores, const int64_t* gidx, int64_t n_rows, int64_t n_groups,
+                     float eps, int norm_by_std, float* mean, float* std, float* count,
+                     float* scalar, void* stream);
+
+/* out[t] = row_scalar[row(t)] * mask[t]  — `scalars.unsqueeze(-1) * response_mask`
+ * (axon/trainer/algos/advantages/advantage.py:108). clamp_abs > 0 applies
+ * compute_advantage's optional clamp (advantages/__init__.py:73-74). */
+int axon_row_broadcast_mask(const float* row_scalar, const void* mask, int mask_kind,
+                            const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                            int64_t uniform_len, float clamp_abs, float* out, void* stream);
+
+/* ------------------------------------------------------------------------- *
+ * (c) elementwise kernels
+ * ------------------------------------------------------------------------- */
+
+int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 0 */
+
+/* Sampler/trainer correction, compute_sampler_correction_and_rejection_mask
+ * (axon/utils/rl/sampler.py:334-446).  lr = old - sampler.
+ *   is_mode: 0 off, 1 token, 2 sequence        (sampler.py:206-231)
+ *   rs_mode: 0 off, 1 token, 2 sequence, 3 geometric   (sampler.py:66-83)
+ *   veto: has_veto != 0, log_veto = fp32 log(threshold) computed by the caller
+ *   rs_lr_lo / rs_lr_hi: the closed log-space interval equivalent to
+ *       lower <= exp(clamp(lr,-20,20)) <= upper in fp32, computed by the caller;
+ * row_cnt,row_sum,row_flag: outputs of axon_row_stats(old, sampler, mask, flag_mode 1,
+ * log_veto); may be NULL when neither a row-level mode nor the veto is on.
+ * Outputs: is_weights [n_slots] (NULL if is_mode 0), new_mask [n_slots] fp32 =
+ * mask * rs * veto.  acc[8] (zero-filled by caller) receives sums for the
+ * metrics: [0] sum mask, [1] sum is_w(before truncation)*mask, [2] sum (1-rs)*mask,
+ * [3] sum catastrophic*mask, [4] rows vetoed, [5] sum truncated is_w * mask. */
+int axon_sampler_correction(const float* old_logp, const float* sampler_logp, const void* mask,
+                            int mask_kind, const int32_t* cu_seqlens, int64_t n_rows,
+                            int64_t n_slots, int64_t uniform_len, int is_mode, float is_threshold,
+                            int rs_mode, float rs_lr_lo, float rs_lr_hi, int has_veto,
+                            float log_veto, const float* row_cnt, const float* row_sum,
+                            const int32_t* row_flag, float* is_weights, float* new_mask,
+                            float* acc, void* stream);
+
+/* Per-row weights of agg_loss (axon/trainer/algos/loss/utils.py:120-251) folded
+ * into one multiplier per row, plus GSPO's per-row mean log-ratio:
+ *   token_reduce: 0 sum, 1 mean, 2 mean-norm, 3 mean-program
+ *   batch_reduce: 0 token-mean, 1 step-mean, 2 program-mean
+ *   row_cnt/row_sum from axon_row_stats(logp, old, mask).
+ *   per_row_token_count / num_program_tokens / num_program_steps: optional
+ *   int64 [n_rows]; valid_count: optional int64 pointer whose element [0] is
+ *   the mini-batch-wide denominator (utils.py:224-229), else computed locally.
+ * Outputs row_scale[n_rows], row_mean[n_rows] (= row_sum / max(row_cnt,1)).
+ * Single workgroup. */
+int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_rows,
+                        int64_t row_len_for_norm, int token_reduce, int batch_reduce,
+                        const int64_t* per_row_token_count, const int64_t* num_program_tokens,
+                        const int64_t* num_program_steps, const int64_t* valid_count,
+                        float* row_scale, float* row_mean, void* stream);
+
+/* Clipped policy loss, forward and gradient in one pass.
+ *   kind 0: ppo_loss_fn  (axon/trainer/algos/loss/loss.py:47-111), dual clip c
+ *   kind 1: gspo_loss_fn (axon/trainer/algos/loss/loss.py:114-180)
+ * ratio_lo / ratio_hi: the clamp bounds 1 - clip_ratio_low and 1 + clip_ratio_high,
+ * evaluated in double by the caller and rounded to fp32 (what torch.clamp does
+ * with Python scalars).  clip_c: dual-clip constant (> 1), PPO only.
+ * row_scale: per-row multiplier from axon_loss_row_scale, or NULL with
+ * uniform_scale (sum / token-mean with a known denominator).
+ * Outputs grad[n_slots] = d loss / d log_probs and acc[8] (zero-filled by
+ * caller): [0] loss, [1] sum mask*(pg2>pg1), [2] sum mask*(-(logp-old)),
+ * [3] sum mask*((c1>pg3)&(A<0)), [4] sum mask. */
+int axon_policy_loss(int kind, const float* logp, const float* old_logp, const float* adv,
+                     const void* mask, int mask_kind, const float* is_weights,
+                     const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                     int64_t uniform_len, const float* row_scale, const float* row_mean,
+                     float uniform_scale, float ratio_lo, float ratio_hi, float clip_c,
+                     float* grad, float* acc, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AXON_AMD_H */

@@ -1,0 +1,107 @@
+"""Oracle: loss aggregation and the PPO / GSPO clipped losses in plain torch (CPU, autograd).
+
+Restates axon/trainer/algos/loss/utils.py:88-251 (``masked_mean``, ``agg_loss``) and
+axon/trainer/algos/loss/loss.py:47-180 (``ppo_loss_fn``, ``gspo_loss_fn``) on plain
+tensors (no DataProto), keeping the order of operations so autograd reproduces the
+reference's gradient conventions (clamp passes gradient at the bound, maximum/min
+split ties evenly).
+"""
+
+from __future__ import annotations
+
+import torch
+
+TOKEN_REDUCE = ("sum", "mean", "mean-norm", "mean-program")
+BATCH_REDUCE = ("token-mean", "step-mean", "program-mean")
+
+
+def masked_mean(values, mask):
+    """utils.py:88-91."""
+    mask = mask.to(values.dtype)
+    return (values * mask).sum() / mask.sum().clamp_min(1.0)
+
+
+def _scalar_count(val, like):
+    """utils.py:224-229: element [0] of a count tensor, clamped to >= 1."""
+    t = torch.as_tensor(val, dtype=like.dtype)
+    if t.dim() > 0:
+        t = t[0]
+    return t.clamp(min=1)
+
+
+def agg_loss(loss_mat, loss_mask, *, token_reduce="sum", batch_reduce="token-mean", num_program_tokens=None,
+             num_program_steps=None, valid_token_count=None, valid_batch_size=None, valid_program_count=None,
+             per_row_token_count=None):
+    """utils.py:120-251: (B,T) -> (B,) by token_reduce, then -> scalar by batch_reduce."""
+    if token_reduce not in TOKEN_REDUCE:
+        raise ValueError(f"Invalid token_reduce: {token_reduce!r}")
+    if batch_reduce not in BATCH_REDUCE:
+        raise ValueError(f"Invalid batch_reduce: {batch_reduce!r}")
+    rows = (loss_mat * loss_mask).sum(-1)
+    if token_reduce == "mean":
+        d = per_row_token_count if per_row_token_count is not None else loss_mask.sum(-1)
+        rows = rows / d.clamp(min=1)
+    elif token_reduce == "mean-norm":
+        rows = rows / loss_mask.shape[-1]
+    elif token_reduce == "mean-program":
+        assert num_program_tokens is not None, "num_program_tokens required"
+        rows = rows / num_program_tokens.clamp(min=1)
+    if batch_reduce == "program-mean":
+        assert num_program_steps is not None, "num_program_steps required"
+        rows = rows / num_program_steps.clamp(min=1)
+    total = rows.sum()
+    if batch_reduce == "token-mean":
+        d = valid_token_count if valid_token_count is not None else loss_mask.sum().clamp_min(1.0)
+        return total / _scalar_count(d, total)
+    if batch_reduce == "step-mean":
+        if valid_batch_size is not None:
+            return total / _scalar_count(valid_batch_size, total)
+        return total / (loss_mask.sum(-1) > 0).float().sum().clamp(min=1)
+    assert valid_program_count is not None, "valid_program_count required for batch_reduce='program-mean'"
+    return total / _scalar_count(valid_program_count, total)
+
+
+def ppo_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0.2, clip_ratio_low=None,
+             clip_ratio_high=None, clip_ratio_c=3.0, sampler_is_weights=None, token_reduce="sum",
+             batch_reduce="token-mean", **agg_kwargs):
+    """loss.py:47-111.  Returns (loss, {pg_clipfrac, ppo_kl, pg_clipfrac_lower})."""
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    assert clip_ratio_c > 1.0, f"clip_ratio_c must be > 1.0, got {clip_ratio_c}"
+    nak = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(nak)
+    kl = masked_mean(-nak, response_mask)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - lo, 1 + hi)
+    c1 = torch.maximum(l1, l2)
+    clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
+    l3 = -advantages * clip_ratio_c
+    c2 = torch.min(l3, c1)
+    clipfrac_lower = masked_mean(torch.gt(c1, l3) * (advantages < 0).float(), response_mask)
+    per_tok = torch.where(advantages < 0, c2, c1)
+    if sampler_is_weights is not None:
+        per_tok = per_tok * sampler_is_weights
+    loss = agg_loss(per_tok, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    return loss, {"pg_clipfrac": clipfrac.item(), "ppo_kl": kl.item(), "pg_clipfrac_lower": clipfrac_lower.item()}
+
+
+def gspo_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0.2, clip_ratio_low=None,
+              clip_ratio_high=None, sampler_is_weights=None, token_reduce="mean", batch_reduce="token-mean",
+              **agg_kwargs):
+    """loss.py:114-180: sequence-level geometric-mean ratio with a stop-gradient token term."""
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    nak = log_prob - old_log_prob
+    lens = response_mask.sum(-1).clamp(min=1)
+    seq = (nak * response_mask).sum(-1) / lens
+    log_s = log_prob - log_prob.detach() + seq.detach().unsqueeze(-1)
+    s = torch.exp(torch.clamp(log_s, min=-20.0, max=20.0))
+    l1 = -advantages * s
+    l2 = -advantages * torch.clamp(s, 1 - lo, 1 + hi)
+    per_tok = torch.maximum(l1, l2)
+    if sampler_is_weights is not None:
+        per_tok = per_tok * sampler_is_weights
+    loss = agg_loss(per_tok, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
+    kl = masked_mean(-nak, response_mask)
+    return loss, {"pg_clipfrac": clipfrac.item(), "ppo_kl": kl.item(), "pg_clipfrac_lower": 0.0}

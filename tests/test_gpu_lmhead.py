@@ -1,0 +1,153 @@
+"""GPU parity: the fused LM head (forward, backward, autograd wiring) and the MFMA main loop,
+through the product API (ctypes -> libaxon_amd.so) against the CPU oracle.
+
+Tolerances (fp): logprob / entropy 1e-3 absolute against the fp32-upcast oracle; gradients
+2e-2 relative-L2 in bf16; plain GEMM 1e-5 relative-L2 against an fp32 matmul of the same
+bf16 inputs."""
+
+import math
+
+import pytest
+import torch
+
+from axon_amd import _ops, workloads as W
+from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+from axon_amd.utils.torch.fused_linear import FusedLinearForPPO
+from oracle import lmhead as OM
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def rel_l2(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (512, 256, 128), (260, 300, 96), (4, 5, 32), (1000, 77, 2880),
+                                   (768, 1024, 896)])
+def test_gemm_nt_vs_fp32_matmul(m, n, k):
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    b = torch.randn(n, k, generator=g).bfloat16()
+    out = _ops.gemm_nt(a.to(DEV), b.to(DEV))
+    ref = b.float() @ a.float().t()
+    assert out.shape == (n, m) and rel_l2(out, ref) < 1e-5
+
+
+CASES = [  # n_tokens, hidden, vocab, temperature, label dtype
+    (64, 128, 1000, 1.0, torch.int64),
+    (300, 96, 777, 0.7, torch.int32),      # hidden % 64 != 0, ragged tiles everywhere
+    (257, 256, 2049, 1.3, torch.int64),
+    (1, 32, 5, 1.0, torch.int32),
+    (513, 2880, 1500, 1.0, torch.int32),   # GPT-OSS hidden size
+]
+
+
+@pytest.mark.parametrize("n,h,v,temp,ldt", CASES)
+def test_forward_vs_oracle(n, h, v, temp, ldt):
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=n + v, label_dtype=ldt)
+    w = (w.float() * 8).bfloat16()  # peaky enough that entropy is far from ln V
+    lp, ent = linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), temp, "none")
+    ref_lp, ref_ent = OM.forward(hid, w, lab, temp)
+    assert lp.dtype == torch.float32 and lp.shape == (n,) and ent.shape == (n,)
+    assert (lp.cpu() - ref_lp).abs().max() < 1e-3
+    assert (ent.cpu() - ref_ent).abs().max() < 1e-3
+
+
+def test_forward_closed_forms_gpu():
+    n, h, v = 130, 64, 3000
+    hid = torch.randn(n, h).bfloat16()
+    lab = torch.randint(0, v, (n,))
+    lp, ent = linear_cross_entropy(hid.to(DEV), torch.zeros(v, h).bfloat16().to(DEV), lab.to(DEV), 1.0, "none")
+    assert torch.allclose(lp.cpu(), torch.full((n,), -math.log(v)), atol=1e-5)
+    assert torch.allclose(ent.cpu(), torch.full((n,), math.log(v)), atol=1e-5)
+    # extreme logits stay finite; out-of-range label contributes logit 0
+    hid2 = torch.full((4, 64), 30.0).bfloat16()
+    w2 = torch.cat([torch.full((1, 64), 2.0), torch.full((1, 64), -2.0), torch.zeros(6, 64)]).bfloat16()
+    lp2, ent2 = linear_cross_entropy(hid2.to(DEV), w2.to(DEV), torch.tensor([0, 1, 2, 99]).to(DEV), 1.0, "none")
+    assert torch.isfinite(lp2).all() and torch.isfinite(ent2).all() and abs(lp2[0].item()) < 1e-5
+    ref = OM.forward(hid2, w2, torch.tensor([0, 1, 2, 0]))[0]
+    assert lp2[1].item() == pytest.approx(ref[1].item(), abs=1e-2)
+    assert lp2[3].item() == pytest.approx(-3840.0, rel=1e-5)  # 0 - logsumexp
+
+
+def test_3d_hidden_reductions_and_errors():
+    hid, w, lab = W.lmhead_inputs(96, 64, 500, seed=3, label_dtype=torch.int64)
+    lp, ent = linear_cross_entropy(hid.view(1, 96, 64).to(DEV), w.to(DEV), lab.view(1, 96).to(DEV), 1.0, "none")
+    assert lp.shape == (96,)  # flat, like the reference
+    ref = OM.forward(hid, w, lab)[0]
+    s, _ = linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1.0, "sum")
+    mn, _ = linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1.0, "mean")
+    assert s.item() == pytest.approx(ref.sum().item(), rel=1e-5) and mn.item() == pytest.approx(ref.mean().item(), rel=1e-5)
+    with pytest.raises(AssertionError, match="temperature must be a float"):
+        linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1, "none")
+    with pytest.raises(Exception):
+        linear_cross_entropy(torch.zeros(4, 40).bfloat16().to(DEV), torch.zeros(8, 40).bfloat16().to(DEV),
+                             torch.zeros(4).long().to(DEV), 1.0, "none")  # hidden % 32 != 0
+    mod = FusedLinearForPPO()
+    lp2, ent2 = mod(hid.view(2, 48, 64).to(DEV), w.to(DEV), lab.view(2, 48).to(DEV).int(), temperature=1.0)
+    assert lp2.shape == (2, 48) and torch.allclose(lp2.flatten().cpu(), ref, atol=1e-3)
+
+
+@pytest.mark.parametrize("n,h,v,temp,ldt", CASES)
+@pytest.mark.parametrize("with_entropy", [False, True])
+def test_backward_vs_oracle(n, h, v, temp, ldt, with_entropy):
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=n + v + 1, label_dtype=ldt)
+    w = (w.float() * 8).bfloat16()
+    g = torch.Generator().manual_seed(5)
+    g_lp = torch.randn(n, generator=g) / n
+    g_en = torch.randn(n, generator=g) / n if with_entropy else None
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = linear_cross_entropy(hd, wd, lab.to(DEV), temp, "none")
+    obj = (lp * g_lp.to(DEV)).sum()
+    if with_entropy:
+        obj = obj + (ent * g_en.to(DEV)).sum()
+    obj.backward()
+    assert hd.grad.dtype == torch.bfloat16 and wd.grad.dtype == torch.bfloat16
+    ref_dh, ref_dw = OM.backward(g_lp, g_en, hid, w, lab, temp)
+    assert rel_l2(hd.grad, ref_dh) < 2e-2
+    assert rel_l2(wd.grad, ref_dw) < 2e-2
+
+
+@pytest.mark.parametrize("chunk", [256, 512, 0])
+def test_backward_vocab_chunks_agree(chunk):
+    n, h, v = 300, 128, 1000
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=8)
+    w = (w.float() * 8).bfloat16()
+    hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
+    lp, ent, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    g_lp = (torch.randn(n) / n).to(DEV)
+    g_en = (torch.randn(n) / n).to(DEV)
+    dh, dw = _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0, vocab_chunk=chunk)
+    ref_dh, ref_dw = OM.backward(g_lp.cpu(), g_en.cpu(), hid, w, lab, 1.0)
+    assert rel_l2(dh, ref_dh) < 2e-2 and rel_l2(dw, ref_dw) < 2e-2
+
+
+def test_backward_properties():
+    """dentropy absent == zeros; rows of dlogit sum to zero => identical weight rows give d_hidden = 0;
+    linearity in the upstream gradient."""
+    n, h, v = 200, 64, 600
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=12)
+    hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
+    _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    g1 = torch.randn(n, device=DEV)
+    a = _ops.lmhead_backward(g1, None, hd, wd, ld, lse, eb, 1.0)
+    b = _ops.lmhead_backward(g1, torch.zeros(n, device=DEV), hd, wd, ld, lse, eb, 1.0)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    c = _ops.lmhead_backward(2 * g1, None, hd, wd, ld, lse, eb, 1.0)
+    assert rel_l2(c[0], 2 * a[0].float()) < 1e-2 and rel_l2(c[1], 2 * a[1].float()) < 1e-2
+    same = torch.randn(1, h).expand(v, h).contiguous().bfloat16().to(DEV)
+    _, _, lse2, eb2 = _ops.lmhead_forward(hd, same, ld, 1.0)
+    dh, _ = _ops.lmhead_backward(g1, torch.randn(n, device=DEV), hd, same, ld, lse2, eb2, 1.0)
+    assert dh.float().abs().max().item() < 1e-2 * g1.abs().max().item()
+
+
+def test_config2_shape_forward():
+    """Qwen2.5-0.5B head shape (config 2): 8192 x 896 x 151936, checked on a token subset."""
+    hid, w, lab = W.lmhead_inputs(8192, 896, 151936, seed=2)
+    lp, ent = linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1.0, "none")
+    idx = torch.arange(0, 8192, 61)
+    ref_lp, ref_ent = OM.forward(hid[idx], w, lab[idx])
+    assert (lp.cpu()[idx] - ref_lp).abs().max() < 1e-3 and (ent.cpu()[idx] - ref_ent).abs().max() < 1e-3
+    assert torch.isfinite(lp).all() and torch.isfinite(ent).all()

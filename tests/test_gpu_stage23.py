@@ -1,0 +1,425 @@
+"""GPU parity: stage 2 (sampler correction) and stage 3 (GRPO advantage, PPO/GSPO loss,
+agg_loss) through the product API (ctypes -> libaxon_amd.so) against the CPU oracle.
+
+Tolerances: masks / kept-row indices bit-exact; loss 1e-4 relative; gradients and fp32
+per-token outputs 1e-5 relative-L2 (fp32 elementwise work)."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from axon_amd import _ops, workloads as W
+from axon_amd.protocol import DataProto
+from axon_amd.trainer.algos.advantages import compute_advantage
+from axon_amd.trainer.algos.loss import agg_loss, compute_loss_fn, masked_mean
+from axon_amd.utils.rl import sampler as S
+from axon_amd.utils.rl.advantage import group_mean_std
+from axon_amd.utils.rl.utils import filter_zero_advantage_samples
+from oracle import advantage as OA
+from oracle import loss as OL
+from oracle import sampler as OS
+
+pytestmark = pytest.mark.gpu
+T = torch.tensor
+DEV = "cuda"
+
+
+def rel_l2(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def pad_to_packed(x, lens):
+    return torch.cat([x[b, :l] for b, l in enumerate(lens)])
+
+
+# ---- (b) row statistics --------------------------------------------------------------------------
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.int64, torch.bool])
+def test_row_stats_ragged_vs_torch(mask_dtype):
+    g = torch.Generator().manual_seed(0)
+    lens = [1, 3, 64, 65, 255, 256, 257, 1023, 4100, 2, 5000, 7]
+    n = sum(lens)
+    cu = W.cu_from_lengths(lens)
+    a, b = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    mask = (torch.rand(n, generator=g) > 0.3).to(mask_dtype)
+    rows = _ops.rows_of(a.to(DEV), cu.to(DEV))
+    cnt, ssum, flag = _ops.row_stats(a.to(DEV), b.to(DEV), mask.to(DEV), rows, flag_mode=1, threshold=-2.5)
+    mf = mask.float()
+    for r, (s, e) in enumerate(zip(cu[:-1].tolist(), cu[1:].tolist())):
+        assert cnt[r].item() == mf[s:e].sum().item()
+        assert ssum[r].item() == pytest.approx(((a - b)[s:e] * mf[s:e]).double().sum().item(), abs=1e-3)
+        assert bool(flag[r].item()) == bool((((a - b)[s:e] < -2.5) & (mf[s:e] != 0)).any())
+
+
+def test_row_stats_empty_rows_and_uniform_layout():
+    cu = T([0, 0, 5, 5, 5, 9, 9], dtype=torch.int32)
+    x = torch.arange(9, dtype=torch.float32)
+    rows = _ops.rows_of(x.to(DEV), cu.to(DEV))
+    cnt, ssum, _ = _ops.row_stats(x.to(DEV), None, None, rows)
+    assert cnt.tolist() == [0, 5, 0, 0, 4, 0] and ssum.tolist() == [0, 10, 0, 0, 26, 0]
+    y = torch.randn(7, 333)
+    rows2 = _ops.rows_of(y.to(DEV))
+    _, s2, _ = _ops.row_stats(y.to(DEV), None, None, rows2)
+    assert torch.allclose(s2.cpu(), y.sum(-1), atol=1e-4)
+
+
+# ---- group_mean_std / GRPO / dynamic sampling (known answers through the HIP path) --------------
+def test_group_mean_std_known_answers_gpu():
+    m, s, c = group_mean_std(T([1.0, 2, 3], device=DEV), T([0, 0, 0], device=DEV))
+    assert s.item() == pytest.approx(1.0) and m.item() == pytest.approx(2.0)
+    _, s, _ = group_mean_std(T([1.0, 3, 2, 4], device=DEV), T([0, 0, 1, 1], device=DEV))
+    assert torch.allclose(s.cpu(), torch.full((2,), math.sqrt(2.0)))
+    m, s, c = group_mean_std(T([5.0], device=DEV), T([0], device=DEV))
+    assert (m.item(), s.item(), c.item()) == (0.0, 1.0, 1.0)
+    m, s, c = group_mean_std(T([10.0, 20], device=DEV), T([0, 5], device=DEV))
+    assert c.tolist() == [1, 0, 0, 0, 0, 1] and (m == 0).all()
+    m, s, _ = group_mean_std(T([5.0, 5, 5], device=DEV), T([0, 0, 0], device=DEV))
+    assert m.item() == pytest.approx(5.0) and s.item() == pytest.approx(math.sqrt(1e-6))
+
+
+def _grpo_proto(tlr, mask, uid, dev=DEV, meta=None):
+    d = DataProto.from_dict(tensors={"token_level_rewards": tlr.to(dev), "response_mask": mask.to(dev)},
+                            meta_info=meta or {})
+    d.non_tensor_batch["uid"] = uid  # per row; in the packed layout rows are sequences, tensors are per token
+    return d
+
+
+@pytest.mark.parametrize("norm", [True, False])
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.int64])
+def test_grpo_config1_vs_oracle(norm, mask_dtype):
+    d = W.c1_loss_only()
+    data = _grpo_proto(d["token_level_rewards"], d["response_mask"].to(mask_dtype), d["uid"])
+    cfg = {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6, "norm_adv_by_std": norm}}
+    out = compute_advantage(data, cfg)
+    gidx = T(np.unique(d["uid"], return_inverse=True)[1])
+    ref = OA.grpo_advantage(d["token_level_rewards"], d["response_mask"], gidx, 1e-6, norm)
+    assert out.batch["advantages"].shape == ref.shape
+    assert torch.allclose(out.batch["advantages"].cpu(), ref, rtol=1e-5, atol=1e-6)
+    assert out.batch["returns"] is out.batch["advantages"]
+    clipped = compute_advantage(data, {"advantage": "grpo", "advantage_args": {"clip_advantages": True}})
+    assert clipped.batch["advantages"].abs().max() <= 1.0
+
+
+def test_grpo_known_answers_and_cpu_staging():
+    rew = T([[0.0, 0, 2], [0, 0, 0]])
+    data = _grpo_proto(rew, torch.ones(2, 3), np.array(["a", "a"], dtype=object), dev="cpu")
+    out = compute_advantage(data, {"advantage": "grpo", "advantage_args": {"norm_adv_by_std": False}})
+    adv = out.batch["advantages"]
+    assert adv.device.type == "cpu"  # driver-side tensors come back where they lived
+    assert torch.equal(adv[0], torch.ones(3)) and torch.equal(adv[1], -torch.ones(3))
+    single = _grpo_proto(rew, torch.ones(2, 3), np.array(["a", "b"], dtype=object))
+    assert (compute_advantage(single, {"advantage": "grpo"}).batch["advantages"] == 0).all()
+
+
+def test_grpo_packed_layout():
+    d = W.packed_rl_inputs(5000, seed=9, lengths=[700, 33, 1200, 64, 2000, 1003])
+    data = _grpo_proto(d["token_level_rewards"], d["response_mask"], W.uids_for(6, 3),
+                       meta={"cu_seqlens": d["cu_seqlens"]})
+    out = compute_advantage(data, {"advantage": "grpo"}).batch["advantages"].cpu()
+    # oracle on the padded equivalent
+    tmax = max(d["lengths"])
+    pad_r, pad_m = torch.zeros(6, tmax), torch.zeros(6, tmax)
+    for b, (s, e) in enumerate(zip(d["cu_seqlens"][:-1].tolist(), d["cu_seqlens"][1:].tolist())):
+        pad_r[b, : e - s] = d["token_level_rewards"][s:e]
+        pad_m[b, : e - s] = d["response_mask"][s:e]
+    ref = OA.grpo_advantage(pad_r, pad_m, T([0, 0, 0, 1, 1, 1]))
+    assert torch.allclose(out, pad_to_packed(ref, d["lengths"]), rtol=1e-5, atol=1e-6)
+
+
+def test_filter_zero_advantage_known_answers_gpu():
+    def proto(adv, uid=None):
+        nt = {"uid": np.array(uid, dtype=object)} if uid else {}
+        return DataProto.from_dict(tensors={"advantages": adv.to(DEV), "other": torch.arange(adv.shape[0]).to(DEV)},
+                                   non_tensors=nt)
+    out = filter_zero_advantage_samples(proto(T([[1.0, 2], [0, 0], [5, 6]])))
+    assert len(out) == 2 and out.batch["other"].tolist() == [0, 2]
+    assert len(filter_zero_advantage_samples(proto(T([[0.0, 0], [0, 0]])))) == 2  # no uid: unchanged
+    out = filter_zero_advantage_samples(proto(T([[1e-7, 1e-8], [1e-5, 0], [0.0, -1.0]]), ["a", "a", "b"]))
+    assert out.batch["other"].tolist() == [2]
+    out = filter_zero_advantage_samples(proto(T([[0.0, 0], [0, 0], [0, 0]]), ["a", "b", "a"]))
+    assert out.batch["other"].tolist() == [0, 2]  # all zero: keep the first uid's group
+    with pytest.raises(AssertionError):
+        filter_zero_advantage_samples(DataProto.from_dict(tensors={"x": torch.zeros(2, 2).to(DEV)}))
+    d = W.c1_loss_only(seed=5)
+    gidx = T(np.unique(d["uid"], return_inverse=True)[1])
+    adv = OA.grpo_advantage(d["token_level_rewards"], d["response_mask"], gidx)
+    kept = filter_zero_advantage_samples(proto(adv)).batch["other"].tolist()
+    assert kept == OA.zero_advantage_keep_rows(adv)  # indices bit-exact
+
+
+# ---- agg_loss / masked_mean known answers through the HIP path --------------------------------
+from tests.test_oracle_loss import AGG_CASES  # noqa: E402  (same table the oracle is pinned with)
+
+
+@pytest.mark.parametrize("loss,mask,tr,br,kw,expect", AGG_CASES)
+def test_agg_loss_known_answers_gpu(loss, mask, tr, br, kw, expect):
+    kw = {k: (v.to(DEV) if isinstance(v, torch.Tensor) else v) for k, v in kw.items()}
+    out = agg_loss(T(loss, dtype=torch.float32, device=DEV), T(mask, dtype=torch.float32, device=DEV),
+                   token_reduce=tr, batch_reduce=br, **kw)
+    assert out.dim() == 0 and out.item() == pytest.approx(expect, rel=1e-6)
+
+
+def test_masked_mean_gpu_with_grad():
+    v = T([1.0, 2, 3], device=DEV, requires_grad=True)
+    out = masked_mean(v, T([1.0, 1, 0], device=DEV))
+    out.backward()
+    assert out.item() == pytest.approx(1.5) and torch.allclose(v.grad.cpu(), T([0.5, 0.5, 0.0]))
+    assert masked_mean(T([1.0, 2], device=DEV), T([0.0, 0], device=DEV)).item() == 0.0
+
+
+# ---- PPO / GSPO --------------------------------------------------------------------------------
+def _loss_proto(d, keys=("log_probs", "old_log_probs", "advantages", "response_mask"), extra=None, meta=None):
+    t = {k: d[k].to(DEV) for k in keys}
+    t.update({k: v.to(DEV) for k, v in (extra or {}).items()})
+    t["log_probs"] = t["log_probs"].clone().requires_grad_(True)
+    return DataProto.from_dict(tensors=t, meta_info=meta or {})
+
+
+def _check_loss(name, oracle_fn, d, cfg, extra=None, agg=None, meta=None, pad=None):
+    data = _loss_proto(d, extra=extra, meta=meta)
+    loss, metrics = compute_loss_fn(data, name, cfg)
+    loss.backward()
+    src = pad if pad is not None else d
+    lp = src["log_probs"].clone().requires_grad_(True)
+    okw = {k: v for k, v in cfg.items() if k.startswith("clip") or k.endswith("_reduce")}
+    ex = {k: v for k, v in (src.get("_extra") or extra or {}).items()}
+    ref, ref_m = oracle_fn(lp, src["old_log_probs"], src["advantages"], src["response_mask"].float(), **okw, **ex,
+                           **(agg or {}))
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4, abs=1e-9)
+    got_g = data.batch["log_probs"].grad.cpu()
+    ref_g = lp.grad if pad is None else pad_to_packed(lp.grad, d["lengths"])
+    assert rel_l2(got_g, ref_g) < 1e-5
+    for k in ("pg_clipfrac", "ppo_kl", "pg_clipfrac_lower"):
+        assert metrics[k] == pytest.approx(ref_m[k], rel=1e-4, abs=1e-7)
+    return loss
+
+
+def _c1_with_adv(seed=1, mask_dtype=torch.float32):
+    d = W.c1_loss_only(seed)
+    gidx = T(np.unique(d["uid"], return_inverse=True)[1])
+    d["advantages"] = OA.grpo_advantage(d["token_level_rewards"], d["response_mask"], gidx)
+    d["response_mask"] = d["response_mask"].to(mask_dtype)
+    return d
+
+
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.int64])
+def test_ppo_config1_vs_oracle(mask_dtype):
+    _check_loss("ppo", OL.ppo_loss, _c1_with_adv(1, mask_dtype),
+                {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"})
+
+
+@pytest.mark.parametrize("tr,br", [("sum", "token-mean"), ("mean", "step-mean"), ("sum", "step-mean"),
+                                   ("mean-norm", "step-mean"), ("mean", "token-mean")])
+@pytest.mark.parametrize("name,fn", [("ppo", OL.ppo_loss), ("gspo", OL.gspo_loss)])
+def test_losses_all_reductions_with_is_weights(name, fn, tr, br):
+    d = _c1_with_adv(2)
+    d["log_probs"] = d["old_log_probs"] + 0.3 * torch.randn(d["old_log_probs"].shape)  # exercise every clip region
+    d["advantages"] = d["advantages"] + 0.0
+    d["response_mask"][5] = 0  # a row without tokens
+    isw = torch.rand(d["old_log_probs"].shape) * 2
+    cfg = {"clip_ratio": 0.2, "clip_ratio_c": 3.0, "token_reduce": tr, "batch_reduce": br}
+    if name == "gspo":
+        cfg.pop("clip_ratio_c")
+        cfg.update(clip_ratio_low=3e-4, clip_ratio_high=4e-4)
+    _check_loss(name, fn, d, cfg, extra={"sampler_is_weights": isw})
+
+
+def test_losses_with_global_counts_and_program_modes():
+    d = _c1_with_adv(3)
+    b = d["old_log_probs"].shape[0]
+    agg = {"valid_token_count": torch.full((b,), 70000), "per_row_token_count": d["response_mask"].sum(-1).long() + 3}
+    _check_loss("ppo", OL.ppo_loss, d, {"token_reduce": "mean", "batch_reduce": "token-mean"}, extra=agg, agg={})
+    prog = {"num_program_steps": torch.randint(1, 4, (b,)), "num_program_tokens": torch.randint(500, 3000, (b,)),
+            "valid_program_count": torch.full((b,), 40)}
+    _check_loss("ppo", OL.ppo_loss, d, {"token_reduce": "mean-program", "batch_reduce": "program-mean"}, extra=prog)
+    _check_loss("gspo", OL.gspo_loss, d, {"token_reduce": "mean", "batch_reduce": "step-mean"},
+                extra={"valid_batch_size": torch.full((b,), 256)})
+
+
+def test_ppo_known_answers_gpu():
+    # reference tests/trainer/algos/loss/test_loss.py:63-87, 670-714
+    lp = T([[-1.0, -2.0, -3.0]], device=DEV)
+    data = DataProto.from_dict(tensors={"log_probs": lp.clone().requires_grad_(True), "old_log_probs": lp,
+                                        "advantages": T([[1.0, 2, 3]], device=DEV),
+                                        "response_mask": torch.ones(1, 3, device=DEV)})
+    loss, m = compute_loss_fn(data, "ppo", {"clip_ratio": 0.2})
+    assert loss.item() == pytest.approx(-2.0) and m["pg_clipfrac"] == 0.0 and m["ppo_kl"] == 0.0
+    data.batch["advantages"] = torch.zeros(1, 3, device=DEV)
+    assert compute_loss_fn(data, "ppo", {})[0].item() == 0.0
+    data.batch["advantages"] = T([[1.0, float("nan"), 3.0]], device=DEV)
+    assert math.isnan(compute_loss_fn(data, "ppo", {})[0].item())
+    data.batch["advantages"] = torch.ones(1, 3, device=DEV)
+    data.batch["log_probs"] = lp + 100.0
+    assert math.isfinite(compute_loss_fn(data, "ppo", {})[0].item())
+    loss, m = compute_loss_fn(data, "gspo", {})
+    assert math.isfinite(loss.item()) and m["pg_clipfrac_lower"] == 0.0
+
+
+def test_ppo_clip_regions_table_gpu():
+    from tests.test_oracle_loss import REGIONS, _ppo_token_scalar
+    lo, hi, c = 0.2, 0.28, 3.0
+    dlt = T([[x for x, _ in REGIONS]])
+    adv = T([[a for _, a in REGIONS]])
+    old = torch.full_like(dlt, -1.0)
+    data = DataProto.from_dict(tensors={"log_probs": (old + dlt).to(DEV).requires_grad_(True),
+                                        "old_log_probs": old.to(DEV), "advantages": adv.to(DEV),
+                                        "response_mask": torch.ones_like(dlt).to(DEV)})
+    loss, _ = compute_loss_fn(data, "ppo", {"clip_ratio_low": lo, "clip_ratio_high": hi, "clip_ratio_c": c})
+    loss.backward()
+    n = len(REGIONS)
+    for k, (x, a) in enumerate(REGIONS):
+        xs = float(T(-1.0 + x, dtype=torch.float32) - T(-1.0))  # the fp32 difference the kernel sees
+        _, g = _ppo_token_scalar(-1.0 + xs, -1.0, a, lo, hi, c)
+        assert data.batch["log_probs"].grad[0, k].item() == pytest.approx(g / n, rel=1e-5, abs=1e-9), REGIONS[k]
+
+
+def test_gspo_packed_config4_vs_oracle():
+    d = W.c4_correction(n_tokens=20000)
+    s = len(d["lengths"])
+    gidx = T(np.unique(d["uid"], return_inverse=True)[1])
+    tmax = max(d["lengths"])
+    pad = {k: torch.zeros(s, tmax) for k in ("log_probs", "old_log_probs", "response_mask", "token_level_rewards")}
+    for b, (st, en) in enumerate(zip(d["cu_seqlens"][:-1].tolist(), d["cu_seqlens"][1:].tolist())):
+        for k in pad:
+            pad[k][b, : en - st] = d[k][st:en]
+    pad["advantages"] = OA.grpo_advantage(pad["token_level_rewards"], pad["response_mask"], gidx)
+    d["advantages"] = pad_to_packed(pad["advantages"], d["lengths"])
+    cfg = {"clip_ratio_low": 3e-4, "clip_ratio_high": 4e-4, "token_reduce": "mean", "batch_reduce": "step-mean"}
+    _check_loss("gspo", OL.gspo_loss, d, cfg, meta={"cu_seqlens": d["cu_seqlens"]}, pad=pad)
+    _check_loss("ppo", OL.ppo_loss, d, {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28},
+                meta={"cu_seqlens": d["cu_seqlens"]}, pad=pad)
+
+
+# ---- stage 2: sampler correction -------------------------------------------------------------------
+def _pad_case(seed=4, b=32, t=700):
+    g = torch.Generator().manual_seed(seed)
+    old = -torch.empty(b, t).exponential_(1.0, generator=g)
+    samp = old + 0.3 * torch.randn(b, t, generator=g)
+    samp[3, 17] = old[3, 17] + 11.0
+    samp[9, 0] = old[9, 0] + 30.0
+    lens = torch.randint(1, t + 1, (b,), generator=g)
+    mask = (torch.arange(t)[None] < lens[:, None]).float()
+    mask[7] = 0
+    return old, samp, mask
+
+
+@pytest.mark.parametrize("is_l,rs_l", [("token", "token"), ("sequence", "sequence"), ("token", "geometric"),
+                                       (None, "token"), ("token", None), (None, None)])
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.int64])
+def test_sampler_correction_vs_oracle(is_l, rs_l, mask_dtype):
+    old, samp, mask = _pad_case()
+    kw = dict(sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l, sampler_rs_threshold=2.0,
+              sampler_token_veto_threshold=1e-4)
+    proto, new, m = S.compute_sampler_correction_and_rejection_mask(old.to(DEV), samp.to(DEV),
+                                                                    mask.to(mask_dtype).to(DEV), **kw)
+    w_ref, new_ref, m_ref = OS.correction(old, samp, mask, **kw)
+    if rs_l in (None, "token"):
+        assert torch.equal(new.cpu(), new_ref)  # bit-exact
+    else:  # row-level ratios depend on summation order: allow rows that sit on the threshold
+        diff_rows = (new.cpu() != new_ref).any(-1).sum().item()
+        assert diff_rows == 0
+    assert new.dtype == torch.float32
+    if is_l is None:
+        assert proto is None
+    else:
+        w = proto.batch["sampler_is_weights"]
+        assert not w.requires_grad and rel_l2(w, w_ref) < 1e-5 and (w.cpu()[mask == 0] == 0).all()
+    for k, v in m_ref.items():
+        assert m["sampler_corr/" + k] == pytest.approx(v, rel=1e-4, abs=1e-7), k
+    assert all(k.startswith("sampler_corr/") for k in m)
+
+
+def test_sampler_masks_bit_exact_at_the_thresholds():
+    """Tokens whose log-ratio sits within a few ulps of +-ln 2 and of ln(1e-4)."""
+    centres = [math.log(2.0), -math.log(2.0), math.log(1e-4)]
+    vals = []
+    for c in centres:
+        x = T(c, dtype=torch.float32)
+        up, dn = x.clone(), x.clone()
+        vals.append(x.clone())
+        for _ in range(20):
+            up = torch.nextafter(up, T(math.inf))
+            dn = torch.nextafter(dn, T(-math.inf))
+            vals += [up.clone(), dn.clone()]
+    lr = torch.stack(vals).repeat(40)  # long enough for the oracle's exp to take the vector path
+    n = lr.numel()
+    lr = lr[: n - n % 8].view(8, -1)
+    old, samp, mask = lr.clone(), torch.zeros_like(lr), torch.ones_like(lr)
+    for veto in (None, 1e-4):
+        kw = dict(sampler_rs="token", sampler_rs_threshold=2.0, sampler_token_veto_threshold=veto)
+        _, new, _ = S.compute_sampler_correction_and_rejection_mask(old.to(DEV), samp.to(DEV), mask.to(DEV), **kw)
+        _, ref, _ = OS.correction(old, samp, mask, **kw)
+        assert torch.equal(new.cpu(), ref)
+    # per-row veto flags at the boundary, one token per row
+    col = torch.stack(vals)[:, None]
+    _, new, _ = S.compute_sampler_correction_and_rejection_mask(col.to(DEV), torch.zeros_like(col).to(DEV),
+                                                                torch.ones_like(col).to(DEV),
+                                                                sampler_token_veto_threshold=1e-4)
+    _, ref, _ = OS.correction(col, torch.zeros_like(col), torch.ones_like(col), sampler_token_veto_threshold=1e-4)
+    assert torch.equal(new.cpu(), ref)
+
+
+def test_sampler_known_answers_gpu():
+    # reference tests/utils/test_rl_sampler.py:199-298
+    z, one = torch.zeros(2, 4, device=DEV), torch.ones(2, 4, device=DEV)
+    proto, new, m = S.compute_sampler_correction_and_rejection_mask(z, z, one, sampler_is="token")
+    assert proto is not None and torch.equal(new, one) and torch.equal(proto.batch["sampler_is_weights"], one)
+    assert m["sampler_corr/sampler_is_mean"] == pytest.approx(1.0)
+    proto, new, _ = S.compute_sampler_correction_and_rejection_mask(z, z, one, sampler_rs="token",
+                                                                    sampler_rs_threshold=2.0)
+    assert proto is None and torch.equal(new, one)
+    proto, new, _ = S.compute_sampler_correction_and_rejection_mask(z, z, one)
+    assert proto is None and torch.equal(new, one)
+    old = z.clone()
+    old[0, 1] = -10.0
+    _, new, m = S.compute_sampler_correction_and_rejection_mask(old, z, one, sampler_token_veto_threshold=0.01)
+    assert new[0].sum() == 0 and new[1].sum() == 4 and m["sampler_corr/sampler_is_veto_fraction"] == 0.5
+    proto, new, m = S.compute_sampler_correction_and_rejection_mask(z, z, z, sampler_is="token", sampler_rs="token")
+    assert proto is None and new is z and m == {}
+    big = T([[70.0, -70.0]], device=DEV)
+    w, _ = S.compute_sampler_correction_weights(big, torch.ones(1, 2, device=DEV), "token", 1e12)
+    assert torch.isfinite(w).all() and w[0, 0].item() == pytest.approx(math.exp(20), rel=1e-4)
+    keep, mm = S.compute_sampler_rejection_mask(torch.full((2, 4), 10.0, device=DEV), one, "token", 2.0)
+    assert keep.sum() == 0 and mm["sampler_rs_masked_fraction"] == pytest.approx(1.0)
+
+
+def test_correction_hook_in_compute_loss_fn_and_mask_side_effect():
+    d = _c1_with_adv(6)
+    samp = d["old_log_probs"] + 0.2 * torch.randn(d["old_log_probs"].shape)
+    data = _loss_proto(d, extra={"sampler_log_probs": samp})
+    args = {"sampler_is": "token", "sampler_is_threshold": 2.0, "sampler_rs": "token", "sampler_rs_threshold": 2.0,
+            "sampler_token_veto_threshold": 1e-4, "clip_ratio_low": 0.2, "clip_ratio_high": 0.28}
+    loss, metrics = compute_loss_fn(data, "ppo", args)
+    loss.backward()
+    w, new_mask, _ = OS.correction(d["old_log_probs"], samp, d["response_mask"], sampler_is="token",
+                                   sampler_rs="token", sampler_token_veto_threshold=1e-4)
+    assert torch.equal(data.batch["response_mask"].cpu(), new_mask)  # the batch's mask is overwritten
+    lp = d["log_probs"].clone().requires_grad_(True)
+    ref, _ = OL.ppo_loss(lp, d["old_log_probs"], d["advantages"], new_mask, clip_ratio_low=0.2, clip_ratio_high=0.28,
+                         sampler_is_weights=w)
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4)
+    assert rel_l2(data.batch["log_probs"].grad, lp.grad) < 1e-5
+    assert "sampler_corr/sampler_is_mean" in metrics and "pg_clipfrac" in metrics
+
+
+def test_config4_full_size_masks_bit_exact():
+    d = W.c4_correction()
+    kw = dict(sampler_is="token", sampler_is_threshold=2.0, sampler_rs="token", sampler_rs_threshold=2.0,
+              sampler_token_veto_threshold=1e-4)
+    proto, new, m = S.compute_sampler_correction_and_rejection_mask(
+        d["old_log_probs"].to(DEV), d["sampler_log_probs"].to(DEV), d["response_mask"].to(DEV),
+        cu_seqlens=d["cu_seqlens"].to(DEV), **kw)
+    s = len(d["lengths"])
+    tmax = max(d["lengths"])
+    pad = {k: torch.zeros(s, tmax) for k in ("old_log_probs", "sampler_log_probs", "response_mask")}
+    for b, (st, en) in enumerate(zip(d["cu_seqlens"][:-1].tolist(), d["cu_seqlens"][1:].tolist())):
+        for k in pad:
+            pad[k][b, : en - st] = d[k][st:en]
+    w_ref, new_ref, m_ref = OS.correction(pad["old_log_probs"], pad["sampler_log_probs"], pad["response_mask"], **kw)
+    assert torch.equal(new.cpu(), pad_to_packed(new_ref, d["lengths"]))
+    assert rel_l2(proto.batch["sampler_is_weights"], pad_to_packed(w_ref, d["lengths"])) < 1e-5
+    assert m["sampler_corr/sampler_is_veto_fraction"] == pytest.approx(m_ref["sampler_is_veto_fraction"])

@@ -1,0 +1,187 @@
+"""CPU-only checks of the host side: registries, DataProto shim, label ranking, threshold
+bisection, argument validation, and the C-ABI surface.  No kernel is launched here."""
+
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from axon_amd import _lib
+from axon_amd.protocol import DataProto
+from axon_amd.trainer.algos.advantages import AdvantageFn, compute_advantage, get_advantage_fn, register_advantage
+from axon_amd.trainer.algos.loss import LossFn, agg_loss, compute_loss_fn, get_loss_fn, register_loss
+from axon_amd.utils.registry import FunctionRegistry
+from axon_amd.utils.rl import sampler as S
+from axon_amd.utils.rl.advantage import as_torch_index, group_mean_std
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- C ABI ------------------------------------------------------------------------------------------
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "axon_amd.h")).read()
+    declared = set(re.findall(r"\b(axon_[a-z0-9_]+)\s*\(", header))
+    assert declared, "no declarations found"
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/axon_amd.h but not exported"
+    assert declared == set(_lib.SIGNATURES), "ctypes bindings and header disagree"
+    assert lib.axon_amd_abi_version() == 1
+    assert lib.axon_amd_error_string(0) == b"ok"
+    assert b"workspace" in lib.axon_amd_error_string(-3)
+
+
+def test_workspace_queries_and_argument_errors_without_gpu():
+    lib = _lib.load()
+    assert lib.axon_lmhead_fwd_workspace_bytes(32768, 4096, 151936) > 0
+    assert lib.axon_lmhead_fwd_workspace_bytes(16, 100, 50) == -1  # hidden % 32 != 0
+    assert lib.axon_lmhead_bwd_workspace_bytes(64, 128, 1000, 100) == -1  # chunk % 256 != 0
+    assert lib.axon_lmhead_bwd_workspace_bytes(64, 128, 1000, 256) > 0
+    # null pointers are rejected before any launch
+    assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None) == -1
+    assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0.8, 1.2, 3.0,
+                                None, None, None) == -1
+    assert lib.axon_fill_zero(None, 3, None) == -1
+
+
+def test_cpu_tensors_fail_loudly():
+    x = torch.zeros(2, 4)
+    with pytest.raises(_lib.AxonAmdError, match="no CPU fallback"):
+        agg_loss(x, x)
+    data = DataProto.from_dict(tensors={"log_probs": x, "old_log_probs": x, "advantages": x, "response_mask": x})
+    with pytest.raises(_lib.AxonAmdError, match="no CPU fallback"):
+        compute_loss_fn(data, "ppo", {})
+    with pytest.raises(_lib.AxonAmdError):
+        S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_is="token")
+    from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+
+    with pytest.raises(_lib.AxonAmdError):
+        linear_cross_entropy(torch.zeros(4, 32).bfloat16(), torch.zeros(8, 32).bfloat16(), torch.zeros(4).long(), 1.0,
+                             "none")
+
+
+# ---- registries (reference tests/utils/registry/test_function_registry.py:46-67) -----------------
+def test_registry_rules():
+    reg = FunctionRegistry(name="thing")
+
+    @reg.register("a")
+    def fa(data, config):
+        return 1
+
+    reg.register("a")(fa)  # same function again: fine
+    with pytest.raises(ValueError, match="already registered with different function"):
+        reg.register("a")(lambda d, c: 2)
+    with pytest.raises(ValueError, match="Unknown thing"):
+        reg.get_fn("missing")
+    assert "a" in reg and reg.keys() == ["a"] and reg.compute("a", None, None) == 1
+
+
+def test_loss_and_advantage_registered():
+    assert get_loss_fn("ppo") is get_loss_fn(LossFn.PPO)
+    assert callable(get_loss_fn("gspo")) and callable(get_advantage_fn(AdvantageFn.GRPO))
+    with pytest.raises(ValueError, match="already registered"):
+        register_loss("ppo")(lambda d, c: None)
+    with pytest.raises(ValueError, match="already registered"):
+        register_advantage("grpo")(lambda d, c: None)
+    with pytest.raises(ValueError, match="must have 'advantage'"):
+        compute_advantage(DataProto.from_dict(tensors={"x": torch.zeros(1)}), {"advantage": None})
+
+
+# ---- DataProto shim (reference tests/test_protocol.py:240-400) ------------------------------------
+def test_dataproto_shim():
+    d = DataProto.from_dict(tensors={"a": torch.arange(6).view(3, 2), "b": torch.ones(3)},
+                            non_tensors={"uid": ["x", "y", "x"]}, meta_info={"k": 1})
+    assert len(d) == 3 and d.non_tensor_batch["uid"].dtype == object
+    assert "a" in d.batch and d.batch.get("zz", None) is None
+    sub = d.select_idxs([0, 2])
+    assert len(sub) == 2 and sub.non_tensor_batch["uid"].tolist() == ["x", "x"]
+    assert d.select(batch_keys=["a"]).batch.keys() == {"a"}
+    d.union(DataProto.from_dict(tensors={"c": torch.zeros(3)}))
+    assert "c" in d.batch
+    with pytest.raises(AssertionError, match="Conflicting"):
+        d.union(DataProto.from_dict(tensors={"b": torch.zeros(3)}))
+    with pytest.raises(AssertionError, match="Batch size mismatch"):
+        DataProto.from_dict(tensors={"a": torch.zeros(3), "b": torch.zeros(4)})
+    with pytest.raises(RuntimeError, match="batch dimension mismatch"):
+        d.batch["bad"] = torch.zeros(5)
+
+
+# ---- as_torch_index (reference tests/utils/test_rl_advantage.py:53-102,402-450) --------------------
+def test_as_torch_index():
+    idx = as_torch_index(np.array(["u1", "u2", "u1", "u3"], dtype=object), device="cpu")
+    assert idx[0] == idx[2] and len({int(i) for i in idx}) == 3 and idx.dtype == torch.long
+    assert as_torch_index(torch.tensor([True, False, True]), device="cpu").tolist() == [1, 0, 1]
+    assert as_torch_index(torch.tensor([0.0, 1.0, 2.0]), device="cpu").tolist() == [0, 1, 2]
+    assert as_torch_index(torch.tensor([0.0, 1.0, 2.0]).bfloat16(), device="cpu").tolist() == [0, 1, 2]
+    frac = as_torch_index(torch.tensor([0.5, 1.5, 0.5]), device="cpu")
+    assert frac[0] == frac[2] != frac[1]
+    assert as_torch_index(torch.tensor([5, 5, 10, 10]), device="cpu").tolist() == [5, 5, 10, 10]
+    assert as_torch_index([3, -1, 3], device="cpu").tolist() == [3, -1, 3]
+    mixed = as_torch_index(np.array([None, "a", None, 1], dtype=object), device="cpu")
+    assert mixed[0] == mixed[2] and mixed.numel() == 4
+
+
+def test_group_mean_std_host_checks():
+    with pytest.raises(ValueError, match="mismatch"):
+        group_mean_std(torch.zeros(2), torch.zeros(1, dtype=torch.long))
+    assert all(t.numel() == 0 for t in group_mean_std(torch.empty(0), torch.empty(0, dtype=torch.long)))
+
+
+# ---- sampler argument validation (reference tests/utils/test_rl_sampler.py:41-49,153-156,272-287) --
+def test_sampler_validation_messages():
+    x = torch.zeros(2, 3)
+    with pytest.raises(ValueError, match="Invalid sampler_rs"):
+        S.compute_sampler_rejection_mask(x, x, "bogus", 2.0)
+    with pytest.raises(ValueError, match="must be provided"):
+        S.compute_sampler_rejection_mask(x, x, "token", None)
+    with pytest.raises(ValueError, match="must be positive"):
+        S.compute_sampler_correction_weights(x, x, "token", 0.0)
+    with pytest.raises(ValueError, match="Invalid sampler_is"):
+        S.compute_sampler_correction_weights(x, x, "geometric", 2.0)
+    with pytest.raises(ValueError, match="must be positive"):
+        S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_token_veto_threshold=-0.1)
+    with pytest.raises(ValueError, match="does not match"):
+        S.compute_sampler_correction_and_rejection_mask(x, torch.zeros(2, 4), x)
+    with pytest.raises(ValueError, match="must be explicitly provided"):
+        S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_rs="token", sampler_rs_threshold=None)
+
+
+def test_log_interval_agrees_with_torch_exp_bitwise():
+    """lo <= x <= hi  <=>  lower <= exp(clamp(x)) <= upper for every fp32 x near the ends."""
+    for lower, upper in [(0.5, 2.0), (1 / 3.0, 3.0), (0.9, 1.1), (1e-3, 5.0)]:
+        lo, hi = S.log_interval_for_ratio_bounds(lower, upper)
+        for centre in (lo, hi):
+            xs = torch.tensor([centre], dtype=torch.float32)
+            near = [xs]
+            up, dn = xs.clone(), xs.clone()
+            for _ in range(40):
+                up = torch.nextafter(up, torch.tensor(math.inf))
+                dn = torch.nextafter(dn, torch.tensor(-math.inf))
+                near += [up.clone(), dn.clone()]
+            x = torch.cat(near).repeat(8)
+            w = torch.exp(torch.clamp(x, -20.0, 20.0))
+            ref = (w >= lower) & (w <= upper)
+            got = (x >= lo) & (x <= hi)
+            assert torch.equal(ref, got), (lower, upper)
+    assert S.log_interval_for_ratio_bounds(1e-12, 1e12) == (-math.inf, math.inf)  # beyond the +-20 clamp
+    assert S._log32(1e-4) == float(torch.log(torch.tensor(1e-4)))
+
+
+def test_loss_config_validation_before_any_launch():
+    x = torch.zeros(1, 3)
+    data = DataProto.from_dict(tensors={"log_probs": x, "old_log_probs": x, "advantages": x, "response_mask": x})
+    for c in (0.5, 1.0):
+        with pytest.raises(AssertionError, match="clip_ratio_c must be > 1.0"):
+            compute_loss_fn(data, "ppo", {"clip_ratio_c": c})
+    with pytest.raises(ValueError, match="Invalid token_reduce"):
+        agg_loss(x, x, token_reduce="nope")
+    with pytest.raises(ValueError, match="Invalid batch_reduce"):
+        agg_loss(x, x, batch_reduce="nope")
+    with pytest.raises(AssertionError, match="valid_program_count required"):
+        agg_loss(x, x, token_reduce="mean", batch_reduce="program-mean", num_program_steps=torch.ones(1))
+    with pytest.raises(ValueError, match="Unknown policy loss"):
+        compute_loss_fn(data, "nonexistent", {})

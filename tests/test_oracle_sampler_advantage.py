@@ -1,0 +1,196 @@
+"""Pins oracle.sampler, oracle.advantage and oracle.layout against the known answers held by
+the reference's tests (tests/utils/test_rl_sampler.py, tests/utils/test_rl_advantage.py,
+tests/trainer/algos/advantages/test_advantages.py, tests/utils/test_rl_utils.py,
+tests/utils/torch/test_ops.py — numbers restated as data) and per-token scalar loops."""
+
+import math
+
+import pytest
+import torch
+
+from oracle import advantage as A
+from oracle import layout as L
+from oracle import sampler as S
+
+T = torch.tensor
+
+
+# ---- rejection sampling, reference test_rl_sampler.py:41-113 ----------------------------------------
+def test_rs_token_known_answers():
+    mask = torch.ones(2, 4)
+    assert torch.equal(S.rejection_mask(torch.zeros(2, 4), mask, "token", 2.0) * mask, mask)
+    assert (S.rejection_mask(torch.full((2, 4), 10.0), mask, "token", 2.0) * mask).sum() == 0
+    assert (S.rejection_mask(torch.full((2, 4), -5.0), mask, "token", 2.0) * mask).sum() == 0
+    _, new, m = S.correction(torch.full((2, 4), 10.0), torch.zeros(2, 4), mask, sampler_rs="token",
+                             sampler_rs_threshold=2.0)
+    assert m["sampler_rs_masked_fraction"] == pytest.approx(1.0)
+
+
+def test_rs_sequence_rejects_whole_row():
+    lr = T([[10.0] * 4, [0.0] * 4])
+    keep = S.rejection_mask(lr, torch.ones(2, 4), "sequence", 2.0)
+    assert keep[0].sum() == 0 and keep[1].sum() == 4
+
+
+def test_rs_errors():
+    with pytest.raises(ValueError, match="Invalid sampler_rs"):
+        S.rejection_mask(torch.zeros(1, 2), torch.ones(1, 2), "bogus", 2.0)
+    with pytest.raises(ValueError, match="must be provided"):
+        S.rejection_mask(torch.zeros(1, 2), torch.ones(1, 2), "token", None)
+
+
+# ---- importance weights, reference test_rl_sampler.py:119-186 -------------------------------------
+def test_is_known_answers():
+    torch.manual_seed(0)
+    lr = torch.randn(3, 5)
+    mask = (torch.rand(3, 5) > 0.3).float()
+    w, _ = S.is_weights(lr, mask, "token", 2.0)
+    assert (w <= 2.0).all() and (w >= 0).all() and not w.requires_grad
+    assert (w[mask == 0] == 0).all()
+    ws, _ = S.is_weights(lr, torch.ones(3, 5), "sequence", 1e9)
+    assert torch.allclose(ws, ws[:, :1].expand_as(ws))
+    w0, raw0 = S.is_weights(torch.zeros(2, 3), torch.ones(2, 3), "token", 2.0)
+    assert torch.equal(w0, torch.ones(2, 3)) and S.masked_mean(raw0, torch.ones(2, 3)).item() == pytest.approx(1.0)
+    wbig, _ = S.is_weights(T([[70.0, -70.0]]), torch.ones(1, 2), "token", 1e12)
+    assert torch.isfinite(wbig).all() and wbig[0, 0].item() == pytest.approx(math.exp(20), rel=1e-4)
+    with pytest.raises(ValueError, match="must be positive"):
+        S.is_weights(lr, mask, "token", 0.0)
+
+
+# ---- unified interface, reference test_rl_sampler.py:199-310 -------------------------------------
+def test_unified_known_answers():
+    old = torch.zeros(2, 4)
+    samp = torch.zeros(2, 4)
+    mask = torch.ones(2, 4)
+    w, new, m = S.correction(old, samp, mask, sampler_is="token")
+    assert w is not None and torch.equal(new, mask)
+    w, new, m = S.correction(old, samp, mask, sampler_rs="token", sampler_rs_threshold=2.0)
+    assert w is None
+    w, new, m = S.correction(old, samp, mask)
+    assert w is None and torch.equal(new, mask)
+    # veto: threshold 0.01, one token at log-ratio -10 vetoes row 0 (fraction 0.5)
+    old2 = old.clone()
+    old2[0, 1] = -10.0
+    _, new, m = S.correction(old2, samp, mask, sampler_token_veto_threshold=0.01)
+    assert new[0].sum() == 0 and new[1].sum() == 4
+    assert m["sampler_is_veto_fraction"] == pytest.approx(0.5)
+    with pytest.raises(ValueError, match="must be positive"):
+        S.correction(old, samp, mask, sampler_token_veto_threshold=-1.0)
+    zero = torch.zeros(2, 4)
+    w, new, m = S.correction(old, samp, zero, sampler_is="token", sampler_rs="token")
+    assert w is None and new is zero and m == {}
+
+
+def test_correction_matches_scalar_loop():
+    torch.manual_seed(3)
+    B, Tn = 5, 9
+    old = -torch.rand(B, Tn) * 3
+    samp = old + torch.randn(B, Tn) * 0.5
+    samp[2, 3] = old[2, 3] + 12.0  # catastrophic token
+    mask = (torch.rand(B, Tn) > 0.25).float()
+    mask[4] = 0
+    for is_l, rs_l in [("token", "token"), ("sequence", "sequence"), ("token", "geometric")]:
+        w, new, _ = S.correction(old, samp, mask, sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l,
+                                 sampler_rs_threshold=2.0, sampler_token_veto_threshold=1e-4)
+        for b in range(B):
+            lrs = [(old[b, t] - samp[b, t]).item() for t in range(Tn)]
+            ms = [mask[b, t].item() for t in range(Tn)]
+            ssum = sum(l * m for l, m in zip(lrs, ms))
+            smean = ssum / (sum(ms) + 1e-8)
+            veto = any(l < math.log(1e-4) and m for l, m in zip(lrs, ms))
+            for t in range(Tn):
+                src = {"token": lrs[t], "sequence": ssum, "geometric": smean}
+                ew = min(math.exp(max(-20, min(20, src[is_l]))) * ms[t], 2.0)
+                assert w[b, t].item() == pytest.approx(ew, rel=2e-6, abs=1e-7)
+                ratio = math.exp(max(-20, min(20, src[rs_l])))
+                if abs(ratio - 2.0) > 1e-5 and abs(ratio - 0.5) > 1e-5:  # away from the fp32 boundary
+                    keep = 0.5 <= ratio <= 2.0
+                    assert new[b, t].item() == ms[t] * keep * (not veto)
+
+
+# ---- group_mean_std, reference test_rl_advantage.py:110-220 --------------------------------------
+def test_group_mean_std_known_answers():
+    m, s, c = A.group_mean_std(T([1.0, 2, 3]), T([0, 0, 0]))
+    assert s.item() == pytest.approx(1.0) and m.item() == pytest.approx(2.0)
+    _, s, _ = A.group_mean_std(T([1.0, 3, 2, 4]), T([0, 0, 1, 1]))
+    assert torch.allclose(s, torch.full((2,), math.sqrt(2.0)))
+    m, s, c = A.group_mean_std(T([5.0]), T([0]))
+    assert (m.item(), s.item(), c.item()) == (0.0, 1.0, 1.0)
+    m, s, c = A.group_mean_std(T([10.0, 1, 2, 3]), T([0, 1, 1, 1]))
+    assert torch.allclose(m, T([0.0, 2.0])) and torch.equal(c, T([1.0, 3.0]))
+    assert all(x.numel() == 0 for x in A.group_mean_std(torch.empty(0), torch.empty(0, dtype=torch.long)))
+    with pytest.raises(ValueError, match="mismatch"):
+        A.group_mean_std(T([1.0, 2]), T([0]))
+    m, s, c = A.group_mean_std(T([10.0, 20]), T([0, 5]))
+    assert c.tolist() == [1, 0, 0, 0, 0, 1] and (m == 0).all()
+    m, s, _ = A.group_mean_std(T([5.0, 5, 5]), T([0, 0, 0]))
+    assert m.item() == pytest.approx(5.0) and s.item() == pytest.approx(math.sqrt(1e-6))
+    x = T([1.0, 3, 5, 7])
+    _, s, _ = A.group_mean_std(x, T([0, 0, 0, 0]))
+    assert s.item() == pytest.approx(torch.std(x).item())
+
+
+def test_group_mean_std_matches_torch_std_per_group():
+    torch.manual_seed(1)
+    x = torch.randn(40)
+    g = torch.randint(0, 6, (40,))
+    m, s, c = A.group_mean_std(x, g)
+    for k in range(6):
+        sel = x[g == k]
+        if sel.numel() > 1:
+            assert m[k].item() == pytest.approx(sel.mean().item(), abs=1e-6)
+            assert s[k].item() == pytest.approx(max(sel.std().item(), 1e-3), rel=1e-4)
+
+
+# ---- GRPO, reference test_advantages.py:70-155,715-755,961-1022 ---------------------------------
+def test_grpo_known_answers():
+    rew = T([[0.0, 0, 2], [0, 0, 0]])
+    mask = torch.ones(2, 3)
+    adv = A.grpo_advantage(rew, mask, T([0, 0]), norm_adv_by_std=False)
+    assert torch.equal(adv[0], torch.ones(3)) and torch.equal(adv[1], -torch.ones(3))
+    assert (A.grpo_advantage(rew, mask, T([0, 1])) == 0).all()  # singleton groups
+    mask2 = T([[1.0, 0, 1], [1, 1, 1]])
+    assert A.grpo_advantage(rew, mask2, T([0, 0]))[0, 1].item() == 0.0
+    same = T([[0.0, 1], [0, 1], [1, 0]])
+    assert A.grpo_advantage(same, torch.ones(3, 2), T([0, 0, 0])).abs().max() < 1e-5
+    assert (A.grpo_advantage(torch.zeros(4, 2), torch.ones(4, 2), T([0, 0, 1, 1])) == 0).all()
+    # sizes 1/2/3: singleton zero, signs follow score - mean
+    rew3 = T([[5.0], [1.0], [3.0], [1.0], [2.0], [6.0]])
+    adv3 = A.grpo_advantage(rew3, torch.ones(6, 1), T([0, 1, 1, 2, 2, 2])).squeeze(1)
+    assert adv3[0] == 0 and adv3[1] < 0 < adv3[2] and adv3[3] < 0 and adv3[5] > 0
+
+
+def test_grpo_std_floor_and_double_eps():
+    """std = sqrt(max(var, eps)) and the divide adds eps again (advantage.py:102)."""
+    rew = T([[1.0], [0.0], [1.0], [0.0]])
+    adv = A.grpo_advantage(rew, torch.ones(4, 1), T([0, 0, 0, 0]), eps=1e-6)
+    std = torch.std(T([1.0, 0, 1, 0])).item()
+    assert adv[0, 0].item() == pytest.approx(0.5 / (std + 1e-6), rel=1e-6)
+
+
+# ---- dynamic sampling, reference test_rl_utils.py:38-104 ------------------------------------------
+def test_zero_advantage_filter_known_answers():
+    assert A.zero_advantage_keep_rows(T([[1.0, 2], [0, 0], [5, 6]])) == [0, 2]
+    assert A.zero_advantage_keep_rows(T([[1e-7, 1e-8]])) == []
+    assert A.zero_advantage_keep_rows(T([[1e-5, 0.0]])) == []  # exactly eps is not > eps
+    assert A.zero_advantage_keep_rows(T([[-1.0, 0.0]])) == [0]
+    assert A.zero_advantage_keep_rows(T([[0.0, 0.0, 0.3]])) == [0]
+
+
+# ---- layout, reference test_ops.py:513-561,723-729 -------------------------------------------------
+def test_unpad_known_answers():
+    idx, cu, mx = L.unpad_data(T([[1, 1, 1, 0, 0], [1, 1, 0, 0, 0]]))
+    assert cu.tolist() == [0, 3, 5] and cu.dtype == torch.int32 and mx == 3
+    assert idx.tolist() == [0, 1, 2, 5, 6]
+    _, cu, _ = L.unpad_data(T([[1] * 5, [1, 0, 0, 0, 0], [1, 1, 1, 0, 0]]))
+    assert cu.tolist() == [0, 5, 6, 9]
+    _, cu, mx = L.unpad_data(torch.zeros(2, 4, dtype=torch.long))
+    assert cu.tolist() == [0, 0, 0] and mx == 0
+
+
+def test_shift_contract():
+    """result[b,t] = head output at position t-1; result[b,0] = 0 (forward_utils.py:164-171)."""
+    am = T([[1, 1, 1, 0], [1, 1, 0, 0]])
+    idx, _, _ = L.unpad_data(am)
+    out = L.head_outputs_to_token_positions(T([10.0, 11, 12, 20, 21]), idx, 2, 4)
+    assert out.tolist() == [[0, 10, 11, 12], [0, 20, 21, 0]]
