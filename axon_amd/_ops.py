@@ -195,8 +195,37 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     return acc, grad
 
 
-def lmhead_forward(hidden, weight, labels, inv_temperature):
-    """Returns logprobs, entropy, lse, entropy_b (all fp32 [N])."""
+# When set to a dict (benchmarks only), the LM-head autograd function routes through the
+# timed entry points and accumulates per-phase HIP-event times here.
+TIMING: dict | None = None
+# vocab chunk of the LM-head backward used when the caller passes 0 (0 = library default)
+DEFAULT_VOCAB_CHUNK = 0
+
+
+def set_timing(timing: dict | None) -> None:
+    global TIMING
+    TIMING = timing
+
+
+def _phase_arrays():
+    import ctypes
+
+    return (ctypes.c_float * 4)(), (ctypes.c_int32 * 4)()
+
+
+def _add_phases(timing: dict, prefix: str, names, ms, launches):
+    for i, name in enumerate(names):
+        key = f"{prefix}/{name}"
+        t = timing.setdefault(key, {"ms": 0.0, "launches": 0})
+        t["ms"] += float(ms[i])
+        t["launches"] += int(launches[i])
+
+
+def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None = None):
+    """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]).
+
+    With ``timing`` (a dict) the timed entry point is used: it synchronises and adds
+    per-phase HIP-event milliseconds and launch counts under ``fwd/...`` keys."""
     lib = _lib.load()
     require_device(hidden, "lmhead_forward")
     n, h = hidden.shape
@@ -207,17 +236,22 @@ def lmhead_forward(hidden, weight, labels, inv_temperature):
     if ws_bytes < 0:
         raise _lib.AxonAmdError(f"axon_lmhead_fwd: unsupported shape tokens={n} hidden={h} vocab={v} (hidden % 32 != 0?)")
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
-    check(
-        lib.axon_lmhead_fwd(ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), n, h, v,
-                            float(inv_temperature), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws),
-                            ws_bytes, stream_ptr()),
-        "axon_lmhead_fwd",
-    )
+    args = (ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), n, h, v,
+            float(inv_temperature), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws), ws_bytes,
+            stream_ptr())
+    if timing is None:
+        check(lib.axon_lmhead_fwd(*args), "axon_lmhead_fwd")
+    else:
+        ms, cnt = _phase_arrays()
+        check(lib.axon_lmhead_fwd_timed(*args, ms, cnt), "axon_lmhead_fwd_timed")
+        _add_phases(timing, "fwd", ("logits_stats", "merge", "label"), ms, cnt)
     return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
 
 
-def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0):
-    """Returns d_hidden [N,H], d_weight [V,H] in bf16."""
+def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
+                    timing: dict | None = None):
+    """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``)."""
+    vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
     lib = _lib.load()
     require_device(hidden, "lmhead_backward")
     n, h = hidden.shape
@@ -231,13 +265,15 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
     g_lp = f32(dlogprobs)  # keep the converted copies alive until the launch is enqueued
     g_en = f32(dentropy) if dentropy is not None else None
-    check(
-        lib.axon_lmhead_bwd(ptr(g_lp), ptr(g_en), ptr(hidden),
-                            ptr(weight), ptr(labels), int(labels.dtype == torch.int64), ptr(lse), ptr(entropy_b), n,
-                            h, v, float(inv_temperature), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
-                            ws_bytes, stream_ptr()),
-        "axon_lmhead_bwd",
-    )
+    args = (ptr(g_lp), ptr(g_en), ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), ptr(lse),
+            ptr(entropy_b), n, h, v, float(inv_temperature), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
+            ws_bytes, stream_ptr())
+    if timing is None:
+        check(lib.axon_lmhead_bwd(*args), "axon_lmhead_bwd")
+    else:
+        ms, cnt = _phase_arrays()
+        check(lib.axon_lmhead_bwd_timed(*args, ms, cnt), "axon_lmhead_bwd_timed")
+        _add_phases(timing, "bwd", ("transpose", "dlogit", "dhidden", "dweight"), ms, cnt)
     return d_hidden, d_weight
 
 

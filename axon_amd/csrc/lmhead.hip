@@ -18,7 +18,6 @@ namespace axon {
 
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-constexpr float kMaskedLogit = -1.0e30f;  // finite stand-in for "row beyond the vocabulary"
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -36,10 +35,68 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 struct FwdParams {
   float* pm;   // [parts][n_tokens] running max, in log2 units of the scaled logit
   float* ps;   // sum 2^(x*c - max)
-  float* pe;   // sum raw_acc * 2^(x*c - max)
+  float* pe;   // sum (x*c - max) * 2^(x*c - max)
   int n_tokens, vocab;
   float c;     // inv_temperature * log2(e)
 };
+
+// Fold one 256x256 logits tile into per-token partials.  TAIL: the tile reaches past
+// the vocabulary; rows beyond it are excluded by predicate (their accumulators hold
+// finite values computed from a clamped weight row).
+constexpr float kEmptyMax = -3.0e38f;  // running max of a partial that saw no vocabulary row
+
+// Partial statistics of a set of scaled logits y = logit * c (log2 units):
+//   M = reference (the set's max), s = sum 2^(y-M), e = sum 2^(y-M) * (y-M).
+// Merge (M2,s2,e2) into (M,s,e) under the common reference Mn >= M, M2.
+__device__ __forceinline__ void merge_stats(float M, float& s, float& e, float M2, float s2,
+                                            float e2, float Mn) {
+  const float d1 = M - Mn, d2 = M2 - Mn;
+  const float f1 = fast_exp2(d1), f2 = fast_exp2(d2);
+  e = f1 * fmaf(s, d1, e) + f2 * fmaf(s2, d2, e2);
+  s = s * f1 + s2 * f2;
+}
+
+template <bool TAIL>
+__device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParams& p,
+                                             const LanePos& lp, int tm, int m0, int n0) {
+  const int part = tm * 2 + lp.wm;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const bool ok = !TAIL || (m0 + lp.m(i, q) < p.vocab);
+        mx = ok ? fmaxf(mx, acc[i][j][q]) : mx;
+      }
+    const float M = (TAIL && mx == -INFINITY) ? kEmptyMax : mx * p.c;
+    float s = 0.f, e = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) {
+        const bool ok = !TAIL || (m0 + lp.m(i, q) < p.vocab);
+        const float t = fmaf(acc[i][j][q], p.c, -M);  // scaled logit relative to the max, <= 0
+        const float w = ok ? fast_exp2(t) : 0.f;
+        s += w;
+        e = fmaf(w, t, e);
+      }
+    // merge the two lanes that hold the same token (lane and lane^32)
+    const float M2 = __shfl_xor(M, 32, 64);
+    const float s2 = __shfl_xor(s, 32, 64);
+    const float e2 = __shfl_xor(e, 32, 64);
+    const float Mn = fmaxf(M, M2);
+    merge_stats(M, s, e, M2, s2, e2, Mn);
+    const int n = n0 + lp.n(j);
+    if (lp.lhi == 0 && n < p.n_tokens) {
+      const int64_t o = (int64_t)part * p.n_tokens + n;
+      p.pm[o] = Mn;
+      p.ps[o] = s;
+      p.pe[o] = e;
+    }
+  }
+}
 
 template <int BK>
 __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
@@ -52,49 +109,10 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g
   gemm_mainloop<BK>(g, m0, n0, acc, smem);
 
   const LanePos lp;
-  const bool tail = (m0 + kTile > p.vocab);
-  const int part = tm * 2 + lp.wm;
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    if (tail) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int q = 0; q < 16; ++q)
-          if (m0 + lp.m(i, q) >= p.vocab) acc[i][j][q] = kMaskedLogit;
-    }
-    float mx = acc[0][j][0];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int q = 0; q < 16; ++q) mx = fmaxf(mx, acc[i][j][q]);
-    const float M = mx * p.c;
-    float s = 0.f, e = 0.f;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const float x = acc[i][j][q];
-        const float w = fast_exp2(fmaf(x, p.c, -M));
-        s += w;
-        e = fmaf(w, x, e);
-      }
-    // merge the two lanes that hold the same token (lane and lane^32)
-    const float M2 = __shfl_xor(M, 32, 64);
-    const float s2 = __shfl_xor(s, 32, 64);
-    const float e2 = __shfl_xor(e, 32, 64);
-    const float Mn = fmaxf(M, M2);
-    const float f1 = fast_exp2(M - Mn), f2 = fast_exp2(M2 - Mn);
-    s = s * f1 + s2 * f2;
-    e = e * f1 + e2 * f2;
-    const int n = n0 + lp.n(j);
-    if (lp.lhi == 0 && n < p.n_tokens) {
-      const int64_t o = (int64_t)part * p.n_tokens + n;
-      p.pm[o] = Mn;
-      p.ps[o] = s;
-      p.pe[o] = e;
-    }
-  }
+  if (m0 + kTile > p.vocab)
+    fwd_epilogue<true>(acc, p, lp, tm, m0, n0);
+  else
+    fwd_epilogue<false>(acc, p, lp, tm, m0, n0);
 }
 
 // Merge partials: lse, entropy_b, entropy.  One thread per token.
@@ -104,7 +122,9 @@ __global__ __launch_bounds__(256) void lmhead_merge_kernel(const float* __restri
                                                            int n_tokens, float inv_temp,
                                                            float* __restrict__ lse,
                                                            float* __restrict__ entropy_b,
-                                                           float* __restrict__ entropy) {
+                                                           float* __restrict__ entropy,
+                                                           float* __restrict__ fin_max,
+                                                           float* __restrict__ fin_log2s) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= n_tokens) return;
   float M = pm[n], s = ps[n], e = pe[n];
@@ -112,16 +132,18 @@ __global__ __launch_bounds__(256) void lmhead_merge_kernel(const float* __restri
     const int64_t o = (int64_t)q * n_tokens + n;
     const float M2 = pm[o], s2 = ps[o], e2 = pe[o];
     const float Mn = fmaxf(M, M2);
-    const float f1 = fast_exp2(M - Mn), f2 = fast_exp2(M2 - Mn);
-    s = s * f1 + s2 * f2;
-    e = e * f1 + e2 * f2;
+    merge_stats(M, s, e, M2, s2, e2, Mn);
     M = Mn;
   }
-  const float l = (M + __log2f(s)) * kLn2;   // logsumexp of logits / T
-  const float eb = (e / s) * inv_temp;       // sum softmax * logits / T
-  lse[n] = l;
-  entropy_b[n] = eb;
-  entropy[n] = l - eb;
+  // log2 units: logsumexp = M + L, sum softmax*logit = M + e/s; differences are taken
+  // before adding M so that large logits do not cancel
+  const float L = __log2f(s);
+  const float d = e / s;
+  lse[n] = (M + L) * kLn2;
+  entropy_b[n] = (M + d) * kLn2;
+  entropy[n] = (L - d) * kLn2;
+  fin_max[n] = M;
+  fin_log2s[n] = L;
 }
 
 // logprob[n] = hidden[n] . W[label[n]] / T - lse[n].  One wave per token.
@@ -129,7 +151,8 @@ template <typename LabelT>
 __global__ __launch_bounds__(256) void lmhead_label_kernel(
     const __bf16* __restrict__ hidden, const __bf16* __restrict__ weight,
     const LabelT* __restrict__ labels, int n_tokens, int hidden_sz, int vocab, float inv_temp,
-    const float* __restrict__ lse, float* __restrict__ logprobs) {
+    const float* __restrict__ fin_max, const float* __restrict__ fin_log2s,
+    float* __restrict__ logprobs) {
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= n_tokens) return;
   const int lane = threadIdx.x & 63;
@@ -149,7 +172,8 @@ __global__ __launch_bounds__(256) void lmhead_label_kernel(
     }
   }
   dot = wave_sum(dot);
-  if (lane == 0) logprobs[n] = dot * inv_temp - lse[n];
+  // (logit*c - M) is formed in one rounding, then log2(sum) is subtracted: no cancellation
+  if (lane == 0) logprobs[n] = (fmaf(dot, inv_temp * kLog2e, -fin_max[n]) - fin_log2s[n]) * kLn2;
 }
 
 // ----------------------------------------------------------------------------
@@ -363,6 +387,7 @@ int set_lds(K kernel, int bytes) {
 
 struct FwdWs {
   float *pm, *ps, *pe;
+  float *fin_max, *fin_log2s;  // [n] merged max and log2(sum), for the label kernel
   int parts;
   int64_t bytes;
 };
@@ -374,7 +399,10 @@ FwdWs fwd_ws(int64_t n, int64_t vocab, void* base) {
   w.pm = reinterpret_cast<float*>(p);
   w.ps = reinterpret_cast<float*>(p + one);
   w.pe = reinterpret_cast<float*>(p + 2 * one);
-  w.bytes = 3 * one;
+  const int64_t fin = round_up(n * 4, kAlign);
+  w.fin_max = reinterpret_cast<float*>(p + 3 * one);
+  w.fin_log2s = reinterpret_cast<float*>(p + 3 * one + fin);
+  w.bytes = 3 * one + 2 * fin;
   return w;
 }
 
@@ -402,6 +430,51 @@ BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
   w.bytes = off;
   return w;
 }
+
+// Optional per-phase timing with HIP events on the launch stream (used by the
+// *_timed entry points only).  A null timer costs nothing.
+struct PhaseTimer {
+  static constexpr int kMaxSpans = 256;
+  hipStream_t st;
+  hipEvent_t ev[kMaxSpans][2];
+  int phase[kMaxSpans];
+  int n = 0;
+  bool open = false;
+  explicit PhaseTimer(hipStream_t s) : st(s) {}
+  void begin(int ph) {
+    if (n >= kMaxSpans) return;
+    if (hipEventCreate(&ev[n][0]) != hipSuccess || hipEventCreate(&ev[n][1]) != hipSuccess) return;
+    phase[n] = ph;
+    hipEventRecord(ev[n][0], st);
+    open = true;
+  }
+  void end() {
+    if (!open) return;
+    hipEventRecord(ev[n][1], st);
+    ++n;
+    open = false;
+  }
+  // synchronises the stream; adds elapsed ms and launch counts per phase
+  void collect(float* ms, int32_t* launches, int n_phases) {
+    hipStreamSynchronize(st);
+    for (int i = 0; i < n; ++i) {
+      float t = 0.f;
+      hipEventElapsedTime(&t, ev[i][0], ev[i][1]);
+      if (phase[i] < n_phases) {
+        ms[phase[i]] += t;
+        launches[phase[i]] += 1;
+      }
+      hipEventDestroy(ev[i][0]);
+      hipEventDestroy(ev[i][1]);
+    }
+    n = 0;
+  }
+};
+struct Span {  // RAII: one timed span around the launches in scope
+  PhaseTimer* t;
+  Span(PhaseTimer* timer, int ph) : t(timer) { if (t) t->begin(ph); }
+  ~Span() { if (t) t->end(); }
+};
 
 int check_head_shape(int64_t n, int64_t h, int64_t v) {
   if (n < 0 || h <= 0 || v <= 0) return AXON_ERR_ARG;
@@ -438,10 +511,10 @@ extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t
   return fwd_ws(n, v, nullptr).bytes + kAlign;
 }
 
-extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
-                               int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
-                               float* logprobs, float* entropy, float* lse, float* entropy_b,
-                               void* workspace, int64_t ws_bytes, void* stream) {
+static int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64,
+                    int64_t n, int64_t h, int64_t v, float inv_temp, float* logprobs, float* entropy,
+                    float* lse, float* entropy_b, void* workspace, int64_t ws_bytes, void* stream,
+                    PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
@@ -461,6 +534,8 @@ extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const voi
   g.k = (int)h;
   FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e};
   const int tiles_m = (int)((v + kTile - 1) / kTile), tiles_n = (int)((n + kTile - 1) / kTile);
+  {
+  Span span(timer, 0);
   if (h % 64 == 0) {
     rc = set_lds(lmhead_fwd_kernel<64>, lds_bytes<64>());
     if (rc != AXON_OK) return rc;
@@ -472,23 +547,50 @@ extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const voi
     hipLaunchKernelGGL(lmhead_fwd_kernel<32>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
                        lds_bytes<32>(), st, g, p, tiles_m, tiles_n);
   }
+  }
   AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.pm,
-                     w.ps, w.pe, w.parts, (int)n, inv_temp, lse, entropy_b, entropy);
+  {
+    Span span(timer, 1);
+    hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       w.pm, w.ps, w.pe, w.parts, (int)n, inv_temp, lse, entropy_b, entropy, w.fin_max,
+                       w.fin_log2s);
+  }
   AXON_CHECK_LAUNCH();
   const dim3 lg((unsigned)((n + 3) / 4));
+  Span span(timer, 2);
   if (labels_i64)
     hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
-                       static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp, lse,
-                       logprobs);
+                       static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp, w.fin_max,
+                       w.fin_log2s, logprobs);
   else
     hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
-                       static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp, lse,
-                       logprobs);
+                       static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp, w.fin_max,
+                       w.fin_log2s, logprobs);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
+}
+
+extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
+                               int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
+                               float* logprobs, float* entropy, float* lse, float* entropy_b,
+                               void* workspace, int64_t ws_bytes, void* stream) {
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, logprobs, entropy, lse,
+                  entropy_b, workspace, ws_bytes, stream, nullptr);
+}
+
+extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, const void* labels,
+                                     int labels_i64, int64_t n, int64_t h, int64_t v,
+                                     float inv_temp, float* logprobs, float* entropy, float* lse,
+                                     float* entropy_b, void* workspace, int64_t ws_bytes,
+                                     void* stream, float* phase_ms, int32_t* phase_launches) {
+  if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
+  PhaseTimer timer((hipStream_t)stream);
+  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, logprobs, entropy,
+                          lse, entropy_b, workspace, ws_bytes, stream, &timer);
+  timer.collect(phase_ms, phase_launches, 4);
+  return rc;
 }
 
 extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t v,
@@ -498,11 +600,11 @@ extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t
   return bwd_ws(n, h, v, chunk, nullptr).bytes + kAlign;
 }
 
-extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
-                               const void* weight, const void* labels, int labels_i64,
-                               const float* lse, const float* entropy_b, int64_t n, int64_t h,
-                               int64_t v, float inv_temp, void* d_hidden, void* d_weight,
-                               int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
+static int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden,
+                    const void* weight, const void* labels, int labels_i64, const float* lse,
+                    const float* entropy_b, int64_t n, int64_t h, int64_t v, float inv_temp,
+                    void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+                    int64_t ws_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
@@ -520,16 +622,20 @@ extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, co
   if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
 
   // K-contiguous copies for the two output GEMMs
-  rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.v_pad, (int)w.v_pad, st);
-  if (rc != AXON_OK) return rc;
-  rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.n_pad, (int)w.n_pad, st);
-  if (rc != AXON_OK) return rc;
+  {
+    Span span(timer, 0);
+    rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.v_pad, (int)w.v_pad, st);
+    if (rc != AXON_OK) return rc;
+    rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.n_pad, (int)w.n_pad, st);
+    if (rc != AXON_OK) return rc;
+  }
 
   for (int ci = 0; ci < w.chunks; ++ci) {
     const int64_t v0 = (int64_t)ci * w.chunk;
     const int64_t vc = (v - v0 < w.chunk) ? (v - v0) : w.chunk;  // valid vocab rows in this chunk
     // B1: dlogit for vocab rows [v0, v0 + vc)
     {
+      Span span(timer, 1);
       GemmOperands g;
       g.a = static_cast<const __bf16*>(weight) + v0 * h;  g.lda = h;  g.m_rows = (int)vc;
       g.b = static_cast<const __bf16*>(hidden);            g.ldb = h;  g.n_rows = (int)n;
@@ -556,6 +662,7 @@ extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, co
     const int64_t vc_red = round_up(vc, 64);  // columns [vc, vc_red) of dl were written as zeros
     // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
     {
+      Span span(timer, 2);
       GemmOperands g;
       g.a = w.wT + v0;  g.lda = w.v_pad;  g.m_rows = (int)h;
       g.b = w.dl;       g.ldb = w.chunk;  g.n_rows = (int)n;
@@ -570,6 +677,7 @@ extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, co
     }
     // B3: dWeight[v0 + v][h] = sum_t dlT[v][t] * hT[h][t]
     {
+      Span span(timer, 3);
       GemmOperands g;
       g.a = w.hT;   g.lda = w.n_pad;  g.m_rows = (int)h;
       g.b = w.dlT;  g.ldb = w.n_pad;  g.n_rows = (int)vc;
@@ -583,6 +691,31 @@ extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, co
     }
   }
   return AXON_OK;
+}
+
+extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
+                               const void* weight, const void* labels, int labels_i64,
+                               const float* lse, const float* entropy_b, int64_t n, int64_t h,
+                               int64_t v, float inv_temp, void* d_hidden, void* d_weight,
+                               int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
+  return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
+                  inv_temp, d_hidden, d_weight, chunk, workspace, ws_bytes, stream, nullptr);
+}
+
+extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy,
+                                     const void* hidden, const void* weight, const void* labels,
+                                     int labels_i64, const float* lse, const float* entropy_b,
+                                     int64_t n, int64_t h, int64_t v, float inv_temp,
+                                     void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+                                     int64_t ws_bytes, void* stream, float* phase_ms,
+                                     int32_t* phase_launches) {
+  if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
+  PhaseTimer timer((hipStream_t)stream);
+  const int rc = bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n,
+                          h, v, inv_temp, d_hidden, d_weight, chunk, workspace, ws_bytes, stream,
+                          &timer);
+  timer.collect(phase_ms, phase_launches, 4);
+  return rc;
 }
 
 extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, float* out,

@@ -48,7 +48,7 @@ class LinearCrossEntropy(torch.autograd.Function):
         assert hidden2.is_contiguous() and weight.is_contiguous() and labels1.is_contiguous()
 
         inv_t = 1.0 / temperature
-        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t)
+        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING)
         ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b)
         ctx.shape, ctx.inv_t, ctx.reduction = shape, inv_t, reduction
         if reduction == "sum":
@@ -69,7 +69,7 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs = (dlogprobs / n).expand(n)
         d_hidden, d_weight = _ops.lmhead_backward(
             dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
-            entropy_b, ctx.inv_t,
+            entropy_b, ctx.inv_t, timing=_ops.TIMING,
         )
         return d_hidden.view(ctx.shape), d_weight, None, None, None, None
 

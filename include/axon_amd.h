@@ -87,6 +87,26 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
                     void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
                     int64_t workspace_bytes, void* stream);
 
+/* Timed variants for benchmarks: same work, plus HIP events recorded on `stream`
+ * around every launch.  They SYNCHRONISE the stream before returning and create
+ * and destroy events (the exception to "never synchronises").  phase_ms[4] and
+ * phase_launches[4] are HOST arrays that are added to (zero them first):
+ *   forward : [0] logits+statistics kernel, [1] merge, [2] label logit
+ *   backward: [0] transposes, [1] dlogit recompute, [2] dHidden GEMM, [3] dWeight GEMM
+ * No reference counterpart (measurement only). */
+int axon_lmhead_fwd_timed(const void* hidden_bf16, const void* weight_bf16, const void* labels,
+                          int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
+                          float inv_temperature, float* logprobs, float* entropy, float* lse,
+                          float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream,
+                          float* phase_ms, int32_t* phase_launches);
+int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
+                          const void* weight_bf16, const void* labels, int labels_are_i64,
+                          const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
+                          int64_t vocab, float inv_temperature, void* d_hidden_bf16,
+                          void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
+                          int64_t workspace_bytes, void* stream, float* phase_ms,
+                          int32_t* phase_launches);
+
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
  * (fp32 accumulate, fp32 output).  No reference counterpart: it exists so tests
  * and the benchmark can measure the main loop in isolation.
