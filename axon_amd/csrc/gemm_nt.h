@@ -1,4 +1,4 @@
-// bf16 "NT" GEMM main loop for gfx950:  D[m][n] = sum_k A[m][k] * B[n][k]
+// bf16 "NT" GEMM main loops for gfx950:  D[m][n] = sum_k A[m][k] * B[n][k]
 //
 // Both operands are K-contiguous, which is the layout the 32x32x16 bf16 MFMA
 // wants on both sides: every lane feeds eight consecutive k of one row.  The
@@ -7,10 +7,20 @@
 // serves the whole path; they differ only in the epilogue.
 //
 // Workgroup: 256 threads = 4 waves in a 2x2 grid, tile 256(m) x 256(n), each
-// wave 128 x 128 = 4x4 MFMA blocks of 32x32 (256 fp32 accumulators per lane).
-// LDS: two stages of (256 + 256) rows x BK bf16, 16-byte chunks XOR-swizzled by
-// row so that the 16-byte fragment reads of 32 consecutive rows spread over all
-// banks.
+// wave 128 x 128 = 4x4 MFMA blocks of 32x32 (256 fp32 accumulators per lane,
+// one wave per SIMD).
+//
+// Two main loops:
+//  * DmaLoop  (the fast path; needs m_rows >= 256, n_rows >= 256, k % 64 == 0)
+//      global -> LDS by `buffer_load_dwordx4 ... lds` (no VGPR staging), two
+//      64 KB stages of 256 x 64 bf16 per operand, 16-byte chunks XOR-swizzled by
+//      row; fragment reads for k-step kk+1 are issued under the MFMAs of k-step
+//      kk; the next tile's DMA is issued one full tile ahead.  Edge tiles are
+//      shifted back inside the matrix (uniform addressing, no per-lane clamps);
+//      the rows that then belong to the neighbouring tile are masked by the
+//      epilogue through `m_lo` / `n_lo`.
+//  * RegLoop<32>  (any shape with k % 32 == 0): loads through registers with
+//      per-row clamping.  Used for small or odd shapes.
 //
 // Accumulator layout of one 32x32 block (v16f32, index q = 4*r + e):
 //   m = 8*r + 4*(lane/32) + e,   n = lane%32.
@@ -29,39 +39,33 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kTile = 256;       // tile edge in m and n
 constexpr int kWaveTile = 128;   // per-wave edge
 constexpr int kGemmThreads = 256;
+constexpr int kGemmLdsBytes = 131072;  // both main loops fit; also the staging area of the dlogit epilogue
 
 struct GemmOperands {
   const __bf16* a;  // [m_rows][lda], K-contiguous
   const __bf16* b;  // [n_rows][ldb]
   int64_t lda, ldb;
-  int m_rows, n_rows;  // valid rows; tile rows beyond are clamped on load
-  int k;               // reduction length, multiple of BK
+  int m_rows, n_rows;  // valid rows
+  int k;               // reduction length
 };
 
-template <int BK>
-struct TileLds {
-  static constexpr int kChunks = BK / 8;                 // 16-byte chunks per row
-  static constexpr int kRowBytes = BK * 2;
-  static constexpr int kRowsPerLine = 256 / kRowBytes;   // rows per 256-byte bank line
-  static constexpr int kOperandBytes = kTile * kRowBytes;
-  static constexpr int kStageBytes = 2 * kOperandBytes;
-  static constexpr int kBytes = 2 * kStageBytes;
-  __device__ static __forceinline__ int offset(int row, int chunk) {
-    const int sw = (row / kRowsPerLine) % kChunks;
-    return row * kRowBytes + ((chunk ^ sw) << 4);
-  }
+// Where a workgroup's tile sits.  (m0, n0) is the first row/column actually
+// computed; rows with tile-relative index < m_lo (columns < n_lo) duplicate the
+// previous tile and must be ignored by the epilogue.
+struct TilePos {
+  int m0, n0, m_lo, n_lo;
 };
 
 // Position of this lane inside the workgroup tile.
 struct LanePos {
-  int lane, l32, lhi, wm, wn;
+  int lane, l32, lhi, wave, wm, wn;
   __device__ __forceinline__ LanePos() {
     lane = threadIdx.x & 63;
     l32 = lane & 31;
     lhi = lane >> 5;
-    const int w = threadIdx.x >> 6;
-    wm = w >> 1;
-    wn = w & 1;
+    wave = threadIdx.x >> 6;
+    wm = wave >> 1;
+    wn = wave & 1;
   }
   // tile-relative coordinates of accumulator (i, j, q)
   __device__ __forceinline__ int m(int i, int q) const {
@@ -70,93 +74,256 @@ struct LanePos {
   __device__ __forceinline__ int n(int j) const { return wn * kWaveTile + j * 32 + l32; }
 };
 
-template <int BK>
-__device__ __forceinline__ void gemm_mainloop(const GemmOperands& g, int m0, int n0,
-                                              f32x16 (&acc)[4][4], char* smem) {
-  using L = TileLds<BK>;
-  constexpr int kLoads = (kTile * L::kChunks) / kGemmThreads;  // 16-byte loads per operand per thread
-  constexpr int kRowStep = kGemmThreads / L::kChunks;
-  const LanePos lp;
-
-  const int ld_chunk = threadIdx.x % L::kChunks;
-  const int ld_row = threadIdx.x / L::kChunks;
-  const uint4* ga[kLoads];
-  const uint4* gb[kLoads];
-  int lds_off[kLoads];
-#pragma unroll
-  for (int i = 0; i < kLoads; ++i) {
-    const int row = ld_row + i * kRowStep;
-    const int ra = min(m0 + row, g.m_rows - 1);
-    const int rb = min(n0 + row, g.n_rows - 1);
-    ga[i] = reinterpret_cast<const uint4*>(g.a + (int64_t)ra * g.lda) + ld_chunk;
-    gb[i] = reinterpret_cast<const uint4*>(g.b + (int64_t)rb * g.ldb) + ld_chunk;
-    lds_off[i] = L::offset(row, ld_chunk);
-  }
-  int a_off[4], b_off[4];  // fragment row offsets (chunk applied per k-step)
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    a_off[i] = lp.wm * kWaveTile + i * 32 + lp.l32;
-    b_off[i] = lp.wn * kWaveTile + i * 32 + lp.l32;
-  }
-
+__device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+}
 
-  uint4 ra[kLoads], rb[kLoads];
-  const int kt_n = g.k / BK;
-#pragma unroll
-  for (int i = 0; i < kLoads; ++i) {
-    ra[i] = ga[i][0];
-    rb[i] = gb[i][0];
-  }
-#pragma unroll
-  for (int i = 0; i < kLoads; ++i) {
-    *reinterpret_cast<uint4*>(smem + lds_off[i]) = ra[i];
-    *reinterpret_cast<uint4*>(smem + L::kOperandBytes + lds_off[i]) = rb[i];
-  }
-  __syncthreads();
+// ---------------------------------------------------------------------------------------
+// DmaLoop
+// ---------------------------------------------------------------------------------------
+struct DmaLoop {
+  static constexpr int kBK = 64;
+  static constexpr int kRowBytes = 128;                    // 64 bf16
+  static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
+  static constexpr int kStageBytes = 2 * kOperandBytes;    // A then B
+  static constexpr bool kShiftsEdgeTiles = true;
 
-  for (int kt = 0; kt < kt_n; ++kt) {
-    const char* cur = smem + (kt & 1) * L::kStageBytes;
-    char* nxt = smem + ((kt + 1) & 1) * L::kStageBytes;
-    const bool more = (kt + 1 < kt_n);
-    if (more) {
-      const int ko = (kt + 1) * L::kChunks;
+  __device__ static __forceinline__ bool supports(const GemmOperands& g) {
+    return g.m_rows >= kTile && g.n_rows >= kTile && (g.k % kBK) == 0;
+  }
+
+  __device__ static __forceinline__ TilePos place(const GemmOperands& g, int tm, int tn) {
+    TilePos t;
+    const int m0 = tm * kTile, n0 = tn * kTile;
+    t.m0 = min(m0, g.m_rows - kTile);
+    t.n0 = min(n0, g.n_rows - kTile);
+    t.m_lo = m0 - t.m0;
+    t.n_lo = n0 - t.n0;
+    return t;
+  }
+
+  __device__ static __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset,
+                                               char* lds) {
+    // LDS destination = lds + 16 * lane (wave-contiguous); memory source = base + voffset + soffset
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16,
+                                             voffset, soffset, 0, 0);
+  }
+
+  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
+                                             f32x16 (&acc)[4][4], char* smem) {
+    const LanePos lp;
+    // --- DMA addressing.  One wave instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns
+    // rows [64w, 64w+64) of each operand (8 instructions).  Lane i lands on row i/8, chunk slot
+    // i%8, and therefore fetches global chunk (i%8) ^ swizzle(row); swizzle(row) = (row/2) % 8.
+    const int lrow = lp.lane >> 3;
+    const int sw_even = (lp.lane >> 4) & 7;        // rows 8j + lrow with j even
+    const int sw_odd = (4 + (lp.lane >> 4)) & 7;   // j odd
+    const int row_a = (lp.wave * 64 + lrow) * (int)g.lda * 2;
+    const int row_b = (lp.wave * 64 + lrow) * (int)g.ldb * 2;
+    const int va_e = row_a + (((lp.lane & 7) ^ sw_even) << 4);
+    const int va_o = row_a + (((lp.lane & 7) ^ sw_odd) << 4);
+    const int vb_e = row_b + (((lp.lane & 7) ^ sw_even) << 4);
+    const int vb_o = row_b + (((lp.lane & 7) ^ sw_odd) << 4);
+    const int step_a = (int)g.lda * 16, step_b = (int)g.ldb * 16;  // 8 rows, in bytes
+    const __bf16* base_a = g.a + (int64_t)t.m0 * g.lda;
+    const __bf16* base_b = g.b + (int64_t)t.n0 * g.ldb;
+    const __amdgpu_buffer_rsrc_t ra =
+        __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb =
+        __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
+    char* const dst = smem + lp.wave * 64 * kRowBytes;
+
+    // --- fragment addressing: row = 128*wm + 32*i + l32, chunk = 2*kk + lhi, swizzle = (l32/2)%8
+    const int sw = (lp.l32 >> 1) & 7;
+    int fa[4], fb[4];
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i) {
-        ra[i] = ga[i][ko];
-        rb[i] = gb[i][ko];
-      }
+    for (int kk = 0; kk < 4; ++kk) {
+      fa[kk] = (lp.wm * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
+      fb[kk] = kOperandBytes + (lp.wn * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
     }
+
+    zero_acc(acc);
+    bf16x8 af[2][4], bf[2][4];
+    const int kt_n = g.k / kBK;
+
+    auto issue = [&](int stage_off, int kt) {
+      const int ko = kt * kRowBytes;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[4], bf[4];
+      for (int j = 0; j < 8; ++j) {
+        dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + stage_off + j * 8 * kRowBytes);
+        dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b,
+              dst + stage_off + kOperandBytes + j * 8 * kRowBytes);
+      }
+    };
+    auto read_frags = [&](int stage_off, int kk, int set) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        af[i] = *reinterpret_cast<const bf16x8*>(cur + L::offset(a_off[i], kk * 2 + lp.lhi));
-        bf[i] = *reinterpret_cast<const bf16x8*>(cur + L::kOperandBytes +
-                                                 L::offset(b_off[i], kk * 2 + lp.lhi));
+        af[set][i] = *reinterpret_cast<const bf16x8*>(smem + stage_off + fa[kk] + i * 32 * kRowBytes);
+        bf[set][i] = *reinterpret_cast<const bf16x8*>(smem + stage_off + fb[kk] + i * 32 * kRowBytes);
       }
+    };
+    auto mfma_block = [&](int set) {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+    };
+
+    // prologue: tiles 0 and 1 in flight, fragments of (tile 0, kk 0) in set 0
+    issue(0, 0);
+    issue(kStageBytes, min(1, kt_n - 1));
+    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): this wave's part of tile 0 has landed
+    __builtin_amdgcn_s_barrier();
+    read_frags(0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+
+    int cur = 0;
+    for (int kt = 0; kt < kt_n; ++kt) {
+      const int nxt = cur ^ kStageBytes;
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i) {
-        *reinterpret_cast<uint4*>(nxt + lds_off[i]) = ra[i];
-        *reinterpret_cast<uint4*>(nxt + L::kOperandBytes + lds_off[i]) = rb[i];
+      for (int kk = 0; kk < 3; ++kk) {
+        read_frags(cur, kk + 1, (kk + 1) & 1);
+        mfma_block(kk & 1);
+        // issue order: one fragment read per MFMA for the first eight, then eight MFMAs
+#pragma unroll
+        for (int r = 0; r < 8; ++r) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
+      // last k-step of this tile: the other stage must have landed for every wave, and every wave
+      // must be done reading this stage (its kk=3 fragments are in registers) before it is refilled.
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      issue(cur, min(kt + 2, kt_n - 1));   // past the end: refetches the last tile, never consumed
+      read_frags(nxt, 0, 0);
+      mfma_block(1);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      cur = nxt;
+    }
+    // DMA issued for tiles past the end is still in flight; drain it before LDS is reused
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __builtin_amdgcn_s_barrier();
+  }
+};
+
+// ---------------------------------------------------------------------------------------
+// RegLoop: loads through registers with per-row clamping; any k % BK == 0
+// ---------------------------------------------------------------------------------------
+template <int BK>
+struct RegLoop {
+  static constexpr int kBK = BK;
+  static constexpr int kChunks = BK / 8;                 // 16-byte chunks per row
+  static constexpr int kRowBytes = BK * 2;
+  static constexpr int kRowsPerLine = 256 / kRowBytes;   // rows per 256-byte bank line
+  static constexpr int kOperandBytes = kTile * kRowBytes;
+  static constexpr int kStageBytes = 2 * kOperandBytes;
+
+  __device__ static __forceinline__ int offset(int row, int chunk) {
+    const int sw = (row / kRowsPerLine) % kChunks;
+    return row * kRowBytes + ((chunk ^ sw) << 4);
+  }
+
+  __device__ static __forceinline__ TilePos place(const GemmOperands&, int tm, int tn) {
+    return TilePos{tm * kTile, tn * kTile, 0, 0};
+  }
+
+  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
+                                             f32x16 (&acc)[4][4], char* smem) {
+    constexpr int kLoads = (kTile * kChunks) / kGemmThreads;  // 16-byte loads per operand per thread
+    constexpr int kRowStep = kGemmThreads / kChunks;
+    const LanePos lp;
+    const int ld_chunk = threadIdx.x % kChunks;
+    const int ld_row = threadIdx.x / kChunks;
+    const uint4* ga[kLoads];
+    const uint4* gb[kLoads];
+    int lds_off[kLoads];
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const int row = ld_row + i * kRowStep;
+      const int ra = min(t.m0 + row, g.m_rows - 1);
+      const int rb = min(t.n0 + row, g.n_rows - 1);
+      ga[i] = reinterpret_cast<const uint4*>(g.a + (int64_t)ra * g.lda) + ld_chunk;
+      gb[i] = reinterpret_cast<const uint4*>(g.b + (int64_t)rb * g.ldb) + ld_chunk;
+      lds_off[i] = offset(row, ld_chunk);
+    }
+    int a_off[4], b_off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a_off[i] = lp.wm * kWaveTile + i * 32 + lp.l32;
+      b_off[i] = lp.wn * kWaveTile + i * 32 + lp.l32;
+    }
+    zero_acc(acc);
+
+    uint4 ra[kLoads], rb[kLoads];
+    const int kt_n = g.k / BK;
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      ra[i] = ga[i][0];
+      rb[i] = gb[i][0];
+    }
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      *reinterpret_cast<uint4*>(smem + lds_off[i]) = ra[i];
+      *reinterpret_cast<uint4*>(smem + kOperandBytes + lds_off[i]) = rb[i];
     }
     __syncthreads();
+
+    for (int kt = 0; kt < kt_n; ++kt) {
+      const char* cur = smem + (kt & 1) * kStageBytes;
+      char* nxt = smem + ((kt + 1) & 1) * kStageBytes;
+      const bool more = (kt + 1 < kt_n);
+      if (more) {
+        const int ko = (kt + 1) * kChunks;
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+          ra[i] = ga[i][ko];
+          rb[i] = gb[i][ko];
+        }
+      }
+#pragma unroll
+      for (int kk = 0; kk < BK / 16; ++kk) {
+        bf16x8 af[4], bf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          af[i] = *reinterpret_cast<const bf16x8*>(cur + offset(a_off[i], kk * 2 + lp.lhi));
+          bf[i] = *reinterpret_cast<const bf16x8*>(cur + kOperandBytes + offset(b_off[i], kk * 2 + lp.lhi));
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      }
+      if (more) {
+#pragma unroll
+        for (int i = 0; i < kLoads; ++i) {
+          *reinterpret_cast<uint4*>(nxt + lds_off[i]) = ra[i];
+          *reinterpret_cast<uint4*>(nxt + kOperandBytes + lds_off[i]) = rb[i];
+        }
+      }
+      __syncthreads();
+    }
   }
-}
+};
 
 // Workgroup id -> (tile_m, tile_n).  Consecutive workgroup ids land on
 // different XCDs (round-robin over 8), so ids are first regrouped so that each

@@ -10,7 +10,7 @@
 //   B2  dHidden[token][h] (+)= sum_v dl[token][v]  * WT[h][v]
 //   B3  dWeight[v][h]      =  sum_t dlT[v][t]      * hiddenT[h][t]
 // WT and hiddenT are bf16 transposes made once per call, so that all four GEMMs
-// run on the same K-contiguous main loop (gemm_nt.h).
+// run on the same K-contiguous main loops (gemm_nt.h).
 #include "common.h"
 #include "gemm_nt.h"
 
@@ -40,9 +40,6 @@ struct FwdParams {
   float c;     // inv_temperature * log2(e)
 };
 
-// Fold one 256x256 logits tile into per-token partials.  TAIL: the tile reaches past
-// the vocabulary; rows beyond it are excluded by predicate (their accumulators hold
-// finite values computed from a clamped weight row).
 constexpr float kEmptyMax = -3.0e38f;  // running max of a partial that saw no vocabulary row
 
 // Partial statistics of a set of scaled logits y = logit * c (log2 units):
@@ -56,9 +53,12 @@ __device__ __forceinline__ void merge_stats(float M, float& s, float& e, float M
   s = s * f1 + s2 * f2;
 }
 
-template <bool TAIL>
+// Fold one 256x256 logits tile into per-token partials.  MASKED: some rows of the tile
+// do not count (beyond the vocabulary, or duplicates of the neighbouring tile); they are
+// excluded by predicate — their accumulators hold finite values.
+template <bool MASKED>
 __device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParams& p,
-                                             const LanePos& lp, int tm, int m0, int n0) {
+                                             const LanePos& lp, const TilePos& t, int tm) {
   const int part = tm * 2 + lp.wm;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -67,20 +67,22 @@ __device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParam
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        const bool ok = !TAIL || (m0 + lp.m(i, q) < p.vocab);
+        const int mr = lp.m(i, q);
+        const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
         mx = ok ? fmaxf(mx, acc[i][j][q]) : mx;
       }
-    const float M = (TAIL && mx == -INFINITY) ? kEmptyMax : mx * p.c;
+    const float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
     float s = 0.f, e = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int q = 0; q < 16; ++q) {
-        const bool ok = !TAIL || (m0 + lp.m(i, q) < p.vocab);
-        const float t = fmaf(acc[i][j][q], p.c, -M);  // scaled logit relative to the max, <= 0
-        const float w = ok ? fast_exp2(t) : 0.f;
+        const int mr = lp.m(i, q);
+        const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
+        const float y = fmaf(acc[i][j][q], p.c, -M);  // scaled logit relative to the max, <= 0
+        const float w = ok ? fast_exp2(y) : 0.f;
         s += w;
-        e = fmaf(w, t, e);
+        e = fmaf(w, y, e);
       }
     // merge the two lanes that hold the same token (lane and lane^32)
     const float M2 = __shfl_xor(M, 32, 64);
@@ -88,8 +90,9 @@ __device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParam
     const float e2 = __shfl_xor(e, 32, 64);
     const float Mn = fmaxf(M, M2);
     merge_stats(M, s, e, M2, s2, e2, Mn);
-    const int n = n0 + lp.n(j);
-    if (lp.lhi == 0 && n < p.n_tokens) {
+    const int nr = lp.n(j);
+    const int n = t.n0 + nr;
+    if (lp.lhi == 0 && nr >= t.n_lo && n < p.n_tokens) {
       const int64_t o = (int64_t)part * p.n_tokens + n;
       p.pm[o] = Mn;
       p.ps[o] = s;
@@ -98,33 +101,27 @@ __device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParam
   }
 }
 
-template <int BK>
+template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
                                                                   int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * kTile, n0 = tn * kTile;
+  const TilePos t = Loop::place(g, tm, tn);
   f32x16 acc[4][4];
-  gemm_mainloop<BK>(g, m0, n0, acc, smem);
-
+  Loop::run(g, t, acc, smem);
   const LanePos lp;
-  if (m0 + kTile > p.vocab)
-    fwd_epilogue<true>(acc, p, lp, tm, m0, n0);
+  if (t.m_lo > 0 || t.m0 + kTile > p.vocab)
+    fwd_epilogue<true>(acc, p, lp, t, tm);
   else
-    fwd_epilogue<false>(acc, p, lp, tm, m0, n0);
+    fwd_epilogue<false>(acc, p, lp, t, tm);
 }
 
 // Merge partials: lse, entropy_b, entropy.  One thread per token.
-__global__ __launch_bounds__(256) void lmhead_merge_kernel(const float* __restrict__ pm,
-                                                           const float* __restrict__ ps,
-                                                           const float* __restrict__ pe, int parts,
-                                                           int n_tokens, float inv_temp,
-                                                           float* __restrict__ lse,
-                                                           float* __restrict__ entropy_b,
-                                                           float* __restrict__ entropy,
-                                                           float* __restrict__ fin_max,
-                                                           float* __restrict__ fin_log2s) {
+__global__ __launch_bounds__(256) void lmhead_merge_kernel(
+    const float* __restrict__ pm, const float* __restrict__ ps, const float* __restrict__ pe,
+    int parts, int n_tokens, float* __restrict__ lse, float* __restrict__ entropy_b,
+    float* __restrict__ entropy, float* __restrict__ fin_max, float* __restrict__ fin_log2s) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= n_tokens) return;
   float M = pm[n], s = ps[n], e = pe[n];
@@ -193,26 +190,32 @@ struct DlogitParams {
   float inv_temp;
 };
 
-constexpr int kStagePitch = kTile + 4;  // bf16 elements per staged row (8-byte aligned rows)
+// Per-wave staging of the wave's 128(n) x 128(m) bf16 sub-tile in its own 32 KB of LDS:
+// row nw (256 bytes = 32 units of 4 bf16), unit u stored at slot u ^ swz(nw),
+// swz(nw) = (nw & 31) ^ (nw >> 5).  The three access patterns (column-of-rows write,
+// row read, 4x4-block read) then each touch 32 distinct slots per 32 lanes.
+__device__ __forceinline__ int stage_off(int nw, int unit) {
+  return nw * 256 + ((unit ^ ((nw & 31) ^ (nw >> 5))) << 3);
+}
 
-template <int BK>
+template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperands g, DlogitParams p,
                                                                      int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * kTile, n0 = tn * kTile;  // m0 relative to the chunk
+  const TilePos t = Loop::place(g, tm, tn);  // t.m0 is relative to the chunk
   f32x16 acc[4][4];
-  gemm_mainloop<BK>(g, m0, n0, acc, smem);
-  // all waves are past their last LDS read (the main loop ends with a barrier)
+  Loop::run(g, t, acc, smem);
+  __syncthreads();  // every wave is past its last main-loop LDS access
 
   const LanePos lp;
   const float c = p.inv_temp * kLog2e;
-  uint16_t* stage = reinterpret_cast<uint16_t*>(smem);  // [256 n][kStagePitch] bf16
+  char* const stage = smem + lp.wave * 32768;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int nrel = lp.n(j);
-    const int n = n0 + nrel;
+    const int nw = j * 32 + lp.l32;  // token row inside the wave's sub-tile
+    const int n = t.n0 + lp.wn * kWaveTile + nw;
     const bool n_ok = n < p.n_tokens;
     const int nn = n_ok ? n : 0;
     const float g_lp = n_ok ? p.dlogprobs[nn] : 0.f;
@@ -223,10 +226,9 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperand
     const float ca = (-g_lp + g_en * eb) * p.inv_temp;
     const float cb = -g_en * p.inv_temp;
     const float gl = g_lp * p.inv_temp;
-    int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[nn]
-                               : (int64_t) static_cast<const int32_t*>(p.labels)[nn];
-    // label position relative to this lane's first row in the wave tile
-    const int64_t lab_rel = lab - (int64_t)(p.v_begin + m0);
+    const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[nn]
+                                     : (int64_t) static_cast<const int32_t*>(p.labels)[nn];
+    const int64_t lab_rel = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -241,35 +243,38 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperand
           const float x = raw * p.inv_temp;
           float v = pr * fmaf(cb, x, ca);
           if ((int64_t)mrel == lab_rel) v += gl;
-          const bool ok = n_ok && (p.v_begin + m0 + mrel < p.vocab);
+          // rows shared with the neighbouring tile keep their (identical) values
+          const bool ok = n_ok && (p.v_begin + t.m0 + mrel < p.vocab);
           d[e] = ok ? v : 0.f;
         }
-        const int mq = lp.m(i, 4 * r);  // first of four consecutive m
         uint2 w;
         w.x = pack_bf16(d[0], d[1]);
         w.y = pack_bf16(d[2], d[3]);
-        *reinterpret_cast<uint2*>(stage + nrel * kStagePitch + mq) = w;
+        *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 8 + 2 * r + lp.lhi)) = w;
       }
     }
   }
-  __syncthreads();
-  // token-major copy: row n, 256 m = 32 chunks of 16 bytes... rows are 8-byte aligned in
-  // LDS, so move 8 bytes per lane: 64 lanes cover one 512-byte row.
+  // the wave reads back only what it wrote itself; LDS operations of one wave complete in order
+  const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
+  const int n_base = t.n0 + lp.wn * kWaveTile;
+  // token-major copy: 32 lanes cover one 256-byte row
   {
-    const int col = (threadIdx.x & 63) * 4;
-    for (int row = threadIdx.x >> 6; row < kTile; row += 4) {
-      const uint2 v = *reinterpret_cast<const uint2*>(stage + row * kStagePitch + col);
-      *reinterpret_cast<uint2*>(p.dl + (int64_t)(n0 + row) * p.ld_dl + m0 + col) = v;
+    const int unit = lp.l32;
+#pragma unroll 4
+    for (int nw = lp.lhi; nw < kWaveTile; nw += 2) {
+      const uint2 v = *reinterpret_cast<const uint2*>(stage + stage_off(nw, unit));
+      *reinterpret_cast<uint2*>(p.dl + (int64_t)(n_base + nw) * p.ld_dl + m_base + unit * 4) = v;
     }
   }
-  // vocab-major copy: 4x4 blocks transposed in registers
+  // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
   {
-    const int nq = threadIdx.x & 63;  // token quad
-    for (int mq = threadIdx.x >> 6; mq < kTile / 4; mq += 4) {
+    const int nq = lp.l32;  // token quad
+#pragma unroll 2
+    for (int unit = lp.lhi; unit < 32; unit += 2) {
       uint2 rws[4];
 #pragma unroll
       for (int f = 0; f < 4; ++f)
-        rws[f] = *reinterpret_cast<const uint2*>(stage + (nq * 4 + f) * kStagePitch + mq * 4);
+        rws[f] = *reinterpret_cast<const uint2*>(stage + stage_off(nq * 4 + f, unit));
       uint2 o[4];
       o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
       o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
@@ -281,7 +286,7 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperand
       o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        *reinterpret_cast<uint2*>(p.dlT + (int64_t)(m0 + mq * 4 + e) * p.ld_dlT + n0 + nq * 4) = o[e];
+        *reinterpret_cast<uint2*>(p.dlT + (int64_t)(m_base + unit * 4 + e) * p.ld_dlT + n_base + nq * 4) = o[e];
     }
   }
 }
@@ -297,26 +302,29 @@ struct StoreParams {
   int accumulate;     // add the previous contents of out_f32 first
 };
 
-template <int BK>
+template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g, StoreParams p,
                                                                   int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
-  const int m0 = tm * kTile, n0 = tn * kTile;
+  const TilePos t = Loop::place(g, tm, tn);
   f32x16 acc[4][4];
-  gemm_mainloop<BK>(g, m0, n0, acc, smem);
+  Loop::run(g, t, acc, smem);
   const LanePos lp;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int n = n0 + lp.n(j);
-    if (n >= p.n_valid) continue;
+    const int nr = lp.n(j);
+    const int n = t.n0 + nr;
+    if (nr < t.n_lo || n >= p.n_valid) continue;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int m = m0 + lp.m(i, 4 * r);
-        if (m >= p.m_valid) continue;  // m_valid % 4 == 0: a quad is all in or all out
+        const int mr = lp.m(i, 4 * r);
+        const int m = t.m0 + mr;
+        // m_valid % 4 == 0 and tile shifts are multiples of 4: a quad is all in or all out
+        if (mr < t.m_lo || m >= p.m_valid) continue;
         float4 v = make_float4(acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2],
                                acc[i][j][4 * r + 3]);
         if (p.out_f32) {
@@ -337,8 +345,8 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g
   }
 }
 
-// out[c][r] = in[r][c] for r < rows, c < cols; zero elsewhere in the padded
-// output [cols_pad][ld_out] for r in [rows, rows_pad).  32x32 tiles through LDS.
+// out[c][r] = in[r][c] for r < rows, c < cols; zero for r in [rows, rows_pad).
+// 64x64 tiles through LDS.
 __global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ in,
                                                              int64_t ld_in, int rows, int cols,
                                                              uint16_t* __restrict__ out,
@@ -358,6 +366,15 @@ __global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __r
   }
 }
 
+// zero the bf16 columns [col0, col0 + ncols) of `rows` rows (reduction padding of dl / dlT)
+__global__ __launch_bounds__(256) void zero_cols_bf16_kernel(uint16_t* p, int64_t ld, int rows,
+                                                             int col0, int ncols) {
+  const int64_t total = (int64_t)rows * ncols;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    p[(i / ncols) * ld + col0 + (i % ncols)] = 0;
+}
+
 }  // namespace axon
 
 using namespace axon;
@@ -367,23 +384,37 @@ namespace {
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 constexpr int64_t kDefaultVocabChunk = 16384;
 constexpr int64_t kAlign = 256;
+using SlowLoop = RegLoop<32>;
 
-template <int BK>
-constexpr int lds_bytes() { return TileLds<BK>::kBytes; }
-// B1 re-uses the stage buffers to hold the bf16 tile it writes out
-template <int BK>
-constexpr int dlogit_lds_bytes() {
-  return TileLds<BK>::kBytes > kTile * kStagePitch * 2 ? TileLds<BK>::kBytes
-                                                       : kTile * kStagePitch * 2;
+inline bool dma_ok(const GemmOperands& g) {
+  return g.m_rows >= kTile && g.n_rows >= kTile && (g.k % DmaLoop::kBK) == 0 &&
+         g.lda < (1 << 21) && g.ldb < (1 << 21);  // byte offsets inside a tile stay below 2^31
 }
 
 template <typename K>
-int set_lds(K kernel, int bytes) {
+int set_lds(K kernel) {
   return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess
+                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                             kGemmLdsBytes) == hipSuccess
              ? AXON_OK
              : AXON_ERR_LAUNCH;
 }
+
+// Launch kernel<DmaLoop> or kernel<SlowLoop> over all tiles of the problem.
+#define AXON_LAUNCH_GEMM(KERNEL, G, P, ST)                                                        \
+  do {                                                                                            \
+    const int tiles_m_ = ((G).m_rows + kTile - 1) / kTile, tiles_n_ = ((G).n_rows + kTile - 1) / kTile; \
+    if (dma_ok(G)) {                                                                              \
+      if (set_lds(KERNEL<DmaLoop>) != AXON_OK) return AXON_ERR_LAUNCH;                            \
+      hipLaunchKernelGGL(KERNEL<DmaLoop>, dim3(tiles_m_ * tiles_n_), dim3(kGemmThreads),          \
+                         kGemmLdsBytes, ST, G, P, tiles_m_, tiles_n_);                            \
+    } else {                                                                                      \
+      if (set_lds(KERNEL<SlowLoop>) != AXON_OK) return AXON_ERR_LAUNCH;                           \
+      hipLaunchKernelGGL(KERNEL<SlowLoop>, dim3(tiles_m_ * tiles_n_), dim3(kGemmThreads),         \
+                         kGemmLdsBytes, ST, G, P, tiles_m_, tiles_n_);                            \
+    }                                                                                             \
+    AXON_CHECK_LAUNCH();                                                                          \
+  } while (0)
 
 struct FwdWs {
   float *pm, *ps, *pe;
@@ -443,29 +474,30 @@ struct PhaseTimer {
   explicit PhaseTimer(hipStream_t s) : st(s) {}
   void begin(int ph) {
     if (n >= kMaxSpans) return;
-    if (hipEventCreate(&ev[n][0]) != hipSuccess || hipEventCreate(&ev[n][1]) != hipSuccess) return;
+    if (hipEventCreate(&ev[n][0]) != hipSuccess) return;
+    if (hipEventCreate(&ev[n][1]) != hipSuccess) { (void)hipEventDestroy(ev[n][0]); return; }
     phase[n] = ph;
-    hipEventRecord(ev[n][0], st);
+    (void)hipEventRecord(ev[n][0], st);
     open = true;
   }
   void end() {
     if (!open) return;
-    hipEventRecord(ev[n][1], st);
+    (void)hipEventRecord(ev[n][1], st);
     ++n;
     open = false;
   }
   // synchronises the stream; adds elapsed ms and launch counts per phase
   void collect(float* ms, int32_t* launches, int n_phases) {
-    hipStreamSynchronize(st);
+    (void)hipStreamSynchronize(st);
     for (int i = 0; i < n; ++i) {
       float t = 0.f;
-      hipEventElapsedTime(&t, ev[i][0], ev[i][1]);
+      (void)hipEventElapsedTime(&t, ev[i][0], ev[i][1]);
       if (phase[i] < n_phases) {
         ms[phase[i]] += t;
         launches[phase[i]] += 1;
       }
-      hipEventDestroy(ev[i][0]);
-      hipEventDestroy(ev[i][1]);
+      (void)hipEventDestroy(ev[i][0]);
+      (void)hipEventDestroy(ev[i][1]);
     }
     n = 0;
   }
@@ -483,14 +515,8 @@ int check_head_shape(int64_t n, int64_t h, int64_t v) {
   return AXON_OK;
 }
 
-template <int BK>
 int launch_store(const GemmOperands& g, const StoreParams& sp, hipStream_t st) {
-  const int tiles_m = (g.m_rows + kTile - 1) / kTile, tiles_n = (g.n_rows + kTile - 1) / kTile;
-  int rc = set_lds(gemm_store_kernel<BK>, lds_bytes<BK>());
-  if (rc != AXON_OK) return rc;
-  hipLaunchKernelGGL(gemm_store_kernel<BK>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
-                     lds_bytes<BK>(), st, g, sp, tiles_m, tiles_n);
-  AXON_CHECK_LAUNCH();
+  AXON_LAUNCH_GEMM(gemm_store_kernel, g, sp, st);
   return AXON_OK;
 }
 
@@ -504,17 +530,20 @@ int launch_transpose(const void* in, int64_t ld_in, int rows, int cols, void* ou
   return AXON_OK;
 }
 
-}  // namespace
-
-extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t v) {
-  if (check_head_shape(n, h, v) != AXON_OK) return -1;
-  return fwd_ws(n, v, nullptr).bytes + kAlign;
+int launch_zero_cols(void* p, int64_t ld, int rows, int col0, int ncols, hipStream_t st) {
+  if (ncols <= 0 || rows <= 0) return AXON_OK;
+  const int64_t total = (int64_t)rows * ncols;
+  const int64_t blocks = (total + 255) / 256;
+  const int grid = (int)(blocks < 2048 ? blocks : 2048);
+  hipLaunchKernelGGL(zero_cols_bf16_kernel, dim3(grid), dim3(256), 0, st, static_cast<uint16_t*>(p),
+                     ld, rows, col0, ncols);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
 }
 
-static int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64,
-                    int64_t n, int64_t h, int64_t v, float inv_temp, float* logprobs, float* entropy,
-                    float* lse, float* entropy_b, void* workspace, int64_t ws_bytes, void* stream,
-                    PhaseTimer* timer) {
+int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64, int64_t n,
+             int64_t h, int64_t v, float inv_temp, float* logprobs, float* entropy, float* lse,
+             float* entropy_b, void* workspace, int64_t ws_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
@@ -533,26 +562,14 @@ static int fwd_impl(const void* hidden, const void* weight, const void* labels, 
   g.b = static_cast<const __bf16*>(hidden);  g.ldb = h;  g.n_rows = (int)n;
   g.k = (int)h;
   FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e};
-  const int tiles_m = (int)((v + kTile - 1) / kTile), tiles_n = (int)((n + kTile - 1) / kTile);
   {
-  Span span(timer, 0);
-  if (h % 64 == 0) {
-    rc = set_lds(lmhead_fwd_kernel<64>, lds_bytes<64>());
-    if (rc != AXON_OK) return rc;
-    hipLaunchKernelGGL(lmhead_fwd_kernel<64>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
-                       lds_bytes<64>(), st, g, p, tiles_m, tiles_n);
-  } else {
-    rc = set_lds(lmhead_fwd_kernel<32>, lds_bytes<32>());
-    if (rc != AXON_OK) return rc;
-    hipLaunchKernelGGL(lmhead_fwd_kernel<32>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
-                       lds_bytes<32>(), st, g, p, tiles_m, tiles_n);
+    Span span(timer, 0);
+    AXON_LAUNCH_GEMM(lmhead_fwd_kernel, g, p, st);
   }
-  }
-  AXON_CHECK_LAUNCH();
   {
     Span span(timer, 1);
     hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                       w.pm, w.ps, w.pe, w.parts, (int)n, inv_temp, lse, entropy_b, entropy, w.fin_max,
+                       w.pm, w.ps, w.pe, w.parts, (int)n, lse, entropy_b, entropy, w.fin_max,
                        w.fin_log2s);
   }
   AXON_CHECK_LAUNCH();
@@ -561,15 +578,109 @@ static int fwd_impl(const void* hidden, const void* weight, const void* labels, 
   if (labels_i64)
     hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
-                       static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp, w.fin_max,
-                       w.fin_log2s, logprobs);
+                       static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
+                       w.fin_max, w.fin_log2s, logprobs);
   else
     hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
-                       static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp, w.fin_max,
-                       w.fin_log2s, logprobs);
+                       static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
+                       w.fin_max, w.fin_log2s, logprobs);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
+}
+
+int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
+             const void* labels, int labels_i64, const float* lse, const float* entropy_b,
+             int64_t n, int64_t h, int64_t v, float inv_temp, void* d_hidden, void* d_weight,
+             int64_t chunk, void* workspace, int64_t ws_bytes, void* stream, PhaseTimer* timer) {
+  int rc = check_head_shape(n, h, v);
+  if (rc != AXON_OK) return rc;
+  if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
+  if (!d_weight || !weight) return AXON_ERR_ARG;
+  const hipStream_t st = (hipStream_t)stream;
+  if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
+  if (!dlogprobs || !hidden || !labels || !lse || !entropy_b || !d_hidden || !workspace)
+    return AXON_ERR_ARG;
+  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
+       reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_weight)) & 15)
+    return AXON_ERR_ARG;
+  char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
+  const BwdWs w = bwd_ws(n, h, v, chunk, base);
+  if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
+
+  // K-contiguous copies for the two output GEMMs
+  {
+    Span span(timer, 0);
+    rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.v_pad, (int)w.v_pad, st);
+    if (rc != AXON_OK) return rc;
+    rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.n_pad, (int)w.n_pad, st);
+    if (rc != AXON_OK) return rc;
+  }
+  const int64_t n_red = round_up(n, 64);  // reduction length of B3
+
+  for (int ci = 0; ci < w.chunks; ++ci) {
+    const int64_t v0 = (int64_t)ci * w.chunk;
+    const int64_t vc = (v - v0 < w.chunk) ? (v - v0) : w.chunk;  // valid vocab rows in this chunk
+    const int64_t vc_red = round_up(vc, 64);                      // reduction length of B2
+    // B1: dlogit for vocab rows [v0, v0 + vc)
+    {
+      Span span(timer, 1);
+      GemmOperands g;
+      g.a = static_cast<const __bf16*>(weight) + v0 * h;  g.lda = h;  g.m_rows = (int)vc;
+      g.b = static_cast<const __bf16*>(hidden);            g.ldb = h;  g.n_rows = (int)n;
+      g.k = (int)h;
+      DlogitParams p;
+      p.lse = lse; p.entropy_b = entropy_b; p.dlogprobs = dlogprobs; p.dentropy = dentropy;
+      p.labels = labels; p.labels_i64 = labels_i64;
+      p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.chunk; p.ld_dlT = w.n_pad;
+      p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
+      AXON_LAUNCH_GEMM(lmhead_dlogit_kernel, g, p, st);
+      // reduction padding the tiles did not cover (the shifted-tile path writes no padding; the
+      // clamped path writes zeros there already, the extra fill is then redundant but harmless)
+      rc = launch_zero_cols(w.dl, w.chunk, (int)n, (int)vc, (int)(vc_red - vc), st);
+      if (rc != AXON_OK) return rc;
+      rc = launch_zero_cols(w.dlT, w.n_pad, (int)vc, (int)n, (int)(n_red - n), st);
+      if (rc != AXON_OK) return rc;
+    }
+    // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
+    {
+      Span span(timer, 2);
+      GemmOperands g;
+      g.a = w.wT + v0;  g.lda = w.v_pad;  g.m_rows = (int)h;
+      g.b = w.dl;       g.ldb = w.chunk;  g.n_rows = (int)n;
+      g.k = (int)vc_red;
+      StoreParams sp;
+      const bool last = (ci == w.chunks - 1);
+      sp.out_f32 = (w.chunks > 1) ? w.dh_acc : nullptr;  sp.ld_f32 = h;
+      sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
+      sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0);
+      rc = launch_store(g, sp, st);
+      if (rc != AXON_OK) return rc;
+    }
+    // B3: dWeight[v0 + v][h] = sum_t dlT[v][t] * hT[h][t]
+    {
+      Span span(timer, 3);
+      GemmOperands g;
+      g.a = w.hT;   g.lda = w.n_pad;  g.m_rows = (int)h;
+      g.b = w.dlT;  g.ldb = w.n_pad;  g.n_rows = (int)vc;
+      g.k = (int)n_red;
+      StoreParams sp;
+      sp.out_f32 = nullptr; sp.ld_f32 = 0;
+      sp.out_bf16 = static_cast<__bf16*>(d_weight) + v0 * h;  sp.ld_bf16 = h;
+      sp.m_valid = (int)h; sp.n_valid = (int)vc; sp.accumulate = 0;
+      rc = launch_store(g, sp, st);
+      if (rc != AXON_OK) return rc;
+    }
+  }
+  return AXON_OK;
+}
+
+}  // namespace
+
+extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t v) {
+  if (check_head_shape(n, h, v) != AXON_OK) return -1;
+  return fwd_ws(n, v, nullptr).bytes + kAlign;
 }
 
 extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
@@ -598,99 +709,6 @@ extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t
   if (check_head_shape(n, h, v) != AXON_OK) return -1;
   if (chunk < 0 || chunk % kTile != 0) return -1;
   return bwd_ws(n, h, v, chunk, nullptr).bytes + kAlign;
-}
-
-static int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden,
-                    const void* weight, const void* labels, int labels_i64, const float* lse,
-                    const float* entropy_b, int64_t n, int64_t h, int64_t v, float inv_temp,
-                    void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
-                    int64_t ws_bytes, void* stream, PhaseTimer* timer) {
-  int rc = check_head_shape(n, h, v);
-  if (rc != AXON_OK) return rc;
-  if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
-  if (!d_weight || !weight) return AXON_ERR_ARG;
-  const hipStream_t st = (hipStream_t)stream;
-  if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
-  if (!dlogprobs || !hidden || !labels || !lse || !entropy_b || !d_hidden || !workspace)
-    return AXON_ERR_ARG;
-  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
-  if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
-       reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_weight)) & 15)
-    return AXON_ERR_ARG;
-  char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
-  const BwdWs w = bwd_ws(n, h, v, chunk, base);
-  if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
-
-  // K-contiguous copies for the two output GEMMs
-  {
-    Span span(timer, 0);
-    rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.v_pad, (int)w.v_pad, st);
-    if (rc != AXON_OK) return rc;
-    rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.n_pad, (int)w.n_pad, st);
-    if (rc != AXON_OK) return rc;
-  }
-
-  for (int ci = 0; ci < w.chunks; ++ci) {
-    const int64_t v0 = (int64_t)ci * w.chunk;
-    const int64_t vc = (v - v0 < w.chunk) ? (v - v0) : w.chunk;  // valid vocab rows in this chunk
-    // B1: dlogit for vocab rows [v0, v0 + vc)
-    {
-      Span span(timer, 1);
-      GemmOperands g;
-      g.a = static_cast<const __bf16*>(weight) + v0 * h;  g.lda = h;  g.m_rows = (int)vc;
-      g.b = static_cast<const __bf16*>(hidden);            g.ldb = h;  g.n_rows = (int)n;
-      g.k = (int)h;
-      DlogitParams p;
-      p.lse = lse; p.entropy_b = entropy_b; p.dlogprobs = dlogprobs; p.dentropy = dentropy;
-      p.labels = labels; p.labels_i64 = labels_i64;
-      p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.chunk; p.ld_dlT = w.n_pad;
-      p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
-      const int tiles_m = (int)((vc + kTile - 1) / kTile), tiles_n = (int)(w.n_pad / kTile);
-      if (h % 64 == 0) {
-        rc = set_lds(lmhead_dlogit_kernel<64>, dlogit_lds_bytes<64>());
-        if (rc != AXON_OK) return rc;
-        hipLaunchKernelGGL(lmhead_dlogit_kernel<64>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
-                           dlogit_lds_bytes<64>(), st, g, p, tiles_m, tiles_n);
-      } else {
-        rc = set_lds(lmhead_dlogit_kernel<32>, dlogit_lds_bytes<32>());
-        if (rc != AXON_OK) return rc;
-        hipLaunchKernelGGL(lmhead_dlogit_kernel<32>, dim3(tiles_m * tiles_n), dim3(kGemmThreads),
-                           dlogit_lds_bytes<32>(), st, g, p, tiles_m, tiles_n);
-      }
-      AXON_CHECK_LAUNCH();
-    }
-    const int64_t vc_red = round_up(vc, 64);  // columns [vc, vc_red) of dl were written as zeros
-    // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
-    {
-      Span span(timer, 2);
-      GemmOperands g;
-      g.a = w.wT + v0;  g.lda = w.v_pad;  g.m_rows = (int)h;
-      g.b = w.dl;       g.ldb = w.chunk;  g.n_rows = (int)n;
-      g.k = (int)vc_red;
-      StoreParams sp;
-      const bool last = (ci == w.chunks - 1);
-      sp.out_f32 = (w.chunks > 1) ? w.dh_acc : nullptr;  sp.ld_f32 = h;
-      sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
-      sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0);
-      rc = launch_store<64>(g, sp, st);
-      if (rc != AXON_OK) return rc;
-    }
-    // B3: dWeight[v0 + v][h] = sum_t dlT[v][t] * hT[h][t]
-    {
-      Span span(timer, 3);
-      GemmOperands g;
-      g.a = w.hT;   g.lda = w.n_pad;  g.m_rows = (int)h;
-      g.b = w.dlT;  g.ldb = w.n_pad;  g.n_rows = (int)vc;
-      g.k = (int)round_up(n, 64);
-      StoreParams sp;
-      sp.out_f32 = nullptr; sp.ld_f32 = 0;
-      sp.out_bf16 = static_cast<__bf16*>(d_weight) + v0 * h;  sp.ld_bf16 = h;
-      sp.m_valid = (int)h; sp.n_valid = (int)vc; sp.accumulate = 0;
-      rc = launch_store<64>(g, sp, st);
-      if (rc != AXON_OK) return rc;
-    }
-  }
-  return AXON_OK;
 }
 
 extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
@@ -732,6 +750,5 @@ extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int6
   StoreParams sp;
   sp.out_f32 = out; sp.ld_f32 = ldo; sp.out_bf16 = nullptr; sp.ld_bf16 = 0;
   sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0;
-  if (k % 64 == 0) return launch_store<64>(g, sp, (hipStream_t)stream);
-  return launch_store<32>(g, sp, (hipStream_t)stream);
+  return launch_store(g, sp, (hipStream_t)stream);
 }
