@@ -67,10 +67,10 @@ def cpu_baseline(hid, w, lab, budget_s):
         OM.backward_bf16_torch_path(lpf.grad.view(-1), h, w, l)
         return time.perf_counter() - t0
 
-    probe_n = 32
+    probe_n = min(512, hid.shape[0])  # one full chunk of the reference's token loop
     t_probe = run(probe_n)
-    n = int(max(probe_n, min(2048, hid.shape[0], probe_n * budget_s / max(t_probe, 1e-6))))
-    n = max(probe_n, (n // 32) * 32)
+    n = int(min(hid.shape[0], probe_n * budget_s / max(t_probe, 1e-6)))
+    n = max(probe_n, (n // 512) * 512)
     t = run(n) if n > probe_n else t_probe
     return {
         "value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",

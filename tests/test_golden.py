@@ -1,0 +1,262 @@
+"""Golden fixtures (tests/golden/*.npz, written by tests/golden/make_fixtures.py).
+
+CPU half: the oracle reproduces every stored output (a changed oracle cannot silently move the
+target), and the stored numbers satisfy facts that do not come from the oracle (closed forms,
+hand-evaluated regions).  GPU half: the HIP path, called through the product API, reproduces the
+stored outputs to the stated tolerances: masks bit-exact, log-prob/entropy 1e-3 absolute, loss
+1e-4 relative, bf16 gradients 2e-2 relative-L2, fp32 per-token outputs 1e-5 relative-L2."""
+
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import advantage as OA
+from oracle import lmhead as OM
+from oracle import loss as OL
+from oracle import sampler as OS
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda"
+
+
+def load(name):
+    with np.load(os.path.join(GOLD, name), allow_pickle=False) as z:
+        return {k: torch.from_numpy(np.asarray(z[k])) for k in z.files}
+
+
+def bf16(bits):
+    return bits.view(torch.bfloat16)
+
+
+def rel_l2(a, b):
+    a, b = a.detach().double().cpu(), b.detach().double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+# ---------------------------------------------------------------------------------------------
+# CPU: oracle vs fixtures, fixtures vs independent facts
+# ---------------------------------------------------------------------------------------------
+def test_fixture_lmhead_oracle_and_textbook():
+    f = load("lmhead_n64_h128_v1000.npz")
+    hid, w, lab, temp = bf16(f["hidden_bf16"]), bf16(f["weight_bf16"]), f["labels"], float(f["temperature"])
+    lp, ent = OM.forward(hid, w, lab, temp)
+    assert torch.equal(lp, f["logprobs"]) or (lp - f["logprobs"]).abs().max() < 1e-6
+    assert (ent - f["entropy"]).abs().max() < 1e-6
+    # library routine in fp64, independent of the oracle's formula
+    logits = (hid.double() @ w.double().t()) / temp
+    lsm = torch.log_softmax(logits, -1)
+    assert (lsm.gather(-1, lab.long()[:, None]).squeeze(-1) - f["logprobs"]).abs().max() < 1e-5
+    assert (-(lsm.exp() * lsm).sum(-1) - f["entropy"]).abs().max() < 1e-5
+    # gradients: autograd through the textbook fp64 forward
+    h64, w64 = hid.double().requires_grad_(True), w.double().requires_grad_(True)
+    l2 = torch.log_softmax((h64 @ w64.t()) / temp, -1)
+    obj = (l2.gather(-1, lab.long()[:, None]).squeeze(-1) * f["dlogprobs"].double()).sum() + \
+          (-(l2.exp() * l2).sum(-1) * f["dentropy"].double()).sum()
+    obj.backward()
+    assert rel_l2(f["dhidden"], h64.grad) < 1e-5 and rel_l2(f["dweight"], w64.grad) < 1e-5
+    dh, dw = OM.backward(f["dlogprobs"], f["dentropy"], hid, w, lab, temp)
+    assert rel_l2(dh, f["dhidden"]) < 1e-6 and rel_l2(dw, f["dweight"]) < 1e-6
+
+
+def _ppo_scalar(x, a, lo=0.2, hi=0.28, c=3.0):
+    """One token by hand: returns (loss, dloss/dlogprob)."""
+    xc = max(-20.0, min(20.0, x))
+    r = math.exp(xc)
+    dr = r if -20.0 <= x <= 20.0 else 0.0
+    rc = max(1 - lo, min(1 + hi, r))
+    drc = dr if 1 - lo <= r <= 1 + hi else 0.0
+    l1, l2 = -a * r, -a * rc
+    if l1 > l2:
+        c1, dc1 = l1, -a * dr
+    elif l2 > l1:
+        c1, dc1 = l2, -a * drc
+    else:
+        c1, dc1 = l1, -a * 0.5 * (dr + drc)
+    if a < 0:
+        l3 = -a * c
+        if l3 < c1:
+            return l3, 0.0
+        if l3 == c1:
+            return c1, 0.5 * dc1
+    return c1, dc1
+
+
+def test_fixture_ppo_regions_by_hand():
+    f = load("ppo_regions.npz")
+    n = f["log_probs"].numel()
+    tot = 0.0
+    for k in range(n):
+        x = float(f["log_probs"][0, k] - f["old_log_probs"][0, k])  # the fp32 difference
+        val, g = _ppo_scalar(x, float(f["advantages"][0, k]))
+        tot += val
+        assert f["grad"][0, k].item() == pytest.approx(g / n, rel=2e-6, abs=1e-12), k
+    assert f["loss"].item() == pytest.approx(tot / n, rel=1e-6)
+    lp = f["log_probs"].clone().requires_grad_(True)
+    loss, m = OL.ppo_loss(lp, f["old_log_probs"], f["advantages"], f["response_mask"], clip_ratio_low=0.2,
+                          clip_ratio_high=0.28, clip_ratio_c=3.0)
+    loss.backward()
+    assert loss.item() == pytest.approx(f["loss"].item(), rel=1e-7) and torch.allclose(lp.grad, f["grad"], rtol=1e-6)
+    assert m["pg_clipfrac"] == pytest.approx(float(f["pg_clipfrac"])) and m["ppo_kl"] == pytest.approx(float(f["ppo_kl"]))
+
+
+def test_fixture_gspo_ragged_by_rows():
+    f = load("gspo_ragged.npz")
+    lo, hi = 3e-4, 4e-4
+    mask, adv, isw = f["response_mask"].double(), f["advantages"].double(), f["sampler_is_weights"].double()
+    nak = (f["log_probs"] - f["old_log_probs"]).double()
+    rows = []
+    for b in range(mask.shape[0]):
+        cnt = mask[b].sum().clamp(min=1)
+        s = math.exp(float((nak[b] * mask[b]).sum() / cnt))
+        sc = min(max(s, 1 - lo), 1 + hi)
+        per = torch.maximum(-adv[b] * s, -adv[b] * sc) * isw[b]
+        rows.append(float((per * mask[b]).sum() / cnt))  # token_reduce=mean
+    assert f["loss"].item() == pytest.approx(sum(rows) / len(rows), rel=1e-5)  # step-mean over all rows
+    lp = f["log_probs"].clone().requires_grad_(True)
+    loss, m = OL.gspo_loss(lp, f["old_log_probs"], f["advantages"], f["response_mask"], clip_ratio_low=lo,
+                           clip_ratio_high=hi, sampler_is_weights=f["sampler_is_weights"], token_reduce="mean",
+                           batch_reduce="step-mean")
+    loss.backward()
+    assert loss.item() == pytest.approx(f["loss"].item(), rel=1e-6) and rel_l2(lp.grad, f["grad"]) < 1e-6
+    assert (f["grad"][f["response_mask"] == 0] == 0).all()
+
+
+def test_fixture_sampler_boundaries():
+    f = load("sampler_boundaries.npz")
+    lr = (f["old_log_probs"] - f["sampler_log_probs"])
+    mask = f["response_mask"]
+    # masks follow from fp32 exp of each value against the fp32 thresholds, nothing else
+    w = torch.exp(lr.clamp(-20, 20))
+    keep = ((w >= 0.5) & (w <= 2.0)).float() * mask
+    assert torch.equal(f["rs_mask"], keep)
+    row_bad = ((lr < torch.log(torch.tensor(1e-4))) & mask.bool()).any(-1, keepdim=True)
+    assert torch.equal(f["veto_mask"], mask * (~row_bad).float())
+    assert torch.equal(f["is_weights"], (w * mask).clamp(max=2.0))
+    # both sides of every boundary are present
+    assert 0 < f["rs_mask"].sum() < mask.sum() and 0 < f["veto_rows"].sum() < f["veto_rows"].numel()
+    wq, rs, _ = OS.correction(f["old_log_probs"], f["sampler_log_probs"], mask, sampler_is="token",
+                              sampler_is_threshold=2.0, sampler_rs="token", sampler_rs_threshold=2.0)
+    assert torch.equal(rs, f["rs_mask"]) and torch.equal(wq, f["is_weights"])
+
+
+def test_fixture_grpo_groups():
+    f = load("grpo_groups.npz")
+    tlr, mask, gidx = f["token_level_rewards"], f["response_mask"], f["gidx"]
+    score = tlr.sum(-1)
+    for g in gidx.unique().tolist():
+        sel = gidx == g
+        k = int(sel.sum())
+        assert f["count"][g].item() == k
+        if k == 1:
+            assert f["mean"][g].item() == 0.0 and f["std"][g].item() == 1.0
+            assert (f["adv_norm1"][sel] == 0).all()
+            continue
+        mu = score[sel].mean()
+        sd = torch.sqrt(torch.clamp(torch.var(score[sel]), min=1e-6))  # library routine, unbiased
+        assert f["mean"][g].item() == pytest.approx(mu.item(), abs=1e-6)
+        assert f["std"][g].item() == pytest.approx(sd.item(), rel=1e-5)
+        want = ((score[sel] - mu) / (sd + 1e-6))[:, None] * mask[sel]
+        assert torch.allclose(f["adv_norm1"][sel], want, atol=1e-5)
+        assert torch.allclose(f["adv_norm0"][sel], (score[sel] - mu)[:, None] * mask[sel], atol=1e-6)
+    assert (f["adv_norm1"][gidx == 4].abs() < 1e-5).all()  # the all-equal group
+    for norm in (True, False):
+        got = OA.grpo_advantage(tlr, mask, gidx, 1e-6, norm)
+        assert torch.allclose(got, f[f"adv_norm{int(norm)}"], atol=1e-7)
+
+
+# ---------------------------------------------------------------------------------------------
+# GPU: HIP path vs fixtures
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_gpu_lmhead_matches_fixture():
+    from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    f = load("lmhead_n64_h128_v1000.npz")
+    hid = bf16(f["hidden_bf16"]).to(DEV).requires_grad_(True)
+    w = bf16(f["weight_bf16"]).to(DEV).requires_grad_(True)
+    lp, ent = linear_cross_entropy(hid, w, f["labels"].to(DEV), float(f["temperature"]), "none")
+    assert (lp.cpu() - f["logprobs"]).abs().max() < 1e-3
+    assert (ent.cpu() - f["entropy"]).abs().max() < 1e-3
+    torch.autograd.backward([lp, ent], [f["dlogprobs"].to(DEV), f["dentropy"].to(DEV)])
+    assert hid.grad.dtype == torch.bfloat16 and w.grad.dtype == torch.bfloat16
+    assert rel_l2(hid.grad, f["dhidden"]) < 2e-2 and rel_l2(w.grad, f["dweight"]) < 2e-2
+
+
+@pytest.mark.gpu
+def test_gpu_ppo_regions_match_fixture():
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    f = load("ppo_regions.npz")
+    t = {k: f[k].to(DEV) for k in ("log_probs", "old_log_probs", "advantages", "response_mask")}
+    t["log_probs"].requires_grad_(True)
+    loss, m = compute_loss_fn(DataProto.from_dict(tensors=t), "ppo",
+                              {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "clip_ratio_c": 3.0})
+    loss.backward()
+    assert loss.item() == pytest.approx(f["loss"].item(), rel=1e-4)
+    g = t["log_probs"].grad.cpu()
+    for k in range(g.numel()):
+        assert g[0, k].item() == pytest.approx(f["grad"][0, k].item(), rel=1e-5, abs=1e-9), k
+    for key in ("pg_clipfrac", "ppo_kl", "pg_clipfrac_lower"):
+        assert m[key] == pytest.approx(float(f[key]), rel=1e-4, abs=1e-7)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", ["padded", "packed"])
+def test_gpu_gspo_ragged_matches_fixture(layout):
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    f = load("gspo_ragged.npz")
+    lens = f["lengths"].tolist()
+    keys = ("log_probs", "old_log_probs", "advantages", "response_mask", "sampler_is_weights")
+    if layout == "padded":
+        t, meta = {k: f[k].to(DEV) for k in keys}, {}
+        want_g = f["grad"]
+    else:
+        t = {k: torch.cat([f[k][b, :l] for b, l in enumerate(lens)]).to(DEV) for k in keys}
+        meta = {"cu_seqlens": f["cu_seqlens"].to(DEV)}
+        want_g = torch.cat([f["grad"][b, :l] for b, l in enumerate(lens)])
+    t["log_probs"].requires_grad_(True)
+    loss, m = compute_loss_fn(DataProto.from_dict(tensors=t, meta_info=meta), "gspo",
+                              {"clip_ratio_low": 3e-4, "clip_ratio_high": 4e-4, "token_reduce": "mean",
+                               "batch_reduce": "step-mean"})
+    loss.backward()
+    assert loss.item() == pytest.approx(f["loss"].item(), rel=1e-4)
+    assert rel_l2(t["log_probs"].grad, want_g) < 1e-5
+    assert m["pg_clipfrac"] == pytest.approx(float(f["pg_clipfrac"]), abs=1e-7)
+    assert m["ppo_kl"] == pytest.approx(float(f["ppo_kl"]), rel=1e-4, abs=1e-8)
+
+
+@pytest.mark.gpu
+def test_gpu_sampler_boundaries_match_fixture():
+    from axon_amd.utils.rl import sampler as S
+    f = load("sampler_boundaries.npz")
+    old, samp, mask = (f[k].to(DEV) for k in ("old_log_probs", "sampler_log_probs", "response_mask"))
+    proto, rs, _ = S.compute_sampler_correction_and_rejection_mask(
+        old, samp, mask, sampler_is="token", sampler_is_threshold=2.0, sampler_rs="token", sampler_rs_threshold=2.0)
+    assert torch.equal(rs.cpu(), f["rs_mask"])  # bit-exact
+    assert rel_l2(proto.batch["sampler_is_weights"], f["is_weights"]) < 1e-6
+    _, veto, m = S.compute_sampler_correction_and_rejection_mask(old, samp, mask, sampler_token_veto_threshold=1e-4)
+    assert torch.equal(veto.cpu(), f["veto_mask"])
+    assert m["sampler_corr/sampler_is_veto_fraction"] == pytest.approx(float(f["veto_fraction"]))
+    col = f["old_log_probs"].reshape(-1, 1)
+    _, rows, _ = S.compute_sampler_correction_and_rejection_mask(
+        col.to(DEV), torch.zeros_like(col).to(DEV), torch.ones_like(col).to(DEV), sampler_token_veto_threshold=1e-4)
+    assert torch.equal(rows.cpu(), f["veto_rows"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("norm", [True, False])
+def test_gpu_grpo_groups_match_fixture(norm):
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.advantages import compute_advantage
+    f = load("grpo_groups.npz")
+    data = DataProto.from_dict(tensors={"token_level_rewards": f["token_level_rewards"].to(DEV),
+                                        "response_mask": f["response_mask"].to(DEV)})
+    data.non_tensor_batch["uid"] = np.array([f"p{int(g)}" for g in f["gidx"]], dtype=object)
+    out = compute_advantage(data, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6, "norm_adv_by_std": norm}})
+    want = f[f"adv_norm{int(norm)}"]
+    got = out.batch["advantages"].cpu()
+    assert torch.allclose(got, want, atol=2e-6, rtol=1e-5)
+    assert (got[f["response_mask"] == 0] == 0).all()
