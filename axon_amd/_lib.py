@@ -37,14 +37,16 @@ SIGNATURES: dict[str, tuple] = {
     "axon_fill_zero": (_i32, [_ptr, _i64, _ptr]),
     "axon_sampler_correction": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
                                        _i32, _f32, _f32, _i32, _f32, _ptr, _ptr, _ptr, _ptr, _ptr,
-                                       _ptr, _ptr]),
+                                       _ptr, _ptr, _ptr]),
+    "axon_reduce_partials_bytes": (_i64, [_i64]),
     "axon_loss_row_scale": (_i32, [_ptr, _ptr, _i64, _i64, _i32, _i32, _ptr, _ptr, _ptr, _ptr,
                                    _ptr, _ptr, _ptr]),
     "axon_policy_loss": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                                _ptr, _ptr, _f32, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
+                                _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr,
+                                _ptr]),
 }
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

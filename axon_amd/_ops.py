@@ -61,6 +61,17 @@ def _zeros(n, device, dtype=torch.float32):
     return torch.zeros(n, device=device, dtype=dtype)
 
 
+def _acc8(n_slots, device):
+    """The eight scalar sums a kernel returns; the library writes all of them unless there are no tokens."""
+    return _zeros(8, device) if n_slots == 0 else torch.empty(8, device=device, dtype=torch.float32)
+
+
+def _partials(n_slots, device):
+    """Uninitialised workspace for the per-workgroup partial sums of the elementwise kernels."""
+    nbytes = _lib.load().axon_reduce_partials_bytes(int(n_slots))
+    return torch.empty(max(nbytes // 4, 8), device=device, dtype=torch.float32)
+
+
 def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=True, want_sum=True):
     """Per-row (count, sum of (a-b)*mask, any-flag); see axon_row_stats."""
     lib = _lib.load()
@@ -134,12 +145,13 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
                                     threshold=log_veto if has_veto else 0.0)
     isw = torch.empty(rows.shape, device=dev, dtype=torch.float32) if is_mode else None
     new_mask = torch.empty(rows.shape, device=dev, dtype=torch.float32)
-    acc = _zeros(8, dev)
+    acc = _acc8(rows.n_slots, dev)
     check(
         lib.axon_sampler_correction(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
                                     rows.uniform_len, is_mode, float(is_threshold), rs_mode, float(rs_lr_lo),
                                     float(rs_lr_hi), int(has_veto), float(log_veto if has_veto else 0.0), ptr(cnt),
-                                    ptr(ssum), ptr(flag), ptr(isw), ptr(new_mask), ptr(acc), stream_ptr()),
+                                    ptr(ssum), ptr(flag), ptr(isw), ptr(new_mask), ptr(acc),
+                                    ptr(_partials(rows.n_slots, dev)), stream_ptr()),
         "axon_sampler_correction",
     )
     return isw, new_mask, acc
@@ -161,7 +173,8 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
                 num_program_steps=None, valid_count=None):
     """Forward + gradient of the clipped policy loss.  Returns (acc[8], grad like log_probs).
 
-    acc[0] is the loss; acc[1:5] are the metric sums (see axon_policy_loss).
+    acc[0] is the loss; acc[1:5] are the metric sums; acc[5] is the factor the returned
+    gradient still has to be multiplied by (see axon_policy_loss).
     """
     lib = _lib.load()
     require_device(log_probs, "policy_loss")
@@ -171,25 +184,31 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     isw = f32(is_weights) if is_weights is not None else None
     tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
 
-    cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
-    row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-    row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
-    prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
-    npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
-    nps = _i64_dev(num_program_steps, dev) if br == 2 else None
     valid = _i64_dev(valid_count, dev)
-    check(
-        lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
-                                ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
-                                stream_ptr()),
-        "axon_loss_row_scale",
-    )
     grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
-    acc = _zeros(8, dev)
+    acc = _acc8(rows.n_slots, dev)
+    # PPO with sum / token-mean needs no per-row quantity: one pass over the tokens, the
+    # division by the token count happens when the last workgroup has the total.
+    one_pass = kind == 0 and tr == 0 and br == 0
+    row_scale = row_mean = None
+    if not one_pass:
+        cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
+        row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
+        row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
+        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        check(
+            lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr,
+                                    br, ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
+                                    stream_ptr()),
+            "axon_loss_row_scale",
+        )
     check(
         lib.axon_policy_loss(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
-                             rows.n_slots, rows.uniform_len, ptr(row_scale), ptr(row_mean), 0.0, float(ratio_lo),
-                             float(ratio_hi), float(clip_c), ptr(grad), ptr(acc), stream_ptr()),
+                             rows.n_slots, rows.uniform_len, ptr(row_scale), ptr(row_mean), 1.0, int(one_pass),
+                             ptr(valid if one_pass else None), float(ratio_lo), float(ratio_hi), float(clip_c),
+                             ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
         "axon_policy_loss",
     )
     return acc, grad

@@ -47,6 +47,30 @@ __device__ __forceinline__ void block_sum(float (&v)[NV], float* lds /* [NV * 4]
   }
 }
 
+// Grid-wide sums without same-address atomics: a streaming kernel runs at most kMaxStreamBlocks
+// workgroups, each walking chunks blockIdx.x, blockIdx.x + gridDim.x, ... and leaving its NV
+// partial sums in partials[blockIdx.x][8]; reduce_partials_kernel (one workgroup, launched
+// next on the same stream) adds them in a fixed order, so results are reproducible.
+constexpr int kMaxStreamBlocks = 2048;  // 8 workgroups per CU
+constexpr int kPartialStride = 8;
+
+template <int NV>
+__device__ __forceinline__ void store_block_partials(float (&v)[NV], float* lds /* [NV * 4] */,
+                                                     float* partials) {
+  static_assert(NV <= kPartialStride, "partials row too small");
+  block_sum<NV>(v, lds);
+  if (threadIdx.x == 0) {
+    float* row = partials + (size_t)blockIdx.x * kPartialStride;
+#pragma unroll
+    for (int k = 0; k < kPartialStride; ++k) row[k] = (k < NV) ? v[k < NV ? k : 0] : 0.f;
+  }
+}
+
+inline unsigned stream_grid(int64_t n_slots) {
+  const int64_t chunks = (n_slots + kChunk - 1) / kChunk;
+  return (unsigned)(chunks < kMaxStreamBlocks ? chunks : kMaxStreamBlocks);
+}
+
 // Mask loads: four consecutive slots as floats.
 template <int KIND>
 __device__ __forceinline__ void load_mask4(const void* mask, int64_t i, float (&m)[4]) {

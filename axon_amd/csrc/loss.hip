@@ -1,6 +1,6 @@
 // (c) Elementwise stage-2/3 kernels: sampler correction and the clipped policy
 // loss with its gradient.  One read of every input, one write of every output;
-// scalar sums leave through one atomic per workgroup per accumulator.
+// scalar sums leave through per-workgroup partials that the last workgroup adds up.
 #include "common.h"
 
 namespace axon {
@@ -19,16 +19,21 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
     int is_mode, float is_thr, int rs_mode, float rs_lo, float rs_hi, int has_veto, float log_veto,
     const float* __restrict__ row_cnt, const float* __restrict__ row_sum,
     const int32_t* __restrict__ row_flag, float* __restrict__ isw, float* __restrict__ new_mask,
-    float* acc) {
+    float* partials) {
   __shared__ int32_t lds_cu[kLdsRows];
   __shared__ float lds_red[6 * (kBlock / kWave)];
-  const int64_t c0 = (int64_t)blockIdx.x * kChunk;
-  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
   const bool need_row = (is_mode == 2) || (rs_mode >= 2) || has_veto;
-  RowFinder rf;
-  if (need_row) rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
-
+  const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int64_t chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+  const int64_t c0 = chunk * kChunk;
+  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+  RowFinder rf;
+  if (need_row) {
+    __syncthreads();  // the previous chunk's row window is no longer read
+    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+  }
 #pragma unroll 1
   for (int it = 0; it < kIter; ++it) {
     const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
@@ -100,14 +105,48 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
       }
     }
   }
+  }  // chunk
   if (blockIdx.x == 0 && has_veto) {
     for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) a[4] += row_flag[r] ? 1.f : 0.f;
   }
-  block_sum<6>(a, lds_red);
-  if (threadIdx.x == 0) {
+  store_block_partials<6>(a, lds_red, partials);
+}
+
+// Adds the per-workgroup partial sums in a fixed order and writes acc[0..7].  post_normalize:
+// acc[0] (a plain masked sum) becomes the token-mean, acc[5] the factor 1/denominator.
+__global__ __launch_bounds__(1024) void reduce_partials_kernel(
+    const float* __restrict__ partials, int n_blocks, int post_normalize,
+    const int64_t* __restrict__ valid, float* __restrict__ acc) {
+  __shared__ float red[16][kPartialStride];
+  float t[kPartialStride];
 #pragma unroll
-    for (int k = 0; k < 6; ++k)
-      if (a[k] != 0.f) atomicAdd(acc + k, a[k]);
+  for (int k = 0; k < kPartialStride; ++k) t[k] = 0.f;
+  for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
+    const float4 lo4 = *reinterpret_cast<const float4*>(partials + (size_t)b * kPartialStride);
+    const float4 hi4 = *reinterpret_cast<const float4*>(partials + (size_t)b * kPartialStride + 4);
+    t[0] += lo4.x; t[1] += lo4.y; t[2] += lo4.z; t[3] += lo4.w;
+    t[4] += hi4.x; t[5] += hi4.y; t[6] += hi4.z; t[7] += hi4.w;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < kPartialStride; ++k) {
+    t[k] = wave_sum(t[k]);
+    if (lane == 0) red[wave][k] = t[k];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float tot[kPartialStride];
+    for (int k = 0; k < kPartialStride; ++k) {
+      float s = 0.f;
+      for (int w = 0; w < (int)(blockDim.x >> 6); ++w) s += red[w][k];
+      tot[k] = s;
+    }
+    if (post_normalize) {  // token-mean over a plain sum: the denominator is known only now
+      const float den = fmaxf(valid != nullptr ? (float)valid[0] : tot[4], 1.f);
+      tot[0] = tot[0] / den;
+      tot[5] = 1.f / den;
+    }
+    for (int k = 0; k < kPartialStride; ++k) acc[k] = tot[k];
   }
 }
 
@@ -166,17 +205,22 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     const float* __restrict__ logp, const float* __restrict__ oldp, const float* __restrict__ adv,
     const void* __restrict__ mask, const float* __restrict__ isw, const int32_t* __restrict__ cu,
     int64_t n_rows, int64_t n_slots, int64_t uniform_len, const float* __restrict__ row_scale,
-    const float* __restrict__ row_mean, float uniform_scale, float lo, float hi,
-    float clip_c, float* __restrict__ grad, float* acc) {
+    const float* __restrict__ row_mean, float uniform_scale, float lo, float hi, float clip_c,
+    float* __restrict__ grad, float* partials) {
   __shared__ int32_t lds_cu[kLdsRows];
-  __shared__ float lds_red[5 * (kBlock / kWave)];
-  const int64_t c0 = (int64_t)blockIdx.x * kChunk;
-  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+  __shared__ float lds_red[6 * (kBlock / kWave)];
   const bool need_row = (row_scale != nullptr) || (KIND == 1);
+  const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
+  float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int64_t chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+  const int64_t c0 = chunk * kChunk;
+  const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
   RowFinder rf;
-  if (need_row) rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
-
-  float a[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  if (need_row) {
+    __syncthreads();  // the previous chunk's row window is no longer read
+    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+  }
 #pragma unroll 1
   for (int it = 0; it < kIter; ++it) {
     const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
@@ -244,17 +288,20 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     else
       for (int j = 0; j < 4 && i + j < n_slots; ++j) grad[i + j] = gv[j];
   }
-  block_sum<5>(a, lds_red);
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int k = 0; k < 5; ++k)
-      if (a[k] != 0.f) atomicAdd(acc + k, a[k]);
-  }
+  }  // chunk
+  if (blockIdx.x == 0 && threadIdx.x == 0) a[5] = 1.f;  // gradient factor unless post-normalised
+  store_block_partials<6>(a, lds_red, partials);
 }
 
 }  // namespace axon
 
 using namespace axon;
+
+extern "C" int64_t axon_reduce_partials_bytes(int64_t n_slots) {
+  if (n_slots < 0) return AXON_ERR_ARG;
+  const int64_t blocks = n_slots > 0 ? (int64_t)stream_grid(n_slots) : 1;
+  return blocks * kPartialStride * (int64_t)sizeof(float);
+}
 
 static int check_rows2(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
                        bool need_row) {
@@ -270,28 +317,31 @@ extern "C" int axon_sampler_correction(
     int64_t n_rows, int64_t n_slots, int64_t uniform_len, int is_mode, float is_thr, int rs_mode,
     float rs_lo, float rs_hi, int has_veto, float log_veto, const float* row_cnt,
     const float* row_sum, const int32_t* row_flag, float* isw, float* new_mask, float* acc,
-    void* stream) {
+    float* partials, void* stream) {
   const bool need_row = (is_mode == 2) || (rs_mode >= 2) || has_veto;
   int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
   if (rc != AXON_OK) return rc;
   if (n_slots == 0) return AXON_OK;
-  if (!oldp || !samp || !mask || !new_mask || !acc) return AXON_ERR_ARG;
+  if (!oldp || !samp || !mask || !new_mask || !acc || !partials) return AXON_ERR_ARG;
   if (is_mode < 0 || is_mode > 2 || rs_mode < 0 || rs_mode > 3) return AXON_ERR_ARG;
   if (is_mode != 0 && isw == nullptr) return AXON_ERR_ARG;
   if ((is_mode == 2 || rs_mode >= 2) && (!row_sum || !row_cnt)) return AXON_ERR_ARG;
   if (has_veto && !row_flag) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
-  const dim3 g((unsigned)((n_slots + kChunk - 1) / kChunk)), blk(kBlock);
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
   if (mask_kind == AXON_MASK_F32)
     hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_F32>, g, blk, 0, (hipStream_t)stream,
                        oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
                        rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
-                       acc);
+                       partials);
   else
     hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_I64>, g, blk, 0, (hipStream_t)stream,
                        oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
                        rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
-                       acc);
+                       partials);
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, partials,
+                     (int)g.x, 0, (const int64_t*)nullptr, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
@@ -320,28 +370,33 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
                                 const void* mask, int mask_kind, const float* isw,
                                 const int32_t* cu, int64_t n_rows, int64_t n_slots,
                                 int64_t uniform_len, const float* row_scale, const float* row_mean,
-                                float uniform_scale, float ratio_lo, float ratio_hi, float clip_c,
-                                float* grad, float* acc, void* stream) {
+                                float uniform_scale, int post_normalize, const int64_t* valid,
+                                float ratio_lo, float ratio_hi, float clip_c, float* grad,
+                                float* acc, float* partials, void* stream) {
   const bool need_row = (row_scale != nullptr) || (kind == 1);
   int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
   if (rc != AXON_OK) return rc;
   if (n_slots == 0) return AXON_OK;
   if (kind != 0 && kind != 1) return AXON_ERR_ARG;
-  if (!logp || !oldp || !adv || !mask || !grad || !acc) return AXON_ERR_ARG;
+  if (!logp || !oldp || !adv || !mask || !grad || !acc || !partials) return AXON_ERR_ARG;
+  if (post_normalize && (row_scale != nullptr || kind != 0)) return AXON_ERR_ARG;
   if (kind == 1 && !row_mean) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
-  const dim3 g((unsigned)((n_slots + kChunk - 1) / kChunk)), blk(kBlock);
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
   const hipStream_t st = (hipStream_t)stream;
 #define AXON_LAUNCH_PL(MK, KD)                                                                   \
   hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
                      n_rows, n_slots, uniform_len, row_scale, row_mean, uniform_scale, ratio_lo, \
-                     ratio_hi, clip_c, grad, acc)
+                     ratio_hi, clip_c, grad, partials)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0); else AXON_LAUNCH_PL(AXON_MASK_F32, 1);
   } else {
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_I64, 0); else AXON_LAUNCH_PL(AXON_MASK_I64, 1);
   }
 #undef AXON_LAUNCH_PL
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
+                     post_normalize, valid, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

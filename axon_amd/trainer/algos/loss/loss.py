@@ -31,16 +31,16 @@ class _ClippedPolicyLoss(torch.autograd.Function):
             kind, log_probs, batch["old_log_probs"], batch["advantages"], batch["response_mask"],
             batch["sampler_is_weights"], rows, **hp,
         )
-        ctx.save_for_backward(grad)
+        ctx.save_for_backward(grad, acc)
         ctx.in_dtype = log_probs.dtype
-        ctx.acc = acc
         ctx.mark_non_differentiable(acc)
         return acc[0].clone(), acc
 
     @staticmethod
     def backward(ctx, g_loss, _g_acc):
-        (grad,) = ctx.saved_tensors
-        return (grad * g_loss).to(ctx.in_dtype), None, None, None, None
+        grad, acc = ctx.saved_tensors
+        # acc[5]: the 1/denominator a one-pass token-mean leaves to this multiply
+        return (grad * (g_loss * acc[5])).to(ctx.in_dtype), None, None, None, None
 
 
 def _run(kind: int, data, config, default_token_reduce: str):

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 1
+#define AXON_AMD_ABI_VERSION 2
 
 enum {
   AXON_OK = 0,
@@ -160,6 +160,15 @@ int axon_row_broadcast_mask(const float* row_scalar, const void* mask, int mask_
 
 int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 0 */
 
+/* Bytes of the `partials` workspace of axon_sampler_correction / axon_policy_loss for
+ * n_slots tokens (8 floats per workgroup; at most 2048 workgroups walk the tokens).  The scalar sums of those two
+ * kernels (the reference's masked_mean metrics and agg_loss totals,
+ * axon/utils/torch/ops.py:131-145, axon/trainer/algos/loss/utils.py:224-251) are added
+ * from per-workgroup partials in a fixed order by a one-workgroup kernel launched right
+ * after, so results are reproducible run to run and no atomics are involved.
+ * Contents need no initialisation. */
+int64_t axon_reduce_partials_bytes(int64_t n_slots);
+
 /* Sampler/trainer correction, compute_sampler_correction_and_rejection_mask
  * (axon/utils/rl/sampler.py:334-446).  lr = old - sampler.
  *   is_mode: 0 off, 1 token, 2 sequence        (sampler.py:206-231)
@@ -170,16 +179,18 @@ int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 
  * row_cnt,row_sum,row_flag: outputs of axon_row_stats(old, sampler, mask, flag_mode 1,
  * log_veto); may be NULL when neither a row-level mode nor the veto is on.
  * Outputs: is_weights [n_slots] (NULL if is_mode 0), new_mask [n_slots] fp32 =
- * mask * rs * veto.  acc[8] (zero-filled by caller) receives sums for the
- * metrics: [0] sum mask, [1] sum is_w(before truncation)*mask, [2] sum (1-rs)*mask,
- * [3] sum catastrophic*mask, [4] rows vetoed, [5] sum truncated is_w * mask. */
+ * mask * rs * veto.  acc[8] (written, not accumulated; untouched when n_slots == 0)
+ * receives sums for the metrics: [0] sum mask,
+ * [1] sum is_w(before truncation)*mask, [2] sum (1-rs)*mask, [3] sum catastrophic*mask,
+ * [4] rows vetoed, [5] sum truncated is_w * mask.
+ * partials: workspace of axon_reduce_partials_bytes(n_slots). */
 int axon_sampler_correction(const float* old_logp, const float* sampler_logp, const void* mask,
                             int mask_kind, const int32_t* cu_seqlens, int64_t n_rows,
                             int64_t n_slots, int64_t uniform_len, int is_mode, float is_threshold,
                             int rs_mode, float rs_lr_lo, float rs_lr_hi, int has_veto,
                             float log_veto, const float* row_cnt, const float* row_sum,
                             const int32_t* row_flag, float* is_weights, float* new_mask,
-                            float* acc, void* stream);
+                            float* acc, float* partials, void* stream);
 
 /* Per-row weights of agg_loss (axon/trainer/algos/loss/utils.py:120-251) folded
  * into one multiplier per row, plus GSPO's per-row mean log-ratio:
@@ -204,16 +215,25 @@ int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_ro
  * evaluated in double by the caller and rounded to fp32 (what torch.clamp does
  * with Python scalars).  clip_c: dual-clip constant (> 1), PPO only.
  * row_scale: per-row multiplier from axon_loss_row_scale, or NULL with
- * uniform_scale (sum / token-mean with a known denominator).
- * Outputs grad[n_slots] = d loss / d log_probs and acc[8] (zero-filled by
- * caller): [0] loss, [1] sum mask*(pg2>pg1), [2] sum mask*(-(logp-old)),
- * [3] sum mask*((c1>pg3)&(A<0)), [4] sum mask. */
+ * uniform_scale applied to every token.
+ * post_normalize != 0 (PPO with row_scale NULL only): `sum` / `token-mean`
+ * aggregation in ONE pass over the tokens (utils.py:224-229): the kernel sums
+ * uniform_scale * loss * mask, then divides the total by max(valid_count[0], 1), or by
+ * max(sum mask, 1) when valid_count is NULL; grad[] is left WITHOUT that division and
+ * acc[5] returns the factor 1/denominator the caller multiplies the gradient by
+ * (it multiplies by the upstream gradient anyway).  Otherwise acc[5] = 1.
+ * Outputs grad[n_slots] = d loss / d log_probs and acc[8] (written, not
+ * accumulated; untouched when n_slots == 0): [0] loss,
+ * [1] sum mask*(pg2>pg1), [2] sum mask*(-(logp-old)), [3] sum mask*((c1>pg3)&(A<0)),
+ * [4] sum mask, [5] gradient factor.
+ * partials: workspace of axon_reduce_partials_bytes(n_slots). */
 int axon_policy_loss(int kind, const float* logp, const float* old_logp, const float* adv,
                      const void* mask, int mask_kind, const float* is_weights,
                      const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
                      int64_t uniform_len, const float* row_scale, const float* row_mean,
-                     float uniform_scale, float ratio_lo, float ratio_hi, float clip_c,
-                     float* grad, float* acc, void* stream);
+                     float uniform_scale, int post_normalize, const int64_t* valid_count,
+                     float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
+                     float* partials, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,7 +30,8 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/axon_amd.h but not exported"
     assert declared == set(_lib.SIGNATURES), "ctypes bindings and header disagree"
-    assert lib.axon_amd_abi_version() == 1
+    m = re.search(r"#define AXON_AMD_ABI_VERSION (\d+)", header)
+    assert lib.axon_amd_abi_version() == int(m.group(1)) == _lib.ABI_VERSION
     assert lib.axon_amd_error_string(0) == b"ok"
     assert b"workspace" in lib.axon_amd_error_string(-3)
 
@@ -43,8 +44,9 @@ def test_workspace_queries_and_argument_errors_without_gpu():
     assert lib.axon_lmhead_bwd_workspace_bytes(64, 128, 1000, 256) > 0
     # null pointers are rejected before any launch
     assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None) == -1
-    assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0.8, 1.2, 3.0,
-                                None, None, None) == -1
+    assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0, None, 0.8, 1.2,
+                                3.0, None, None, None, None) == -1
+    assert lib.axon_reduce_partials_bytes(4097) == 2 * 8 * 4 and lib.axon_reduce_partials_bytes(1 << 30) == 2048 * 32 and lib.axon_reduce_partials_bytes(-1) == -1
     assert lib.axon_fill_zero(None, 3, None) == -1
 
 
