@@ -24,6 +24,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E, published
 
 WORKLOADS = {
     # name: (tokens, hidden, vocab, group size, seed)
@@ -42,6 +43,8 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (debugging)")
     ap.add_argument("--vocab-chunk", type=int, default=0)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
+    ap.add_argument("--hbm-tokens", type=int, default=1 << 26,
+                    help="token count for the HBM-bound stage-2/3 kernels' bandwidth figures; 0 disables them")
     return ap.parse_args()
 
 
@@ -76,6 +79,73 @@ def cpu_baseline(hid, w, lab, budget_s):
         "value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",
         "sample": f"{n} of the workload's tokens, full hidden and vocab, fwd+loss+bwd, {t:.1f} s; linear in tokens",
     }
+
+
+def hbm_kernels(n_tokens, dev):
+    """Stage-2/3 kernels on a packed batch large enough to show the bandwidth asymptote
+    (same lognormal length law as the headline workload).  Each figure is algorithmic bytes
+    (one read of every input, one write of every output, fp32) over the median of 20 timed
+    calls of the whole operator, every launch it makes included."""
+    import math
+
+    import torch
+
+    from axon_amd import _ops, workloads as W
+
+    g = torch.Generator().manual_seed(11)
+    lens = torch.exp(torch.randn(max(n_tokens // 300, 8), generator=g) * 0.8 + 6.5).round().clamp(32, 8192).long()
+    lens = lens[: int((torch.cumsum(lens, 0) <= n_tokens).sum())].tolist()
+    if n_tokens - sum(lens):
+        lens.append(n_tokens - sum(lens))
+    cu = W.cu_from_lengths(lens).to(dev)
+    gd = torch.Generator(device=dev).manual_seed(12)
+    old = -torch.empty(n_tokens, device=dev).exponential_(1.0, generator=gd)
+    new = old + 0.05 * torch.randn(n_tokens, device=dev, generator=gd)
+    samp = old + 0.01 * torch.randn(n_tokens, device=dev, generator=gd)
+    adv = torch.randn(n_tokens, device=dev, generator=gd)
+    mask = torch.ones(n_tokens, device=dev)
+    mask[cu[:-1].long()] = 0
+    rows = _ops.rows_of(new, cu)
+    seq_scalar = torch.randn(len(lens), device=dev, generator=gd)
+
+    def median_ms(fn, iters=20, warm=5):
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(iters):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            b.synchronize()
+            ts.append(a.elapsed_time(b))
+        return sorted(ts)[len(ts) // 2]
+
+    ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
+    gspo = dict(token_reduce="mean", batch_reduce="step-mean", ratio_lo=1 - 3e-4, ratio_hi=1 + 4e-4, clip_c=3.0)
+    corr = dict(is_mode=1, is_threshold=2.0, rs_mode=1, rs_lr_lo=-math.log(2.0), rs_lr_hi=math.log(2.0))
+    x = torch.empty_like(old)
+    cases = [  # name, bytes per token, callable
+        ("device-to-device copy (calibration)", 8, lambda: x.copy_(old)),
+        ("policy_loss_kernel: PPO/DAPO loss + gradient, sum/token-mean (one pass)", 20,
+         lambda: _ops.policy_loss(0, new, old, adv, mask, None, rows, **ppo)),
+        ("row_stats + policy_loss_kernel: GSPO loss + gradient (two reads of log_probs, old, mask)", 32,
+         lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
+        ("sampler_correction_kernel: token IS weights + rejection mask", 20,
+         lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=None, **corr)),
+        ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads)", 32,
+         lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4), **corr)),
+        ("row_stats_kernel: per-sequence count and masked sum", 12, lambda: _ops.row_stats(new, old, mask, rows)),
+        ("row_broadcast_kernel: GRPO advantage = per-sequence scalar * mask", 8,
+         lambda: _ops.row_broadcast_mask(seq_scalar, mask, rows)),
+    ]
+    out = []
+    for name, bpt, fn in cases:
+        ms = median_ms(fn)
+        gbs = n_tokens * bpt / (ms * 1e-3) / 1e9
+        out.append({"kernel": name, "bytes_per_token": bpt, "ms": ms, "achieved": gbs, "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS})
+    return {"tokens": n_tokens, "sequences": len(lens), "bound": "hbm", "kernels": out}
 
 
 def main():
@@ -196,6 +266,10 @@ def main():
         "roofline": roofline,
         "parity": {"logprob_max_abs_err_subset": lp_err},
     }
+    if args.hbm_tokens > 0:
+        del hd, wd, dh, dw
+        torch.cuda.empty_cache()
+        out["hbm_kernels"] = hbm_kernels(args.hbm_tokens, dev)
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(hid, w, lab, args.cpu_seconds)
     print(json.dumps(out))

@@ -161,7 +161,7 @@ int axon_row_broadcast_mask(const float* row_scalar, const void* mask, int mask_
 int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 0 */
 
 /* Bytes of the `partials` workspace of axon_sampler_correction / axon_policy_loss for
- * n_slots tokens (8 floats per workgroup; at most 2048 workgroups walk the tokens).  The scalar sums of those two
+ * n_slots tokens (8 floats per workgroup; at most 16384 workgroups walk the tokens).  The scalar sums of those two
  * kernels (the reference's masked_mean metrics and agg_loss totals,
  * axon/utils/torch/ops.py:131-145, axon/trainer/algos/loss/utils.py:224-251) are added
  * from per-workgroup partials in a fixed order by a one-workgroup kernel launched right
