@@ -28,6 +28,7 @@
 // quad: per-n statistics need no cross-lane traffic beyond lane^32, and stores
 // to an [n][m] output are 4-element vectors.
 #pragma once
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -54,6 +55,7 @@ struct GemmOperands {
 // previous tile and must be ignored by the epilogue.
 struct TilePos {
   int m0, n0, m_lo, n_lo;
+  int kt0 = 0;  // k-tile this workgroup starts its walk over k at (it wraps around)
 };
 
 // Position of this lane inside the workgroup tile.
@@ -86,7 +88,12 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 // ---------------------------------------------------------------------------------------
 // DmaLoop
 // ---------------------------------------------------------------------------------------
-struct DmaLoop {
+// C3, C0, C1, C2: how many of a wave's 16 DMA instructions for the next-but-one k-tile are issued
+// under the last k-step of the current tile (right after the barrier that frees the stage) and
+// under k-steps 0, 1, 2 of the next tile.
+template <int C3, int C0, int C1, int C2>
+struct DmaLoopT {
+  static_assert(C3 + C0 + C1 + C2 == 16 && C3 >= 1, "16 DMA instructions per wave and k-tile");
   static constexpr int kBK = 64;
   static constexpr int kRowBytes = 128;                    // 64 bf16
   static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
@@ -104,6 +111,7 @@ struct DmaLoop {
     t.n0 = min(n0, g.n_rows - kTile);
     t.m_lo = m0 - t.m0;
     t.n_lo = n0 - t.n0;
+    t.kt0 = ((tm + 2 * tn) & 7) % (g.k / kBK);
     return t;
   }
 
@@ -151,14 +159,24 @@ struct DmaLoop {
     bf16x8 af[2][4], bf[2][4];
     const int kt_n = g.k / kBK;
 
-    auto issue = [&](int stage_off, int kt) {
-      const int ko = kt * kRowBytes;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
+    // byte offset inside a row of k-tile number kt of this workgroup's walk
+    auto k_byte = [&](int kt) {
+      const int ks = kt + t.kt0;
+      return (ks >= kt_n ? ks - kt_n : ks) * kRowBytes;
+    };
+    // instruction idx of the 16 that bring one k-tile: even = A, odd = B
+    auto dma_one = [&](int stage_off, int ko, int idx) {
+      const int j = idx >> 1;
+      if ((idx & 1) == 0)
         dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + stage_off + j * 8 * kRowBytes);
+      else
         dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b,
               dst + stage_off + kOperandBytes + j * 8 * kRowBytes);
-      }
+    };
+    auto issue = [&](int stage_off, int kt, int first, int count) {
+#pragma unroll
+      for (int idx = 0; idx < 16; ++idx)
+        if (idx >= first && idx < first + count) dma_one(stage_off, k_byte(kt), idx);
     };
     auto read_frags = [&](int stage_off, int kk, int set) {
 #pragma unroll
@@ -167,18 +185,43 @@ struct DmaLoop {
         bf[set][i] = *reinterpret_cast<const bf16x8*>(smem + stage_off + fb[kk] + i * 32 * kRowBytes);
       }
     };
-    auto mfma_block = [&](int set) {
+    // One k-step: 16 MFMAs on fragment set `mm_set`; under them the eight fragments of the next
+    // k-step are read into the other set (one per MFMA, in the order the next step consumes them)
+    // and `vmem` DMA instructions [dma_first, dma_first + vmem) of k-tile dma_kt are issued, evenly
+    // spread.  Source order is issue order: an LDS DMA and a fragment read are both LDS accesses
+    // to the compiler, so it will not move one across the other.
+    auto step = [&](int rd_stage, int rd_kk, int mm_set, int dma_stage, int dma_kt, int dma_first,
+                    auto vmem_c) {
+      constexpr int vmem = decltype(vmem_c)::value;
+      const int rd_set = mm_set ^ 1;
+      const int ko = k_byte(dma_kt);
+      const char* const fr = smem + rd_stage;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int m = 0; m < 16; ++m) {
+        const int before = (m * vmem) / 16, due = ((m + 1) * vmem) / 16 - before;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[set][i], bf[set][j], acc[i][j], 0, 0, 0);
+        for (int d = 0; d < due; ++d) dma_one(dma_stage, ko, dma_first + before + d);
+        // a0 b0 b1 b2 b3 a1 a2 a3
+        if (m == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(fr + fa[rd_kk]);
+        if (m >= 1 && m <= 4)
+          bf[rd_set][m - 1] = *reinterpret_cast<const bf16x8*>(fr + fb[rd_kk] + (m - 1) * 32 * kRowBytes);
+        if (m >= 5 && m <= 7)
+          af[rd_set][m - 4] = *reinterpret_cast<const bf16x8*>(fr + fa[rd_kk] + (m - 4) * 32 * kRowBytes);
+        acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mm_set][m >> 2], bf[mm_set][m & 3],
+                                                                     acc[m >> 2][m & 3], 0, 0, 0);
+        if (due == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (due == 2) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        if (due > 2) __builtin_amdgcn_sched_group_barrier(0x020, 16, 0);
+        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     };
 
-    // prologue: tiles 0 and 1 in flight, fragments of (tile 0, kk 0) in set 0
-    issue(0, 0);
-    issue(kStageBytes, min(1, kt_n - 1));
-    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): this wave's part of tile 0 has landed
+    // prologue: tile 0 whole, the first C3 instructions of tile 1; fragments of (tile 0, kk 0) in set 0
+    issue(0, 0, 0, 16);
+    issue(kStageBytes, min(1, kt_n - 1), 0, C3);
+    __builtin_amdgcn_s_waitcnt(C3 == 16 ? 0x4F70 : (0x0F70 | (C3 & 15)));  // vmcnt(C3): tile 0 has landed
     __builtin_amdgcn_s_barrier();
     read_frags(0, 0, 0);
     __builtin_amdgcn_sched_barrier(0);
@@ -186,37 +229,16 @@ struct DmaLoop {
     int cur = 0;
     for (int kt = 0; kt < kt_n; ++kt) {
       const int nxt = cur ^ kStageBytes;
-#pragma unroll
-      for (int kk = 0; kk < 3; ++kk) {
-        read_frags(cur, kk + 1, (kk + 1) & 1);
-        mfma_block(kk & 1);
-        // issue order: one fragment read per MFMA for the first eight, then eight MFMAs
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      const int kt1 = min(kt + 1, kt_n - 1);  // past the end: refetches the last tile, never consumed
+      // k-steps 0..2: fragments of the next k-step, the rest of tile kt+1 into the other stage
+      step(cur, 1, 0, nxt, kt1, C3, std::integral_constant<int, C0>{});
+      step(cur, 2, 1, nxt, kt1, C3 + C0, std::integral_constant<int, C1>{});
+      step(cur, 3, 0, nxt, kt1, C3 + C0 + C1, std::integral_constant<int, C2>{});
       // last k-step of this tile: the other stage must have landed for every wave, and every wave
       // must be done reading this stage (its kk=3 fragments are in registers) before it is refilled.
       __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
-      issue(cur, min(kt + 2, kt_n - 1));   // past the end: refetches the last tile, never consumed
-      read_frags(nxt, 0, 0);
-      mfma_block(1);
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+      step(nxt, 0, 1, cur, min(kt + 2, kt_n - 1), 0, std::integral_constant<int, C3>{});
       cur = nxt;
     }
     // DMA issued for tiles past the end is still in flight; drain it before LDS is reused
@@ -224,6 +246,8 @@ struct DmaLoop {
     __builtin_amdgcn_s_barrier();
   }
 };
+
+using DmaLoop = DmaLoopT<4, 4, 4, 4>;
 
 // ---------------------------------------------------------------------------------------
 // RegLoop: loads through registers with per-row clamping; any k % BK == 0
