@@ -40,7 +40,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kTile = 256;       // tile edge in m and n
 constexpr int kWaveTile = 128;   // per-wave edge
 constexpr int kGemmThreads = 256;
-constexpr int kGemmLdsBytes = 131072;  // both main loops fit; also the staging area of the dlogit epilogue
+constexpr int kGemmLdsBytes = 163840;  // both main loops fit; also the staging area of the dlogit epilogue
 
 struct GemmOperands {
   const __bf16* a;  // [m_rows][lda], K-contiguous
@@ -111,7 +111,10 @@ struct DmaLoopT {
     t.n0 = min(n0, g.n_rows - kTile);
     t.m_lo = m0 - t.m0;
     t.n_lo = n0 - t.n0;
-    t.kt0 = ((tm + 2 * tn) & 7) % (g.k / kBK);
+#ifndef AXON_K_SKEW
+#define AXON_K_SKEW 0
+#endif
+    t.kt0 = (AXON_K_SKEW) % (g.k / kBK);
     return t;
   }
 
@@ -247,7 +250,166 @@ struct DmaLoopT {
   }
 };
 
-using DmaLoop = DmaLoopT<4, 4, 4, 4>;
+// ---------------------------------------------------------------------------------------
+// DmaLoop32: the same k-tile of 64 and LDS layout, but the 160 KB of LDS hold THREE slots for
+// the A operand and TWO for B.  B for k-tile t+2 is issued in one burst of eight instructions per
+// wave right after the barrier that frees its slot (one k-tile of time to land, half the burst
+// of a symmetric double buffer); A for k-tile t+2 is issued a whole k-tile earlier, spread
+// under the MFMAs of k-steps 0..2, into the slot freed one barrier before.
+// ---------------------------------------------------------------------------------------
+struct DmaLoop32 {
+  static constexpr int kBK = 64;
+  static constexpr int kRowBytes = 128;
+  static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
+  static constexpr int kBBase = 3 * kOperandBytes;         // A slots at 0/32/64 KB, B slots at 96/128 KB
+  static constexpr bool kShiftsEdgeTiles = true;
+
+  __device__ static __forceinline__ TilePos place(const GemmOperands& g, int tm, int tn) {
+    return DmaLoopT<4, 4, 4, 4>::place(g, tm, tn);
+  }
+
+  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
+                                             f32x16 (&acc)[4][4], char* smem) {
+    using Base = DmaLoopT<4, 4, 4, 4>;
+    const LanePos lp;
+    // DMA addressing as in DmaLoopT: one instruction = 8 rows x 128 B, wave w owns rows [64w, 64w+64)
+    const int lrow = lp.lane >> 3;
+    const int sw_even = (lp.lane >> 4) & 7;
+    const int sw_odd = (4 + (lp.lane >> 4)) & 7;
+    const int row_a = (lp.wave * 64 + lrow) * (int)g.lda * 2;
+    const int row_b = (lp.wave * 64 + lrow) * (int)g.ldb * 2;
+    const int va_e = row_a + (((lp.lane & 7) ^ sw_even) << 4);
+    const int va_o = row_a + (((lp.lane & 7) ^ sw_odd) << 4);
+    const int vb_e = row_b + (((lp.lane & 7) ^ sw_even) << 4);
+    const int vb_o = row_b + (((lp.lane & 7) ^ sw_odd) << 4);
+    const int step_a = (int)g.lda * 16, step_b = (int)g.ldb * 16;
+    const __bf16* base_a = g.a + (int64_t)t.m0 * g.lda;
+    const __bf16* base_b = g.b + (int64_t)t.n0 * g.ldb;
+    const __amdgpu_buffer_rsrc_t ra =
+        __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rb =
+        __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
+    char* const dst = smem + lp.wave * 64 * kRowBytes;
+
+    const int sw = (lp.l32 >> 1) & 7;
+    int fa[4], fb[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      fa[kk] = (lp.wm * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
+      fb[kk] = kBBase + (lp.wn * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
+    }
+
+    zero_acc(acc);
+    bf16x8 af[2][4], bf[2][4];
+    const int kt_n = g.k / kBK;
+    auto k_byte = [&](int kt) {
+      const int ks = min(kt, kt_n - 1) + t.kt0;  // past the end: refetches the last tile, never consumed
+      return (ks >= kt_n ? ks - kt_n : ks) * kRowBytes;
+    };
+    auto dma_a = [&](int slot_off, int ko, int j) {
+      Base::dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + slot_off + j * 8 * kRowBytes);
+    };
+    auto dma_b = [&](int slot_off, int ko, int j) {
+      Base::dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b, dst + kBBase + slot_off + j * 8 * kRowBytes);
+    };
+    // One k-step: 16 MFMAs on fragment set mm_set; the eight fragments of the next k-step are read
+    // one per MFMA; `NA` A instructions [a_first, a_first + NA) and `NB` B instructions [0, NB) are
+    // issued in between, in source order (the compiler keeps LDS DMA and LDS reads ordered).
+    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, int a_ko, int a_first,
+                    auto na_c, int b_slot, int b_ko, auto nb_c) {
+      constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
+      constexpr int vmem = NA + NB;
+      const int rd_set = mm_set ^ 1;
+#pragma unroll
+      for (int m = 0; m < 16; ++m) {
+#ifdef AXON_B_FRONT
+        const int before = (NB > 0) ? min(m, NB) : (m * vmem) / 16;
+        const int due = (NB > 0) ? (m < NB ? 1 : 0) : ((m + 1) * vmem) / 16 - before;
+#else
+        const int before = (m * vmem) / 16, due = ((m + 1) * vmem) / 16 - before;
+#endif
+#pragma unroll
+        for (int d = 0; d < due; ++d) {
+          const int idx = before + d;  // B first: it has the shorter time to land
+          if (idx < NB) dma_b(b_slot, b_ko, idx);
+          else dma_a(a_slot, a_ko, a_first + idx - NB);
+        }
+        if (m == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk]);
+        if (m >= 1 && m <= 4)
+          bf[rd_set][m - 1] =
+              *reinterpret_cast<const bf16x8*>(smem + rd_b + fb[rd_kk] + (m - 1) * 32 * kRowBytes);
+        if (m >= 5 && m <= 7)
+          af[rd_set][m - 4] =
+              *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk] + (m - 4) * 32 * kRowBytes);
+        acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mm_set][m >> 2], bf[mm_set][m & 3],
+                                                                     acc[m >> 2][m & 3], 0, 0, 0);
+        if (due == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (due >= 2) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I8 = std::integral_constant<int, 8>;
+#ifndef AXON_A_SPREAD
+#define AXON_A_SPREAD 3, 3, 2
+#endif
+    constexpr int kA[3] = {AXON_A_SPREAD};  // A instructions under k-steps 0, 1, 2
+    static_assert(kA[0] + kA[1] + kA[2] == 8, "eight A instructions per wave and k-tile");
+    using A0 = std::integral_constant<int, kA[0]>;
+    using A1 = std::integral_constant<int, kA[1]>;
+    using A2 = std::integral_constant<int, kA[2]>;
+
+    // prologue: tiles 0 and 1 whole (A slots 0, 1; B slots 0, 1)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dma_a(0, k_byte(0), j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dma_b(0, k_byte(0), j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, k_byte(1), j);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dma_b(kOperandBytes, k_byte(1), j);
+    __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 has landed
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      af[0][i] = *reinterpret_cast<const bf16x8*>(smem + fa[0] + i * 32 * kRowBytes);
+      bf[0][i] = *reinterpret_cast<const bf16x8*>(smem + fb[0] + i * 32 * kRowBytes);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    int a_cur = 0, b_cur = 0;  // slots of the tile being consumed
+    for (int kt = 0; kt < kt_n; ++kt) {
+      const int a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
+      const int a_fill = (a_nxt == 2 * kOperandBytes) ? 0 : a_nxt + kOperandBytes;  // freed one barrier ago
+      const int b_nxt = b_cur ^ kOperandBytes;
+      const int ko2 = k_byte(kt + 2);
+      // k-steps 0..2: A of tile kt+2
+      step(a_cur, b_cur, 1, 0, a_fill, ko2, 0, A0{}, 0, 0, I0{});
+      step(a_cur, b_cur, 2, 1, a_fill, ko2, kA[0], A1{}, 0, 0, I0{});
+      step(a_cur, b_cur, 3, 0, a_fill, ko2, kA[0] + kA[1], A2{}, 0, 0, I0{});
+      // last k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
+      // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
+      __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
+      __builtin_amdgcn_s_barrier();
+      step(a_nxt, b_nxt, 0, 1, 0, 0, 0, I0{}, b_cur, ko2, I8{});
+      a_cur = a_nxt;
+      b_cur = b_nxt;
+    }
+    __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
+    __builtin_amdgcn_s_barrier();
+  }
+};
+
+#ifndef AXON_DMA_SPREAD
+#define AXON_DMA_SPREAD 4, 4, 4, 4
+#endif
+#ifdef AXON_DMA_SYMMETRIC
+using DmaLoop = DmaLoopT<AXON_DMA_SPREAD>;
+#else
+using DmaLoop = DmaLoop32;
+#endif
 
 // ---------------------------------------------------------------------------------------
 // RegLoop: loads through registers with per-row clamping; any k % BK == 0

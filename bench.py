@@ -45,6 +45,9 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
     ap.add_argument("--hbm-tokens", type=int, default=1 << 26,
                     help="token count for the HBM-bound stage-2/3 kernels' bandwidth figures; 0 disables them")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="run a 1 GiB calibration copy, one head forward and one head backward, then exit: the "
+                         "command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken on")
     return ap.parse_args()
 
 
@@ -148,8 +151,34 @@ def hbm_kernels(n_tokens, dev):
     return {"tokens": n_tokens, "sequences": len(lens), "bound": "hbm", "kernels": out}
 
 
+# HBM-side bytes of ONE launch of the dominant kernel at the default workload, from rocprofv3 --pmc passes
+# over `bench.py --traffic-probe` (FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0, the factors a 1 GiB
+# device copy in the same run calibrates): 6.59e9 read + 0.36e9 written.
+TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 6.95e9}
+
+
+def traffic_probe(workload):
+    import torch
+
+    from axon_amd import _ops, workloads as W
+
+    n, h, v, _, seed = WORKLOADS[workload]
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed)
+    hd, wd, ld = hid.to("cuda"), w.to("cuda"), lab.to("cuda")
+    src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()  # 1 GiB
+    dst = torch.empty_like(src)
+    dst.copy_(src)  # calibration kernel: reads 1 GiB, writes 1 GiB
+    _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    g = torch.randn(n, device="cuda")
+    _ops.lmhead_backward(g, torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0)
+    torch.cuda.synchronize()
+
+
 def main():
     args = parse_args()
+    if args.traffic_probe:
+        traffic_probe(args.workload)
+        return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it",
               file=sys.stderr)
@@ -247,7 +276,8 @@ def main():
         "bound": "mfma", "kernel": dom["kernel"], "achieved": dom["algorithmic_tflops"] or dom["executed_tflops"],
         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": (dom["algorithmic_tflops"] or dom["executed_tflops"]) / MFMA_BF16_PEAK_TFLOPS,
-        "avg_launch_ms": dom["avg_launch_ms"], "traffic": None,
+        "avg_launch_ms": dom["avg_launch_ms"],
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if not args.tokens and "gemm_store" in dom["kernel"] else None,
         "kernels": kernels,
         "path_algorithmic_tflops": 6 * nhv / (ms_per_step * 1e-3) / 1e12,
         "path_frac_of_peak": 6 * nhv / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
