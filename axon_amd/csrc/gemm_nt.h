@@ -12,10 +12,10 @@
 //
 // Two main loops:
 //  * DmaLoop  (the fast path; needs m_rows >= 256, n_rows >= 256, k % 64 == 0)
-//      global -> LDS by `buffer_load_dwordx4 ... lds` (no VGPR staging), two
-//      64 KB stages of 256 x 64 bf16 per operand, 16-byte chunks XOR-swizzled by
-//      row; fragment reads for k-step kk+1 are issued under the MFMAs of k-step
-//      kk; the next tile's DMA is issued one full tile ahead.  Edge tiles are
+//      global -> LDS by `buffer_load_dwordx4 ... lds` (no VGPR staging), 32 KB
+//      slots of 256 x 64 bf16 (three for A, two for B), 16-byte chunks
+//      XOR-swizzled by row; fragment reads for k-step kk+1 are issued under the
+//      MFMAs of k-step kk; A is fetched two k-tiles ahead, B one.  Edge tiles are
 //      shifted back inside the matrix (uniform addressing, no per-lane clamps);
 //      the rows that then belong to the neighbouring tile are masked by the
 //      epilogue through `m_lo` / `n_lo`.
@@ -40,7 +40,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kTile = 256;       // tile edge in m and n
 constexpr int kWaveTile = 128;   // per-wave edge
 constexpr int kGemmThreads = 256;
-constexpr int kGemmLdsBytes = 163840;  // both main loops fit; also the staging area of the dlogit epilogue
+constexpr int kGemmLdsBytes = 163840;  // all of a CU's LDS: five 32 KB operand slots; the dlogit epilogue stages in the first 128 KB
 
 struct GemmOperands {
   const __bf16* a;  // [m_rows][lda], K-contiguous
@@ -55,7 +55,6 @@ struct GemmOperands {
 // previous tile and must be ignored by the epilogue.
 struct TilePos {
   int m0, n0, m_lo, n_lo;
-  int kt0 = 0;  // k-tile this workgroup starts its walk over k at (it wraps around)
 };
 
 // Position of this lane inside the workgroup tile.
@@ -86,24 +85,26 @@ __device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
 }
 
 // ---------------------------------------------------------------------------------------
-// DmaLoop
+// DmaLoop: k-tiles of 64 go global -> LDS by buffer_load ... lds (no register staging) into
+// XOR-swizzled [row][128 B] slots.  The 160 KB of LDS hold THREE slots for the A operand and
+// TWO for B.  B of k-tile t+2 is issued right after the barrier that frees its slot and has one
+// k-tile of time to land; A of k-tile t+2 is issued a whole k-tile earlier, spread under the
+// MFMAs of k-steps 0..2, into the slot freed one barrier before.  Compared with a symmetric
+// double buffer this halves the data that has only one k-tile to arrive, which is what keeps the
+// single wave per SIMD from waiting at the barrier (measured: +20 % on long-k GEMMs).
 // ---------------------------------------------------------------------------------------
-// C3, C0, C1, C2: how many of a wave's 16 DMA instructions for the next-but-one k-tile are issued
-// under the last k-step of the current tile (right after the barrier that frees the stage) and
-// under k-steps 0, 1, 2 of the next tile.
-template <int C3, int C0, int C1, int C2>
-struct DmaLoopT {
-  static_assert(C3 + C0 + C1 + C2 == 16 && C3 >= 1, "16 DMA instructions per wave and k-tile");
+struct DmaLoop {
   static constexpr int kBK = 64;
-  static constexpr int kRowBytes = 128;                    // 64 bf16
+  static constexpr int kRowBytes = 128;
   static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
-  static constexpr int kStageBytes = 2 * kOperandBytes;    // A then B
+  static constexpr int kBBase = 3 * kOperandBytes;         // A slots at 0/32/64 KB, B slots at 96/128 KB
   static constexpr bool kShiftsEdgeTiles = true;
 
   __device__ static __forceinline__ bool supports(const GemmOperands& g) {
     return g.m_rows >= kTile && g.n_rows >= kTile && (g.k % kBK) == 0;
   }
 
+  // Edge tiles are shifted back inside the matrix; the epilogue skips the duplicated rows.
   __device__ static __forceinline__ TilePos place(const GemmOperands& g, int tm, int tn) {
     TilePos t;
     const int m0 = tm * kTile, n0 = tn * kTile;
@@ -111,10 +112,6 @@ struct DmaLoopT {
     t.n0 = min(n0, g.n_rows - kTile);
     t.m_lo = m0 - t.m0;
     t.n_lo = n0 - t.n0;
-#ifndef AXON_K_SKEW
-#define AXON_K_SKEW 0
-#endif
-    t.kt0 = (AXON_K_SKEW) % (g.k / kBK);
     return t;
   }
 
@@ -131,148 +128,6 @@ struct DmaLoopT {
     // --- DMA addressing.  One wave instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns
     // rows [64w, 64w+64) of each operand (8 instructions).  Lane i lands on row i/8, chunk slot
     // i%8, and therefore fetches global chunk (i%8) ^ swizzle(row); swizzle(row) = (row/2) % 8.
-    const int lrow = lp.lane >> 3;
-    const int sw_even = (lp.lane >> 4) & 7;        // rows 8j + lrow with j even
-    const int sw_odd = (4 + (lp.lane >> 4)) & 7;   // j odd
-    const int row_a = (lp.wave * 64 + lrow) * (int)g.lda * 2;
-    const int row_b = (lp.wave * 64 + lrow) * (int)g.ldb * 2;
-    const int va_e = row_a + (((lp.lane & 7) ^ sw_even) << 4);
-    const int va_o = row_a + (((lp.lane & 7) ^ sw_odd) << 4);
-    const int vb_e = row_b + (((lp.lane & 7) ^ sw_even) << 4);
-    const int vb_o = row_b + (((lp.lane & 7) ^ sw_odd) << 4);
-    const int step_a = (int)g.lda * 16, step_b = (int)g.ldb * 16;  // 8 rows, in bytes
-    const __bf16* base_a = g.a + (int64_t)t.m0 * g.lda;
-    const __bf16* base_b = g.b + (int64_t)t.n0 * g.ldb;
-    const __amdgpu_buffer_rsrc_t ra =
-        __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rb =
-        __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
-    char* const dst = smem + lp.wave * 64 * kRowBytes;
-
-    // --- fragment addressing: row = 128*wm + 32*i + l32, chunk = 2*kk + lhi, swizzle = (l32/2)%8
-    const int sw = (lp.l32 >> 1) & 7;
-    int fa[4], fb[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      fa[kk] = (lp.wm * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
-      fb[kk] = kOperandBytes + (lp.wn * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
-    }
-
-    zero_acc(acc);
-    bf16x8 af[2][4], bf[2][4];
-    const int kt_n = g.k / kBK;
-
-    // byte offset inside a row of k-tile number kt of this workgroup's walk
-    auto k_byte = [&](int kt) {
-      const int ks = kt + t.kt0;
-      return (ks >= kt_n ? ks - kt_n : ks) * kRowBytes;
-    };
-    // instruction idx of the 16 that bring one k-tile: even = A, odd = B
-    auto dma_one = [&](int stage_off, int ko, int idx) {
-      const int j = idx >> 1;
-      if ((idx & 1) == 0)
-        dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + stage_off + j * 8 * kRowBytes);
-      else
-        dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b,
-              dst + stage_off + kOperandBytes + j * 8 * kRowBytes);
-    };
-    auto issue = [&](int stage_off, int kt, int first, int count) {
-#pragma unroll
-      for (int idx = 0; idx < 16; ++idx)
-        if (idx >= first && idx < first + count) dma_one(stage_off, k_byte(kt), idx);
-    };
-    auto read_frags = [&](int stage_off, int kk, int set) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        af[set][i] = *reinterpret_cast<const bf16x8*>(smem + stage_off + fa[kk] + i * 32 * kRowBytes);
-        bf[set][i] = *reinterpret_cast<const bf16x8*>(smem + stage_off + fb[kk] + i * 32 * kRowBytes);
-      }
-    };
-    // One k-step: 16 MFMAs on fragment set `mm_set`; under them the eight fragments of the next
-    // k-step are read into the other set (one per MFMA, in the order the next step consumes them)
-    // and `vmem` DMA instructions [dma_first, dma_first + vmem) of k-tile dma_kt are issued, evenly
-    // spread.  Source order is issue order: an LDS DMA and a fragment read are both LDS accesses
-    // to the compiler, so it will not move one across the other.
-    auto step = [&](int rd_stage, int rd_kk, int mm_set, int dma_stage, int dma_kt, int dma_first,
-                    auto vmem_c) {
-      constexpr int vmem = decltype(vmem_c)::value;
-      const int rd_set = mm_set ^ 1;
-      const int ko = k_byte(dma_kt);
-      const char* const fr = smem + rd_stage;
-#pragma unroll
-      for (int m = 0; m < 16; ++m) {
-        const int before = (m * vmem) / 16, due = ((m + 1) * vmem) / 16 - before;
-#pragma unroll
-        for (int d = 0; d < due; ++d) dma_one(dma_stage, ko, dma_first + before + d);
-        // a0 b0 b1 b2 b3 a1 a2 a3
-        if (m == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(fr + fa[rd_kk]);
-        if (m >= 1 && m <= 4)
-          bf[rd_set][m - 1] = *reinterpret_cast<const bf16x8*>(fr + fb[rd_kk] + (m - 1) * 32 * kRowBytes);
-        if (m >= 5 && m <= 7)
-          af[rd_set][m - 4] = *reinterpret_cast<const bf16x8*>(fr + fa[rd_kk] + (m - 4) * 32 * kRowBytes);
-        acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mm_set][m >> 2], bf[mm_set][m & 3],
-                                                                     acc[m >> 2][m & 3], 0, 0, 0);
-        if (due == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        if (due == 2) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-        if (due > 2) __builtin_amdgcn_sched_group_barrier(0x020, 16, 0);
-        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    };
-
-    // prologue: tile 0 whole, the first C3 instructions of tile 1; fragments of (tile 0, kk 0) in set 0
-    issue(0, 0, 0, 16);
-    issue(kStageBytes, min(1, kt_n - 1), 0, C3);
-    __builtin_amdgcn_s_waitcnt(C3 == 16 ? 0x4F70 : (0x0F70 | (C3 & 15)));  // vmcnt(C3): tile 0 has landed
-    __builtin_amdgcn_s_barrier();
-    read_frags(0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-
-    int cur = 0;
-    for (int kt = 0; kt < kt_n; ++kt) {
-      const int nxt = cur ^ kStageBytes;
-      const int kt1 = min(kt + 1, kt_n - 1);  // past the end: refetches the last tile, never consumed
-      // k-steps 0..2: fragments of the next k-step, the rest of tile kt+1 into the other stage
-      step(cur, 1, 0, nxt, kt1, C3, std::integral_constant<int, C0>{});
-      step(cur, 2, 1, nxt, kt1, C3 + C0, std::integral_constant<int, C1>{});
-      step(cur, 3, 0, nxt, kt1, C3 + C0 + C1, std::integral_constant<int, C2>{});
-      // last k-step of this tile: the other stage must have landed for every wave, and every wave
-      // must be done reading this stage (its kk=3 fragments are in registers) before it is refilled.
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-      __builtin_amdgcn_s_barrier();
-      step(nxt, 0, 1, cur, min(kt + 2, kt_n - 1), 0, std::integral_constant<int, C3>{});
-      cur = nxt;
-    }
-    // DMA issued for tiles past the end is still in flight; drain it before LDS is reused
-    __builtin_amdgcn_s_waitcnt(0x0070);
-    __builtin_amdgcn_s_barrier();
-  }
-};
-
-// ---------------------------------------------------------------------------------------
-// DmaLoop32: the same k-tile of 64 and LDS layout, but the 160 KB of LDS hold THREE slots for
-// the A operand and TWO for B.  B for k-tile t+2 is issued in one burst of eight instructions per
-// wave right after the barrier that frees its slot (one k-tile of time to land, half the burst
-// of a symmetric double buffer); A for k-tile t+2 is issued a whole k-tile earlier, spread
-// under the MFMAs of k-steps 0..2, into the slot freed one barrier before.
-// ---------------------------------------------------------------------------------------
-struct DmaLoop32 {
-  static constexpr int kBK = 64;
-  static constexpr int kRowBytes = 128;
-  static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
-  static constexpr int kBBase = 3 * kOperandBytes;         // A slots at 0/32/64 KB, B slots at 96/128 KB
-  static constexpr bool kShiftsEdgeTiles = true;
-
-  __device__ static __forceinline__ TilePos place(const GemmOperands& g, int tm, int tn) {
-    return DmaLoopT<4, 4, 4, 4>::place(g, tm, tn);
-  }
-
-  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
-                                             f32x16 (&acc)[4][4], char* smem) {
-    using Base = DmaLoopT<4, 4, 4, 4>;
-    const LanePos lp;
-    // DMA addressing as in DmaLoopT: one instruction = 8 rows x 128 B, wave w owns rows [64w, 64w+64)
     const int lrow = lp.lane >> 3;
     const int sw_even = (lp.lane >> 4) & 7;
     const int sw_odd = (4 + (lp.lane >> 4)) & 7;
@@ -291,6 +146,7 @@ struct DmaLoop32 {
         __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
     char* const dst = smem + lp.wave * 64 * kRowBytes;
 
+    // --- fragment addressing: row = 128*wm + 32*i + l32, chunk = 2*kk + lhi, swizzle = (l32/2)%8
     const int sw = (lp.l32 >> 1) & 7;
     int fa[4], fb[4];
 #pragma unroll
@@ -302,15 +158,13 @@ struct DmaLoop32 {
     zero_acc(acc);
     bf16x8 af[2][4], bf[2][4];
     const int kt_n = g.k / kBK;
-    auto k_byte = [&](int kt) {
-      const int ks = min(kt, kt_n - 1) + t.kt0;  // past the end: refetches the last tile, never consumed
-      return (ks >= kt_n ? ks - kt_n : ks) * kRowBytes;
-    };
+    // byte offset of k-tile kt inside a row; past the end: refetches the last tile, never consumed
+    auto k_byte = [&](int kt) { return min(kt, kt_n - 1) * kRowBytes; };
     auto dma_a = [&](int slot_off, int ko, int j) {
-      Base::dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + slot_off + j * 8 * kRowBytes);
+      dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + slot_off + j * 8 * kRowBytes);
     };
     auto dma_b = [&](int slot_off, int ko, int j) {
-      Base::dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b, dst + kBBase + slot_off + j * 8 * kRowBytes);
+      dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b, dst + kBBase + slot_off + j * 8 * kRowBytes);
     };
     // One k-step: 16 MFMAs on fragment set mm_set; the eight fragments of the next k-step are read
     // one per MFMA; `NA` A instructions [a_first, a_first + NA) and `NB` B instructions [0, NB) are
@@ -322,12 +176,7 @@ struct DmaLoop32 {
       const int rd_set = mm_set ^ 1;
 #pragma unroll
       for (int m = 0; m < 16; ++m) {
-#ifdef AXON_B_FRONT
-        const int before = (NB > 0) ? min(m, NB) : (m * vmem) / 16;
-        const int due = (NB > 0) ? (m < NB ? 1 : 0) : ((m + 1) * vmem) / 16 - before;
-#else
         const int before = (m * vmem) / 16, due = ((m + 1) * vmem) / 16 - before;
-#endif
 #pragma unroll
         for (int d = 0; d < due; ++d) {
           const int idx = before + d;  // B first: it has the shorter time to land
@@ -352,10 +201,7 @@ struct DmaLoop32 {
     };
     using I0 = std::integral_constant<int, 0>;
     using I8 = std::integral_constant<int, 8>;
-#ifndef AXON_A_SPREAD
-#define AXON_A_SPREAD 3, 3, 2
-#endif
-    constexpr int kA[3] = {AXON_A_SPREAD};  // A instructions under k-steps 0, 1, 2
+    constexpr int kA[3] = {3, 3, 2};  // A instructions under k-steps 0, 1, 2
     static_assert(kA[0] + kA[1] + kA[2] == 8, "eight A instructions per wave and k-tile");
     using A0 = std::integral_constant<int, kA[0]>;
     using A1 = std::integral_constant<int, kA[1]>;
@@ -401,15 +247,6 @@ struct DmaLoop32 {
     __builtin_amdgcn_s_barrier();
   }
 };
-
-#ifndef AXON_DMA_SPREAD
-#define AXON_DMA_SPREAD 4, 4, 4, 4
-#endif
-#ifdef AXON_DMA_SYMMETRIC
-using DmaLoop = DmaLoopT<AXON_DMA_SPREAD>;
-#else
-using DmaLoop = DmaLoop32;
-#endif
 
 // ---------------------------------------------------------------------------------------
 // RegLoop: loads through registers with per-row clamping; any k % BK == 0
