@@ -144,7 +144,8 @@ struct DmaLoop {
         __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
     const __amdgpu_buffer_rsrc_t rb =
         __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
-    char* const dst = smem + lp.wave * 64 * kRowBytes;
+    // wave-uniform, so the LDS destination of every DMA instruction is scalar arithmetic into M0
+    char* const dst = smem + __builtin_amdgcn_readfirstlane(lp.wave) * 64 * kRowBytes;
 
     // --- fragment addressing: row = 128*wm + 32*i + l32, chunk = 2*kk + lhi, swizzle = (l32/2)%8
     const int sw = (lp.l32 >> 1) & 7;
