@@ -157,6 +157,32 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
     return isw, new_mask, acc
 
 
+DIAG_OUT = 72
+
+
+def sampler_diag(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_lo, is_hi, rs_mode, rs_lo, rs_hi, rs_lr_lo,
+                 rs_lr_hi, log_is_lo, log_is_hi, log_rs_lo, log_rs_hi):
+    """All mismatch diagnostics as one float64 device tensor of DIAG_OUT raw sums / extrema
+    (layout: axon_sampler_diag in include/axon_amd.h).  No host synchronisation."""
+    lib = _lib.load()
+    require_device(old_lp, "sampler_diag")
+    dev = old_lp.device
+    old_lp, samp_lp = f32(old_lp), f32(samp_lp)
+    mk, kind = mask_arg(mask)
+    nbytes = lib.axon_sampler_diag_workspace_bytes(rows.n_rows, rows.n_slots)
+    ws = torch.empty(nbytes // 4, device=dev, dtype=torch.float32)
+    ws[: 6 * rows.n_rows].zero_()
+    out = torch.empty(DIAG_OUT, device=dev, dtype=torch.float64)
+    check(
+        lib.axon_sampler_diag(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                              rows.uniform_len, int(is_mode), float(is_lo), float(is_hi), int(rs_mode), float(rs_lo),
+                              float(rs_hi), float(rs_lr_lo), float(rs_lr_hi), float(log_is_lo), float(log_is_hi),
+                              float(log_rs_lo), float(log_rs_hi), ptr(ws), ptr(out), stream_ptr()),
+        "axon_sampler_diag",
+    )
+    return out
+
+
 TOKEN_REDUCE = {"sum": 0, "mean": 1, "mean-norm": 2, "mean-program": 3}
 BATCH_REDUCE = {"token-mean": 0, "step-mean": 1, "program-mean": 2}
 

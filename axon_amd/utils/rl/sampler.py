@@ -33,6 +33,7 @@ import math
 import struct
 from typing import Any
 
+import numpy as np
 import torch
 
 from axon_amd import _ops
@@ -143,6 +144,60 @@ def _check_shapes(old_log_prob, sampler_log_prob, response_mask):
         raise ValueError(f"log_prob shape {old_log_prob.shape} does not match response_mask shape {response_mask.shape}.")
 
 
+# --- metrics from the raw sums of axon_sampler_diag ------------------------------------------------
+
+def _soft(n: float) -> float:
+    """``mask.sum() + 1e-8`` as fp32 arithmetic gives it (axon/utils/torch/ops.py:131-145)."""
+    return float(np.float32(n) + np.float32(1e-8))
+
+
+def _weight_metrics(prefix, d, n_rows, level, s_e, s_hi, s_lo, s_c, s_c2, row, lvl, mm_x, mm_dev, mm_l):
+    """The diagnostics of untruncated weights (sampler.py:106-173 / :259-326) from raw sums.
+
+    ``d``: the 72 values; token-level slots s_*; row-statistics slots ``row`` (sum x, sum x^2, #hi, #lo);
+    row-level-mode slots ``lvl`` (#L>hi, #L<lo, sum w*cnt, sum clamp*cnt, sum clamp^2*cnt); extrema slots.
+    """
+    n = d[0]
+    soft = _soft(n)
+    m = {}
+    if level == "token":
+        m["mean"] = d[s_e] / soft
+        m["ratio_fraction_high"] = d[s_hi] / soft
+        m["ratio_fraction_low"] = d[s_lo] / soft
+        m["max"], m["min"] = d[50], d[60]
+        c1, c2 = d[s_c] / soft, d[s_c2] / soft
+    else:
+        m["max"] = math.exp(min(d[50 + mm_l], SAFETY_BOUND))
+        m["min"] = math.exp(d[60 + mm_l])
+        m["mean"] = d[lvl + 2] / soft
+        m["ratio_fraction_high"] = d[lvl] / n_rows
+        m["ratio_fraction_low"] = d[lvl + 1] / n_rows
+        c1, c2 = d[lvl + 3] / soft, d[lvl + 4] / soft
+    m["std"] = math.sqrt(max(c2 - c1 * c1, 0.0)) if n > 1 else 0.0
+    m["eff_sample_size"] = (c1 + 1e-8) ** 2 / c2 if c2 > 0 else float("inf")
+    sx, sx2 = d[row], d[row + 1]
+    m["seq_mean"] = sx / n_rows
+    m["seq_std"] = math.sqrt(max((sx2 - sx * sx / n_rows) / (n_rows - 1), 0.0)) if n_rows > 1 else 0.0
+    m["seq_max"], m["seq_min"] = d[50 + mm_x], d[60 + mm_x]
+    m["seq_max_deviation"] = d[50 + mm_dev]
+    m["seq_fraction_high"] = d[row + 2] / n_rows
+    m["seq_fraction_low"] = d[row + 3] / n_rows
+    return {f"{prefix}_{k}": v for k, v in m.items()}
+
+
+def _offpolicy_from_diag(d, n_rows) -> dict[str, float]:
+    soft = _soft(d[0])
+    return {
+        "training_ppl": d[42] / n_rows, "training_log_ppl": d[43] / n_rows,
+        "kl": -d[3] / soft, "k3_kl": d[4] / soft,
+        "sampler_ppl": d[44] / n_rows, "sampler_log_ppl": d[45] / n_rows,
+        "log_ppl_diff": d[46] / n_rows, "log_ppl_abs_diff": d[47] / n_rows,
+        "log_ppl_diff_max": d[59], "log_ppl_diff_min": d[69],
+        "ppl_ratio": d[48] / n_rows,
+        "chi2_token": d[2] / soft - 1.0, "chi2_seq": d[49] / n_rows - 1.0,
+    }
+
+
 # --- public API -------------------------------------------------------------------------------
 
 def compute_sampler_correction_and_rejection_mask(
@@ -191,15 +246,28 @@ def compute_sampler_correction_and_rejection_mask(
         is_threshold=sampler_is_threshold if use_is else 1.0,
         rs_mode=_ops.RS_MODES[sampler_rs], rs_lr_lo=rs_lo, rs_lr_hi=rs_hi, log_veto=log_veto,
     )
-    sums = acc.tolist()  # single readback for the empty-mask test and every metric
+    is_hi = float(sampler_is_threshold) if use_is else 1.0
+    is_lo = 1.0 / is_hi
+    rs_hi_t = float(sampler_rs_threshold) if sampler_rs is not None else 1.0
+    rs_lo_t = (float(sampler_rs_threshold_lower) if sampler_rs_threshold_lower is not None else 1.0 / rs_hi_t) \
+        if sampler_rs is not None else 1.0
+    tok_lo, tok_hi = (rs_lo, rs_hi) if sampler_rs == "token" else (-math.inf, math.inf)
+    diag = _ops.sampler_diag(
+        old_log_prob, sampler_log_prob, response_mask, rows,
+        is_mode=_ops.IS_MODES[sampler_is] if use_is else 0, is_lo=is_lo, is_hi=is_hi,
+        rs_mode=_ops.RS_MODES[sampler_rs], rs_lo=rs_lo_t, rs_hi=rs_hi_t, rs_lr_lo=tok_lo, rs_lr_hi=tok_hi,
+        log_is_lo=_log32(is_lo), log_is_hi=_log32(is_hi), log_rs_lo=_log32(rs_lo_t), log_rs_hi=_log32(rs_hi_t),
+    )
+    both = torch.cat([acc.double(), diag]).tolist()  # single readback: empty-mask test and every metric
+    sums, d = both[:8], both[8:]
     n_valid = sums[0]
     if n_valid == 0:
         return None, response_mask, {}
 
     metrics: dict[str, float] = {}
-    soft = n_valid + 1e-8  # denominator of the reference's masked_mean (axon/utils/torch/ops.py:131-145)
+    soft = _soft(n_valid)
     if use_is:
-        metrics["sampler_is_mean"] = sums[1] / soft
+        metrics.update(_weight_metrics("sampler_is", d, rows.n_rows, sampler_is, 1, 5, 6, 7, 8, 23, 31, 3, 4, 7))
         if sampler_is_batch_normalize:
             mean_w = sums[5] / soft
             if sampler_is == "sequence":
@@ -213,7 +281,9 @@ def compute_sampler_correction_and_rejection_mask(
             else:
                 metrics["sampler_is_batch_norm_factor"] = 1.0
     if sampler_rs is not None:
+        metrics.update(_weight_metrics("sampler_rs", d, rows.n_rows, sampler_rs, 1, 9, 10, 11, 12, 27, 36, 5, 6, 8))
         metrics["sampler_rs_masked_fraction"] = sums[2] / soft
+        metrics["sampler_rs_seq_masked_fraction"] = d[41] / rows.n_rows
     if log_veto is not None:
         metrics["sampler_is_veto_fraction"] = sums[4] / max(rows.n_rows, 1)
         metrics["sampler_is_catastrophic_token_fraction"] = sums[3] / soft
@@ -265,6 +335,33 @@ def compute_sampler_rejection_mask(
         raise ValueError("response_mask must contain at least one valid token (1).")
     short = {k[len("sampler_corr/"):]: v for k, v in metrics.items() if "veto" not in k and "catastrophic" not in k}
     return new_mask, short
+
+
+def _diag_plain(old_log_prob, sampler_log_prob, response_mask, cu_seqlens):
+    rows = _ops.rows_of(old_log_prob, cu_seqlens)
+    d = _ops.sampler_diag(old_log_prob, sampler_log_prob, response_mask, rows, is_mode=0, is_lo=1.0, is_hi=1.0,
+                          rs_mode=0, rs_lo=1.0, rs_hi=1.0, rs_lr_lo=-math.inf, rs_lr_hi=math.inf, log_is_lo=0.0,
+                          log_is_hi=0.0, log_rs_lo=0.0, log_rs_hi=0.0)
+    return d.tolist(), rows.n_rows
+
+
+def compute_offpolicy_metrics(old_log_prob, sampler_log_prob, response_mask,
+                              cu_seqlens: torch.Tensor | None = None) -> dict[str, Any]:
+    """Off-policy diagnostics (sampler.py:454-518): perplexities, KL / K3, chi-squared; no prefix.
+    One token pass, one row pass, one readback."""
+    _ops.require_device(old_log_prob, "compute_offpolicy_metrics")
+    if sampler_log_prob is None:
+        rows = _ops.rows_of(old_log_prob, cu_seqlens)
+        cnt, ssum, _ = _ops.row_stats(old_log_prob, None, response_mask, rows)
+        a = ssum / (cnt + 1e-8)
+        vals = torch.stack([cnt.sum(), torch.exp(-a).mean(), (-a).mean()]).tolist()
+        if vals[0] == 0:
+            return {}
+        return {"training_ppl": vals[1], "training_log_ppl": vals[2]}
+    d, n_rows = _diag_plain(old_log_prob, sampler_log_prob, response_mask, cu_seqlens)
+    if d[0] == 0:
+        return {}
+    return _offpolicy_from_diag(d, n_rows)
 
 
 def compute_sampler_correction_and_add_to_batch(batch: DataProto, config: dict[str, Any]) -> tuple[DataProto, dict]:

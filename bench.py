@@ -139,6 +139,11 @@ def hbm_kernels(n_tokens, dev):
         ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads)", 32,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4), **corr)),
         ("row_stats_kernel: per-sequence count and masked sum", 12, lambda: _ops.row_stats(new, old, mask, rows)),
+        ("sampler_diag kernels: all IS / rejection / off-policy / mismatch diagnostics (token pass + row pass)", 12,
+         lambda: _ops.sampler_diag(old, samp, mask, rows, is_mode=1, is_lo=0.5, is_hi=2.0, rs_mode=1, rs_lo=0.5,
+                                   rs_hi=2.0, rs_lr_lo=-math.log(2.0), rs_lr_hi=math.log(2.0),
+                                   log_is_lo=-math.log(2.0), log_is_hi=math.log(2.0), log_rs_lo=-math.log(2.0),
+                                   log_rs_hi=math.log(2.0))),
         ("row_broadcast_kernel: GRPO advantage = per-sequence scalar * mask", 8,
          lambda: _ops.row_broadcast_mask(seq_scalar, mask, rows)),
     ]

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 2
+#define AXON_AMD_ABI_VERSION 3
 
 enum {
   AXON_OK = 0,
@@ -191,6 +191,39 @@ int axon_sampler_correction(const float* old_logp, const float* sampler_logp, co
                             float log_veto, const float* row_cnt, const float* row_sum,
                             const int32_t* row_flag, float* is_weights, float* new_mask,
                             float* acc, float* partials, void* stream);
+
+/* Diagnostics of the sampler / trainer mismatch in one token pass and one row pass, for a single
+ * host readback.  Replaces the ~60 separate reductions (each with its own .item()) of
+ * _compute_is_metrics / _compute_rs_metrics (axon/utils/rl/sampler.py:106-173, 259-326),
+ * compute_offpolicy_metrics (sampler.py:454-518) and compute_trainer_sampler_mismatch_metrics
+ * (axon/utils/metrics/trainer_sampler_mismatch_metrics.py:36-80).
+ *   lr = old - sampler, e = exp(clamp(lr, -20, 20)), pa = exp(old), ps = exp(sampler); every
+ *   quantity is taken over tokens with mask != 0.
+ *   is_mode / rs_mode as in axon_sampler_correction; is_lo/is_hi, rs_lo/rs_hi: ratio thresholds
+ *   (lower, upper) in fp32; rs_lr_lo/rs_lr_hi: the log-space interval of the token-level rejection
+ *   (same values as passed to axon_sampler_correction); log_*: fp32 log of the ratio thresholds.
+ *   workspace: axon_sampler_diag_workspace_bytes(n_rows, n_slots) bytes whose first
+ *   6 * n_rows floats the caller has zero-filled.
+ * out[72] (double):
+ *   sums   [0] mask  [1] e  [2] e^2  [3] lr  [4] exp(lr)-lr-1  [5] e>is_hi  [6] e<is_lo
+ *          [7] clamp(e,is)  [8] clamp(e,is)^2  [9] e>rs_hi  [10] e<rs_lo  [11] clamp(e,rs)
+ *          [12] clamp(e,rs)^2  [13] |pa-ps|  [14] |pa-ps|^2  [15] |lr|  [16] lr^2  [17] pa  [18] ps
+ *          [19] pa^2  [20] ps^2  [21] pa*ps  [22] token-level rejected
+ *   rows   x = masked row mean of the untruncated weight:
+ *          [23..26] IS: sum x, sum x^2, #x>is_hi, #x<is_lo      [27..30] RS: the same
+ *          row-level modes, L = row log-ratio (sum, or masked mean for geometric), w = exp(clamp L):
+ *          [31..35] IS: #L>log_is_hi, #L<log_is_lo, sum w*cnt, sum clamp(w)*cnt, sum clamp(w)^2*cnt
+ *          [36..40] RS: the same   [41] rows rejected (token mode: rows with a rejected valid token)
+ *          a, b = masked row means of old / sampler:  [42] sum exp(-a)  [43] sum -a  [44] sum exp(-b)
+ *          [45] sum -b  [46] sum (b-a)  [47] sum |b-a|  [48] sum exp(b-a)  [49] sum exp(2 clamp(sum lr))
+ *   maxima [50] e  [51] |pa-ps|  [52] |lr|  [53] IS x  [54] IS |x-1|  [55] RS x  [56] RS |x-1|
+ *          [57] IS L  [58] RS L  [59] b-a          minima [60..69]: the same slots ([64],[66] unused) */
+int64_t axon_sampler_diag_workspace_bytes(int64_t n_rows, int64_t n_slots);
+int axon_sampler_diag(const float* old_logp, const float* sampler_logp, const void* mask, int mask_kind,
+                      const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
+                      int is_mode, float is_lo, float is_hi, int rs_mode, float rs_lo, float rs_hi,
+                      float rs_lr_lo, float rs_lr_hi, float log_is_lo, float log_is_hi,
+                      float log_rs_lo, float log_rs_hi, float* workspace, double* out, void* stream);
 
 /* Per-row weights of agg_loss (axon/trainer/algos/loss/utils.py:120-251) folded
  * into one multiplier per row, plus GSPO's per-row mean log-ratio:

@@ -423,3 +423,92 @@ def test_config4_full_size_masks_bit_exact():
     assert torch.equal(new.cpu(), pad_to_packed(new_ref, d["lengths"]))
     assert rel_l2(proto.batch["sampler_is_weights"], pad_to_packed(w_ref, d["lengths"])) < 1e-5
     assert m["sampler_corr/sampler_is_veto_fraction"] == pytest.approx(m_ref["sampler_is_veto_fraction"])
+
+
+# ---- diagnostics: every sampler_is_* / sampler_rs_* metric, off-policy and mismatch statistics ----
+def _assert_metrics(got, ref, prefix="", rel=2e-4, abs_=2e-6):
+    for k, v in ref.items():
+        g = got[prefix + k]
+        if math.isinf(v):
+            assert math.isinf(g) and (g > 0) == (v > 0), k
+        else:
+            # variances are differences of fp32 second moments close to 1 (in the reference too):
+            # their square roots agree to ~1e-5 absolute, not 1e-4 relative
+            tol_abs = 5e-5 if k.endswith("std") else abs_
+            assert g == pytest.approx(v, rel=rel, abs=tol_abs), (k, g, v)
+
+
+@pytest.mark.parametrize("is_l,rs_l", [("token", "token"), ("sequence", "sequence"), ("token", "geometric"),
+                                       ("sequence", "token"), (None, "geometric"), ("token", None)])
+def test_sampler_full_metrics_vs_oracle(is_l, rs_l):
+    old, samp, mask = _pad_case(seed=9, b=24, t=300)
+    samp = old + 0.02 * (samp - old)  # keep row sums inside the +-20 clamp for most rows
+    samp[3, 17] = old[3, 17] + 3.0
+    kw = dict(sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l, sampler_rs_threshold=1.5,
+              sampler_rs_threshold_lower=0.6)
+    _, _, m = S.compute_sampler_correction_and_rejection_mask(old.to(DEV), samp.to(DEV), mask.to(DEV), **kw)
+    ref = OS.full_metrics(old, samp, mask, **kw)
+    assert set(ref) <= {k[len("sampler_corr/"):] for k in m}
+    assert set(m) == {"sampler_corr/" + k for k in ref} | {"sampler_corr/sampler_is_veto_fraction",
+                                                            "sampler_corr/sampler_is_catastrophic_token_fraction"}
+    _assert_metrics(m, ref, "sampler_corr/")
+
+
+def test_sampler_full_metrics_packed_layout_matches_padded():
+    old, samp, mask = _pad_case(seed=10, b=16, t=200)
+    samp = old + 0.05 * (samp - old)
+    lens = mask.sum(-1).long().clamp(min=1).tolist()
+    cu = W.cu_from_lengths(lens)
+    pk = lambda x: pad_to_packed(x, lens)  # noqa: E731
+    kw = dict(sampler_is="sequence", sampler_is_threshold=2.0, sampler_rs="geometric", sampler_rs_threshold=1.2)
+    _, _, mp = S.compute_sampler_correction_and_rejection_mask(pk(old).to(DEV), pk(samp).to(DEV), pk(mask).to(DEV),
+                                                               cu_seqlens=cu.to(DEV), **kw)
+    ref = OS.full_metrics(old, samp, mask, **kw)
+    _assert_metrics(mp, ref, "sampler_corr/")
+
+
+def test_offpolicy_metrics_gpu():
+    old, samp, mask = _pad_case(seed=11, b=20, t=150)
+    samp = old + 0.03 * (samp - old)
+    got = S.compute_offpolicy_metrics(old.to(DEV), samp.to(DEV), mask.to(DEV))
+    ref = OS.offpolicy_metrics(old, samp, mask)
+    assert set(got) == set(ref) and len(got) == 13
+    _assert_metrics(got, ref)
+    # known answers of the reference's tests
+    o2, s2 = T([[-1.5, -2.5]]), T([[-1.0, -2.0]])
+    assert S.compute_offpolicy_metrics(o2.to(DEV), s2.to(DEV), torch.ones(1, 2).to(DEV))["kl"] == pytest.approx(0.5)
+    same = S.compute_offpolicy_metrics(o2.to(DEV), o2.to(DEV), torch.ones(1, 2).to(DEV))
+    assert same["kl"] == 0 and same["k3_kl"] == 0 and same["chi2_token"] == pytest.approx(0, abs=1e-7)
+    assert same["ppl_ratio"] == pytest.approx(1.0)
+    assert S.compute_offpolicy_metrics(o2.to(DEV), s2.to(DEV), torch.zeros(1, 2).to(DEV)) == {}
+    only = S.compute_offpolicy_metrics(o2.to(DEV), None, torch.ones(1, 2).to(DEV))
+    assert set(only) == {"training_ppl", "training_log_ppl"} and only["training_log_ppl"] == pytest.approx(2.0)
+
+
+def test_mismatch_metrics_gpu_and_aggregation():
+    from axon_amd.utils.metrics import aggregate_trainer_sampler_metrics, compute_trainer_sampler_mismatch_metrics
+    old, samp, mask = _pad_case(seed=12, b=10, t=90)
+    samp = old + 0.05 * (samp - old)
+    halves = []
+    for sl in (slice(0, 5), slice(5, 10)):
+        data = DataProto.from_dict(tensors={"old_log_probs": old[sl].to(DEV), "sampler_log_probs": samp[sl].to(DEV),
+                                            "response_mask": mask[sl].to(torch.int64).to(DEV)})
+        got = compute_trainer_sampler_mismatch_metrics(data)
+        ref = OS.mismatch_stats(old[sl], samp[sl], mask[sl])
+        assert set(got) == set(ref)
+        _assert_metrics(got, ref)
+        halves.append(got)
+    agg = aggregate_trainer_sampler_metrics(halves)
+    mb = mask.bool()
+    dp = (old.exp() - samp.exp()).abs()[mb]
+    dl = (old - samp).abs()[mb]
+    assert agg["batch/sampler_probs_diff_mean"] == pytest.approx(dp.mean().item(), rel=1e-4)
+    assert agg["batch/sampler_probs_diff_std"] == pytest.approx(dp.std(unbiased=False).item(), rel=1e-3)
+    assert agg["batch/sampler_logprobs_diff_max"] == pytest.approx(dl.max().item(), rel=1e-6)
+    pear = torch.corrcoef(torch.stack([old.exp()[mb], samp.exp()[mb]]))[0, 1].item()
+    assert agg["batch/sampler_actor_probs_pearson_corr"] == pytest.approx(pear, rel=1e-3)
+    assert aggregate_trainer_sampler_metrics([]) == {}
+    empty = DataProto.from_dict(tensors={"old_log_probs": old[:2].to(DEV), "sampler_log_probs": samp[:2].to(DEV),
+                                         "response_mask": torch.zeros(2, 90).to(DEV)})
+    z = aggregate_trainer_sampler_metrics([compute_trainer_sampler_mismatch_metrics(empty)])
+    assert len(z) == 9 and all(v == 0.0 for v in z.values())

@@ -194,3 +194,48 @@ def test_shift_contract():
     idx, _, _ = L.unpad_data(am)
     out = L.head_outputs_to_token_positions(T([10.0, 11, 12, 20, 21]), idx, 2, 4)
     assert out.tolist() == [[0, 10, 11, 12], [0, 20, 21, 0]]
+
+
+# ---- diagnostics: known answers of tests/utils/test_rl_sampler.py:158-178, 317-368 ----------------
+def test_oracle_offpolicy_known_answers():
+    old = torch.tensor([[-1.5, -2.5]])
+    samp = torch.tensor([[-1.0, -2.0]])
+    m = S.offpolicy_metrics(old, samp, torch.ones(1, 2))
+    assert m["kl"] == pytest.approx(0.5)
+    assert set(m) == {"training_ppl", "training_log_ppl", "kl", "k3_kl", "sampler_ppl", "sampler_log_ppl",
+                      "log_ppl_diff", "log_ppl_abs_diff", "log_ppl_diff_max", "log_ppl_diff_min", "ppl_ratio",
+                      "chi2_token", "chi2_seq"}
+    same = S.offpolicy_metrics(old, old, torch.ones(1, 2))
+    assert same["kl"] == 0 and same["k3_kl"] == 0 and same["chi2_token"] == 0 and same["ppl_ratio"] == 1
+    assert S.offpolicy_metrics(old, samp, torch.zeros(1, 2)) == {}
+    assert set(S.offpolicy_metrics(old, None, torch.ones(1, 2))) == {"training_ppl", "training_log_ppl"}
+
+
+def test_oracle_weight_metrics_known_answers():
+    lr, mask = torch.zeros(3, 5), torch.ones(3, 5)
+    m = S.full_metrics(lr, torch.zeros(3, 5), mask, sampler_is="token", sampler_rs="token")
+    assert m["sampler_is_mean"] == pytest.approx(1.0) and m["sampler_is_eff_sample_size"] == pytest.approx(1.0)
+    assert m["sampler_rs_masked_fraction"] == 0.0 and m["sampler_rs_seq_masked_fraction"] == 0.0
+    # lr = +-70 with a huge threshold: finite, the upper weight is e^20 (the +-20 clamp)
+    big = torch.tensor([[70.0, -70.0]])
+    mm = S.full_metrics(big, torch.zeros(1, 2), torch.ones(1, 2), sampler_is="token", sampler_is_threshold=1e12)
+    assert all(math.isfinite(v) for v in mm.values())
+    assert mm["sampler_is_max"] == pytest.approx(math.exp(20.0), rel=1e-4)
+    # a row of lr = 10 is rejected whole at sequence level, a row of 0 kept
+    seq = S.full_metrics(torch.tensor([[10.0] * 4, [0.0] * 4]), torch.zeros(2, 4), torch.ones(2, 4),
+                          sampler_rs="sequence", sampler_rs_threshold=2.0)
+    assert seq["sampler_rs_seq_masked_fraction"] == 0.5 and seq["sampler_rs_masked_fraction"] == pytest.approx(0.5)
+    assert seq["sampler_rs_ratio_fraction_high"] == 0.5 and seq["sampler_rs_max"] == pytest.approx(math.exp(20.0))
+
+
+def test_oracle_mismatch_stats_by_hand():
+    old = torch.tensor([[-1.0, -2.0, -9.0]])
+    samp = torch.tensor([[-1.5, -2.0, -1.0]])
+    mask = torch.tensor([[1.0, 1.0, 0.0]])
+    s = S.mismatch_stats(old, samp, mask)
+    pa, ps = [math.exp(-1.0), math.exp(-2.0)], [math.exp(-1.5), math.exp(-2.0)]
+    assert s["_valid_count"] == 2
+    assert s["_sum"] == pytest.approx(abs(pa[0] - ps[0])) and s["batch/sampler_probs_diff_min"] == 0.0
+    assert s["_logprobs_sum"] == pytest.approx(0.5) and s["batch/sampler_logprobs_diff_max"] == pytest.approx(0.5)
+    assert s["_product_sum"] == pytest.approx(pa[0] * ps[0] + pa[1] * ps[1])
+    assert S.mismatch_stats(old, samp, torch.zeros(1, 3))["_valid_count"] == 0
