@@ -240,6 +240,72 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     return acc, grad
 
 
+KL_TYPES = {"kl": 1, "k1": 1, "abs": 2, "mse": 3, "k2": 3, "low_var_kl": 4, "k3": 4}
+
+
+def kl_type_of(kl_penalty_type: str):
+    """(type code, straight-through flag) of a kl_penalty type string (kl.py:176-187, 216-245)."""
+    base = kl_penalty_type.rstrip("+")
+    if base == "full":
+        raise NotImplementedError("Full KL divergence requires logits, not just log probs")
+    if base not in KL_TYPES:
+        raise NotImplementedError(f"Unknown KL penalty type: {kl_penalty_type}")
+    plus = kl_penalty_type.endswith("+") and kl_penalty_type not in ("mse", "k2")
+    return KL_TYPES[base], int(plus)
+
+
+def kl_penalty(logprob, ref_logprob, kl_type: int, kl_plus: int):
+    """Per-token estimate and its derivative w.r.t. logprob (both fp32, shape of logprob)."""
+    lib = _lib.load()
+    require_device(logprob, "kl_penalty")
+    lp, ref = f32(logprob), f32(ref_logprob)
+    out, grad = torch.empty_like(lp), torch.empty_like(lp)
+    check(lib.axon_kl_penalty(ptr(lp), ptr(ref), lp.numel(), kl_type, kl_plus, ptr(out), ptr(grad), stream_ptr()),
+          "axon_kl_penalty")
+    return out, grad
+
+
+def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_reduce, batch_reduce, kl_type=0,
+               kl_plus=0, per_row_token_count=None, num_program_tokens=None, num_program_steps=None,
+               valid_count=None):
+    """Aggregated entropy and KL penalty with their gradient arrays.  Returns (acc[8], agg_w | None,
+    grad_kl | None); see axon_side_terms."""
+    lib = _lib.load()
+    anchor = entropy if entropy is not None else log_probs
+    require_device(anchor, "side_terms")
+    dev = anchor.device
+    ent = f32(entropy) if entropy is not None else None
+    lp = f32(log_probs) if kl_type else None
+    ref = f32(ref_log_probs) if kl_type else None
+    mk, mkind = mask_arg(mask)
+    tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
+    valid = _i64_dev(valid_count, dev)
+    one_pass = tr == 0 and br == 0
+    row_scale = None
+    if not one_pass:
+        cnt, _, _ = row_stats(anchor, None, mk, rows, want_sum=False)
+        row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
+        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        check(
+            lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
+                                    ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),
+            "axon_loss_row_scale",
+        )
+    agg_w = torch.empty(rows.shape, device=dev, dtype=torch.float32) if ent is not None else None
+    grad_kl = torch.empty(rows.shape, device=dev, dtype=torch.float32) if kl_type else None
+    acc = _acc8(rows.n_slots, dev)
+    check(
+        lib.axon_side_terms(ptr(ent), ptr(lp), ptr(ref), ptr(mk), mkind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                            rows.uniform_len, ptr(row_scale), 1.0, int(one_pass), ptr(valid if one_pass else None),
+                            int(kl_type), int(kl_plus), ptr(agg_w), ptr(grad_kl), ptr(acc),
+                            ptr(_partials(rows.n_slots, dev)), stream_ptr()),
+        "axon_side_terms",
+    )
+    return acc, agg_w, grad_kl
+
+
 # When set to a dict (benchmarks only), the LM-head autograd function routes through the
 # timed entry points and accumulates per-phase HIP-event times here.
 TIMING: dict | None = None

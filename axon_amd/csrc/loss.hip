@@ -112,10 +112,10 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
   store_block_partials<6>(a, lds_red, partials);
 }
 
-// Adds the per-workgroup partial sums in a fixed order and writes acc[0..7].  post_normalize:
-// acc[0] (a plain masked sum) becomes the token-mean, acc[5] the factor 1/denominator.
+// Adds the per-workgroup partial sums in a fixed order and writes acc[0..7].  norm_slots != 0:
+// the slots in that bit mask (plain masked sums) become token-means, acc[5] the factor 1/denominator.
 __global__ __launch_bounds__(1024) void reduce_partials_kernel(
-    const float* __restrict__ partials, int n_blocks, int post_normalize,
+    const float* __restrict__ partials, int n_blocks, int norm_slots,
     const int64_t* __restrict__ valid, float* __restrict__ acc) {
   __shared__ float red[16][kPartialStride];
   float t[kPartialStride];
@@ -141,9 +141,10 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(
       for (int w = 0; w < (int)(blockDim.x >> 6); ++w) s += red[w][k];
       tot[k] = s;
     }
-    if (post_normalize) {  // token-mean over a plain sum: the denominator is known only now
+    if (norm_slots) {  // token-mean over a plain sum: the denominator is known only now
       const float den = fmaxf(valid != nullptr ? (float)valid[0] : tot[4], 1.f);
-      tot[0] = tot[0] / den;
+      for (int k = 0; k < kPartialStride; ++k)
+        if ((norm_slots >> k) & 1) tot[k] = tot[k] / den;
       tot[5] = 1.f / den;
     }
     for (int k = 0; k < kPartialStride; ++k) acc[k] = tot[k];
@@ -293,6 +294,130 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
   store_block_partials<6>(a, lds_red, partials);
 }
 
+// KL penalty estimators of axon/utils/rl/kl.py:154-245 with PyTorch's gradient conventions.
+//   type 1: k1 = lp - ref   2: abs   3: k2 = 0.5 (lp - ref)^2   4: k3 = low-variance (clamped)
+//   plus != 0 ("k1+", "k3+"): forward value of the type, gradient of k2 (straight-through, :184-190)
+__device__ __forceinline__ ValGrad kl_term(float lp, float ref, int type, int plus) {
+  const float d = lp - ref;
+  ValGrad r{0.f, 0.f};
+  if (type == 1) {
+    r = ValGrad{d, 1.f};
+  } else if (type == 2) {
+    r = ValGrad{fabsf(d), (d > 0.f) ? 1.f : ((d < 0.f) ? -1.f : 0.f)};
+  } else if (type == 3) {
+    r = ValGrad{0.5f * d * d, d};
+  } else if (type == 4) {
+    const float k = ref - lp;
+    const bool in1 = (k >= -kSafetyBound && k <= kSafetyBound);
+    const float kc = clampf(k, -kSafetyBound, kSafetyBound);
+    const float ratio = expf(kc);
+    const float v = ratio - kc - 1.f;
+    const bool in2 = (v >= -10.f && v <= 10.f);
+    r = ValGrad{clampf(v, -10.f, 10.f), (in1 && in2) ? (1.f - ratio) : 0.f};
+  }
+  if (plus && type != 3) r.g = d;
+  return r;
+}
+
+__global__ __launch_bounds__(kBlock) void kl_penalty_kernel(const float* __restrict__ lp,
+                                                            const float* __restrict__ ref, int64_t n,
+                                                            int type, int plus, float* __restrict__ out,
+                                                            float* __restrict__ grad) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    const ValGrad r = kl_term(lp[i], ref[i], type, plus);
+    out[i] = r.v;
+    grad[i] = r.g;
+  }
+}
+
+// Side terms of the actor loss, aggregated exactly like the policy-gradient term
+// (axon/models/fsdp_models.py:247-273): entropy bonus and KL penalty against a reference
+// policy.  partial slots: [0] sum entropy*w  [1] sum kld*w  [2] sum entropy*mask  [4] sum mask,
+// w = mask * scale.  Outputs agg_w[t] = w (the gradient of slot 0 w.r.t. entropy) and
+// grad_kl[t] = w * d kld / d log_prob.
+template <int MK>
+__global__ __launch_bounds__(kBlock) void side_terms_kernel(
+    const float* __restrict__ entropy, const float* __restrict__ logp, const float* __restrict__ ref,
+    const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots,
+    int64_t uniform_len, const float* __restrict__ row_scale, float uniform_scale, int kl_type,
+    int kl_plus, float* __restrict__ agg_w, float* __restrict__ grad_kl, float* partials) {
+  __shared__ int32_t lds_cu[kLdsRows];
+  __shared__ float lds_red[6 * (kBlock / kWave)];
+  const bool need_row = (row_scale != nullptr);
+  const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
+  float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+  for (int64_t chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const int64_t c0 = chunk * kChunk;
+    const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+    RowFinder rf;
+    if (need_row) {
+      __syncthreads();
+      rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+    }
+#pragma unroll 1
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      if (i >= c1) continue;
+      float ev[4] = {0.f, 0.f, 0.f, 0.f}, lv[4] = {0.f, 0.f, 0.f, 0.f}, rv[4] = {0.f, 0.f, 0.f, 0.f};
+      float mv[4], wv[4], gv[4];
+      const bool full = (i + kVec <= n_slots);
+      if (full) {
+        if (entropy) load4(entropy, i, ev);
+        if (kl_type) { load4(logp, i, lv); load4(ref, i, rv); }
+        load_mask4<MK>(mask, i, mv);
+      } else {
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = i + j < n_slots;
+          ev[j] = (ok && entropy) ? entropy[i + j] : 0.f;
+          lv[j] = (ok && kl_type) ? logp[i + j] : 0.f;
+          rv[j] = (ok && kl_type) ? ref[i + j] : 0.f;
+          mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+        }
+      }
+      int64_t rend = -1;
+      float scale = uniform_scale;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int64_t p = i + j;
+        if (p >= n_slots) { wv[j] = 0.f; gv[j] = 0.f; continue; }
+        if (need_row && p >= rend) {
+          const int r = rf.row(p);
+          rend = rf.row_end(r);
+          scale = row_scale[r];
+        }
+        const float m = mv[j];
+        const float w = m * scale;
+        wv[j] = w;
+        a[4] += m;
+        if (entropy) {
+          a[0] += ev[j] * w;
+          a[2] += ev[j] * m;
+        }
+        float g = 0.f;
+        if (kl_type) {
+          const ValGrad k = kl_term(lv[j], rv[j], kl_type, kl_plus);
+          a[1] += k.v * w;
+          g = k.g * w;
+        }
+        gv[j] = g;
+      }
+      if (full) {
+        if (agg_w) store4(agg_w, i, wv);
+        if (grad_kl) store4(grad_kl, i, gv);
+      } else {
+        for (int j = 0; j < 4 && i + j < n_slots; ++j) {
+          if (agg_w) agg_w[i + j] = wv[j];
+          if (grad_kl) grad_kl[i + j] = gv[j];
+        }
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) a[5] = 1.f;
+  store_block_partials<6>(a, lds_red, partials);
+}
+
 }  // namespace axon
 
 using namespace axon;
@@ -396,7 +521,54 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
 #undef AXON_LAUNCH_PL
   AXON_CHECK_LAUNCH();
   hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
-                     post_normalize, valid, acc);
+                     post_normalize ? 1 : 0, valid, acc);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_kl_penalty(const float* logp, const float* ref_logp, int64_t n, int kl_type,
+                               int kl_plus, float* out, float* grad, void* stream) {
+  if (n < 0) return AXON_ERR_ARG;
+  if (n == 0) return AXON_OK;
+  if (!logp || !ref_logp || !out || !grad) return AXON_ERR_ARG;
+  if (kl_type < 1 || kl_type > 4) return AXON_ERR_ARG;
+  int64_t nb = (n + kBlock - 1) / kBlock;
+  const int grid = (int)(nb < 8192 ? nb : 8192);
+  hipLaunchKernelGGL(kl_penalty_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, logp,
+                     ref_logp, n, kl_type, kl_plus, out, grad);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_side_terms(const float* entropy, const float* logp, const float* ref_logp,
+                               const void* mask, int mask_kind, const int32_t* cu, int64_t n_rows,
+                               int64_t n_slots, int64_t uniform_len, const float* row_scale,
+                               float uniform_scale, int post_normalize, const int64_t* valid,
+                               int kl_type, int kl_plus, float* agg_w, float* grad_kl, float* acc,
+                               float* partials, void* stream) {
+  const bool need_row = (row_scale != nullptr);
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0) return AXON_OK;
+  if (!mask || !acc || !partials) return AXON_ERR_ARG;
+  if (kl_type < 0 || kl_type > 4) return AXON_ERR_ARG;
+  if (kl_type != 0 && (!logp || !ref_logp || !grad_kl)) return AXON_ERR_ARG;
+  if (entropy == nullptr && kl_type == 0) return AXON_ERR_ARG;
+  if (post_normalize && row_scale != nullptr) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
+  const hipStream_t st = (hipStream_t)stream;
+  if (mask_kind == AXON_MASK_F32)
+    hipLaunchKernelGGL(side_terms_kernel<AXON_MASK_F32>, g, blk, 0, st, entropy, logp, ref_logp, mask,
+                       cu, n_rows, n_slots, uniform_len, row_scale, uniform_scale, kl_type, kl_plus,
+                       agg_w, grad_kl, partials);
+  else
+    hipLaunchKernelGGL(side_terms_kernel<AXON_MASK_I64>, g, blk, 0, st, entropy, logp, ref_logp, mask,
+                       cu, n_rows, n_slots, uniform_len, row_scale, uniform_scale, kl_type, kl_plus,
+                       agg_w, grad_kl, partials);
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
+                     post_normalize ? 3 : 0, valid, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

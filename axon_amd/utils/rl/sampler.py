@@ -364,6 +364,14 @@ def compute_offpolicy_metrics(old_log_prob, sampler_log_prob, response_mask,
     return _offpolicy_from_diag(d, n_rows)
 
 
+def compute_sampler_corr_metrics_from_logprobs(log_prob, sampler_log_prob, response_mask,
+                                               cu_seqlens: torch.Tensor | None = None) -> dict[str, float]:
+    """Off-policy gap of the CURRENT policy against the sampler, "sampler_corr/"-prefixed
+    (sampler.py:566-597); called inside the actor update as the policy moves."""
+    m = compute_offpolicy_metrics(log_prob.detach(), sampler_log_prob, response_mask, cu_seqlens=cu_seqlens)
+    return {f"sampler_corr/{k}": v for k, v in m.items()}
+
+
 def compute_sampler_correction_and_add_to_batch(batch: DataProto, config: dict[str, Any]) -> tuple[DataProto, dict]:
     """Overwrite ``batch.batch["response_mask"]`` and union ``sampler_is_weights`` into the batch
     (sampler.py:526-563); ``config`` is the loss_args dict."""

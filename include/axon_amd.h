@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 3
+#define AXON_AMD_ABI_VERSION 4
 
 enum {
   AXON_OK = 0,
@@ -267,6 +267,28 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
                      float uniform_scale, int post_normalize, const int64_t* valid_count,
                      float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                      float* partials, void* stream);
+
+/* Per-token KL penalty against a reference policy, kl_penalty / kl_penalty_forward
+ * (axon/utils/rl/kl.py:154-245): kl_type 1 "kl"/"k1", 2 "abs", 3 "mse"/"k2", 4 "low_var_kl"/"k3";
+ * kl_plus != 0 for "k1+"/"k3+" (forward value of the type, gradient of k2, kl.py:184-190).
+ * out[n] = the estimate, grad[n] = d out / d logp. */
+int axon_kl_penalty(const float* logp, const float* ref_logp, int64_t n, int kl_type, int kl_plus,
+                    float* out, float* grad, void* stream);
+
+/* Entropy bonus and KL penalty of the actor loss, aggregated with agg_loss like the
+ * policy-gradient term (CausalLM.forward_backward_fn, axon/models/fsdp_models.py:247-273), in one
+ * pass: entropy (NULL: no entropy term), logp/ref_logp (kl_type 0: no KL term).
+ * row_scale / uniform_scale / post_normalize / valid_count as in axon_policy_loss.
+ * Outputs: agg_w[n_slots] = mask*scale (= d acc[0] / d entropy; may be NULL),
+ * grad_kl[n_slots] = mask*scale * d kld / d logp (NULL when kl_type 0);
+ * acc[8] (written): [0] aggregated entropy, [1] aggregated KL penalty, [2] sum entropy*mask,
+ * [4] sum mask, [5] the factor the two gradient arrays still have to be multiplied by.
+ * partials: workspace of axon_reduce_partials_bytes(n_slots). */
+int axon_side_terms(const float* entropy, const float* logp, const float* ref_logp, const void* mask,
+                    int mask_kind, const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                    int64_t uniform_len, const float* row_scale, float uniform_scale,
+                    int post_normalize, const int64_t* valid_count, int kl_type, int kl_plus,
+                    float* agg_w, float* grad_kl, float* acc, float* partials, void* stream);
 
 #ifdef __cplusplus
 }

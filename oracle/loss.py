@@ -105,3 +105,53 @@ def gspo_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0
     clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
     kl = masked_mean(-nak, response_mask)
     return loss, {"pg_clipfrac": clipfrac.item(), "ppo_kl": kl.item(), "pg_clipfrac_lower": 0.0}
+
+
+def kl_penalty(logprob, ref_logprob, kl_penalty_type="low_var_kl"):
+    """axon/utils/rl/kl.py:154-245.  "+" types: forward value of the base type, gradient of k2."""
+    base = kl_penalty_type.rstrip("+")
+    d = logprob - ref_logprob
+    if base in ("kl", "k1"):
+        fwd = d
+    elif base == "abs":
+        fwd = d.abs()
+    elif base in ("mse", "k2"):
+        fwd = 0.5 * d.square()
+    elif base in ("low_var_kl", "k3"):
+        k = torch.clamp(ref_logprob - logprob, min=-20, max=20)
+        fwd = torch.clamp(torch.exp(k) - k - 1, min=-10, max=10)
+    elif base == "full":
+        raise NotImplementedError("Full KL divergence requires logits, not just log probs")
+    else:
+        raise NotImplementedError(f"Unknown KL penalty type: {kl_penalty_type}")
+    if not kl_penalty_type.endswith("+") or kl_penalty_type in ("mse", "k2"):
+        return fwd
+    bwd = 0.5 * d.square()
+    return bwd - bwd.detach() + fwd.detach()
+
+
+def actor_loss(loss_fn, log_prob, entropy, old_log_prob, advantages, response_mask, *, loss_args, ref_log_prob=None,
+               side_mask=None, dp_replicas=1, n_micro_batches=1, **agg_kwargs):
+    """axon/models/fsdp_models.py:226-276: pg loss - entropy_coef * agg(entropy) + kl_coef * agg(kld), times
+    dp_replicas.  ``side_mask``: the mask the side terms aggregate over (the one captured before the
+    sampler correction hook); defaults to ``response_mask``."""
+    tr = loss_args.get("token_reduce", "sum")
+    br = loss_args.get("batch_reduce", "token-mean")
+    clip = {k: v for k, v in loss_args.items() if k.startswith("clip")}
+    loss, m = loss_fn(log_prob, old_log_prob, advantages, response_mask, token_reduce=tr, batch_reduce=br, **clip,
+                      **agg_kwargs)
+    metrics = dict(m)
+    metrics["pg_loss"] = loss.item() * n_micro_batches
+    sm = response_mask if side_mask is None else side_mask
+    ent_agg = agg_loss(entropy, sm, token_reduce=tr, batch_reduce=br, **agg_kwargs)
+    metrics["entropy"] = ent_agg.item() * n_micro_batches
+    metrics["entropy_token_mean"] = agg_loss(entropy, sm, token_reduce="sum", batch_reduce="token-mean").item()
+    if loss_args.get("entropy_coef", 0) != 0:
+        loss = loss - ent_agg * loss_args["entropy_coef"]
+    if loss_args.get("kl_coef", 0) != 0:
+        kld = kl_penalty(log_prob, ref_log_prob, loss_args.get("kl_type", "low_var_kl"))
+        kl_loss = agg_loss(kld, sm, token_reduce=tr, batch_reduce=br, **agg_kwargs)
+        loss = loss + kl_loss * loss_args["kl_coef"]
+        metrics["kl_loss"] = kl_loss.item() * n_micro_batches
+        metrics["kl_coef"] = loss_args["kl_coef"]
+    return loss * dp_replicas, metrics

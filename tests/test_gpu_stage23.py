@@ -512,3 +512,82 @@ def test_mismatch_metrics_gpu_and_aggregation():
                                          "response_mask": torch.zeros(2, 90).to(DEV)})
     z = aggregate_trainer_sampler_metrics([compute_trainer_sampler_mismatch_metrics(empty)])
     assert len(z) == 9 and all(v == 0.0 for v in z.values())
+
+
+# ---- KL penalty and the actor-loss side terms ---------------------------------------------------------
+@pytest.mark.parametrize("ktype", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3", "k1+", "k3+"])
+def test_kl_penalty_gpu_vs_oracle(ktype):
+    from axon_amd.utils.rl.kl import kl_penalty, kl_penalty_forward
+    g = torch.Generator().manual_seed(21)
+    lp = -torch.empty(7, 33).exponential_(1.0, generator=g)
+    ref = lp + 0.5 * torch.randn(7, 33, generator=g)
+    ref[0, 0], ref[0, 1], ref[0, 2] = lp[0, 0] + 25.0, lp[0, 1] - 25.0, lp[0, 2]  # clamps and the tie at 0
+    a = lp.clone().to(DEV).requires_grad_(True)
+    out = kl_penalty(a, ref.to(DEV), ktype)
+    w = torch.randn(7, 33, generator=g)
+    (out * w.to(DEV)).sum().backward()
+    b = lp.clone().requires_grad_(True)
+    want = OL.kl_penalty(b, ref, ktype)
+    (want * w).sum().backward()
+    assert torch.allclose(out.detach().cpu(), want.detach(), rtol=1e-5, atol=1e-6)
+    assert torch.allclose(a.grad.cpu(), b.grad, rtol=1e-5, atol=1e-6)
+    assert torch.allclose(kl_penalty_forward(a.detach(), ref.to(DEV), ktype).cpu(), want.detach(), rtol=1e-5, atol=1e-6)
+
+
+def test_kl_penalty_errors():
+    from axon_amd.utils.rl.kl import kl_penalty
+    x = torch.zeros(2, 3, device=DEV)
+    with pytest.raises(NotImplementedError):
+        kl_penalty(x, x, "full")
+    with pytest.raises(NotImplementedError):
+        kl_penalty(x, x, "nope")
+
+
+@pytest.mark.parametrize("loss_name,tr,br", [("ppo", "sum", "token-mean"), ("ppo", "mean", "step-mean"),
+                                             ("gspo", "mean", "token-mean")])
+@pytest.mark.parametrize("kl_type", ["low_var_kl", "k1+"])
+def test_actor_loss_assembly_vs_oracle(loss_name, tr, br, kl_type):
+    from axon_amd.models.fsdp_models import CausalLM
+    d = _c1_with_adv(3)
+    g = torch.Generator().manual_seed(33)
+    entropy = torch.rand(d["log_probs"].shape, generator=g) * 3
+    ref = d["log_probs"] + 0.1 * torch.randn(d["log_probs"].shape, generator=g)
+    args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": tr, "batch_reduce": br,
+            "entropy_coef": 0.01, "kl_coef": 0.05, "kl_type": kl_type}
+    meta = {"loss_fn": loss_name, "loss_fn_args": args, "temperature": 1.0, "dp_replicas": 2, "n_micro_batches": 4}
+    lp_dev = d["log_probs"].to(DEV).requires_grad_(True)
+    ent_dev = entropy.to(DEV).requires_grad_(True)
+    data = DataProto.from_dict(tensors={"old_log_probs": d["old_log_probs"].to(DEV), "advantages": d["advantages"].to(DEV),
+                                        "response_mask": d["response_mask"].to(DEV), "ref_log_prob": ref.to(DEV)})
+    module = lambda inputs, m: {"log_probs": lp_dev, "entropys": ent_dev}  # noqa: E731
+    loss, metrics = CausalLM.forward_backward_fn(module, data, meta)
+    loss.backward()
+    lp = d["log_probs"].clone().requires_grad_(True)
+    en = entropy.clone().requires_grad_(True)
+    fn = OL.ppo_loss if loss_name == "ppo" else OL.gspo_loss
+    want, wm = OL.actor_loss(fn, lp, en, d["old_log_probs"], d["advantages"], d["response_mask"], loss_args=args,
+                             ref_log_prob=ref, dp_replicas=2, n_micro_batches=4)
+    want.backward()
+    assert loss.item() == pytest.approx(want.item(), rel=1e-4)
+    assert rel_l2(lp_dev.grad, lp.grad) < 1e-5 and rel_l2(ent_dev.grad, en.grad) < 1e-5
+    for k in ("pg_loss", "entropy", "entropy_token_mean", "kl_loss", "kl_coef", "pg_clipfrac", "ppo_kl"):
+        assert metrics[k] == pytest.approx(wm[k], rel=1e-4, abs=1e-7), k
+
+
+def test_actor_loss_without_side_terms_and_with_sampler_metrics():
+    from axon_amd.models.fsdp_models import loss_from_outputs
+    d = _c1_with_adv(4)
+    entropy = torch.ones_like(d["log_probs"])
+    samp = d["old_log_probs"] + 0.01
+    data = DataProto.from_dict(tensors={"old_log_probs": d["old_log_probs"].to(DEV), "advantages": d["advantages"].to(DEV),
+                                        "response_mask": d["response_mask"].to(DEV), "sampler_log_probs": samp.to(DEV)})
+    lp_dev = d["log_probs"].to(DEV).requires_grad_(True)
+    ent_dev = entropy.to(DEV).requires_grad_(True)
+    meta = {"loss_fn": "ppo", "loss_fn_args": {}, "temperature": 1.0, "dp_replicas": 1}
+    loss, m = loss_from_outputs(data, lp_dev, ent_dev, meta)
+    loss.backward()
+    assert ent_dev.grad is None or float(ent_dev.grad.abs().max()) == 0.0  # entropy_coef 0: metric only
+    assert m["entropy"] == pytest.approx(1.0, rel=1e-5) and m["entropy_token_mean"] == pytest.approx(1.0, rel=1e-5)
+    assert "kl_loss" not in m and m["pg_loss"] == pytest.approx(loss.item(), rel=1e-6)
+    ref = OS.offpolicy_metrics(d["log_probs"], samp, d["response_mask"])
+    _assert_metrics(m, ref, "sampler_corr/")

@@ -197,3 +197,47 @@ def test_dp_scaling_invariant():
             O.agg_loss(x[sh] * w2, mask[sh], token_reduce=tr, batch_reduce=br, **{key: count}).backward()
             acc += w2.grad.item()
         assert acc == pytest.approx(full, rel=1e-5)
+
+
+# ---- KL penalty: facts the reference's tests/utils/test_kl.py:178-340 asserts ---------------------
+KL_TYPES = ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3", "k1+", "k3+"]
+
+
+def test_oracle_kl_penalty_closed_forms():
+    lp = torch.tensor([[-1.0, -2.0, -3.0], [-0.5, -1.5, -2.5]])
+    ref = torch.tensor([[-1.5, -1.0, -3.5], [-0.5, -2.0, -2.0]])
+    d = (lp - ref).tolist()
+    for name, f in [("kl", lambda x: x), ("abs", abs), ("mse", lambda x: 0.5 * x * x),
+                    ("low_var_kl", lambda x: math.exp(-x) + x - 1)]:
+        got = O.kl_penalty(lp, ref, name).tolist()
+        for gr, dr in zip(got, d):
+            for g, x in zip(gr, dr):
+                assert g == pytest.approx(f(x), abs=1e-6), name
+    assert torch.equal(O.kl_penalty(lp, ref, "k1"), O.kl_penalty(lp, ref, "kl"))
+    assert torch.equal(O.kl_penalty(lp, ref, "k2"), O.kl_penalty(lp, ref, "mse"))
+    assert torch.equal(O.kl_penalty(lp, ref, "k3"), O.kl_penalty(lp, ref, "low_var_kl"))
+    assert torch.equal(O.kl_penalty(lp, ref, "k1+"), O.kl_penalty(lp, ref, "k1"))  # forward of "+" = base
+    assert torch.equal(O.kl_penalty(lp, ref, "k3+"), O.kl_penalty(lp, ref, "k3"))
+    for t in KL_TYPES:
+        assert torch.allclose(O.kl_penalty(lp, lp, t), torch.zeros_like(lp), atol=1e-6)
+    for t in ("abs", "mse", "low_var_kl"):
+        assert (O.kl_penalty(lp, ref, t) >= -1e-7).all()
+    big = O.kl_penalty(torch.tensor([[100.0]]), torch.tensor([[-100.0]]), "low_var_kl")
+    assert -10.0 <= big.item() <= 10.0
+    for t in KL_TYPES:
+        assert torch.isfinite(O.kl_penalty(torch.tensor([[100.0, -100.0, 50.0]]),
+                                            torch.tensor([[-100.0, 100.0, -50.0]]), t)).all()
+    with pytest.raises(NotImplementedError):
+        O.kl_penalty(lp, ref, "full")
+    with pytest.raises(NotImplementedError):
+        O.kl_penalty(lp, ref, "nope")
+
+
+def test_oracle_kl_penalty_gradients():
+    ref = torch.tensor([[-1.5, -1.0, -3.5]])
+    for t, g in [("kl", lambda x: 1.0), ("mse", lambda x: x), ("low_var_kl", lambda x: 1 - math.exp(-x)),
+                 ("k1+", lambda x: x), ("k3+", lambda x: x), ("abs", lambda x: math.copysign(1.0, x))]:
+        lp = torch.tensor([[-1.0, -2.0, -3.0]], requires_grad=True)
+        O.kl_penalty(lp, ref, t).sum().backward()
+        for got, x in zip(lp.grad[0].tolist(), (lp.detach() - ref)[0].tolist()):
+            assert got == pytest.approx(g(x), abs=1e-6), t
