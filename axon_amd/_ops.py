@@ -215,7 +215,7 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     acc = _acc8(rows.n_slots, dev)
     # PPO with sum / token-mean needs no per-row quantity: one pass over the tokens, the
     # division by the token count happens when the last workgroup has the total.
-    one_pass = kind == 0 and tr == 0 and br == 0
+    one_pass = kind != 1 and tr == 0 and br == 0
     row_scale = row_mean = None
     if not one_pass:
         cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))

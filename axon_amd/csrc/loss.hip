@@ -258,6 +258,26 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
       }
       const float A = av[j], m = mv[j];
       const float d = lv[j] - ov[j];
+      const float w = wv[j];
+      a[4] += m;
+      if (KIND == 2) {  // REINFORCE / GPG (loss.py:471-512): -A * log_prob * w
+        a[2] += -d * m;
+        a[0] += (-A * lv[j] * w) * m * scale;
+        gv[j] = -A * w * m * scale;
+        continue;
+      }
+      if (KIND == 3) {  // CISPO (loss.py:411-468): -sg(clip(r)) * A * log_prob, IS weights not used
+        const float xc = clampf(d, -kSafetyBound, kSafetyBound);
+        const float r_ = expf(xc);
+        const float rc = clampf(r_, lo, hi);
+        float tm = 1.f;  // optional token-level mask of the unified formulation (clip_c != 0)
+        if (clip_c != 0.f && ((A > 0.f && r_ > hi) || (A < 0.f && r_ < lo))) tm = 0.f;
+        a[1] += (r_ > hi || r_ < lo) ? m : 0.f;
+        a[2] += -xc * m;
+        a[0] += (-rc * A * lv[j] * tm) * m * scale;
+        gv[j] = -rc * A * tm * m * scale;
+        continue;
+      }
       float x;  // exponent before the +-20 clamp
       if (KIND == 0) x = d;
       else x = (lv[j] - lv[j]) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
@@ -280,8 +300,6 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
           else if (!(pg3 > c.v)) c = ValGrad{pg3 + c.v, 0.f};
         }
       }
-      a[4] += m;
-      const float w = wv[j];
       a[0] += (c.v * w) * m * scale;
       gv[j] = (pass ? c.g : 0.f) * w * m * scale;
     }
@@ -502,9 +520,9 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
   int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
   if (rc != AXON_OK) return rc;
   if (n_slots == 0) return AXON_OK;
-  if (kind != 0 && kind != 1) return AXON_ERR_ARG;
+  if (kind < 0 || kind > 3) return AXON_ERR_ARG;
   if (!logp || !oldp || !adv || !mask || !grad || !acc || !partials) return AXON_ERR_ARG;
-  if (post_normalize && (row_scale != nullptr || kind != 0)) return AXON_ERR_ARG;
+  if (post_normalize && (row_scale != nullptr || kind == 1)) return AXON_ERR_ARG;
   if (kind == 1 && !row_mean) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
   const dim3 g(stream_grid(n_slots)), blk(kBlock);
@@ -514,9 +532,15 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
                      n_rows, n_slots, uniform_len, row_scale, row_mean, uniform_scale, ratio_lo, \
                      ratio_hi, clip_c, grad, partials)
   if (mask_kind == AXON_MASK_F32) {
-    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0); else AXON_LAUNCH_PL(AXON_MASK_F32, 1);
+    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0);
+    else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_F32, 1);
+    else if (kind == 2) AXON_LAUNCH_PL(AXON_MASK_F32, 2);
+    else AXON_LAUNCH_PL(AXON_MASK_F32, 3);
   } else {
-    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_I64, 0); else AXON_LAUNCH_PL(AXON_MASK_I64, 1);
+    if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_I64, 0);
+    else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_I64, 1);
+    else if (kind == 2) AXON_LAUNCH_PL(AXON_MASK_I64, 2);
+    else AXON_LAUNCH_PL(AXON_MASK_I64, 3);
   }
 #undef AXON_LAUNCH_PL
   AXON_CHECK_LAUNCH();

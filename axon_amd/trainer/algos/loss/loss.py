@@ -21,7 +21,7 @@ from axon_amd import _lib, _ops
 from axon_amd.trainer.algos.constants import VALID_BATCH_REDUCE, VALID_TOKEN_REDUCE
 from axon_amd.trainer.algos.loss.registry import LossFn, register_loss
 
-_KIND_PPO, _KIND_GSPO = 0, 1
+_KIND_PPO, _KIND_GSPO, _KIND_REINFORCE, _KIND_CISPO = 0, 1, 2, 3
 
 
 class _ClippedPolicyLoss(torch.autograd.Function):
@@ -49,11 +49,14 @@ def _run(kind: int, data, config, default_token_reduce: str):
     clip = config.get("clip_ratio", 0.2)
     lo = config.get("clip_ratio_low", None)
     hi = config.get("clip_ratio_high", None)
-    lo = clip if lo is None else lo
+    # CISPO leaves the lower side effectively unclipped unless asked to (loss.py:435-436)
+    lo = (1e10 if kind == _KIND_CISPO else clip) if lo is None else lo
     hi = clip if hi is None else hi
     clip_c = config.get("clip_ratio_c", 3.0)
     if kind == _KIND_PPO:
         assert clip_c > 1.0, f"clip_ratio_c must be > 1.0, got {clip_c}"
+    if kind == _KIND_CISPO:  # the slot carries the token_level_mask switch instead
+        clip_c = 1.0 if config.get("token_level_mask", False) else 0.0
     token_reduce = config.get("token_reduce", default_token_reduce)
     batch_reduce = config.get("batch_reduce", "token-mean")
     if token_reduce not in VALID_TOKEN_REDUCE:
@@ -79,7 +82,8 @@ def _run(kind: int, data, config, default_token_reduce: str):
         "old_log_probs": b["old_log_probs"],
         "advantages": b["advantages"],
         "response_mask": b["response_mask"],
-        "sampler_is_weights": b.get("sampler_is_weights", None),
+        # CISPO does not read the sampler weights (loss.py:421-468)
+        "sampler_is_weights": None if kind == _KIND_CISPO else b.get("sampler_is_weights", None),
     }
     hp = dict(
         token_reduce=token_reduce, batch_reduce=batch_reduce,
@@ -91,11 +95,11 @@ def _run(kind: int, data, config, default_token_reduce: str):
     loss, acc = _ClippedPolicyLoss.apply(log_probs, kind, tensors, rows, hp)
     sums = acc.tolist()  # the only host sync of the loss
     denom = max(sums[4], 1.0)
-    metrics: dict[str, Any] = {
-        "pg_clipfrac": sums[1] / denom,
-        "ppo_kl": sums[2] / denom,
-        "pg_clipfrac_lower": (sums[3] / denom) if kind == _KIND_PPO else 0.0,
-    }
+    metrics: dict[str, Any] = {"ppo_kl": sums[2] / denom}
+    if kind != _KIND_REINFORCE:
+        metrics["pg_clipfrac"] = sums[1] / denom
+    if kind in (_KIND_PPO, _KIND_GSPO):
+        metrics["pg_clipfrac_lower"] = (sums[3] / denom) if kind == _KIND_PPO else 0.0
     return loss, metrics
 
 
@@ -109,3 +113,21 @@ def ppo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
 def gspo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
     """GSPO sequence-level ratio loss (loss.py:114-180); code defaults mean / token-mean (:165-166)."""
     return _run(_KIND_GSPO, data, config, "mean")
+
+
+@register_loss(LossFn.REINFORCE)
+def reinforce_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """``-log_prob * A`` (times the sampler weights when present), loss.py:471-512; sum / token-mean."""
+    return _run(_KIND_REINFORCE, data, config, "sum")
+
+
+@register_loss(LossFn.GPG)
+def gpg_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """Same objective as REINFORCE; pairs with the GPG advantage (loss.py:183-197)."""
+    return reinforce_loss_fn(data, config)
+
+
+@register_loss(LossFn.CISPO)
+def cispo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """Clipped, stop-gradient importance weight times ``A * log_prob`` (loss.py:411-468)."""
+    return _run(_KIND_CISPO, data, config, "sum")

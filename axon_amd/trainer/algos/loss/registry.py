@@ -19,11 +19,14 @@ LossRegistryEntry = FunctionRegistryEntry
 
 
 class LossFn(str, Enum):
-    """Losses this path provides (the reference enum also lists gpg, clip_cov, kl_cov,
-    geo_mean, cispo, reinforce, value — outside this path)."""
+    """Losses this path provides (the reference enum also lists clip_cov, kl_cov, geo_mean and
+    value, which are not on it)."""
 
     PPO = "ppo"
     GSPO = "gspo"
+    GPG = "gpg"
+    CISPO = "cispo"
+    REINFORCE = "reinforce"
 
 
 _loss_registry: FunctionRegistry = FunctionRegistry(name="policy loss")

@@ -244,12 +244,15 @@ int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_ro
 /* Clipped policy loss, forward and gradient in one pass.
  *   kind 0: ppo_loss_fn  (axon/trainer/algos/loss/loss.py:47-111), dual clip c
  *   kind 1: gspo_loss_fn (axon/trainer/algos/loss/loss.py:114-180)
+ *   kind 2: reinforce_loss_fn / gpg_loss_fn (loss.py:183-197, 471-512): -A * logp * is_weights
+ *   kind 3: cispo_loss_fn (loss.py:411-468): -sg(clamp(ratio)) * A * logp; clip_c != 0 switches
+ *           the optional token-level mask on; is_weights must be NULL
  * ratio_lo / ratio_hi: the clamp bounds 1 - clip_ratio_low and 1 + clip_ratio_high,
  * evaluated in double by the caller and rounded to fp32 (what torch.clamp does
  * with Python scalars).  clip_c: dual-clip constant (> 1), PPO only.
  * row_scale: per-row multiplier from axon_loss_row_scale, or NULL with
  * uniform_scale applied to every token.
- * post_normalize != 0 (PPO with row_scale NULL only): `sum` / `token-mean`
+ * post_normalize != 0 (row_scale NULL, any kind but 1): `sum` / `token-mean`
  * aggregation in ONE pass over the tokens (utils.py:224-229): the kernel sums
  * uniform_scale * loss * mask, then divides the total by max(valid_count[0], 1), or by
  * max(sum mask, 1) when valid_count is NULL; grad[] is left WITHOUT that division and

@@ -155,3 +155,30 @@ def actor_loss(loss_fn, log_prob, entropy, old_log_prob, advantages, response_ma
         metrics["kl_loss"] = kl_loss.item() * n_micro_batches
         metrics["kl_coef"] = loss_args["kl_coef"]
     return loss * dp_replicas, metrics
+
+
+def reinforce_loss(log_prob, old_log_prob, advantages, response_mask, *, sampler_is_weights=None, token_reduce="sum",
+                   batch_reduce="token-mean", **agg_kwargs):
+    """loss.py:471-512 (also GPG, :183-197).  Returns (loss, {ppo_kl})."""
+    per_tok = -advantages * log_prob
+    if sampler_is_weights is not None:
+        per_tok = -advantages * log_prob * sampler_is_weights
+    loss = agg_loss(per_tok, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    return loss, {"ppo_kl": masked_mean(-(log_prob - old_log_prob), response_mask).item()}
+
+
+def cispo_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0.2, clip_ratio_low=None,
+               clip_ratio_high=None, token_level_mask=False, token_reduce="sum", batch_reduce="token-mean",
+               **agg_kwargs):
+    """loss.py:411-468: the clipped importance weight is a constant, gradients flow through log_prob only."""
+    lo = 1e10 if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    nak = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(nak)
+    per_tok = -torch.clamp(ratio, 1 - lo, 1 + hi).detach() * advantages * log_prob
+    if token_level_mask:
+        drop = ((advantages > 0) & (ratio > 1 + hi)) | ((advantages < 0) & (ratio < 1 - lo))
+        per_tok = per_tok * (~drop).float()
+    loss = agg_loss(per_tok, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    clipfrac = masked_mean(((ratio > 1 + hi) | (ratio < 1 - lo)).float(), response_mask)
+    return loss, {"pg_clipfrac": clipfrac.item(), "ppo_kl": masked_mean(-nak, response_mask).item()}

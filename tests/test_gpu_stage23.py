@@ -591,3 +591,42 @@ def test_actor_loss_without_side_terms_and_with_sampler_metrics():
     assert "kl_loss" not in m and m["pg_loss"] == pytest.approx(loss.item(), rel=1e-6)
     ref = OS.offpolicy_metrics(d["log_probs"], samp, d["response_mask"])
     _assert_metrics(m, ref, "sampler_corr/")
+
+
+# ---- REINFORCE / GPG / CISPO ---------------------------------------------------------------------
+@pytest.mark.parametrize("tr,br", [("sum", "token-mean"), ("mean", "step-mean")])
+@pytest.mark.parametrize("name", ["reinforce", "gpg", "cispo", "cispo-mask"])
+def test_more_registry_losses_vs_oracle(name, tr, br):
+    d = _c1_with_adv(5)
+    g = torch.Generator().manual_seed(44)
+    d["log_probs"] = d["old_log_probs"] + 0.3 * torch.randn(d["old_log_probs"].shape, generator=g)
+    isw = (1.0 + 0.2 * torch.randn(d["log_probs"].shape, generator=g)).clamp(0.1, 2.0) * d["response_mask"]
+    cfg = {"token_reduce": tr, "batch_reduce": br}
+    if name.startswith("cispo"):
+        cfg.update(clip_ratio_low=0.2, clip_ratio_high=0.28, token_level_mask=name.endswith("mask"))
+        okw = dict(clip_ratio_low=0.2, clip_ratio_high=0.28, token_level_mask=name.endswith("mask"))
+        fn, reg = OL.cispo_loss, "cispo"
+    else:
+        okw = dict(sampler_is_weights=isw)
+        fn, reg = OL.reinforce_loss, name
+    data = _loss_proto(d, extra={"sampler_is_weights": isw})
+    loss, metrics = compute_loss_fn(data, reg, cfg)
+    loss.backward()
+    lp = d["log_probs"].clone().requires_grad_(True)
+    ref, ref_m = fn(lp, d["old_log_probs"], d["advantages"], d["response_mask"], token_reduce=tr, batch_reduce=br, **okw)
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4, abs=1e-9)
+    assert rel_l2(data.batch["log_probs"].grad, lp.grad) < 1e-5
+    assert set(metrics) == set(ref_m)
+    for k, v in ref_m.items():
+        assert metrics[k] == pytest.approx(v, rel=1e-4, abs=1e-7), k
+
+
+def test_reinforce_known_answers_gpu():
+    lp, adv = T([[1.0, 2.0]]), T([[3.0, 4.0]])
+    data = DataProto.from_dict(tensors={"log_probs": lp.to(DEV), "old_log_probs": lp.to(DEV), "advantages": adv.to(DEV),
+                                        "response_mask": torch.ones(1, 2).to(DEV)})
+    assert compute_loss_fn(data, "reinforce", {})[0].item() == pytest.approx(-5.5)
+    assert compute_loss_fn(data, "gpg", {})[0].item() == pytest.approx(-5.5)
+    data.batch["sampler_is_weights"] = torch.full((1, 2), 2.0).to(DEV)
+    assert compute_loss_fn(data, "reinforce", {})[0].item() == pytest.approx(-11.0)

@@ -241,3 +241,31 @@ def test_oracle_kl_penalty_gradients():
         O.kl_penalty(lp, ref, t).sum().backward()
         for got, x in zip(lp.grad[0].tolist(), (lp.detach() - ref)[0].tolist()):
             assert got == pytest.approx(g(x), abs=1e-6), t
+
+
+def test_oracle_reinforce_known_answers():
+    """tests/trainer/algos/loss/test_loss.py:228-259: lp=[1,2], A=[3,4] -> -5.5; IS weight 2 doubles it."""
+    lp, adv, m = torch.tensor([[1.0, 2.0]]), torch.tensor([[3.0, 4.0]]), torch.ones(1, 2)
+    loss, met = O.reinforce_loss(lp, lp, adv, m)
+    assert loss.item() == pytest.approx(-5.5) and met["ppo_kl"] == 0.0
+    loss2, _ = O.reinforce_loss(lp, lp, adv, m, sampler_is_weights=torch.full((1, 2), 2.0))
+    assert loss2.item() == pytest.approx(-11.0)
+
+
+def test_oracle_cispo_by_hand():
+    old = torch.tensor([[-1.0, -1.0, -1.0, -1.0]])
+    lp = (old + torch.tensor([[0.0, 0.5, -0.5, 0.5]])).requires_grad_(True)
+    adv, m = torch.tensor([[1.0, 1.0, -2.0, -1.0]]), torch.ones(1, 4)
+    loss, met = O.cispo_loss(lp, old, adv, m, clip_ratio_low=0.2, clip_ratio_high=0.28, token_level_mask=True)
+    loss.backward()
+    r = [1.0, math.exp(0.5), math.exp(-0.5), math.exp(0.5)]
+    rc = [min(max(x, 0.8), 1.28) for x in r]
+    keep = [1.0, 0.0, 0.0, 1.0]  # A>0 with r>1.28 dropped; A<0 with r<0.8 dropped
+    want = sum(-rc[i] * adv[0, i].item() * lp[0, i].item() * keep[i] for i in range(4)) / 4
+    assert loss.item() == pytest.approx(want, rel=1e-6)
+    for i in range(4):
+        assert lp.grad[0, i].item() == pytest.approx(-rc[i] * adv[0, i].item() * keep[i] / 4, rel=1e-6, abs=1e-9)
+    assert met["pg_clipfrac"] == pytest.approx(0.75)
+    # default: no lower bound, no token mask
+    l2, m2 = O.cispo_loss(lp.detach(), old, adv, m)
+    assert m2["pg_clipfrac"] == pytest.approx(0.5)  # only r > 1.2 counts
