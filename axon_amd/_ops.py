@@ -102,7 +102,7 @@ def group_stats(scores, gidx, n_groups, eps, norm_by_std=True, want_scalar=True)
     stats = _zeros(3 * max(n_groups, 1), dev).view(3, -1)
     scalar = torch.empty(n, device=dev, dtype=torch.float32) if want_scalar else None
     check(
-        lib.axon_group_stats(ptr(scores), ptr(gidx), n, int(n_groups), float(eps), int(bool(norm_by_std)),
+        lib.axon_group_stats(ptr(scores), ptr(gidx), n, int(n_groups), float(eps), int(norm_by_std),
                              ptr(stats[0]), ptr(stats[1]), ptr(stats[2]), ptr(scalar), stream_ptr()),
         "axon_group_stats",
     )

@@ -105,11 +105,15 @@ __global__ __launch_bounds__(1024) void group_stats_kernel(
     const float* __restrict__ scores, const int64_t* __restrict__ gidx, int64_t n_rows,
     int64_t n_groups, float eps, int norm_by_std, float* mean, float* stdv, float* count,
     float* scalar) {
+  __shared__ int nonzero;  // rows with a non-zero score (GPG's alpha)
+  if (threadIdx.x == 0) nonzero = 0;
+  __syncthreads();
   // phase 1: count -> count[], s1 -> mean[], s2 -> stdv[] (zero-filled by caller)
   for (int64_t i = threadIdx.x; i < n_rows; i += blockDim.x) {
     const int64_t g = gidx[i];
-    if (g < 0 || g >= n_groups) continue;
     const float x = scores[i];
+    if (norm_by_std == 3 && x != 0.f) atomicAdd(&nonzero, 1);
+    if (g < 0 || g >= n_groups) continue;
     atomicAdd(count + g, 1.f);
     atomicAdd(mean + g, x);
     atomicAdd(stdv + g, x * x);
@@ -134,8 +138,18 @@ __global__ __launch_bounds__(1024) void group_stats_kernel(
     const int64_t g = gidx[i];
     if (g < 0 || g >= n_groups) { scalar[i] = 0.f; continue; }
     const float x = scores[i];
-    float v = norm_by_std ? (x - mean[g]) / (stdv[g] + eps) : (x - mean[g]);
-    v = v * ((count[g] > 1.f) ? 1.f : 0.f);
+    const float c = count[g];
+    float v;
+    if (norm_by_std == 2) {  // RLOO / LOOP: (n*s - S) / (n - 1), S = n * mean (advantage.py:112-146)
+      v = (c * x - c * mean[g]) / fmaxf(c - 1.f, 1.f);
+    } else if (norm_by_std == 3) {  // GPG: alpha * (s - mean) / f_norm, eps carries f_norm (:336-371)
+      const float alpha = (float)n_rows / (float)max(nonzero, 1);
+      scalar[i] = alpha * (x - mean[g]) / eps;  // singleton groups have mean 0 and keep their score
+      continue;
+    } else {
+      v = norm_by_std ? (x - mean[g]) / (stdv[g] + eps) : (x - mean[g]);
+    }
+    v = v * ((c > 1.f) ? 1.f : 0.f);
     scalar[i] = v;
   }
 }

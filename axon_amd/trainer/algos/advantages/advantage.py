@@ -25,13 +25,13 @@ def _stage(t: torch.Tensor):
     return t.cuda(), t.device
 
 
-@register_advantage(AdvantageFn.GRPO)
-def grpo_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
+def _group_advantage(data, mode: int, eps: float, clamp_abs: float):
+    """score = sum of token rewards per row -> per-row scalar by group (mode: axon_group_stats) ->
+    broadcast over the response mask."""
     rewards, home = _stage(data.batch["token_level_rewards"])
     mask, _ = _stage(data.batch["response_mask"])
     uid = data.non_tensor_batch["uid"]
-    eps = config.get("epsilon", 1e-6)
-    norm = config.get("norm_adv_by_std", True)
+    norm = mode
 
     cu = data.meta_info.get("cu_seqlens", None) if data.meta_info else None
     rows = _ops.rows_of(rewards, cu)
@@ -45,3 +45,24 @@ def grpo_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tenso
     if home is not None:
         adv = adv.to(home)
     return adv, adv
+
+
+@register_advantage(AdvantageFn.GRPO)
+def grpo_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
+    """Group-normalised outcome advantage (advantage.py:78-109)."""
+    mode = 1 if config.get("norm_adv_by_std", True) else 0
+    return _group_advantage(data, mode, config.get("epsilon", 1e-6), clamp_abs)
+
+
+@register_advantage(AdvantageFn.RLOO)
+@register_advantage(AdvantageFn.LOOP)
+def rloo_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
+    """Leave-one-out advantage ``(n*s_i - S_g)/(n-1)``, 0 for singleton groups (advantage.py:112-146)."""
+    return _group_advantage(data, 2, 1e-6, clamp_abs)
+
+
+@register_advantage(AdvantageFn.GPG)
+def gpg_advantage_fn(data, config, clamp_abs: float = 0.0) -> tuple[torch.Tensor, torch.Tensor]:
+    """``alpha * (score - group_mean) / f_norm`` with ``alpha = rows / count_nonzero(scores)``
+    (advantage.py:336-371)."""
+    return _group_advantage(data, 3, float(config.get("f_norm", 1.0)), clamp_abs)

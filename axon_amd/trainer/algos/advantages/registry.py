@@ -10,9 +10,13 @@ AdvantageRegistryEntry = FunctionRegistryEntry
 
 
 class AdvantageFn(str, Enum):
-    """Estimators this path provides (the reference lists twelve more)."""
+    """Estimators this path provides (the outcome-reward, group-baseline family; the reference also
+    lists GAE and other value- or return-based estimators)."""
 
     GRPO = "grpo"
+    RLOO = "rloo"
+    LOOP = "loop"  # alias of RLOO
+    GPG = "gpg"
 
 
 _advantage_registry: FunctionRegistry = FunctionRegistry(name="advantage estimator")

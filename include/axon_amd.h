@@ -140,7 +140,10 @@ int axon_row_stats(const float* a, const float* b, const void* mask, int mask_ki
  * (axon/trainer/algos/advantages/advantage.py:98-107):
  *   count/s1/s2 by group, mean, var with Bessel, std = sqrt(max(var, eps)),
  *   count<=1 -> mean 0, std 1;
- *   scalar[i] = (score[i]-mean[g])/(std[g]+eps) or score-mean; * (count[g] > 1).
+ *   norm_by_std 1 / 0: scalar[i] = (score[i]-mean[g])/(std[g]+eps) or score-mean; * (count[g] > 1);
+ *   norm_by_std 2: RLOO / LOOP (advantage.py:112-146): (n*s - S_g)/(n-1), 0 for singleton groups;
+ *   norm_by_std 3: GPG (advantage.py:336-371): rows/count_nonzero(scores) * (s - mean[g]) / eps,
+ *                  with eps carrying f_norm.
  * mean/std/count [n_groups] are outputs AND scratch: zero-fill them first.
  * scalar may be NULL (plain group_mean_std).  Single workgroup; n_rows < 2^31. */
 int axon_group_stats(const float* scores, const int64_t* gidx, int64_t n_rows, int64_t n_groups,

@@ -47,6 +47,25 @@ def grpo_advantage(token_level_rewards, response_mask, gidx, eps=1e-6, norm_adv_
     return torch.clamp(adv, -1, 1) if clip else adv
 
 
+def rloo_advantage(token_level_rewards, response_mask, gidx):
+    """advantages/advantage.py:112-146: leave-one-out baseline (n*s_i - S_g)/(n-1); singleton groups 0."""
+    scores = token_level_rewards.sum(-1)
+    c = torch.bincount(gidx)[gidx].to(scores.dtype)
+    gsum = torch.bincount(gidx, weights=scores)[gidx]
+    a = ((c * scores - gsum) / (c - 1).clamp_min(1)) * (c > 1)
+    return a.unsqueeze(-1) * response_mask
+
+
+def gpg_advantage(token_level_rewards, response_mask, gidx, f_norm=1.0):
+    """advantages/advantage.py:336-371: alpha * (score - group mean) / f_norm, alpha = rows / nonzero scores."""
+    scores = token_level_rewards.sum(-1)
+    alpha = scores.shape[0] / torch.count_nonzero(scores).clamp(min=1).to(scores.dtype)
+    c = torch.bincount(gidx)[gidx].to(scores.dtype)
+    gsum = torch.bincount(gidx, weights=scores)[gidx]
+    gmean = torch.where(c > 1, gsum / c, torch.zeros_like(gsum))
+    return (alpha * (scores - gmean) / f_norm).unsqueeze(-1) * response_mask
+
+
 def zero_advantage_keep_rows(advantages, eps=1e-5):
     """Row indices with any |advantage| > eps (strict), as a python list."""
     return torch.nonzero((advantages.abs() > eps).any(dim=1)).squeeze(1).tolist()

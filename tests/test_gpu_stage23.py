@@ -630,3 +630,26 @@ def test_reinforce_known_answers_gpu():
     assert compute_loss_fn(data, "gpg", {})[0].item() == pytest.approx(-5.5)
     data.batch["sampler_is_weights"] = torch.full((1, 2), 2.0).to(DEV)
     assert compute_loss_fn(data, "reinforce", {})[0].item() == pytest.approx(-11.0)
+
+
+# ---- RLOO / LOOP / GPG advantages ------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["rloo", "loop", "gpg"])
+def test_group_baseline_advantages_vs_oracle(name):
+    d = W.c1_loss_only(7)
+    d["token_level_rewards"][5] = 0  # a zero score for GPG's alpha
+    uid = d["uid"].copy()
+    uid[3] = "alone"  # a singleton group
+    gidx = T(np.unique(uid, return_inverse=True)[1])
+    data = DataProto.from_dict(tensors={"token_level_rewards": d["token_level_rewards"].to(DEV),
+                                        "response_mask": d["response_mask"].to(DEV)})
+    data.non_tensor_batch["uid"] = uid
+    args = {"f_norm": 1.5} if name == "gpg" else {}
+    out = compute_advantage(data, {"advantage": name, "advantage_args": args})
+    if name == "gpg":
+        ref = OA.gpg_advantage(d["token_level_rewards"], d["response_mask"], gidx, f_norm=1.5)
+    else:
+        ref = OA.rloo_advantage(d["token_level_rewards"], d["response_mask"], gidx)
+    got = out.batch["advantages"].cpu()
+    assert torch.allclose(got, ref, rtol=1e-5, atol=1e-6)
+    assert torch.equal(out.batch["returns"].cpu(), got)
+    assert (got[d["response_mask"] == 0] == 0).all()

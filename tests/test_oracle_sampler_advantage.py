@@ -239,3 +239,20 @@ def test_oracle_mismatch_stats_by_hand():
     assert s["_logprobs_sum"] == pytest.approx(0.5) and s["batch/sampler_logprobs_diff_max"] == pytest.approx(0.5)
     assert s["_product_sum"] == pytest.approx(pa[0] * ps[0] + pa[1] * ps[1])
     assert S.mismatch_stats(old, samp, torch.zeros(1, 3))["_valid_count"] == 0
+
+
+def test_oracle_rloo_and_gpg_by_hand():
+    # groups: {0,1,2} scores 1,2,6 ; {3} score 5 ; {4,5} scores 0,4
+    tlr = torch.zeros(6, 3)
+    tlr[:, 1] = torch.tensor([1.0, 2.0, 6.0, 5.0, 0.0, 4.0])
+    mask = torch.ones(6, 3)
+    mask[2, 2] = 0
+    g = torch.tensor([0, 0, 0, 1, 2, 2])
+    r = A.rloo_advantage(tlr, mask, g)
+    # (n*s - S)/(n-1): (3*1-9)/2=-3, (6-9)/2=-1.5, (18-9)/2=4.5 ; singleton 0 ; (0-4)/1=-4, (8-4)/1=4
+    assert r[:, 0].tolist() == pytest.approx([-3.0, -1.5, 4.5, 0.0, -4.0, 4.0])
+    assert r[2, 2].item() == 0.0
+    gp = A.gpg_advantage(tlr, mask, g, f_norm=2.0)
+    alpha = 6 / 5  # one zero score
+    assert gp[:, 0].tolist() == pytest.approx([alpha * (1 - 3) / 2, alpha * (2 - 3) / 2, alpha * (6 - 3) / 2,
+                                               alpha * 5 / 2, alpha * (0 - 2) / 2, alpha * (4 - 2) / 2])
