@@ -3,9 +3,10 @@
 ``agg_loss`` keeps the signature of axon/trainer/algos/loss/utils.py:120-187
 (two-axis reduction: token_reduce x batch_reduce) and ``masked_mean`` that of
 :88-91.  Both are differentiable with respect to their first argument.  The
-reductions run in libaxon_amd.so: one row-statistics pass, one single-workgroup
-pass that folds every denominator into a per-row multiplier, and one
-elementwise pass that produces the scalar and its gradient.
+reductions run in libaxon_amd.so: for ``sum`` / ``token-mean`` one pass over the tokens;
+otherwise a row-statistics pass and a single-workgroup pass that folds every denominator
+into a per-row multiplier come first.  Scalars are added from per-workgroup partials in a fixed
+order (no atomics).
 """
 
 from __future__ import annotations
@@ -19,41 +20,23 @@ __all__ = ["agg_loss", "masked_mean"]
 
 
 class _WeightedRowSum(torch.autograd.Function):
-    """sum_t loss[t] * mask[t] * row_scale[row(t)] with gradient mask*row_scale."""
+    """sum_t loss[t] * mask[t] * row_scale[row(t)] with gradient mask*row_scale: the entropy slot of
+    ``axon_side_terms`` (one pass for sum / token-mean, a row pass first otherwise)."""
 
     @staticmethod
-    def forward(ctx, loss_mat, mask, rows, tr, br, extras):
-        lib = _lib.load()
-        dev = loss_mat.device
-        x = _ops.f32(loss_mat)
-        mk, kind = _ops.mask_arg(mask)
-        cnt, _, _ = _ops.row_stats(x, None, mk, rows, want_sum=False)
-        scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        prtc, npt, nps, valid = (_ops._i64_dev(e, dev) for e in extras)
-        _lib.check(
-            lib.axon_loss_row_scale(_lib.ptr(cnt), None, rows.n_rows, rows.uniform_len, tr, br,
-                                    _lib.ptr(prtc if tr == 1 else None), _lib.ptr(npt if tr == 3 else None),
-                                    _lib.ptr(nps if br == 2 else None), _lib.ptr(valid), _lib.ptr(scale), None,
-                                    _lib.stream_ptr()),
-            "axon_loss_row_scale",
-        )
-        weights = _ops.row_broadcast_mask(scale, mk, rows)  # d out / d loss[t]
-        ssum = torch.zeros(1, device=dev, dtype=torch.float32)
-        # total = sum_t x[t] * weights[t]: a single row over all slots
-        one_row = _ops.Rows(1, rows.n_slots, rows.n_slots, None, rows.shape)
-        _lib.check(
-            lib.axon_row_stats(_lib.ptr(x), None, _lib.ptr(weights), _lib.MASK_F32, None, 1, one_row.n_slots,
-                               one_row.uniform_len, 0, 0.0, None, _lib.ptr(ssum), None, _lib.stream_ptr()),
-            "axon_row_stats",
-        )
-        ctx.save_for_backward(weights)
+    def forward(ctx, loss_mat, mask, rows, token_reduce, batch_reduce, extras):
+        prtc, npt, nps, valid = extras
+        acc, agg_w, _ = _ops.side_terms(loss_mat, None, None, mask, rows, token_reduce=token_reduce,
+                                        batch_reduce=batch_reduce, per_row_token_count=prtc, num_program_tokens=npt,
+                                        num_program_steps=nps, valid_count=valid)
+        ctx.save_for_backward(agg_w, acc)
         ctx.in_dtype = loss_mat.dtype
-        return ssum[0]
+        return acc[0].clone()
 
     @staticmethod
     def backward(ctx, g):
-        (weights,) = ctx.saved_tensors
-        return (weights * g).to(ctx.in_dtype), None, None, None, None, None
+        agg_w, acc = ctx.saved_tensors
+        return (agg_w * (g * acc[5])).to(ctx.in_dtype), None, None, None, None, None
 
 
 def agg_loss(
@@ -89,7 +72,7 @@ def agg_loss(
     _lib.require_device(loss_mat, "agg_loss")
     rows = _ops.rows_of(loss_mat, cu_seqlens)
     return _WeightedRowSum.apply(
-        loss_mat, loss_mask, rows, _ops.TOKEN_REDUCE[token_reduce], _ops.BATCH_REDUCE[batch_reduce],
+        loss_mat, loss_mask, rows, token_reduce, batch_reduce,
         (per_row_token_count, num_program_tokens, num_program_steps, valid),
     )
 
