@@ -39,6 +39,8 @@ SIGNATURES: dict[str, tuple] = {
                                        _i32, _f32, _f32, _i32, _f32, _ptr, _ptr, _ptr, _ptr, _ptr,
                                        _ptr, _ptr, _ptr]),
     "axon_reduce_partials_bytes": (_i64, [_i64]),
+    "axon_gmpo_loss": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr,
+                              _ptr, _ptr]),
     "axon_kl_penalty": (_i32, [_ptr, _ptr, _i64, _i32, _i32, _ptr, _ptr, _ptr]),
     "axon_side_terms": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _ptr, _f32, _i32, _ptr, _i32,
                                _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
@@ -52,7 +54,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -240,6 +240,27 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     return acc, grad
 
 
+def gmpo_loss(log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows, *, clip_low, clip_high):
+    """GMPO loss and gradient; returns (acc[8], grad).  See axon_gmpo_loss."""
+    lib = _lib.load()
+    require_device(log_probs, "gmpo_loss")
+    dev = log_probs.device
+    lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
+    mk, mkind = mask_arg(mask)
+    isw = f32(is_weights) if is_weights is not None else None
+    row_ws = torch.empty(5 * rows.n_rows, device=dev, dtype=torch.float32)
+    row_ws[: 4 * rows.n_rows].zero_()
+    grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    acc = _acc8(rows.n_slots, dev)
+    check(
+        lib.axon_gmpo_loss(ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
+                           rows.n_slots, rows.uniform_len, float(clip_low), float(clip_high), ptr(row_ws), ptr(grad),
+                           ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
+        "axon_gmpo_loss",
+    )
+    return acc, grad
+
+
 KL_TYPES = {"kl": 1, "k1": 1, "abs": 2, "mse": 3, "k2": 3, "low_var_kl": 4, "k3": 4}
 
 

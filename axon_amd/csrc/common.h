@@ -108,6 +108,41 @@ __device__ __forceinline__ void store4(float* p, int64_t i, const float (&v)[4])
   __builtin_nontemporal_store(x, reinterpret_cast<f32x4*>(p + i));
 }
 
+// Per-row sums of NV values from a token-parallel kernel: a lane folds its slots into a RowSeg,
+// the wave runs a segmented shuffle reduction keyed by row id (row ids are non-decreasing across
+// lanes) and the first lane of each run adds the run total to row_vals[k][row] with one atomic.
+template <int NV>
+struct RowSeg {
+  int row;
+  float v[NV];
+};
+
+template <int NV>
+__device__ __forceinline__ void row_seg_flush(const RowSeg<NV>& s, float* row_vals, int64_t n_rows) {
+  if (s.row < 0) return;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+    if (s.v[k] != 0.f) atomicAdd(row_vals + (int64_t)k * n_rows + s.row, s.v[k]);
+}
+
+template <int NV>
+__device__ __forceinline__ void row_seg_wave_reduce_flush(RowSeg<NV> s, float* row_vals, int64_t n_rows) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int off = 1; off < kWave; off <<= 1) {
+    const int r2 = __shfl_down(s.row, off, kWave);
+    float t[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) t[k] = __shfl_down(s.v[k], off, kWave);
+    if (lane + off < kWave && r2 == s.row) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k) s.v[k] += t[k];
+    }
+  }
+  const int prev = __shfl_up(s.row, 1, kWave);
+  if (lane == 0 || prev != s.row) row_seg_flush(s, row_vals, n_rows);
+}
+
 // Row lookup.  row(pos) = number of s in [1, n_rows] with cu[s] <= pos, i.e. the
 // row whose half-open range contains pos; empty rows are skipped.  A workgroup
 // owns the contiguous slots [c0, c1); it caches the cu_seqlens entries covering

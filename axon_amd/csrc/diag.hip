@@ -21,33 +21,13 @@ __device__ __forceinline__ float clampf3(float x, float lo, float hi) {
   return (x != x) ? x : fminf(fmaxf(x, lo), hi);
 }
 
-struct DiagSeg {
-  int row;
-  float v[kDiagRowVals];
-};
+using DiagSeg = RowSeg<kDiagRowVals>;
 
 __device__ __forceinline__ void diag_flush(const DiagSeg& s, float* row_vals, int64_t n_rows) {
-  if (s.row < 0) return;
-#pragma unroll
-  for (int k = 0; k < kDiagRowVals; ++k)
-    if (s.v[k] != 0.f) atomicAdd(row_vals + (int64_t)k * n_rows + s.row, s.v[k]);
+  row_seg_flush(s, row_vals, n_rows);
 }
-
 __device__ __forceinline__ void diag_wave_reduce_flush(DiagSeg s, float* row_vals, int64_t n_rows) {
-  const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const int r2 = __shfl_down(s.row, off, kWave);
-    float t[kDiagRowVals];
-#pragma unroll
-    for (int k = 0; k < kDiagRowVals; ++k) t[k] = __shfl_down(s.v[k], off, kWave);
-    if (lane + off < kWave && r2 == s.row) {
-#pragma unroll
-      for (int k = 0; k < kDiagRowVals; ++k) s.v[k] += t[k];
-    }
-  }
-  const int prev = __shfl_up(s.row, 1, kWave);
-  if (lane == 0 || prev != s.row) diag_flush(s, row_vals, n_rows);
+  row_seg_wave_reduce_flush(s, row_vals, n_rows);
 }
 
 template <int MK>

@@ -436,6 +436,161 @@ __global__ __launch_bounds__(kBlock) void side_terms_kernel(
   store_block_partials<6>(a, lds_red, partials);
 }
 
+// ---- GMPO (geo_mean_loss_fn, axon/trainer/algos/loss/loss.py:355-408) ------------------------------
+// Per token: nak_min = sgn(A) * min(sgn(A) * nak, sgn(A) * clamp(nak, -lo, hi)), nak = logp - old.
+// Per row: ratio = exp(sum(nak_min * m) / (cnt + 1e-8)), adv = sum(A * m) / (cnt + 1e-8),
+// w = exp(sum(log(is_w + 1e-10) * m) / (cnt + 1e-8)); loss = mean over rows with tokens of -adv*ratio*w.
+__device__ __forceinline__ ValGrad gmpo_term(float nak, float A, float lo, float hi) {
+  const float sg = (A > 0.f) ? 1.f : ((A < 0.f) ? -1.f : 0.f);
+  const float c = clampf(nak, -lo, hi);
+  const float dclamp = (nak >= -lo && nak <= hi) ? 1.f : 0.f;
+  const float a1 = sg * nak, a2 = sg * c;
+  float v, g;
+  if (a1 < a2) { v = a1; g = sg; }
+  else if (a1 > a2) { v = a2; g = sg * dclamp; }
+  else { v = a1; g = 0.5f * (sg + sg * dclamp); }  // torch.min splits the gradient on ties
+  return ValGrad{sg * v, sg * g};
+}
+
+constexpr int kGmpoRowVals = 4;  // cnt, sum nak_min*m, sum A*m, sum log(is_w + 1e-10)*m
+
+// PASS 0: row sums and metric partials.  PASS 1: gradient from the per-row coefficients.
+template <int MK, int PASS>
+__global__ __launch_bounds__(kBlock) void gmpo_kernel(
+    const float* __restrict__ logp, const float* __restrict__ oldp, const float* __restrict__ adv,
+    const void* __restrict__ mask, const float* __restrict__ isw, const int32_t* __restrict__ cu,
+    int64_t n_rows, int64_t n_slots, int64_t uniform_len, float lo, float hi, float* row_vals,
+    const float* __restrict__ row_coef, float* __restrict__ grad, float* partials) {
+  __shared__ int32_t lds_cu[kLdsRows];
+  __shared__ float lds_red[5 * (kBlock / kWave)];
+  float a[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+  const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
+#pragma unroll 1
+  for (int64_t chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const int64_t c0 = chunk * kChunk;
+    const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+    __syncthreads();
+    RowFinder rf;
+    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+#pragma unroll 1
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      RowSeg<kGmpoRowVals> s;
+      s.row = -1;
+#pragma unroll
+      for (int k = 0; k < kGmpoRowVals; ++k) s.v[k] = 0.f;
+      if (i < c1) {
+        float lv[4], ov[4], av[4], mv[4], wv[4] = {1.f, 1.f, 1.f, 1.f}, gv[4];
+        const bool full = (i + kVec <= n_slots);
+        if (full) {
+          load4(logp, i, lv);
+          load4(oldp, i, ov);
+          load4(adv, i, av);
+          load_mask4<MK>(mask, i, mv);
+          if (PASS == 0 && isw) load4(isw, i, wv);
+        } else {
+          for (int j = 0; j < 4; ++j) {
+            const bool ok = i + j < n_slots;
+            lv[j] = ok ? logp[i + j] : 0.f;
+            ov[j] = ok ? oldp[i + j] : 0.f;
+            av[j] = ok ? adv[i + j] : 0.f;
+            mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+            wv[j] = (ok && PASS == 0 && isw) ? isw[i + j] : 1.f;
+          }
+        }
+        int r = rf.row(i);
+        int64_t rend = rf.row_end(r);
+        s.row = r;
+        float coef = (PASS == 1) ? row_coef[r] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t p = i + j;
+          if (p >= n_slots) { gv[j] = 0.f; continue; }
+          if (p >= rend) {
+            if (PASS == 0) row_seg_flush(s, row_vals, n_rows);
+            r = rf.row(p);
+            rend = rf.row_end(r);
+            s.row = r;
+#pragma unroll
+            for (int k = 0; k < kGmpoRowVals; ++k) s.v[k] = 0.f;
+            if (PASS == 1) coef = row_coef[r];
+          }
+          const float m = mv[j], A = av[j];
+          const float nak = lv[j] - ov[j];
+          const ValGrad t = gmpo_term(nak, A, lo, hi);
+          if (PASS == 0) {
+            const bool clipped = (nak != clampf(nak, -lo, hi));
+            a[1] += (clipped && A > 0.f) ? m : 0.f;
+            a[2] += -nak * m;
+            a[3] += (clipped && A < 0.f) ? m : 0.f;
+            a[4] += m;
+            s.v[0] += m;
+            s.v[1] += t.v * m;
+            s.v[2] += A * m;
+            if (isw) s.v[3] += logf(wv[j] + 1e-10f) * m;
+          } else {
+            gv[j] = coef * m * t.g;
+          }
+        }
+        if (PASS == 1) {
+          if (full) store4(grad, i, gv);
+          else
+            for (int j = 0; j < 4 && i + j < n_slots; ++j) grad[i + j] = gv[j];
+        }
+      }
+      if (PASS == 0) row_seg_wave_reduce_flush(s, row_vals, n_rows);
+    }
+  }
+  if (PASS == 0) store_block_partials<5>(a, lds_red, partials);
+}
+
+// One workgroup: per-row loss terms -> acc[0] (mean over rows with tokens; over all rows when no row
+// has any) and row_coef[r] = d loss / d (sum nak_min*m)_r.
+__global__ __launch_bounds__(1024) void gmpo_rows_kernel(const float* __restrict__ row_vals, int64_t n_rows,
+                                                         int has_isw, float* __restrict__ row_coef,
+                                                         float* __restrict__ acc) {
+  __shared__ double red[16][3];
+  __shared__ double tot[3];
+  const float* cnt_a = row_vals;
+  const float* s1_a = row_vals + n_rows;
+  const float* s2_a = row_vals + 2 * n_rows;
+  const float* s3_a = row_vals + 3 * n_rows;
+  double t[3] = {0.0, 0.0, 0.0};  // valid rows, sum of valid rows' losses, sum of all rows' losses
+  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+    const float cnt = cnt_a[r], den = cnt + 1e-8f;
+    const float ratio = expf(s1_a[r] / den);
+    const float w = has_isw ? expf(s3_a[r] / den) : 1.f;
+    const float l = -(s2_a[r] / den) * ratio * w;
+    if (cnt > 0.f) { t[0] += 1.0; t[1] += (double)l; }
+    t[2] += (double)l;
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int k = 0; k < 3; ++k) {
+    double v = t[k];
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);
+    if (lane == 0) red[wave][k] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 0; k < 3; ++k) {
+      double v = 0.0;
+      for (int w = 0; w < (int)(blockDim.x >> 6); ++w) v += red[w][k];
+      tot[k] = v;
+    }
+    acc[0] = (float)(tot[0] > 0.0 ? tot[1] / tot[0] : tot[2] / (double)n_rows);
+  }
+  __syncthreads();
+  const bool any_valid = tot[0] > 0.0;
+  const float inv_n = (float)(1.0 / (any_valid ? tot[0] : (double)n_rows));
+  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+    const float cnt = cnt_a[r], den = cnt + 1e-8f;
+    const float ratio = expf(s1_a[r] / den);
+    const float w = has_isw ? expf(s3_a[r] / den) : 1.f;
+    const float l = -(s2_a[r] / den) * ratio * w;
+    row_coef[r] = (any_valid && !(cnt > 0.f)) ? 0.f : l * inv_n / den;
+  }
+}
+
 }  // namespace axon
 
 using namespace axon;
@@ -593,6 +748,36 @@ extern "C" int axon_side_terms(const float* entropy, const float* logp, const fl
   AXON_CHECK_LAUNCH();
   hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
                      post_normalize ? 3 : 0, valid, acc);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_gmpo_loss(const float* logp, const float* oldp, const float* adv, const void* mask,
+                              int mask_kind, const float* isw, const int32_t* cu, int64_t n_rows,
+                              int64_t n_slots, int64_t uniform_len, float clip_low, float clip_high,
+                              float* row_ws, float* grad, float* acc, float* partials, void* stream) {
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, true);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0 || n_rows == 0) return AXON_OK;
+  if (!logp || !oldp || !adv || !mask || !row_ws || !grad || !acc || !partials) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  float* row_vals = row_ws;                          // [4][n_rows], zero-filled by the caller
+  float* row_coef = row_ws + kGmpoRowVals * n_rows;  // [n_rows]
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
+  const hipStream_t st = (hipStream_t)stream;
+#define AXON_LAUNCH_GMPO(MK, PASS)                                                                  \
+  hipLaunchKernelGGL((gmpo_kernel<MK, PASS>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, n_rows, \
+                     n_slots, uniform_len, clip_low, clip_high, row_vals, row_coef, grad, partials)
+  if (mask_kind == AXON_MASK_F32) AXON_LAUNCH_GMPO(AXON_MASK_F32, 0); else AXON_LAUNCH_GMPO(AXON_MASK_I64, 0);
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x, 0,
+                     (const int64_t*)nullptr, acc);
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(gmpo_rows_kernel, dim3(1), dim3(1024), 0, st, row_vals, n_rows, isw != nullptr,
+                     row_coef, acc);
+  AXON_CHECK_LAUNCH();
+  if (mask_kind == AXON_MASK_F32) AXON_LAUNCH_GMPO(AXON_MASK_F32, 1); else AXON_LAUNCH_GMPO(AXON_MASK_I64, 1);
+#undef AXON_LAUNCH_GMPO
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

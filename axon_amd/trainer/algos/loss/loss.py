@@ -131,3 +131,40 @@ def gpg_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
 def cispo_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
     """Clipped, stop-gradient importance weight times ``A * log_prob`` (loss.py:411-468)."""
     return _run(_KIND_CISPO, data, config, "sum")
+
+
+class _GmpoLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, batch, rows, clip_low, clip_high):
+        acc, grad = _ops.gmpo_loss(log_probs, batch["old_log_probs"], batch["advantages"], batch["response_mask"],
+                                   batch["sampler_is_weights"], rows, clip_low=clip_low, clip_high=clip_high)
+        ctx.save_for_backward(grad)
+        ctx.in_dtype = log_probs.dtype
+        ctx.mark_non_differentiable(acc)
+        return acc[0].clone(), acc
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_acc):
+        (grad,) = ctx.saved_tensors
+        return (grad * g_loss).to(ctx.in_dtype), None, None, None, None
+
+
+@register_loss(LossFn.GEO_MEAN)
+def geo_mean_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """GMPO: sequence-level geometric-mean ratio with token-level clipping of the log-ratio
+    (loss.py:355-408).  Ignores token_reduce / batch_reduce like the reference."""
+    b = data.batch
+    clip = config.get("clip_ratio", 0.2)
+    lo = config.get("clip_ratio_low", None)
+    hi = config.get("clip_ratio_high", None)
+    lo = clip if lo is None else lo
+    hi = clip if hi is None else hi
+    log_probs = b["log_probs"]
+    _lib.require_device(log_probs, "policy loss")
+    rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
+    tensors = {"old_log_probs": b["old_log_probs"], "advantages": b["advantages"], "response_mask": b["response_mask"],
+               "sampler_is_weights": b.get("sampler_is_weights", None)}
+    loss, acc = _GmpoLoss.apply(log_probs, tensors, rows, lo, hi)
+    sums = acc.tolist()
+    denom = max(sums[4], 1.0)
+    return loss, {"pg_clipfrac": sums[1] / denom, "ppo_kl": sums[2] / denom, "pg_clipfrac_lower": sums[3] / denom}

@@ -19,14 +19,15 @@ LossRegistryEntry = FunctionRegistryEntry
 
 
 class LossFn(str, Enum):
-    """Losses this path provides (the reference enum also lists clip_cov, kl_cov, geo_mean and
-    value, which are not on it)."""
+    """Losses this path provides (the reference enum also lists clip_cov, kl_cov and value, which are
+    not on it)."""
 
     PPO = "ppo"
     GSPO = "gspo"
     GPG = "gpg"
     CISPO = "cispo"
     REINFORCE = "reinforce"
+    GEO_MEAN = "geo_mean"
 
 
 _loss_registry: FunctionRegistry = FunctionRegistry(name="policy loss")

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 4
+#define AXON_AMD_ABI_VERSION 5
 
 enum {
   AXON_OK = 0,
@@ -295,6 +295,17 @@ int axon_side_terms(const float* entropy, const float* logp, const float* ref_lo
                     int64_t uniform_len, const float* row_scale, float uniform_scale,
                     int post_normalize, const int64_t* valid_count, int kl_type, int kl_plus,
                     float* agg_w, float* grad_kl, float* acc, float* partials, void* stream);
+
+/* GMPO, geo_mean_loss_fn (axon/trainer/algos/loss/loss.py:355-408): the sequence-level loss
+ * -adv_r * exp(mean_t nak_min) * geo-mean(is_weights), averaged over rows that have tokens, with
+ * its gradient w.r.t. logp.  clip_low / clip_high are the log-ratio clip ranges.
+ * row_ws: 5 * n_rows floats, the first 4 * n_rows zero-filled by the caller.
+ * acc[8] (written): [0] loss, [1] sum mask*(clipped & A>0), [2] sum mask*(old-logp),
+ * [3] sum mask*(clipped & A<0), [4] sum mask.  partials: axon_reduce_partials_bytes(n_slots). */
+int axon_gmpo_loss(const float* logp, const float* old_logp, const float* adv, const void* mask,
+                   int mask_kind, const float* is_weights, const int32_t* cu_seqlens, int64_t n_rows,
+                   int64_t n_slots, int64_t uniform_len, float clip_low, float clip_high, float* row_ws,
+                   float* grad, float* acc, float* partials, void* stream);
 
 #ifdef __cplusplus
 }

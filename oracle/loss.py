@@ -182,3 +182,27 @@ def cispo_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=
     loss = agg_loss(per_tok, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
     clipfrac = masked_mean(((ratio > 1 + hi) | (ratio < 1 - lo)).float(), response_mask)
     return loss, {"pg_clipfrac": clipfrac.item(), "ppo_kl": masked_mean(-nak, response_mask).item()}
+
+
+def geo_mean_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0.2, clip_ratio_low=None,
+                  clip_ratio_high=None, sampler_is_weights=None, **_ignored):
+    """loss.py:355-408 (GMPO): token-level clipping of the log-ratio in the direction of the advantage,
+    geometric-mean ratio per sequence, mean over sequences that have tokens."""
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    nak = log_prob - old_log_prob
+    sgn = torch.sign(advantages)
+    nak_c = torch.clamp(nak, -lo, hi)
+    nak_min = sgn * torch.min(sgn * nak, sgn * nak_c)
+    cnt = response_mask.sum(dim=-1)
+    ratio = torch.exp((nak_min * response_mask).sum(dim=-1) / (cnt + 1e-8))
+    adv = (advantages * response_mask).sum(dim=-1) / (cnt + 1e-8)
+    per_row = -adv * ratio
+    if sampler_is_weights is not None:
+        per_row = per_row * torch.exp((torch.log(sampler_is_weights + 1e-10) * response_mask).sum(dim=-1) / (cnt + 1e-8))
+    valid = cnt > 0
+    loss = per_row[valid].mean() if valid.any() else per_row.mean()
+    clipped = torch.ne(nak, nak_c)
+    return loss, {"pg_clipfrac": masked_mean((clipped * (advantages > 0)).float(), response_mask).item(),
+                  "ppo_kl": masked_mean(-nak, response_mask).item(),
+                  "pg_clipfrac_lower": masked_mean((clipped * (advantages < 0)).float(), response_mask).item()}

@@ -653,3 +653,44 @@ def test_group_baseline_advantages_vs_oracle(name):
     assert torch.allclose(got, ref, rtol=1e-5, atol=1e-6)
     assert torch.equal(out.batch["returns"].cpu(), got)
     assert (got[d["response_mask"] == 0] == 0).all()
+
+
+# ---- GMPO (geo_mean) -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("with_isw", [False, True])
+def test_geo_mean_loss_vs_oracle(with_isw):
+    d = _c1_with_adv(6)
+    g = torch.Generator().manual_seed(55)
+    d["log_probs"] = d["old_log_probs"] + 0.3 * torch.randn(d["old_log_probs"].shape, generator=g)
+    d["log_probs"][0, 0] = d["old_log_probs"][0, 0] + 0.2   # on the clip boundary
+    d["advantages"][1] = 0.0                                  # sign 0
+    d["response_mask"][2] = 0.0                               # a row without tokens
+    isw = (1.0 + 0.2 * torch.randn(d["log_probs"].shape, generator=g)).clamp(0.1, 2.0) * d["response_mask"]
+    extra = {"sampler_is_weights": isw} if with_isw else None
+    data = _loss_proto(d, extra=extra)
+    loss, metrics = compute_loss_fn(data, "geo_mean", {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28})
+    loss.backward()
+    lp = d["log_probs"].clone().requires_grad_(True)
+    ref, ref_m = OL.geo_mean_loss(lp, d["old_log_probs"], d["advantages"], d["response_mask"], clip_ratio_low=0.2,
+                                  clip_ratio_high=0.28, sampler_is_weights=isw if with_isw else None)
+    ref.backward()
+    assert loss.item() == pytest.approx(ref.item(), rel=1e-4)
+    assert rel_l2(data.batch["log_probs"].grad, lp.grad) < 1e-5
+    for k, v in ref_m.items():
+        assert metrics[k] == pytest.approx(v, rel=1e-4, abs=1e-7), k
+
+
+def test_geo_mean_known_answer_and_packed_gpu():
+    lp, adv = T([[-1.0, -2.0, -3.0]]), T([[1.0, 2.0, 3.0]])
+    data = DataProto.from_dict(tensors={"log_probs": lp.to(DEV), "old_log_probs": lp.to(DEV), "advantages": adv.to(DEV),
+                                        "response_mask": torch.ones(1, 3).to(DEV)})
+    loss, m = compute_loss_fn(data, "geo_mean", {})
+    assert loss.item() == pytest.approx(-2.0, rel=1e-6) and m["pg_clipfrac"] == 0.0
+    # packed layout == padded layout
+    d = _c1_with_adv(8)
+    lens = d["lengths"].tolist()
+    pk = {k: pad_to_packed(d[k], lens).to(DEV) for k in ("log_probs", "old_log_probs", "advantages", "response_mask")}
+    packed = DataProto.from_dict(tensors=pk, meta_info={"cu_seqlens": W.cu_from_lengths(lens).to(DEV)})
+    l_pk, _ = compute_loss_fn(packed, "geo_mean", {})
+    l_pad, _ = compute_loss_fn(_loss_proto(d), "geo_mean", {})
+    # the mean of +-O(1) row terms cancels to ~3e-4: compare on the scale of the terms
+    assert l_pk.item() == pytest.approx(l_pad.item(), abs=1e-6)

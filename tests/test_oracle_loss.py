@@ -269,3 +269,21 @@ def test_oracle_cispo_by_hand():
     # default: no lower bound, no token mask
     l2, m2 = O.cispo_loss(lp.detach(), old, adv, m)
     assert m2["pg_clipfrac"] == pytest.approx(0.5)  # only r > 1.2 counts
+
+
+def test_oracle_geo_mean_known_answer_and_by_hand():
+    """tests/trainer/algos/loss/test_loss.py:391-403: ratio one, A=[1,2,3] -> -2.0."""
+    lp, adv, m = torch.tensor([[-1.0, -2.0, -3.0]]), torch.tensor([[1.0, 2.0, 3.0]]), torch.ones(1, 3)
+    loss, met = O.geo_mean_loss(lp, lp, adv, m)
+    assert loss.item() == pytest.approx(-2.0, rel=1e-6) and met["pg_clipfrac"] == 0 and met["ppo_kl"] == 0
+    # two rows by hand: row 0 A=+1 with nak = [0.5 (clipped to 0.2), -0.5 (kept: min picks the smaller)],
+    # row 1 A=-1 with nak = [-0.5 (clipped to -0.2), 0.1]; a fully masked third row is left out of the mean
+    old = torch.zeros(3, 2)
+    new = torch.tensor([[0.5, -0.5], [-0.5, 0.1], [9.0, 9.0]])
+    adv2 = torch.tensor([[1.0, 1.0], [-1.0, -1.0], [5.0, 5.0]])
+    m2 = torch.tensor([[1.0, 1.0], [1.0, 1.0], [0.0, 0.0]])
+    loss2, met2 = O.geo_mean_loss(new, old, adv2, m2, clip_ratio=0.2)
+    r0 = math.exp((0.2 - 0.5) / 2)
+    r1 = math.exp((-0.2 + 0.1) / 2)
+    assert loss2.item() == pytest.approx((-1.0 * r0 + 1.0 * r1) / 2, rel=1e-6)
+    assert met2["pg_clipfrac"] == pytest.approx(0.5) and met2["pg_clipfrac_lower"] == pytest.approx(0.25)
