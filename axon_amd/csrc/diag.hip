@@ -93,9 +93,10 @@ __global__ __launch_bounds__(kBlock) void sampler_diag_tokens_kernel(
           if (m == 0.f) continue;  // every quantity below is masked
           const float o = ov[j], sp = sv[j];
           const float lr = o - sp;
-          const float e = expf(clampf3(lr, -kBound, kBound));
-          const float eu = expf(lr);
-          const float pa = expf(o), ps = expf(sp);
+          // diagnostics tolerate the ~1e-6 relative error of the hardware exp2 path
+          const float e = __expf(clampf3(lr, -kBound, kBound));
+          const float eu = (lr >= -kBound && lr <= kBound) ? e : __expf(lr);
+          const float pa = __expf(o), ps = __expf(sp);
           const float dp = fabsf(pa - ps), dl = fabsf(lr);
           const float rej = (lr >= rs_lr_lo && lr <= rs_lr_hi) ? 0.f : 1.f;
           const float ci = clampf3(e, is_lo, is_hi), cr = clampf3(e, rs_lo, rs_hi);
@@ -185,9 +186,12 @@ __device__ __forceinline__ double wave_sum_d(double v) {
   return v;
 }
 
+// Workgroup b of the grid takes token partials b, b + gridDim.x, ... and rows likewise, and leaves its
+// 70 sums / maxima / minima in out[b][kDiagOut]; sampler_diag_final_kernel folds the workgroups.
 __global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
     const float* __restrict__ partials, int n_blocks, const float* __restrict__ row_vals,
-    int64_t n_rows, DiagCfg cfg, double* __restrict__ out) {
+    int64_t n_rows, DiagCfg cfg, double* __restrict__ out_all) {
+  double* out = out_all + (size_t)blockIdx.x * kDiagOut;
   __shared__ double red[16][kOutSums];
   __shared__ float red_mx[16][kOutMM], red_mn[16][kOutMM];
   const float kInf = __builtin_huge_valf();
@@ -199,7 +203,7 @@ __global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
   for (int k = 0; k < kOutMM; ++k) { mx[k] = -kInf; mn[k] = kInf; }
 
   // (a) token partials: sums -> acc[0..22]; (max, min) pairs -> slots 0..2
-  for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
+  for (int b = blockIdx.x * blockDim.x + threadIdx.x; b < n_blocks; b += gridDim.x * blockDim.x) {
     const float* row = partials + (size_t)b * kDiagStride;
 #pragma unroll
     for (int k = 0; k < kDiagSums; ++k) acc[k] += (double)row[k];
@@ -216,7 +220,8 @@ __global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
   const float* sl_a = row_vals + 3 * n_rows;
   const float* se_a = row_vals + 4 * n_rows;
   const float* sr_a = row_vals + 5 * n_rows;
-  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+  for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < n_rows;
+       r += (int64_t)gridDim.x * blockDim.x) {
     const float cnt = cnt_a[r], s_lr = sl_a[r];
     const float den = cnt + 1e-8f;  // masked_mean over a row, axon/utils/torch/ops.py:131-145
     if (cfg.is_mode != 0) {
@@ -310,15 +315,38 @@ __global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
   }
 }
 
+__global__ __launch_bounds__(128) void sampler_diag_final_kernel(const double* __restrict__ parts, int n_parts,
+                                                                 double* __restrict__ out) {
+  const int k = threadIdx.x;
+  if (k >= kOutSums + 2 * kOutMM) return;
+  double v = parts[k];
+  for (int b = 1; b < n_parts; ++b) {
+    const double x = parts[(size_t)b * kDiagOut + k];
+    if (k < kOutSums) v += x;
+    else if (k < kOutSums + kOutMM) v = fmax(v, x);
+    else v = fmin(v, x);
+  }
+  out[k] = v;
+}
+
 }  // namespace axon
 
 using namespace axon;
 
+static inline int diag_row_blocks(int64_t n_rows, int64_t token_blocks) {
+  const int64_t work = n_rows > token_blocks ? n_rows : token_blocks;
+  const int64_t b = (work + 1023) / 1024;
+  return (int)(b < 1 ? 1 : (b > 128 ? 128 : b));
+}
+
 extern "C" int64_t axon_sampler_diag_workspace_bytes(int64_t n_rows, int64_t n_slots) {
   if (n_rows < 0 || n_slots < 0) return AXON_ERR_ARG;
   const int64_t blocks = n_slots > 0 ? (int64_t)stream_grid(n_slots) : 1;
-  // [6][n_rows] row sums (zero-filled by the caller), then the per-workgroup partials
-  return (kDiagRowVals * n_rows + blocks * kDiagStride) * (int64_t)sizeof(float);
+  // [6][n_rows] row sums (zero-filled by the caller), the per-workgroup token partials, then the
+  // row pass's per-workgroup results (doubles, 8-byte aligned)
+  const int64_t floats = kDiagRowVals * n_rows + blocks * kDiagStride;
+  return ((floats + 1) / 2 * 2) * (int64_t)sizeof(float) +
+         (int64_t)diag_row_blocks(n_rows, blocks) * kDiagOut * (int64_t)sizeof(double);
 }
 
 extern "C" int axon_sampler_diag(const float* oldp, const float* samp, const void* mask, int mask_kind,
@@ -332,6 +360,7 @@ extern "C" int axon_sampler_diag(const float* oldp, const float* samp, const voi
   if (uniform_len == 0 && cu == nullptr) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
   if (!oldp || !samp || !mask || !workspace || !out) return AXON_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(workspace) & 7) return AXON_ERR_WORKSPACE;
   if (is_mode < 0 || is_mode > 2 || rs_mode < 0 || rs_mode > 3) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
   float* row_vals = workspace;
@@ -352,8 +381,13 @@ extern "C" int axon_sampler_diag(const float* oldp, const float* samp, const voi
   cfg.is_lo = is_lo; cfg.is_hi = is_hi; cfg.rs_lo = rs_lo; cfg.rs_hi = rs_hi;
   cfg.log_is_lo = log_is_lo; cfg.log_is_hi = log_is_hi;
   cfg.log_rs_lo = log_rs_lo; cfg.log_rs_hi = log_rs_hi;
-  hipLaunchKernelGGL(sampler_diag_rows_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x, row_vals,
-                     n_rows, cfg, out);
+  const int64_t floats = kDiagRowVals * n_rows + (int64_t)g.x * kDiagStride;
+  double* parts = reinterpret_cast<double*>(workspace + (floats + 1) / 2 * 2);
+  const int rb = diag_row_blocks(n_rows, g.x);
+  hipLaunchKernelGGL(sampler_diag_rows_kernel, dim3(rb), dim3(1024), 0, st, partials, (int)g.x, row_vals,
+                     n_rows, cfg, parts);
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(sampler_diag_final_kernel, dim3(1), dim3(128), 0, st, parts, rb, out);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

@@ -205,8 +205,8 @@ int axon_sampler_correction(const float* old_logp, const float* sampler_logp, co
  *   is_mode / rs_mode as in axon_sampler_correction; is_lo/is_hi, rs_lo/rs_hi: ratio thresholds
  *   (lower, upper) in fp32; rs_lr_lo/rs_lr_hi: the log-space interval of the token-level rejection
  *   (same values as passed to axon_sampler_correction); log_*: fp32 log of the ratio thresholds.
- *   workspace: axon_sampler_diag_workspace_bytes(n_rows, n_slots) bytes whose first
- *   6 * n_rows floats the caller has zero-filled.
+ *   workspace: axon_sampler_diag_workspace_bytes(n_rows, n_slots) bytes, 8-byte aligned, whose
+ *   first 6 * n_rows floats the caller has zero-filled.
  * out[72] (double):
  *   sums   [0] mask  [1] e  [2] e^2  [3] lr  [4] exp(lr)-lr-1  [5] e>is_hi  [6] e<is_lo
  *          [7] clamp(e,is)  [8] clamp(e,is)^2  [9] e>rs_hi  [10] e<rs_lo  [11] clamp(e,rs)
