@@ -158,8 +158,8 @@ def hbm_kernels(n_tokens, dev):
 
 # HBM-side bytes of ONE launch of the dominant kernel at the default workload, from rocprofv3 --pmc passes
 # over `bench.py --traffic-probe` (FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0, the factors a 1 GiB
-# device copy in the same run calibrates): 6.59e9 read + 0.36e9 written.
-TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 6.95e9}
+# device copy in the same run calibrates): 6.29e9 read + 0.37e9 written.
+TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 6.65e9}
 
 
 def traffic_probe(workload):
