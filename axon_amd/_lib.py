@@ -20,15 +20,15 @@ SIGNATURES: dict[str, tuple] = {
     "axon_amd_abi_version": (_i32, []),
     "axon_amd_error_string": (ctypes.c_char_p, [_i32]),
     "axon_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
-    "axon_lmhead_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32,
+    "axon_lmhead_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32,
                                _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "axon_lmhead_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "axon_lmhead_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                               _f32, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
-    "axon_lmhead_fwd_timed": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32,
+                               _f32, _f32, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
+    "axon_lmhead_fwd_timed": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32,
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                                     _f32, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
+                                     _f32, _f32, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
     "axon_gemm_nt_bf16": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "axon_row_stats": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
                               _ptr, _ptr, _ptr, _ptr]),
@@ -54,7 +54,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()
@@ -73,6 +73,11 @@ def load() -> ctypes.CDLL:
     with _lock:
         if _lib is not None:
             return _lib
+        # The process must hold ONE HIP runtime: torch ships its own libamdhip64, so torch is loaded
+        # first and the library's dependency then resolves to that copy (loaded the other way round,
+        # the library's runtime sees no device).
+        import torch  # noqa: F401
+
         path = _build.ensure_built()
         if not os.path.exists(path):
             raise AxonAmdError(f"{path} is missing and could not be built")

@@ -38,7 +38,13 @@ struct FwdParams {
   float* pe;   // sum (x*c - max) * 2^(x*c - max)
   int n_tokens, vocab;
   float c;     // inv_temperature * log2(e)
+  float cap, inv_cap;  // logit soft-capping cap * tanh(logit / cap) (SOFTCAP kernels only)
 };
+
+// tanh(u) = 1 - 2 / (e^(2u) + 1): saturates cleanly at +-1 (2^x -> inf gives rcp 0, 2^x -> 0 gives -1)
+__device__ __forceinline__ float fast_tanh(float u) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(u * (2.f * kLog2e)) + 1.f);
+}
 
 constexpr float kEmptyMax = -3.0e38f;  // running max of a partial that saw no vocabulary row
 
@@ -101,20 +107,42 @@ __device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParam
   }
 }
 
-template <class Loop>
-__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
-                                                                  int tiles_m, int tiles_n) {
+// SOFTCAP: the logits go through cap * tanh(. / cap) before the statistics (fused_linear.py:19-23).
+template <class Loop, bool SOFTCAP>
+__device__ __forceinline__ void fwd_body(const GemmOperands& g, const FwdParams& p, int tiles_m,
+                                         int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);
   f32x16 acc[4][4];
   Loop::run(g, t, acc, smem);
+  if (SOFTCAP) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) acc[i][j][q] = p.cap * fast_tanh(acc[i][j][q] * p.inv_cap);
+  }
   const LanePos lp;
   if (t.m_lo > 0 || t.m0 + kTile > p.vocab)
     fwd_epilogue<true>(acc, p, lp, t, tm);
   else
     fwd_epilogue<false>(acc, p, lp, t, tm);
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
+                                                                  int tiles_m, int tiles_n) {
+  fwd_body<Loop, false>(g, p, tiles_m, tiles_n);
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_softcap_kernel(GemmOperands g,
+                                                                          FwdParams p, int tiles_m,
+                                                                          int tiles_n) {
+  fwd_body<Loop, true>(g, p, tiles_m, tiles_n);
 }
 
 // Merge partials: lse, entropy_b, entropy.  One thread per token.
@@ -143,12 +171,12 @@ __global__ __launch_bounds__(256) void lmhead_merge_kernel(
   fin_log2s[n] = L;
 }
 
-// logprob[n] = hidden[n] . W[label[n]] / T - lse[n].  One wave per token.
+// logprob[n] = softcap(hidden[n] . W[label[n]]) / T - lse[n].  One wave per token.
 template <typename LabelT>
 __global__ __launch_bounds__(256) void lmhead_label_kernel(
     const __bf16* __restrict__ hidden, const __bf16* __restrict__ weight,
     const LabelT* __restrict__ labels, int n_tokens, int hidden_sz, int vocab, float inv_temp,
-    const float* __restrict__ fin_max, const float* __restrict__ fin_log2s,
+    float cap, const float* __restrict__ fin_max, const float* __restrict__ fin_log2s,
     float* __restrict__ logprobs) {
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= n_tokens) return;
@@ -169,6 +197,7 @@ __global__ __launch_bounds__(256) void lmhead_label_kernel(
     }
   }
   dot = wave_sum(dot);
+  if (cap != 0.f) dot = cap * fast_tanh(dot / cap);
   // (logit*c - M) is formed in one rounding, then log2(sum) is subtracted: no cancellation
   if (lane == 0) logprobs[n] = (fmaf(dot, inv_temp * kLog2e, -fin_max[n]) - fin_log2s[n]) * kLn2;
 }
@@ -188,6 +217,7 @@ struct DlogitParams {
   int64_t ld_dl, ld_dlT;
   int n_tokens, vocab, v_begin;  // v_begin: first vocab row of this chunk
   float inv_temp;
+  float cap, inv_cap;  // soft-capping (SOFTCAP kernels only)
 };
 
 // Per-wave staging of the wave's 128(n) x 128(m) bf16 sub-tile in its own 32 KB of LDS:
@@ -198,9 +228,11 @@ __device__ __forceinline__ int stage_off(int nw, int unit) {
   return nw * 256 + ((unit ^ ((nw & 31) ^ (nw >> 5))) << 3);
 }
 
-template <class Loop>
-__global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperands g, DlogitParams p,
-                                                                     int tiles_m, int tiles_n) {
+// SOFTCAP: the recomputed logit goes through cap * tanh(. / cap) and the gradient is multiplied by
+// the derivative 1 - tanh^2 (fused_linear.py:80-83).
+template <class Loop, bool SOFTCAP>
+__device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitParams& p,
+                                            int tiles_m, int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
@@ -238,11 +270,18 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperand
         for (int e = 0; e < 4; ++e) {
           const int q = 4 * r + e;
           const int mrel = lp.m(i, q);
-          const float raw = acc[i][j][q];
+          float raw = acc[i][j][q];
+          float dcap = 1.f;
+          if (SOFTCAP) {
+            const float th = fast_tanh(raw * p.inv_cap);
+            raw = p.cap * th;
+            dcap = fmaf(-th, th, 1.f);
+          }
           const float pr = fast_exp2(fmaf(raw, c, -lse2));
           const float x = raw * p.inv_temp;
           float v = pr * fmaf(cb, x, ca);
           if ((int64_t)mrel == lab_rel) v += gl;
+          if (SOFTCAP) v *= dcap;
           // rows shared with the neighbouring tile keep their (identical) values
           const bool ok = n_ok && (p.v_begin + t.m0 + mrel < p.vocab);
           d[e] = ok ? v : 0.f;
@@ -289,6 +328,20 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperand
         *reinterpret_cast<uint2*>(p.dlT + (int64_t)(m_base + unit * 4 + e) * p.ld_dlT + n_base + nq * 4) = o[e];
     }
   }
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_kernel(GemmOperands g, DlogitParams p,
+                                                                     int tiles_m, int tiles_n) {
+  dlogit_body<Loop, false>(g, p, tiles_m, tiles_n);
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_softcap_kernel(GemmOperands g,
+                                                                             DlogitParams p,
+                                                                             int tiles_m,
+                                                                             int tiles_n) {
+  dlogit_body<Loop, true>(g, p, tiles_m, tiles_n);
 }
 
 // ----------------------------------------------------------------------------
@@ -550,14 +603,15 @@ int launch_zero_cols(void* p, int64_t ld, int rows, int col0, int ncols, hipStre
 }
 
 int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64, int64_t n,
-             int64_t h, int64_t v, float inv_temp, float* logprobs, float* entropy, float* lse,
-             float* entropy_b, void* workspace, int64_t ws_bytes, void* stream, PhaseTimer* timer) {
+             int64_t h, int64_t v, float inv_temp, float softcap, float* logprobs, float* entropy,
+             float* lse, float* entropy_b, void* workspace, int64_t ws_bytes, void* stream,
+             PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
   if (!hidden || !weight || !labels || !logprobs || !entropy || !lse || !entropy_b || !workspace)
     return AXON_ERR_ARG;
-  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
+  if (!(inv_temp > 0.f) || !(softcap >= 0.f)) return AXON_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight)) & 15)
     return AXON_ERR_ARG;
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
@@ -569,10 +623,14 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
   g.a = static_cast<const __bf16*>(weight);  g.lda = h;  g.m_rows = (int)v;
   g.b = static_cast<const __bf16*>(hidden);  g.ldb = h;  g.n_rows = (int)n;
   g.k = (int)h;
-  FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e};
+  FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e, softcap,
+              softcap > 0.f ? 1.f / softcap : 0.f};
   {
     Span span(timer, 0);
-    AXON_LAUNCH_GEMM(lmhead_fwd_kernel, g, p, st);
+    if (softcap > 0.f)
+      AXON_LAUNCH_GEMM(lmhead_fwd_softcap_kernel, g, p, st);
+    else
+      AXON_LAUNCH_GEMM(lmhead_fwd_kernel, g, p, st);
   }
   {
     Span span(timer, 1);
@@ -587,20 +645,21 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
     hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       w.fin_max, w.fin_log2s, logprobs);
+                       softcap, w.fin_max, w.fin_log2s, logprobs);
   else
     hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       w.fin_max, w.fin_log2s, logprobs);
+                       softcap, w.fin_max, w.fin_log2s, logprobs);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
 
 int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
              const void* labels, int labels_i64, const float* lse, const float* entropy_b,
-             int64_t n, int64_t h, int64_t v, float inv_temp, void* d_hidden, void* d_weight,
-             int64_t chunk, void* workspace, int64_t ws_bytes, void* stream, PhaseTimer* timer) {
+             int64_t n, int64_t h, int64_t v, float inv_temp, float softcap, void* d_hidden,
+             void* d_weight, int64_t chunk, void* workspace, int64_t ws_bytes, void* stream,
+             PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
@@ -609,7 +668,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
   if (!dlogprobs || !hidden || !labels || !lse || !entropy_b || !d_hidden || !workspace)
     return AXON_ERR_ARG;
-  if (!(inv_temp > 0.f)) return AXON_ERR_ARG;
+  if (!(inv_temp > 0.f) || !(softcap >= 0.f)) return AXON_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
        reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_weight)) & 15)
     return AXON_ERR_ARG;
@@ -643,7 +702,11 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       p.labels = labels; p.labels_i64 = labels_i64;
       p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.ld_c; p.ld_dlT = w.ld_n;
       p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
-      AXON_LAUNCH_GEMM(lmhead_dlogit_kernel, g, p, st);
+      p.cap = softcap; p.inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+      if (softcap > 0.f)
+        AXON_LAUNCH_GEMM(lmhead_dlogit_softcap_kernel, g, p, st);
+      else
+        AXON_LAUNCH_GEMM(lmhead_dlogit_kernel, g, p, st);
       // reduction padding the tiles did not cover (the shifted-tile path writes no padding; the
       // clamped path writes zeros there already, the extra fill is then redundant but harmless)
       rc = launch_zero_cols(w.dl, w.ld_c, (int)n, (int)vc, (int)(vc_red - vc), st);
@@ -686,6 +749,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
 
 }  // namespace
 
+
 extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t v) {
   if (check_head_shape(n, h, v) != AXON_OK) return -1;
   return fwd_ws(n, v, nullptr).bytes + kAlign;
@@ -693,21 +757,21 @@ extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t
 
 extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
                                int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
-                               float* logprobs, float* entropy, float* lse, float* entropy_b,
+                               float softcap, float* logprobs, float* entropy, float* lse, float* entropy_b,
                                void* workspace, int64_t ws_bytes, void* stream) {
-  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, logprobs, entropy, lse,
-                  entropy_b, workspace, ws_bytes, stream, nullptr);
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, logprobs, entropy,
+                  lse, entropy_b, workspace, ws_bytes, stream, nullptr);
 }
 
 extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, const void* labels,
                                      int labels_i64, int64_t n, int64_t h, int64_t v,
-                                     float inv_temp, float* logprobs, float* entropy, float* lse,
-                                     float* entropy_b, void* workspace, int64_t ws_bytes,
+                                     float inv_temp, float softcap, float* logprobs, float* entropy,
+                                     float* lse, float* entropy_b, void* workspace, int64_t ws_bytes,
                                      void* stream, float* phase_ms, int32_t* phase_launches) {
   if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
   PhaseTimer timer((hipStream_t)stream);
-  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, logprobs, entropy,
-                          lse, entropy_b, workspace, ws_bytes, stream, &timer);
+  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, logprobs,
+                          entropy, lse, entropy_b, workspace, ws_bytes, stream, &timer);
   timer.collect(phase_ms, phase_launches, 4);
   return rc;
 }
@@ -722,24 +786,24 @@ extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t
 extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
                                const void* weight, const void* labels, int labels_i64,
                                const float* lse, const float* entropy_b, int64_t n, int64_t h,
-                               int64_t v, float inv_temp, void* d_hidden, void* d_weight,
-                               int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
+                               int64_t v, float inv_temp, float softcap, void* d_hidden,
+                               void* d_weight, int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
   return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
-                  inv_temp, d_hidden, d_weight, chunk, workspace, ws_bytes, stream, nullptr);
+                  inv_temp, softcap, d_hidden, d_weight, chunk, workspace, ws_bytes, stream, nullptr);
 }
 
 extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy,
                                      const void* hidden, const void* weight, const void* labels,
                                      int labels_i64, const float* lse, const float* entropy_b,
                                      int64_t n, int64_t h, int64_t v, float inv_temp,
-                                     void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+                                     float softcap, void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
                                      int64_t ws_bytes, void* stream, float* phase_ms,
                                      int32_t* phase_launches) {
   if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
   PhaseTimer timer((hipStream_t)stream);
   const int rc = bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n,
-                          h, v, inv_temp, d_hidden, d_weight, chunk, workspace, ws_bytes, stream,
-                          &timer);
+                          h, v, inv_temp, softcap, d_hidden, d_weight, chunk, workspace, ws_bytes,
+                          stream, &timer);
   timer.collect(phase_ms, phase_launches, 4);
   return rc;
 }

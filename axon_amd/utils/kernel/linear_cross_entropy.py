@@ -11,7 +11,10 @@ Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntro
 * differentiable w.r.t. ``hidden`` and ``weight``; gradients come back in the input dtype;
 * ``reduction`` "sum"/"mean" reduce the log-probs as the reference's epilogue does
   (kernels.py:369-378); the trainer path uses "none";
-* a ``dist_process_group`` (vocab-parallel head) is refused: one GPU only.
+* a ``dist_process_group`` (vocab-parallel head) is refused: one GPU only;
+* ``logit_softcapping`` (an extra trailing argument the reference's Triton op does not have; its
+  models fall back to the torch path for it, dense_common.py:201-219) applies
+  ``cap * tanh(logits / cap)`` before the temperature (fused_linear.py:19-23), forward and backward.
 
 The [tokens x vocab] logits are never written to memory, forward or backward.
 """
@@ -27,7 +30,8 @@ _REDUCTIONS = ("none", "sum", "mean")
 
 class LinearCrossEntropy(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+    def forward(ctx, hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None,
+                logit_softcapping=None):
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
         reduction = reduction.lower()
@@ -48,9 +52,13 @@ class LinearCrossEntropy(torch.autograd.Function):
         assert hidden2.is_contiguous() and weight.is_contiguous() and labels1.is_contiguous()
 
         inv_t = 1.0 / temperature
-        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING)
+        cap = 0.0 if logit_softcapping is None else float(logit_softcapping)
+        if not cap >= 0.0:
+            raise ValueError(f"logit_softcapping must be positive, got {logit_softcapping}")
+        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING,
+                                                                softcap=cap)
         ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b)
-        ctx.shape, ctx.inv_t, ctx.reduction = shape, inv_t, reduction
+        ctx.shape, ctx.inv_t, ctx.reduction, ctx.cap = shape, inv_t, reduction, cap
         if reduction == "sum":
             logprobs = logprobs.sum()
         elif reduction == "mean":
@@ -69,9 +77,9 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs = (dlogprobs / n).expand(n)
         d_hidden, d_weight = _ops.lmhead_backward(
             dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
-            entropy_b, ctx.inv_t, timing=_ops.TIMING,
+            entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap,
         )
-        return d_hidden.view(ctx.shape), d_weight, None, None, None, None
+        return d_hidden.view(ctx.shape), d_weight, None, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply

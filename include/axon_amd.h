@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 5
+#define AXON_AMD_ABI_VERSION 6
 
 enum {
   AXON_OK = 0,
@@ -63,11 +63,17 @@ const char* axon_amd_error_string(int code);
  *        lse = logsumexp(logits/T), entropy_b = sum softmax*logits/T  [n_tokens]
  *        fp32, the statistics the backward needs (the reference saves
  *        maximum/accumulate/entropy_b, linear_cross_entropy.py:93).
+ *   softcap > 0 applies Gemma-style logit soft-capping, logits = softcap *
+ *        tanh(logits / softcap), before the temperature
+ *        (_apply_logit_softcapping, axon/utils/torch/fused_linear.py:19-23;
+ *        the reference's Triton kernels have no such option and its models fall
+ *        back to the torch path, axon/models/transformers/dense_common.py:201-219);
+ *        0 = none.  Pass the same value to the backward.
  * Constraints: hidden % 32 == 0, hidden >= 32, vocab >= 1, n_tokens >= 0. */
 int64_t axon_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab);
 int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void* labels,
                     int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
-                    float inv_temperature, float* logprobs, float* entropy, float* lse,
+                    float inv_temperature, float softcap, float* logprobs, float* entropy, float* lse,
                     float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Backward.  Replaces efficient_entropy_backward
@@ -75,7 +81,8 @@ int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void
  * _fused_linear_for_ppo_bwd (axon/utils/torch/fused_linear.py:49-89):
  *   dlogit = [g*(onehot - p) - gH*p*(logit/T - entropy_b)] / T, rounded to bf16,
  *   d_hidden = dlogit @ W, d_weight = dlogit^T @ hidden, both written as bf16.
- * dentropy may be NULL (treated as zeros).  vocab_chunk (multiple of 256, or 0
+ * With softcap > 0 dlogit is additionally multiplied by 1 - tanh^2(raw logit / softcap)
+ * (fused_linear.py:80-83).  dentropy may be NULL (treated as zeros).  vocab_chunk (multiple of 256, or 0
  * for the library default) bounds the bf16 dlogit scratch to
  * 2 * n_tokens_padded * vocab_chunk * 2 bytes. */
 int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab,
@@ -83,7 +90,7 @@ int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_
 int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                     const void* weight_bf16, const void* labels, int labels_are_i64,
                     const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
-                    int64_t vocab, float inv_temperature, void* d_hidden_bf16,
+                    int64_t vocab, float inv_temperature, float softcap, void* d_hidden_bf16,
                     void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
                     int64_t workspace_bytes, void* stream);
 
@@ -96,13 +103,13 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
  * No reference counterpart (measurement only). */
 int axon_lmhead_fwd_timed(const void* hidden_bf16, const void* weight_bf16, const void* labels,
                           int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
-                          float inv_temperature, float* logprobs, float* entropy, float* lse,
-                          float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream,
-                          float* phase_ms, int32_t* phase_launches);
+                          float inv_temperature, float softcap, float* logprobs, float* entropy,
+                          float* lse, float* entropy_b, void* workspace, int64_t workspace_bytes,
+                          void* stream, float* phase_ms, int32_t* phase_launches);
 int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                           const void* weight_bf16, const void* labels, int labels_are_i64,
                           const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
-                          int64_t vocab, float inv_temperature, void* d_hidden_bf16,
+                          int64_t vocab, float inv_temperature, float softcap, void* d_hidden_bf16,
                           void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
                           int64_t workspace_bytes, void* stream, float* phase_ms,
                           int32_t* phase_launches);

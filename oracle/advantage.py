@@ -69,3 +69,14 @@ def gpg_advantage(token_level_rewards, response_mask, gidx, f_norm=1.0):
 def zero_advantage_keep_rows(advantages, eps=1e-5):
     """Row indices with any |advantage| > eps (strict), as a python list."""
     return torch.nonzero((advantages.abs() > eps).any(dim=1)).squeeze(1).tolist()
+
+
+def mini_batch_counts(response_mask, program_uids=None):
+    """axon/driver/driver_utils.py:436-474 (``process_mini_batch``): rows with a valid token, valid
+    tokens, tokens per row, distinct program uids among valid rows (None without uids)."""
+    per_row = response_mask.sum(dim=-1).to(torch.long)
+    valid = response_mask.sum(dim=-1) > 0
+    programs = None
+    if program_uids is not None:
+        programs = len({program_uids[i] for i in valid.nonzero(as_tuple=True)[0].tolist()})
+    return int(valid.sum().item()), int(response_mask.sum().item()), per_row, programs

@@ -14,8 +14,13 @@ from __future__ import annotations
 import torch
 
 
-def forward(hidden, weight, labels, temperature: float = 1.0, chunk: int = 512):
-    """logits = (h @ W^T)/T in fp32; returns (logprob[label], entropy) as fp32 [N].
+def _softcap(logits, softcap):
+    """fused_linear.py:19-23: tanh(logits / cap) * cap, applied to the raw logits before the temperature."""
+    return logits if softcap is None else torch.tanh(logits / softcap) * softcap
+
+
+def forward(hidden, weight, labels, temperature: float = 1.0, chunk: int = 512, softcap: float | None = None):
+    """logits = softcap(h @ W^T)/T in fp32; returns (logprob[label], entropy) as fp32 [N].
 
     fused_linear.py:33-44: log_softmax + gather, entropy = logsumexp - sum softmax*logits.
     Token-chunked like the reference (:125-136) to bound memory.
@@ -28,7 +33,7 @@ def forward(hidden, weight, labels, temperature: float = 1.0, chunk: int = 512):
     ent = torch.empty(n, dtype=torch.float32)
     for s in range(0, n, chunk):
         e = min(s + chunk, n)
-        logits = (h[s:e] @ w.t()) / temperature
+        logits = _softcap(h[s:e] @ w.t(), softcap) / temperature
         lse = torch.logsumexp(logits, dim=-1)
         probs = torch.softmax(logits, dim=-1)
         logp[s:e] = logits.gather(-1, ids[s:e, None]).squeeze(-1) - lse
@@ -37,10 +42,10 @@ def forward(hidden, weight, labels, temperature: float = 1.0, chunk: int = 512):
 
 
 def backward(dlogp, dent, hidden, weight, labels, temperature: float = 1.0, chunk: int = 512,
-             round_dlogits_bf16: bool = False):
+             round_dlogits_bf16: bool = False, softcap: float | None = None):
     """Closed-form gradients (fused_linear.py:49-89):
 
-        dlogits = [ g*(onehot - p) - gH * p * (log p + H) ] / T
+        dlogits = [ g*(onehot - p) - gH * p * (log p + H) ] / T   (* (1 - tanh^2(raw / cap)) with a softcap, :80-83)
         d_hidden = dlogits @ W,   d_weight = dlogits^T @ hidden      (fp32)
 
     ``round_dlogits_bf16`` reproduces the rounding of dlogits to the input dtype
@@ -55,7 +60,8 @@ def backward(dlogp, dent, hidden, weight, labels, temperature: float = 1.0, chun
     d_w = torch.zeros_like(w)
     for s in range(0, n, chunk):
         e = min(s + chunk, n)
-        logits = (h[s:e] @ w.t()) / temperature
+        raw = h[s:e] @ w.t()
+        logits = _softcap(raw, softcap) / temperature
         logp_all = torch.log_softmax(logits, dim=-1)
         p = logp_all.exp()
         dl = torch.zeros_like(logits)
@@ -66,6 +72,8 @@ def backward(dlogp, dent, hidden, weight, labels, temperature: float = 1.0, chun
             entropy = -(p * logp_all).sum(-1, keepdim=True)
             dl = dl - dent[s:e].float()[:, None] * p * (logp_all + entropy)
         dl = dl / temperature
+        if softcap is not None:
+            dl = dl * (1.0 - torch.tanh(raw / softcap) ** 2)
         if round_dlogits_bf16:
             dl = dl.bfloat16().float()
         d_h[s:e] = dl @ w

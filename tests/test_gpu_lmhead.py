@@ -110,6 +110,45 @@ def test_backward_vs_oracle(n, h, v, temp, ldt, with_entropy):
     assert rel_l2(wd.grad, ref_dw) < 2e-2
 
 
+# ---- logit soft-capping (fused_linear.py:19-23,80-83): DMA-loop and register-loop shapes ----------------
+SOFTCAP_CASES = [(300, 96, 777, 0.7, 4.0), (513, 256, 1500, 1.0, 30.0), (64, 128, 1000, 1.3, 2.0)]
+
+
+@pytest.mark.parametrize("n,h,v,temp,cap", SOFTCAP_CASES)
+def test_softcap_forward_backward_vs_oracle(n, h, v, temp, cap):
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=n + v + 2)
+    w = (w.float() * 8).bfloat16()
+    g = torch.Generator().manual_seed(6)
+    g_lp, g_en = torch.randn(n, generator=g) / n, torch.randn(n, generator=g) / n
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = linear_cross_entropy(hd, wd, lab.to(DEV), temp, "none", None, cap)
+    ref_lp, ref_ent = OM.forward(hid, w, lab, temp, softcap=cap)
+    assert (lp.cpu() - ref_lp).abs().max() < 1e-3 and (ent.cpu() - ref_ent).abs().max() < 1e-3
+    if cap < 30:  # the cap changes the answer on these inputs
+        assert (ref_lp - OM.forward(hid, w, lab, temp)[0]).abs().max() > 1e-2
+    ((lp * g_lp.to(DEV)).sum() + (ent * g_en.to(DEV)).sum()).backward()
+    ref_dh, ref_dw = OM.backward(g_lp, g_en, hid, w, lab, temp, softcap=cap)
+    assert rel_l2(hd.grad, ref_dh) < 2e-2 and rel_l2(wd.grad, ref_dw) < 2e-2
+    # the module face of the same path
+    lp2, ent2 = FusedLinearForPPO()(hid.to(DEV), w.to(DEV), lab.to(DEV), temperature=temp, logit_softcapping=cap)
+    assert torch.equal(lp2, lp.detach()) and torch.equal(ent2, ent.detach())
+
+
+def test_softcap_saturated_logits_and_errors():
+    # every logit far beyond the cap: capped logits are +-cap exactly, gradients vanish, nothing overflows
+    hid = torch.full((256, 64), 30.0).bfloat16()
+    w = torch.cat([torch.full((300, 64), 2.0), torch.full((300, 64), -2.0)]).bfloat16()
+    lab = torch.arange(256) % 600
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = linear_cross_entropy(hd, wd, lab.to(DEV), 1.0, "none", None, 10.0)
+    ref_lp, ref_ent = OM.forward(hid, w, lab, 1.0, softcap=10.0)
+    assert torch.isfinite(lp).all() and (lp.cpu() - ref_lp).abs().max() < 1e-3 and (ent.cpu() - ref_ent).abs().max() < 1e-3
+    (lp.sum() + ent.sum()).backward()
+    assert hd.grad.float().abs().max() == 0 and wd.grad.float().abs().max() == 0
+    with pytest.raises(ValueError):
+        linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1.0, "none", None, -1.0)
+
+
 @pytest.mark.parametrize("chunk", [256, 512, 0])
 def test_backward_vocab_chunks_agree(chunk):
     n, h, v = 300, 128, 1000

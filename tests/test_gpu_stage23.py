@@ -149,6 +149,38 @@ def test_filter_zero_advantage_known_answers_gpu():
     assert kept == OA.zero_advantage_keep_rows(adv)  # indices bit-exact
 
 
+# ---- process_mini_batch (reference tests/driver/test_driver_utils.py:260-281) -------------------
+@pytest.mark.parametrize("mask_dtype", [torch.int64, torch.float32, torch.bool])
+@pytest.mark.parametrize("where", ["cpu", "gpu"])
+def test_process_mini_batch(mask_dtype, where):
+    from axon_amd.driver.driver_utils import process_mini_batch
+    dev = DEV if where == "gpu" else "cpu"
+    mask = T([[1, 1, 0], [1, 0, 0], [0, 0, 0]]).to(mask_dtype).to(dev)
+    batch = DataProto.from_dict(
+        tensors={"response_mask": mask},
+        non_tensors={"program_uids": np.array(["program-a", "program-a", "program-padding"], dtype=object)})
+    process_mini_batch(batch)
+    assert batch.batch["valid_batch_size"].tolist() == [2, 2, 2]
+    assert batch.batch["valid_token_count"].tolist() == [3, 3, 3]
+    assert batch.batch["valid_program_count"].tolist() == [1, 1, 1]
+    assert batch.batch["per_row_token_count"].tolist() == [2, 1, 0]
+    for k in ("valid_batch_size", "valid_token_count", "per_row_token_count"):
+        assert batch.batch[k].dtype == torch.long and batch.batch[k].device.type == mask.device.type
+    # no mask: untouched; a seeded ragged batch against the oracle
+    empty = DataProto.from_dict(tensors={"x": torch.zeros(2, 2)})
+    process_mini_batch(empty)
+    assert "valid_batch_size" not in empty.batch
+    d = W.c1_loss_only(seed=9)
+    m = d["response_mask"].clone()
+    m[3] = 0
+    b2 = DataProto.from_dict(tensors={"response_mask": m.to(mask_dtype).to(dev)})
+    process_mini_batch(b2)
+    rows, tokens, per_row, _ = OA.mini_batch_counts(m)
+    assert b2.batch["valid_batch_size"][0].item() == rows and b2.batch["valid_token_count"][-1].item() == tokens
+    assert torch.equal(b2.batch["per_row_token_count"].cpu(), per_row)
+    assert "valid_program_count" not in b2.batch
+
+
 # ---- agg_loss / masked_mean known answers through the HIP path --------------------------------
 from tests.test_oracle_loss import AGG_CASES  # noqa: E402  (same table the oracle is pinned with)
 

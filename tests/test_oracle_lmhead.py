@@ -133,3 +133,53 @@ def test_dlogits_rows_sum_to_zero():
     w = torch.randn(1, h).expand(v, h).contiguous().bfloat16()
     dh, _ = M.backward(torch.randn(n), torch.randn(n), hid, w, torch.randint(0, v, (n,)))
     assert dh.abs().max() < 1e-5
+
+
+# ---- logit soft-capping (fused_linear.py:19-23,80-83) -------------------------------------------------
+def test_softcap_forward_closed_forms():
+    hid, w, lab = _case(n=5, h=16, v=24, seed=3)
+    w = (w.float() * 8).bfloat16()  # logits large enough for the cap to bite
+    lp, ent = M.forward(hid, w, lab, temperature=0.8, softcap=5.0)
+    raw = hid.double() @ w.double().t()
+    logits = torch.tanh(raw / 5.0) * 5.0 / 0.8  # cap first, temperature second
+    ref_lp = torch.log_softmax(logits, -1).gather(-1, lab[:, None]).squeeze(-1)
+    p = torch.softmax(logits, -1)
+    assert torch.allclose(lp.double(), ref_lp, atol=1e-5)
+    assert torch.allclose(ent.double(), -(p * torch.log(p)).sum(-1), atol=1e-5)
+    assert (raw.abs() > 5.0).any() and not torch.allclose(lp, M.forward(hid, w, lab, temperature=0.8)[0], atol=1e-2)
+    # a cap far above every logit is the identity; capped logits lie in (-cap, cap), so the
+    # log-probabilities are bounded below by -(2 cap / T + ln V)
+    lp_inf, ent_inf = M.forward(hid, w, lab, temperature=0.8, softcap=1e6)
+    lp0, ent0 = M.forward(hid, w, lab, temperature=0.8)
+    assert torch.allclose(lp_inf, lp0, atol=1e-4) and torch.allclose(ent_inf, ent0, atol=1e-4)
+    assert (lp >= -(2 * 5.0 / 0.8 + math.log(24))).all()
+
+
+def test_softcap_backward_matches_autograd_and_finite_differences():
+    hid, w, lab = _case(n=4, h=8, v=12, seed=5)
+    w = (w.float() * 6).bfloat16()
+    g1, g2 = torch.randn(4), torch.randn(4)
+    cap, temp = 3.0, 0.7
+
+    def f(hm, wm):
+        logits = torch.tanh((hm @ wm.t()) / cap) * cap / temp
+        lse = torch.logsumexp(logits, -1)
+        lp = logits.gather(-1, lab[:, None]).squeeze(-1) - lse
+        ent = lse - (torch.softmax(logits, -1) * logits).sum(-1)
+        return (lp * g1.to(hm.dtype)).sum() + (ent * g2.to(hm.dtype)).sum()
+
+    hf, wf = hid.float().requires_grad_(True), w.float().requires_grad_(True)
+    f(hf, wf).backward()
+    dh, dw = M.backward(g1, g2, hid, w, lab, temperature=temp, chunk=3, softcap=cap)
+    assert torch.allclose(dh, hf.grad, atol=1e-5, rtol=1e-4)
+    assert torch.allclose(dw, wf.grad, atol=1e-5, rtol=1e-4)
+    hd, wd = hid.double(), w.double()
+    eps = 1e-6
+    for (i, k) in [(0, 0), (1, 3), (3, 7)]:
+        d = torch.zeros_like(hd); d[i, k] = eps
+        fd = (f(hd + d, wd) - f(hd - d, wd)).item() / (2 * eps)
+        assert dh[i, k].item() == pytest.approx(fd, abs=2e-4)
+    for (j, k) in [(0, 0), (5, 2), (11, 7), (int(lab[0]), 1)]:
+        d = torch.zeros_like(wd); d[j, k] = eps
+        fd = (f(hd, wd + d) - f(hd, wd - d)).item() / (2 * eps)
+        assert dw[j, k].item() == pytest.approx(fd, abs=2e-4)

@@ -177,6 +177,15 @@ def test_zero_advantage_filter_known_answers():
     assert A.zero_advantage_keep_rows(T([[0.0, 0.0, 0.3]])) == [0]
 
 
+# ---- mini-batch counts, reference tests/driver/test_driver_utils.py:260-281 -----------------------
+def test_mini_batch_counts_known_answer():
+    mask = T([[1, 1, 0], [1, 0, 0], [0, 0, 0]])
+    rows, tokens, per_row, programs = A.mini_batch_counts(mask, ["program-a", "program-a", "program-padding"])
+    assert (rows, tokens, programs) == (2, 3, 1)
+    assert per_row.tolist() == [2, 1, 0] and per_row.dtype == torch.long
+    assert A.mini_batch_counts(mask)[3] is None
+
+
 # ---- layout, reference test_ops.py:513-561,723-729 -------------------------------------------------
 def test_unpad_known_answers():
     idx, cu, mx = L.unpad_data(T([[1, 1, 1, 0, 0], [1, 1, 0, 0, 0]]))
