@@ -353,9 +353,22 @@ def _add_phases(timing: dict, prefix: str, names, ms, launches):
         t["launches"] += int(launches[i])
 
 
-def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None = None, softcap: float = 0.0):
+def seq_start_flags(cu_seqlens, n_tokens: int):
+    """uint8 [N] (padded to a multiple of 4): 1 where a non-empty sequence begins."""
+    lib = _lib.load()
+    require_device(cu_seqlens, "seq_start_flags")
+    cu = cu_seqlens.to(torch.int32).contiguous()
+    flags = torch.empty((int(n_tokens) + 3) // 4 * 4, device=cu.device, dtype=torch.uint8)
+    check(lib.axon_seq_start_flags(ptr(cu), int(cu.numel()) - 1, int(n_tokens), ptr(flags), stream_ptr()),
+          "axon_seq_start_flags")
+    return flags
+
+
+def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None = None, softcap: float = 0.0,
+                   seq_start=None):
     """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]).  ``softcap`` > 0 soft-caps the logits
-    (cap * tanh(logit / cap)) before the temperature.
+    (cap * tanh(logit / cap)) before the temperature.  With ``seq_start`` (``seq_start_flags``) ``labels`` is
+    the packed id stream and logprobs / entropy come back aligned to token positions.
 
     With ``timing`` (a dict) the timed entry point is used: it synchronises and adds
     per-phase HIP-event milliseconds and launch counts under ``fwd/...`` keys."""
@@ -370,7 +383,7 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None 
         raise _lib.AxonAmdError(f"axon_lmhead_fwd: unsupported shape tokens={n} hidden={h} vocab={v} (hidden % 32 != 0?)")
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
     args = (ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), n, h, v,
-            float(inv_temperature), float(softcap), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws), ws_bytes,
+            float(inv_temperature), float(softcap), ptr(seq_start), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws), ws_bytes,
             stream_ptr())
     if timing is None:
         check(lib.axon_lmhead_fwd(*args), "axon_lmhead_fwd")
@@ -382,7 +395,7 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None 
 
 
 def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
-                    timing: dict | None = None, softcap: float = 0.0):
+                    timing: dict | None = None, softcap: float = 0.0, seq_start=None):
     """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``)."""
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
     lib = _lib.load()
@@ -399,7 +412,7 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     g_lp = f32(dlogprobs)  # keep the converted copies alive until the launch is enqueued
     g_en = f32(dentropy) if dentropy is not None else None
     args = (ptr(g_lp), ptr(g_en), ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), ptr(lse),
-            ptr(entropy_b), n, h, v, float(inv_temperature), float(softcap), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
+            ptr(entropy_b), n, h, v, float(inv_temperature), float(softcap), ptr(seq_start), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
             ws_bytes, stream_ptr())
     if timing is None:
         check(lib.axon_lmhead_bwd(*args), "axon_lmhead_bwd")

@@ -145,11 +145,32 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_softcap_kernel(GemmOp
   fwd_body<Loop, true>(g, p, tiles_m, tiles_n);
 }
 
+// Token-aligned packed layout.  With `is_start` (one byte per packed position, 1 where a sequence
+// begins) the head works on a packed stream of token ids directly: hidden position n predicts the
+// token at position n + 1, so its label is ids[n + 1] and its outputs land at position n + 1; a
+// sequence's first position receives 0 (there is no prediction for it) and its upstream gradient
+// is ignored.  This is roll(ids, -1) before and the shift-right after the head
+// (axon/utils/fsdp/forward_utils.py:131,180-182) without the extra passes.  The position after the
+// last one wraps to 0, which is always a sequence start.
+__device__ __forceinline__ int aligned_pos(int n, int n_tokens, const uint8_t* is_start) {
+  if (is_start == nullptr) return n;
+  return (n + 1 == n_tokens) ? 0 : n + 1;
+}
+
+__global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restrict__ cu, int n_seqs,
+                                                        int n_tokens, uint8_t* __restrict__ is_start) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_seqs) return;
+  const int s0 = cu[i];
+  if (s0 >= 0 && s0 < n_tokens && cu[i + 1] > s0) is_start[s0] = 1;  // empty sequences own no position
+}
+
 // Merge partials: lse, entropy_b, entropy.  One thread per token.
 __global__ __launch_bounds__(256) void lmhead_merge_kernel(
     const float* __restrict__ pm, const float* __restrict__ ps, const float* __restrict__ pe,
     int parts, int n_tokens, float* __restrict__ lse, float* __restrict__ entropy_b,
-    float* __restrict__ entropy, float* __restrict__ fin_max, float* __restrict__ fin_log2s) {
+    float* __restrict__ entropy, float* __restrict__ fin_max, float* __restrict__ fin_log2s,
+    const uint8_t* __restrict__ is_start) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= n_tokens) return;
   float M = pm[n], s = ps[n], e = pe[n];
@@ -166,7 +187,8 @@ __global__ __launch_bounds__(256) void lmhead_merge_kernel(
   const float d = e / s;
   lse[n] = (M + L) * kLn2;
   entropy_b[n] = (M + d) * kLn2;
-  entropy[n] = (L - d) * kLn2;
+  const int dst = aligned_pos(n, n_tokens, is_start);
+  entropy[dst] = (is_start && is_start[dst]) ? 0.f : (L - d) * kLn2;
   fin_max[n] = M;
   fin_log2s[n] = L;
 }
@@ -177,11 +199,12 @@ __global__ __launch_bounds__(256) void lmhead_label_kernel(
     const __bf16* __restrict__ hidden, const __bf16* __restrict__ weight,
     const LabelT* __restrict__ labels, int n_tokens, int hidden_sz, int vocab, float inv_temp,
     float cap, const float* __restrict__ fin_max, const float* __restrict__ fin_log2s,
-    float* __restrict__ logprobs) {
+    float* __restrict__ logprobs, const uint8_t* __restrict__ is_start) {
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= n_tokens) return;
   const int lane = threadIdx.x & 63;
-  const int64_t lab = (int64_t)labels[n];
+  const int dst = aligned_pos(n, n_tokens, is_start);
+  const int64_t lab = (int64_t)labels[dst];
   float dot = 0.f;
   if (lab >= 0 && lab < vocab) {
     const uint4* h = reinterpret_cast<const uint4*>(hidden + (int64_t)n * hidden_sz);
@@ -199,7 +222,10 @@ __global__ __launch_bounds__(256) void lmhead_label_kernel(
   dot = wave_sum(dot);
   if (cap != 0.f) dot = cap * fast_tanh(dot / cap);
   // (logit*c - M) is formed in one rounding, then log2(sum) is subtracted: no cancellation
-  if (lane == 0) logprobs[n] = (fmaf(dot, inv_temp * kLog2e, -fin_max[n]) - fin_log2s[n]) * kLn2;
+  if (lane == 0) {
+    const float lpv = (fmaf(dot, inv_temp * kLog2e, -fin_max[n]) - fin_log2s[n]) * kLn2;
+    logprobs[dst] = (is_start && is_start[dst]) ? 0.f : lpv;
+  }
 }
 
 // ----------------------------------------------------------------------------
@@ -218,6 +244,7 @@ struct DlogitParams {
   int n_tokens, vocab, v_begin;  // v_begin: first vocab row of this chunk
   float inv_temp;
   float cap, inv_cap;  // soft-capping (SOFTCAP kernels only)
+  const uint8_t* is_start;  // token-aligned packed layout (see aligned_pos), or null
 };
 
 // Per-wave staging of the wave's 128(n) x 128(m) bf16 sub-tile in its own 32 KB of LDS:
@@ -250,16 +277,18 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
     const int n = t.n0 + lp.wn * kWaveTile + nw;
     const bool n_ok = n < p.n_tokens;
     const int nn = n_ok ? n : 0;
-    const float g_lp = n_ok ? p.dlogprobs[nn] : 0.f;
-    const float g_en = (n_ok && p.dentropy) ? p.dentropy[nn] : 0.f;
+    const int src = aligned_pos(nn, p.n_tokens, p.is_start);  // where the label and the gradients live
+    const bool g_ok = n_ok && !(p.is_start && p.is_start[src]);
+    const float g_lp = g_ok ? p.dlogprobs[src] : 0.f;
+    const float g_en = (g_ok && p.dentropy) ? p.dentropy[src] : 0.f;
     const float lse2 = p.lse[nn] * kLog2e;
     const float eb = p.entropy_b[nn];
     // dlogit = p * (a + b * x) + onehot * g / T,  x = logit / T
     const float ca = (-g_lp + g_en * eb) * p.inv_temp;
     const float cb = -g_en * p.inv_temp;
     const float gl = g_lp * p.inv_temp;
-    const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[nn]
-                                     : (int64_t) static_cast<const int32_t*>(p.labels)[nn];
+    const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[src]
+                                     : (int64_t) static_cast<const int32_t*>(p.labels)[src];
     const int64_t lab_rel = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -603,9 +632,9 @@ int launch_zero_cols(void* p, int64_t ld, int rows, int col0, int ncols, hipStre
 }
 
 int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64, int64_t n,
-             int64_t h, int64_t v, float inv_temp, float softcap, float* logprobs, float* entropy,
-             float* lse, float* entropy_b, void* workspace, int64_t ws_bytes, void* stream,
-             PhaseTimer* timer) {
+             int64_t h, int64_t v, float inv_temp, float softcap, const uint8_t* is_start,
+             float* logprobs, float* entropy, float* lse, float* entropy_b, void* workspace,
+             int64_t ws_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
@@ -636,7 +665,7 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
     Span span(timer, 1);
     hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
                        w.pm, w.ps, w.pe, w.parts, (int)n, lse, entropy_b, entropy, w.fin_max,
-                       w.fin_log2s);
+                       w.fin_log2s, is_start);
   }
   AXON_CHECK_LAUNCH();
   const dim3 lg((unsigned)((n + 3) / 4));
@@ -645,21 +674,21 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
     hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       softcap, w.fin_max, w.fin_log2s, logprobs);
+                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start);
   else
     hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       softcap, w.fin_max, w.fin_log2s, logprobs);
+                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
 
 int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
              const void* labels, int labels_i64, const float* lse, const float* entropy_b,
-             int64_t n, int64_t h, int64_t v, float inv_temp, float softcap, void* d_hidden,
-             void* d_weight, int64_t chunk, void* workspace, int64_t ws_bytes, void* stream,
-             PhaseTimer* timer) {
+             int64_t n, int64_t h, int64_t v, float inv_temp, float softcap,
+             const uint8_t* is_start, void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+             int64_t ws_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
@@ -703,6 +732,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.ld_c; p.ld_dlT = w.ld_n;
       p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
       p.cap = softcap; p.inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+      p.is_start = is_start;
       if (softcap > 0.f)
         AXON_LAUNCH_GEMM(lmhead_dlogit_softcap_kernel, g, p, st);
       else
@@ -750,6 +780,21 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
 }  // namespace
 
 
+extern "C" int axon_seq_start_flags(const int32_t* cu_seqlens, int64_t n_seqs, int64_t n_tokens,
+                                    uint8_t* flags, void* stream) {
+  if (n_seqs < 0 || n_tokens < 0 || n_tokens >= (int64_t)INT32_MAX || n_seqs >= (int64_t)INT32_MAX)
+    return AXON_ERR_SHAPE;
+  if (n_tokens == 0) return AXON_OK;
+  if (!flags || (n_seqs > 0 && !cu_seqlens)) return AXON_ERR_ARG;
+  int rc = axon_fill_zero(flags, round_up(n_tokens, 4), stream);
+  if (rc != AXON_OK) return rc;
+  if (n_seqs == 0) return AXON_OK;
+  hipLaunchKernelGGL(seq_start_kernel, dim3((unsigned)((n_seqs + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, cu_seqlens, (int)n_seqs, (int)n_tokens, flags);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
 extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t v) {
   if (check_head_shape(n, h, v) != AXON_OK) return -1;
   return fwd_ws(n, v, nullptr).bytes + kAlign;
@@ -757,21 +802,24 @@ extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t
 
 extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
                                int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
-                               float softcap, float* logprobs, float* entropy, float* lse, float* entropy_b,
-                               void* workspace, int64_t ws_bytes, void* stream) {
-  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, logprobs, entropy,
-                  lse, entropy_b, workspace, ws_bytes, stream, nullptr);
+                               float softcap, const uint8_t* seq_start, float* logprobs,
+                               float* entropy, float* lse, float* entropy_b, void* workspace,
+                               int64_t ws_bytes, void* stream) {
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start,
+                  logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stream, nullptr);
 }
 
 extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, const void* labels,
                                      int labels_i64, int64_t n, int64_t h, int64_t v,
-                                     float inv_temp, float softcap, float* logprobs, float* entropy,
-                                     float* lse, float* entropy_b, void* workspace, int64_t ws_bytes,
+                                     float inv_temp, float softcap, const uint8_t* seq_start,
+                                     float* logprobs, float* entropy, float* lse,
+                                     float* entropy_b, void* workspace, int64_t ws_bytes,
                                      void* stream, float* phase_ms, int32_t* phase_launches) {
   if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
   PhaseTimer timer((hipStream_t)stream);
-  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, logprobs,
-                          entropy, lse, entropy_b, workspace, ws_bytes, stream, &timer);
+  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap,
+                          seq_start, logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stream,
+                          &timer);
   timer.collect(phase_ms, phase_launches, 4);
   return rc;
 }
@@ -786,24 +834,27 @@ extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t
 extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
                                const void* weight, const void* labels, int labels_i64,
                                const float* lse, const float* entropy_b, int64_t n, int64_t h,
-                               int64_t v, float inv_temp, float softcap, void* d_hidden,
-                               void* d_weight, int64_t chunk, void* workspace, int64_t ws_bytes, void* stream) {
+                               int64_t v, float inv_temp, float softcap, const uint8_t* seq_start,
+                               void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+                               int64_t ws_bytes, void* stream) {
   return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
-                  inv_temp, softcap, d_hidden, d_weight, chunk, workspace, ws_bytes, stream, nullptr);
+                  inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes,
+                  stream, nullptr);
 }
 
 extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy,
                                      const void* hidden, const void* weight, const void* labels,
                                      int labels_i64, const float* lse, const float* entropy_b,
                                      int64_t n, int64_t h, int64_t v, float inv_temp,
-                                     float softcap, void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
+                                     float softcap, const uint8_t* seq_start, void* d_hidden,
+                                     void* d_weight, int64_t chunk, void* workspace,
                                      int64_t ws_bytes, void* stream, float* phase_ms,
                                      int32_t* phase_launches) {
   if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
   PhaseTimer timer((hipStream_t)stream);
   const int rc = bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n,
-                          h, v, inv_temp, softcap, d_hidden, d_weight, chunk, workspace, ws_bytes,
-                          stream, &timer);
+                          h, v, inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace,
+                          ws_bytes, stream, &timer);
   timer.collect(phase_ms, phase_launches, 4);
   return rc;
 }

@@ -61,3 +61,14 @@ def shift_packed(values: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor
     starts = cu_seqlens[:-1].long()
     out[starts[starts < values.numel()]] = 0
     return out
+
+
+def packed_logprobs(hidden, weight, packed_ids, cu_seqlens, temperature: float = 1.0, logit_softcapping=None):
+    """Head of the remove-padding path in one call: packed hidden states ``[N, H]`` and the packed token ids
+    ``[N]`` (or ``[1, N]``) in, ``(log_probs, entropy)`` ``[N]`` aligned to token positions out — what
+    ``rolled_labels`` + the fused head + ``shift_packed`` produce, without the roll and shift passes
+    (forward_utils.py:131,164-182 in packed form)."""
+    from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+
+    return linear_cross_entropy(hidden, weight, packed_ids.reshape(-1), float(temperature), "none", None,
+                                logit_softcapping, cu_seqlens)

@@ -14,7 +14,12 @@ Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntro
 * a ``dist_process_group`` (vocab-parallel head) is refused: one GPU only;
 * ``logit_softcapping`` (an extra trailing argument the reference's Triton op does not have; its
   models fall back to the torch path for it, dense_common.py:201-219) applies
-  ``cap * tanh(logits / cap)`` before the temperature (fused_linear.py:19-23), forward and backward.
+  ``cap * tanh(logits / cap)`` before the temperature (fused_linear.py:19-23), forward and backward;
+* ``cu_seqlens`` (a second extra trailing argument, int32 ``[S+1]``) selects the token-aligned packed
+  layout: ``labels`` is then the packed stream of token ids itself, and the outputs come back aligned
+  to token positions (``out[p]`` = log-prob of token ``p`` given its prefix, 0 at the first position of
+  every sequence).  That is ``torch.roll(ids, -1)`` before the head and the shift-right after it
+  (axon/utils/fsdp/forward_utils.py:131,164-182) done inside the kernels, forward and backward.
 
 The [tokens x vocab] logits are never written to memory, forward or backward.
 """
@@ -31,7 +36,7 @@ _REDUCTIONS = ("none", "sum", "mean")
 class LinearCrossEntropy(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None,
-                logit_softcapping=None):
+                logit_softcapping=None, cu_seqlens=None):
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
         reduction = reduction.lower()
@@ -55,9 +60,10 @@ class LinearCrossEntropy(torch.autograd.Function):
         cap = 0.0 if logit_softcapping is None else float(logit_softcapping)
         if not cap >= 0.0:
             raise ValueError(f"logit_softcapping must be positive, got {logit_softcapping}")
+        seq_start = None if cu_seqlens is None else _ops.seq_start_flags(cu_seqlens, hidden2.shape[0])
         logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING,
-                                                                softcap=cap)
-        ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b)
+                                                                softcap=cap, seq_start=seq_start)
+        ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b, seq_start)
         ctx.shape, ctx.inv_t, ctx.reduction, ctx.cap = shape, inv_t, reduction, cap
         if reduction == "sum":
             logprobs = logprobs.sum()
@@ -67,7 +73,7 @@ class LinearCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dlogprobs, dentropy):
-        hidden2, weight, labels1, lse, entropy_b = ctx.saved_tensors
+        hidden2, weight, labels1, lse, entropy_b, seq_start = ctx.saved_tensors
         n = hidden2.shape[0]
         if dlogprobs is None:
             dlogprobs = torch.zeros(n, device=hidden2.device, dtype=torch.float32)
@@ -77,9 +83,9 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs = (dlogprobs / n).expand(n)
         d_hidden, d_weight = _ops.lmhead_backward(
             dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
-            entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap,
+            entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap, seq_start=seq_start,
         )
-        return d_hidden.view(ctx.shape), d_weight, None, None, None, None, None
+        return d_hidden.view(ctx.shape), d_weight, None, None, None, None, None, None
 
 
 linear_cross_entropy = LinearCrossEntropy.apply

@@ -195,8 +195,7 @@ def main():
     from axon_amd.protocol import DataProto
     from axon_amd.trainer.algos.advantages import compute_advantage
     from axon_amd.trainer.algos.loss import compute_loss_fn
-    from axon_amd.utils.fsdp.forward_utils import shift_packed
-    from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs
     from oracle import lmhead as OM
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
@@ -214,12 +213,14 @@ def main():
     uid = rl["uid"]
 
     # old log-probs: one forward, detached, perturbed (as the trainer's first pass would give)
+    # (`lab` is the packed stream of token ids: the head rolls and shifts inside its kernels)
     with torch.no_grad():
-        lp0, _ = linear_cross_entropy(hd, wd, ld, 1.0, "none")
-        old = shift_packed(lp0, cu) - 0.05 * torch.randn(n, device=dev)
-    # parity gate on a token subset before anything is timed
-    idx = torch.arange(0, n, max(1, n // 48))
-    ref_lp, _ = OM.forward(hid[idx], w, lab[idx])
+        lp0, _ = packed_logprobs(hd, wd, ld, cu)
+        old = lp0 - 0.05 * torch.randn(n, device=dev)
+    # parity gate on a token subset before anything is timed: token p is predicted from hidden p - 1
+    idx = torch.arange(1, n, max(1, n // 48))
+    idx = idx[rl["response_mask"][idx] > 0]
+    ref_lp, _ = OM.forward(hid[idx - 1], w, lab[idx])
     lp_err = (lp0.cpu()[idx] - ref_lp).abs().max().item()
     assert lp_err < 1e-3, f"log-prob parity failed: {lp_err}"
 
@@ -227,8 +228,7 @@ def main():
 
     def step():
         hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
-        lp_head, _ent = linear_cross_entropy(hg, wg, ld, 1.0, "none")
-        lp_tok = shift_packed(lp_head, cu)
+        lp_tok, _ent = packed_logprobs(hg, wg, ld, cu)
         adv_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
                                      meta_info={"cu_seqlens": cu})
         adv_in.non_tensor_batch["uid"] = uid

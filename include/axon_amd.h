@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 6
+#define AXON_AMD_ABI_VERSION 7
 
 enum {
   AXON_OK = 0,
@@ -69,11 +69,26 @@ const char* axon_amd_error_string(int code);
  *        the reference's Triton kernels have no such option and its models fall
  *        back to the torch path, axon/models/transformers/dense_common.py:201-219);
  *        0 = none.  Pass the same value to the backward.
+ *   seq_start (may be NULL): token-aligned packed layout.  `labels` is then the
+ *        packed stream of token ids itself and seq_start[p] = 1 where a sequence
+ *        begins (axon_seq_start_flags).  Hidden position n predicts the token at
+ *        n + 1: the label is labels[n + 1] and logprobs / entropy are written at
+ *        n + 1; sequence starts receive 0.  This is torch.roll(ids, -1) before the
+ *        head (axon/utils/fsdp/forward_utils.py:131) and the shift-right after it
+ *        (rmpad_postprocess, forward_utils.py:164-182) folded into the kernels.
+ *        lse / entropy_b stay indexed by hidden position.  The backward takes the
+ *        same flags and reads dlogprobs / dentropy in the aligned layout, ignoring
+ *        them at sequence starts.
  * Constraints: hidden % 32 == 0, hidden >= 32, vocab >= 1, n_tokens >= 0. */
 int64_t axon_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab);
+/* flags[p] = 1 where a non-empty sequence of cu_seqlens[n_seqs + 1] begins, else 0.
+ * `flags` holds n_tokens bytes rounded up to a multiple of 4. */
+int axon_seq_start_flags(const int32_t* cu_seqlens, int64_t n_seqs, int64_t n_tokens,
+                         uint8_t* flags, void* stream);
 int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void* labels,
                     int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
-                    float inv_temperature, float softcap, float* logprobs, float* entropy, float* lse,
+                    float inv_temperature, float softcap, const uint8_t* seq_start,
+                    float* logprobs, float* entropy, float* lse,
                     float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Backward.  Replaces efficient_entropy_backward
@@ -90,9 +105,9 @@ int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_
 int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                     const void* weight_bf16, const void* labels, int labels_are_i64,
                     const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
-                    int64_t vocab, float inv_temperature, float softcap, void* d_hidden_bf16,
-                    void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
-                    int64_t workspace_bytes, void* stream);
+                    int64_t vocab, float inv_temperature, float softcap,
+                    const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
+                    int64_t vocab_chunk, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Timed variants for benchmarks: same work, plus HIP events recorded on `stream`
  * around every launch.  They SYNCHRONISE the stream before returning and create
@@ -103,15 +118,16 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
  * No reference counterpart (measurement only). */
 int axon_lmhead_fwd_timed(const void* hidden_bf16, const void* weight_bf16, const void* labels,
                           int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
-                          float inv_temperature, float softcap, float* logprobs, float* entropy,
-                          float* lse, float* entropy_b, void* workspace, int64_t workspace_bytes,
+                          float inv_temperature, float softcap, const uint8_t* seq_start,
+                          float* logprobs, float* entropy, float* lse, float* entropy_b, void* workspace, int64_t workspace_bytes,
                           void* stream, float* phase_ms, int32_t* phase_launches);
 int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                           const void* weight_bf16, const void* labels, int labels_are_i64,
                           const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
-                          int64_t vocab, float inv_temperature, float softcap, void* d_hidden_bf16,
-                          void* d_weight_bf16, int64_t vocab_chunk, void* workspace,
-                          int64_t workspace_bytes, void* stream, float* phase_ms,
+                          int64_t vocab, float inv_temperature, float softcap,
+                          const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
+                          int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
+                          void* stream, float* phase_ms,
                           int32_t* phase_launches);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]

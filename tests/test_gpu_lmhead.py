@@ -149,6 +149,55 @@ def test_softcap_saturated_logits_and_errors():
         linear_cross_entropy(hid.to(DEV), w.to(DEV), lab.to(DEV), 1.0, "none", None, -1.0)
 
 
+# ---- token-aligned packed layout: roll(ids, -1) before and shift-right after the head, inside the kernels --
+def _aligned_reference(hid, w, ids, lens, temp, cap=None):
+    """forward_utils.py:131,164-182 on the oracle: labels = roll(ids, -1), outputs shifted right inside each
+    sequence, 0 at sequence starts."""
+    lp, ent = OM.forward(hid, w, torch.roll(ids, -1), temp, softcap=cap)
+    out_lp, out_ent = torch.zeros_like(lp), torch.zeros_like(ent)
+    out_lp[1:], out_ent[1:] = lp[:-1], ent[:-1]
+    cu = torch.tensor([0] + lens).cumsum(0)
+    starts = cu[:-1][cu[:-1] < len(ids)]
+    out_lp[starts] = 0
+    out_ent[starts] = 0
+    return out_lp, out_ent, cu
+
+
+@pytest.mark.parametrize("n,h,v,lens,cap", [
+    (300, 96, 777, [1, 0, 120, 1, 78, 100], None),      # single-token and empty sequences, register loop
+    (513, 256, 1500, [256, 1, 256], 4.0),               # DMA loop, boundary on a tile edge, soft-capping
+    (64, 128, 1000, [64], None),
+])
+def test_aligned_packed_layout(n, h, v, lens, cap):
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs, rolled_labels, shift_packed
+    assert sum(lens) == n
+    hid, w, ids = W.lmhead_inputs(n, h, v, seed=n + v + 3, label_dtype=torch.int64)
+    w = (w.float() * 8).bfloat16()
+    temp = 0.9
+    ref_lp, ref_ent, cu = _aligned_reference(hid, w, ids, lens, temp, cap)
+    cu_d = cu.to(torch.int32).to(DEV)
+    flags = _ops.seq_start_flags(cu_d, n)[:n].cpu()
+    expect = torch.zeros(n, dtype=torch.uint8)
+    expect[[int(a) for a, b in zip(cu[:-1], cu[1:]) if b > a]] = 1
+    assert torch.equal(flags, expect)  # bit-exact
+
+    g = torch.Generator().manual_seed(9)
+    g_lp, g_en = (torch.randn(n, generator=g) / n).to(DEV), (torch.randn(n, generator=g) / n).to(DEV)
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = packed_logprobs(hd, wd, ids.to(DEV).view(1, -1), cu_d, temp, cap)
+    assert (lp.cpu() - ref_lp).abs().max() < 1e-3 and (ent.cpu() - ref_ent).abs().max() < 1e-3
+    assert (lp[cu_d[:-1].long()[cu_d[:-1] < n]] == 0).all()
+    ((lp * g_lp).sum() + (ent * g_en).sum()).backward()
+
+    # the unfused composition of the same kernels gives the same bits, forward and backward
+    h2, w2 = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp_h, ent_h = linear_cross_entropy(h2, w2, rolled_labels(ids.to(DEV)), temp, "none", None, cap)
+    lp2, ent2 = shift_packed(lp_h, cu_d), shift_packed(ent_h, cu_d)
+    ((lp2 * g_lp).sum() + (ent2 * g_en).sum()).backward()
+    assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
+    assert torch.equal(hd.grad, h2.grad) and torch.equal(wd.grad, w2.grad)
+
+
 @pytest.mark.parametrize("chunk", [256, 512, 0])
 def test_backward_vocab_chunks_agree(chunk):
     n, h, v = 300, 128, 1000
