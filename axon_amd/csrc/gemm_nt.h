@@ -1,14 +1,17 @@
 // bf16 "NT" GEMM main loops for gfx950:  D[m][n] = sum_k A[m][k] * B[n][k]
 //
-// Both operands are K-contiguous, which is the layout the 32x32x16 bf16 MFMA
+// Both operands are K-contiguous, which is the layout the 16x16x32 bf16 MFMA
 // wants on both sides: every lane feeds eight consecutive k of one row.  The
 // LM-head forward, its logit recompute, dHidden and dWeight are all brought to
 // this one form (by pre-transposed copies where needed), so one main loop
 // serves the whole path; they differ only in the epilogue.
 //
 // Workgroup: 256 threads = 4 waves in a 2x2 grid, tile 256(m) x 256(n), each
-// wave 128 x 128 = 4x4 MFMA blocks of 32x32 (256 fp32 accumulators per lane,
-// one wave per SIMD).
+// wave 128 x 128 = 8x8 MFMA blocks of 16x16 (256 fp32 accumulators per lane,
+// one wave per SIMD).  The 16x16x32 shape reads and writes each accumulator once
+// per 32 k (the 32x32x16 shape once per 16 k); under sustained load the part
+// holds a higher clock with it (MFMA-only loop on random data: 2047 vs 1795
+// TFLOP/s), which is worth more than the larger block's operand reuse.
 //
 // Two main loops:
 //  * DmaLoop  (the fast path; needs m_rows >= 256, n_rows >= 256, k % 64 == 0)
@@ -22,11 +25,11 @@
 //  * RegLoop<32>  (any shape with k % 32 == 0): loads through registers with
 //      per-row clamping.  Used for small or odd shapes.
 //
-// Accumulator layout of one 32x32 block (v16f32, index q = 4*r + e):
-//   m = 8*r + 4*(lane/32) + e,   n = lane%32.
-// So a lane owns ONE n per block column and four consecutive m per register
-// quad: per-n statistics need no cross-lane traffic beyond lane^32, and stores
-// to an [n][m] output are 4-element vectors.
+// Accumulator layout of one 16x16 block (four floats, index r):
+//   m = 4*(lane/16) + r,   n = lane%16.
+// So a lane owns ONE n per block column and four consecutive m per block: per-n
+// statistics need cross-lane traffic only over lane^16 and lane^32, and stores to
+// an [n][m] output are 4-element vectors, 16 consecutive m per four lanes.
 #pragma once
 #include <type_traits>
 #include <hip/hip_runtime.h>
@@ -35,10 +38,12 @@
 namespace axon {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float acc4;
 
 constexpr int kTile = 256;       // tile edge in m and n
 constexpr int kWaveTile = 128;   // per-wave edge
+constexpr int kBlk = 16;         // MFMA block edge
+constexpr int kBlocks = kWaveTile / kBlk;  // 8 x 8 blocks per wave
 constexpr int kGemmThreads = 256;
 constexpr int kGemmLdsBytes = 163840;  // all of a CU's LDS: five 32 KB operand slots; the dlogit epilogue stages in the first 128 KB
 
@@ -59,39 +64,50 @@ struct TilePos {
 
 // Position of this lane inside the workgroup tile.
 struct LanePos {
-  int lane, l32, lhi, wave, wm, wn;
+  int lane, l16, lq, wave, wm, wn;
   __device__ __forceinline__ LanePos() {
     lane = threadIdx.x & 63;
-    l32 = lane & 31;
-    lhi = lane >> 5;
+    l16 = lane & 15;
+    lq = lane >> 4;
     wave = threadIdx.x >> 6;
     wm = wave >> 1;
     wn = wave & 1;
   }
-  // tile-relative coordinates of accumulator (i, j, q)
-  __device__ __forceinline__ int m(int i, int q) const {
-    return wm * kWaveTile + i * 32 + 8 * (q >> 2) + 4 * lhi + (q & 3);
-  }
-  __device__ __forceinline__ int n(int j) const { return wn * kWaveTile + j * 32 + l32; }
+  // tile-relative coordinates of accumulator (i, j, r)
+  __device__ __forceinline__ int m(int i, int r) const { return wm * kWaveTile + i * kBlk + 4 * lq + r; }
+  __device__ __forceinline__ int n(int j) const { return wn * kWaveTile + j * kBlk + l16; }
 };
 
-__device__ __forceinline__ void zero_acc(f32x16 (&acc)[4][4]) {
+typedef acc4 AccTile[kBlocks][kBlocks];
+
+__device__ __forceinline__ void zero_acc(AccTile& acc) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < kBlocks; ++j)
 #pragma unroll
-      for (int q = 0; q < 16; ++q) acc[i][j][q] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 }
+
+// c += a * b on one 16x16 block, accumulator held in place in the AGPR file.  Written as an
+// instruction because the register allocator otherwise rotates the 64 four-register accumulators
+// through the VGPR file on every trip of the unrolled loop (hundreds of copies per k-tile).
+__device__ __forceinline__ void mfma_16x16x32(acc4& c, const bf16x8& a, const bf16x8& b) {
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+
+// The compiler does not see the matrix instructions above, so it cannot count the wait states
+// between the last of them and the first read of an accumulator: spend them here.
+__device__ __forceinline__ void settle_acc() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 // ---------------------------------------------------------------------------------------
 // DmaLoop: k-tiles of 64 go global -> LDS by buffer_load ... lds (no register staging) into
 // XOR-swizzled [row][128 B] slots.  The 160 KB of LDS hold THREE slots for the A operand and
-// TWO for B.  B of k-tile t+2 is issued right after the barrier that frees its slot and has one
-// k-tile of time to land; A of k-tile t+2 is issued a whole k-tile earlier, spread under the
-// MFMAs of k-steps 0..2, into the slot freed one barrier before.  Compared with a symmetric
-// double buffer this halves the data that has only one k-tile to arrive, which is what keeps the
-// single wave per SIMD from waiting at the barrier (measured: +20 % on long-k GEMMs).
+// TWO for B.  A k-tile is two k-steps of 32 (64 MFMAs per wave each).  A of k-tile t+2 is
+// issued under the first k-step of tile t into the slot freed one barrier before; the one
+// barrier of the tile follows; B of k-tile t+2 is issued under the second k-step into the B slot
+// that the barrier has just freed.  Compared with a symmetric double buffer this halves the data
+// that has only one k-tile to arrive.
 // ---------------------------------------------------------------------------------------
 struct DmaLoop {
   static constexpr int kBK = 64;
@@ -122,8 +138,8 @@ struct DmaLoop {
                                              voffset, soffset, 0, 0);
   }
 
-  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
-                                             f32x16 (&acc)[4][4], char* smem) {
+  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t, AccTile& acc,
+                                             char* smem) {
     const LanePos lp;
     // --- DMA addressing.  One wave instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns
     // rows [64w, 64w+64) of each operand (8 instructions).  Lane i lands on row i/8, chunk slot
@@ -147,17 +163,18 @@ struct DmaLoop {
     // wave-uniform, so the LDS destination of every DMA instruction is scalar arithmetic into M0
     char* const dst = smem + __builtin_amdgcn_readfirstlane(lp.wave) * 64 * kRowBytes;
 
-    // --- fragment addressing: row = 128*wm + 32*i + l32, chunk = 2*kk + lhi, swizzle = (l32/2)%8
-    const int sw = (lp.l32 >> 1) & 7;
-    int fa[4], fb[4];
+    // --- fragment addressing: row = 128*wm + 16*i + l16, chunk = 4*kk + lq, swizzle = (l16/2)%8.
+    // Sixteen lanes (one chunk column of sixteen rows) cover all 64 banks once.
+    const int sw = (lp.l16 >> 1) & 7;
+    int fa[2], fb[2];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      fa[kk] = (lp.wm * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
-      fb[kk] = kBBase + (lp.wn * kWaveTile + lp.l32) * kRowBytes + (((kk * 2 + lp.lhi) ^ sw) << 4);
+    for (int kk = 0; kk < 2; ++kk) {
+      fa[kk] = (lp.wm * kWaveTile + lp.l16) * kRowBytes + (((kk * 4 + lp.lq) ^ sw) << 4);
+      fb[kk] = kBBase + (lp.wn * kWaveTile + lp.l16) * kRowBytes + (((kk * 4 + lp.lq) ^ sw) << 4);
     }
 
     zero_acc(acc);
-    bf16x8 af[2][4], bf[2][4];
+    bf16x8 af[2][kBlocks], bf[2][kBlocks];
     const int kt_n = g.k / kBK;
     // byte offset of k-tile kt inside a row; past the end: refetches the last tile, never consumed
     auto k_byte = [&](int kt) { return min(kt, kt_n - 1) * kRowBytes; };
@@ -167,46 +184,44 @@ struct DmaLoop {
     auto dma_b = [&](int slot_off, int ko, int j) {
       dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b, dst + kBBase + slot_off + j * 8 * kRowBytes);
     };
-    // One k-step: 16 MFMAs on fragment set mm_set; the eight fragments of the next k-step are read
-    // one per MFMA; `NA` A instructions [a_first, a_first + NA) and `NB` B instructions [0, NB) are
-    // issued in between, in source order (the compiler keeps LDS DMA and LDS reads ordered).
-    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, int a_ko, int a_first,
-                    auto na_c, int b_slot, int b_ko, auto nb_c) {
+    // One k-step of 32: 64 MFMAs on fragment set mm_set.  The sixteen fragments of the next k-step
+    // (k-step rd_kk of the slots rd_a / rd_b) are read one per four MFMAs into the other set, and
+    // NA A-operand or NB B-operand DMA instructions are issued one per eight MFMAs.  The scheduling
+    // fence after every MFMA keeps the source order: the compiler treats an LDS DMA and an LDS read
+    // as aliasing accesses and would otherwise bunch them.
+    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, int a_ko, auto na_c,
+                    int b_slot, int b_ko, auto nb_c) {
       constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
       constexpr int vmem = NA + NB;
       const int rd_set = mm_set ^ 1;
 #pragma unroll
-      for (int m = 0; m < 16; ++m) {
-        const int before = (m * vmem) / 16, due = ((m + 1) * vmem) / 16 - before;
+      for (int i = 0; i < kBlocks; ++i) {
 #pragma unroll
-        for (int d = 0; d < due; ++d) {
-          const int idx = before + d;  // B first: it has the shorter time to land
-          if (idx < NB) dma_b(b_slot, b_ko, idx);
-          else dma_a(a_slot, a_ko, a_first + idx - NB);
+        for (int j = 0; j < kBlocks; ++j) {
+          const int m = i * kBlocks + j;
+          const int before = (m * vmem) / 64, due = ((m + 1) * vmem) / 64 - before;
+#pragma unroll
+          for (int d = 0; d < due; ++d) {
+            const int idx = before + d;
+            if (idx < NB) dma_b(b_slot, b_ko, idx);
+            else dma_a(a_slot, a_ko, idx - NB);
+          }
+          const bool rd = (j & 3) == 0;
+          const int r = i * 2 + (j >> 2);  // A block 0, then the eight B blocks, then A blocks 1..7
+          if (rd && r == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk]);
+          if (rd && r >= 1 && r <= 8)
+            bf[rd_set][r - 1] =
+                *reinterpret_cast<const bf16x8*>(smem + rd_b + fb[rd_kk] + (r - 1) * kBlk * kRowBytes);
+          if (rd && r >= 9)
+            af[rd_set][r - 8] =
+                *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk] + (r - 8) * kBlk * kRowBytes);
+          mfma_16x16x32(acc[i][j], af[mm_set][i], bf[mm_set][j]);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        if (m == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk]);
-        if (m >= 1 && m <= 4)
-          bf[rd_set][m - 1] =
-              *reinterpret_cast<const bf16x8*>(smem + rd_b + fb[rd_kk] + (m - 1) * 32 * kRowBytes);
-        if (m >= 5 && m <= 7)
-          af[rd_set][m - 4] =
-              *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk] + (m - 4) * 32 * kRowBytes);
-        acc[m >> 2][m & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[mm_set][m >> 2], bf[mm_set][m & 3],
-                                                                     acc[m >> 2][m & 3], 0, 0, 0);
-        if (due == 1) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        if (due >= 2) __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
-        if (m < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       }
-      __builtin_amdgcn_sched_barrier(0);
     };
     using I0 = std::integral_constant<int, 0>;
     using I8 = std::integral_constant<int, 8>;
-    constexpr int kA[3] = {3, 3, 2};  // A instructions under k-steps 0, 1, 2
-    static_assert(kA[0] + kA[1] + kA[2] == 8, "eight A instructions per wave and k-tile");
-    using A0 = std::integral_constant<int, kA[0]>;
-    using A1 = std::integral_constant<int, kA[1]>;
-    using A2 = std::integral_constant<int, kA[2]>;
 
     // prologue: tiles 0 and 1 whole (A slots 0, 1; B slots 0, 1)
 #pragma unroll
@@ -220,9 +235,9 @@ struct DmaLoop {
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 has landed
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      af[0][i] = *reinterpret_cast<const bf16x8*>(smem + fa[0] + i * 32 * kRowBytes);
-      bf[0][i] = *reinterpret_cast<const bf16x8*>(smem + fb[0] + i * 32 * kRowBytes);
+    for (int i = 0; i < kBlocks; ++i) {
+      af[0][i] = *reinterpret_cast<const bf16x8*>(smem + fa[0] + i * kBlk * kRowBytes);
+      bf[0][i] = *reinterpret_cast<const bf16x8*>(smem + fb[0] + i * kBlk * kRowBytes);
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -232,20 +247,19 @@ struct DmaLoop {
       const int a_fill = (a_nxt == 2 * kOperandBytes) ? 0 : a_nxt + kOperandBytes;  // freed one barrier ago
       const int b_nxt = b_cur ^ kOperandBytes;
       const int ko2 = k_byte(kt + 2);
-      // k-steps 0..2: A of tile kt+2
-      step(a_cur, b_cur, 1, 0, a_fill, ko2, 0, A0{}, 0, 0, I0{});
-      step(a_cur, b_cur, 2, 1, a_fill, ko2, kA[0], A1{}, 0, 0, I0{});
-      step(a_cur, b_cur, 3, 0, a_fill, ko2, kA[0] + kA[1], A2{}, 0, 0, I0{});
-      // last k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
+      // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read
+      step(a_cur, b_cur, 1, 0, a_fill, ko2, I8{}, 0, 0, I0{});
+      // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
-      step(a_nxt, b_nxt, 0, 1, 0, 0, 0, I0{}, b_cur, ko2, I8{});
+      step(a_nxt, b_nxt, 0, 1, 0, 0, I0{}, b_cur, ko2, I8{});
       a_cur = a_nxt;
       b_cur = b_nxt;
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
     __builtin_amdgcn_s_barrier();
+    settle_acc();
   }
 };
 
@@ -254,6 +268,7 @@ struct DmaLoop {
 // ---------------------------------------------------------------------------------------
 template <int BK>
 struct RegLoop {
+  static_assert(BK == 32, "one 16x16x32 k-step per staged tile");
   static constexpr int kBK = BK;
   static constexpr int kChunks = BK / 8;                 // 16-byte chunks per row
   static constexpr int kRowBytes = BK * 2;
@@ -270,8 +285,8 @@ struct RegLoop {
     return TilePos{tm * kTile, tn * kTile, 0, 0};
   }
 
-  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t,
-                                             f32x16 (&acc)[4][4], char* smem) {
+  __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t, AccTile& acc,
+                                             char* smem) {
     constexpr int kLoads = (kTile * kChunks) / kGemmThreads;  // 16-byte loads per operand per thread
     constexpr int kRowStep = kGemmThreads / kChunks;
     const LanePos lp;
@@ -289,11 +304,11 @@ struct RegLoop {
       gb[i] = reinterpret_cast<const uint4*>(g.b + (int64_t)rb * g.ldb) + ld_chunk;
       lds_off[i] = offset(row, ld_chunk);
     }
-    int a_off[4], b_off[4];
+    int a_off[kBlocks], b_off[kBlocks];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      a_off[i] = lp.wm * kWaveTile + i * 32 + lp.l32;
-      b_off[i] = lp.wn * kWaveTile + i * 32 + lp.l32;
+    for (int i = 0; i < kBlocks; ++i) {
+      a_off[i] = offset(lp.wm * kWaveTile + i * kBlk + lp.l16, lp.lq);
+      b_off[i] = kOperandBytes + offset(lp.wn * kWaveTile + i * kBlk + lp.l16, lp.lq);
     }
     zero_acc(acc);
 
@@ -323,20 +338,16 @@ struct RegLoop {
           rb[i] = gb[i][ko];
         }
       }
+      bf16x8 af[kBlocks], bf[kBlocks];
 #pragma unroll
-      for (int kk = 0; kk < BK / 16; ++kk) {
-        bf16x8 af[4], bf[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          af[i] = *reinterpret_cast<const bf16x8*>(cur + offset(a_off[i], kk * 2 + lp.lhi));
-          bf[i] = *reinterpret_cast<const bf16x8*>(cur + kOperandBytes + offset(b_off[i], kk * 2 + lp.lhi));
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < kBlocks; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(cur + a_off[i]);
+        bf[i] = *reinterpret_cast<const bf16x8*>(cur + b_off[i]);
       }
+#pragma unroll
+      for (int i = 0; i < kBlocks; ++i)
+#pragma unroll
+        for (int j = 0; j < kBlocks; ++j) mfma_16x16x32(acc[i][j], af[i], bf[j]);
       if (more) {
 #pragma unroll
         for (int i = 0; i < kLoads; ++i) {
@@ -346,6 +357,7 @@ struct RegLoop {
       }
       __syncthreads();
     }
+    settle_acc();
   }
 };
 

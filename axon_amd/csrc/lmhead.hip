@@ -63,44 +63,48 @@ __device__ __forceinline__ void merge_stats(float M, float& s, float& e, float M
 // do not count (beyond the vocabulary, or duplicates of the neighbouring tile); they are
 // excluded by predicate — their accumulators hold finite values.
 template <bool MASKED>
-__device__ __forceinline__ void fwd_epilogue(f32x16 (&acc)[4][4], const FwdParams& p,
-                                             const LanePos& lp, const TilePos& t, int tm) {
+__device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, const LanePos& lp,
+                                             const TilePos& t, int tm) {
   const int part = tm * 2 + lp.wm;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < kBlocks; ++j) {
     float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const int mr = lp.m(i, q);
+      for (int r = 0; r < 4; ++r) {
+        const int mr = lp.m(i, r);
         const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
-        mx = ok ? fmaxf(mx, acc[i][j][q]) : mx;
+        mx = ok ? fmaxf(mx, acc[i][j][r]) : mx;
       }
-    const float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
+    float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
     float s = 0.f, e = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-      for (int q = 0; q < 16; ++q) {
-        const int mr = lp.m(i, q);
+      for (int r = 0; r < 4; ++r) {
+        const int mr = lp.m(i, r);
         const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
-        const float y = fmaf(acc[i][j][q], p.c, -M);  // scaled logit relative to the max, <= 0
+        const float y = fmaf(acc[i][j][r], p.c, -M);  // scaled logit relative to the max, <= 0
         const float w = ok ? fast_exp2(y) : 0.f;
         s += w;
         e = fmaf(w, y, e);
       }
-    // merge the two lanes that hold the same token (lane and lane^32)
-    const float M2 = __shfl_xor(M, 32, 64);
-    const float s2 = __shfl_xor(s, 32, 64);
-    const float e2 = __shfl_xor(e, 32, 64);
-    const float Mn = fmaxf(M, M2);
-    merge_stats(M, s, e, M2, s2, e2, Mn);
+    // merge the four lanes that hold the same token (lane ^ 16, lane ^ 32)
+#pragma unroll
+    for (int off = 16; off <= 32; off <<= 1) {
+      const float M2 = __shfl_xor(M, off, 64);
+      const float s2 = __shfl_xor(s, off, 64);
+      const float e2 = __shfl_xor(e, off, 64);
+      const float Mn = fmaxf(M, M2);
+      merge_stats(M, s, e, M2, s2, e2, Mn);
+      M = Mn;
+    }
     const int nr = lp.n(j);
     const int n = t.n0 + nr;
-    if (lp.lhi == 0 && nr >= t.n_lo && n < p.n_tokens) {
+    if (lp.lq == 0 && nr >= t.n_lo && n < p.n_tokens) {
       const int64_t o = (int64_t)part * p.n_tokens + n;
-      p.pm[o] = Mn;
+      p.pm[o] = M;
       p.ps[o] = s;
       p.pe[o] = e;
     }
@@ -115,15 +119,15 @@ __device__ __forceinline__ void fwd_body(const GemmOperands& g, const FwdParams&
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);
-  f32x16 acc[4][4];
+  AccTile acc;
   Loop::run(g, t, acc, smem);
   if (SOFTCAP) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kBlocks; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < kBlocks; ++j)
 #pragma unroll
-        for (int q = 0; q < 16; ++q) acc[i][j][q] = p.cap * fast_tanh(acc[i][j][q] * p.inv_cap);
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = p.cap * fast_tanh(acc[i][j][r] * p.inv_cap);
   }
   const LanePos lp;
   if (t.m_lo > 0 || t.m0 + kTile > p.vocab)
@@ -248,11 +252,14 @@ struct DlogitParams {
 };
 
 // Per-wave staging of the wave's 128(n) x 128(m) bf16 sub-tile in its own 32 KB of LDS:
-// row nw (256 bytes = 32 units of 4 bf16), unit u stored at slot u ^ swz(nw),
-// swz(nw) = (nw & 31) ^ (nw >> 5).  The three access patterns (column-of-rows write,
-// row read, 4x4-block read) then each touch 32 distinct slots per 32 lanes.
+// row nw (256 bytes = 32 units of 4 bf16), unit u stored at slot perm(u) ^ swz(nw),
+// swz(nw) = (nw & 31) ^ (nw >> 5), perm(u) = u rotated right by two bits (unit = 4 * block + lane
+// quarter: the quarter's low bit becomes the slot's high bit).  The three access patterns
+// (accumulator write: sixteen rows x two quarters per 32 lanes; row read; 4x4-block read) then each
+// touch 32 distinct slots per 32 lanes.
 __device__ __forceinline__ int stage_off(int nw, int unit) {
-  return nw * 256 + ((unit ^ ((nw & 31) ^ (nw >> 5))) << 3);
+  const int pu = ((unit & 1) << 4) | ((unit & 2) << 2) | (unit >> 2);
+  return nw * 256 + ((pu ^ ((nw & 31) ^ (nw >> 5))) << 3);
 }
 
 // SOFTCAP: the recomputed logit goes through cap * tanh(. / cap) and the gradient is multiplied by
@@ -264,16 +271,17 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);  // t.m0 is relative to the chunk
-  f32x16 acc[4][4];
+  AccTile acc;
   Loop::run(g, t, acc, smem);
   __syncthreads();  // every wave is past its last main-loop LDS access
 
   const LanePos lp;
+  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
   const float c = p.inv_temp * kLog2e;
   char* const stage = smem + lp.wave * 32768;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int nw = j * 32 + lp.l32;  // token row inside the wave's sub-tile
+  for (int j = 0; j < kBlocks; ++j) {
+    const int nw = j * kBlk + lp.l16;  // token row inside the wave's sub-tile
     const int n = t.n0 + lp.wn * kWaveTile + nw;
     const bool n_ok = n < p.n_tokens;
     const int nn = n_ok ? n : 0;
@@ -291,35 +299,31 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
                                      : (int64_t) static_cast<const int32_t*>(p.labels)[src];
     const int64_t lab_rel = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kBlocks; ++i) {
+      float d[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        float d[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int q = 4 * r + e;
-          const int mrel = lp.m(i, q);
-          float raw = acc[i][j][q];
-          float dcap = 1.f;
-          if (SOFTCAP) {
-            const float th = fast_tanh(raw * p.inv_cap);
-            raw = p.cap * th;
-            dcap = fmaf(-th, th, 1.f);
-          }
-          const float pr = fast_exp2(fmaf(raw, c, -lse2));
-          const float x = raw * p.inv_temp;
-          float v = pr * fmaf(cb, x, ca);
-          if ((int64_t)mrel == lab_rel) v += gl;
-          if (SOFTCAP) v *= dcap;
-          // rows shared with the neighbouring tile keep their (identical) values
-          const bool ok = n_ok && (p.v_begin + t.m0 + mrel < p.vocab);
-          d[e] = ok ? v : 0.f;
+        const int mrel = lp.m(i, r);
+        float raw = acc[i][j][r];
+        float dcap = 1.f;
+        if (SOFTCAP) {
+          const float th = fast_tanh(raw * p.inv_cap);
+          raw = p.cap * th;
+          dcap = fmaf(-th, th, 1.f);
         }
-        uint2 w;
-        w.x = pack_bf16(d[0], d[1]);
-        w.y = pack_bf16(d[2], d[3]);
-        *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 8 + 2 * r + lp.lhi)) = w;
+        const float pr = fast_exp2(fmaf(raw, c, -lse2));
+        const float x = raw * p.inv_temp;
+        float v = pr * fmaf(cb, x, ca);
+        if ((int64_t)mrel == lab_rel) v += gl;
+        if (SOFTCAP) v *= dcap;
+        // rows shared with the neighbouring tile keep their (identical) values
+        const bool ok = n_ok && (p.v_begin + t.m0 + mrel < p.vocab);
+        d[r] = ok ? v : 0.f;
       }
+      uint2 w;
+      w.x = pack_bf16(d[0], d[1]);
+      w.y = pack_bf16(d[2], d[3]);
+      *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 4 + lp.lq)) = w;
     }
   }
   // the wave reads back only what it wrote itself; LDS operations of one wave complete in order
@@ -327,18 +331,18 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   const int n_base = t.n0 + lp.wn * kWaveTile;
   // token-major copy: 32 lanes cover one 256-byte row
   {
-    const int unit = lp.l32;
+    const int unit = l32;
 #pragma unroll 4
-    for (int nw = lp.lhi; nw < kWaveTile; nw += 2) {
+    for (int nw = lhi; nw < kWaveTile; nw += 2) {
       const uint2 v = *reinterpret_cast<const uint2*>(stage + stage_off(nw, unit));
       *reinterpret_cast<uint2*>(p.dl + (int64_t)(n_base + nw) * p.ld_dl + m_base + unit * 4) = v;
     }
   }
   // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
   {
-    const int nq = lp.l32;  // token quad
+    const int nq = l32;  // token quad
 #pragma unroll 2
-    for (int unit = lp.lhi; unit < 32; unit += 2) {
+    for (int unit = lhi; unit < 32; unit += 2) {
       uint2 rws[4];
 #pragma unroll
       for (int f = 0; f < 4; ++f)
@@ -391,39 +395,36 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);
-  f32x16 acc[4][4];
+  AccTile acc;
   Loop::run(g, t, acc, smem);
   const LanePos lp;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < kBlocks; ++j) {
     const int nr = lp.n(j);
     const int n = t.n0 + nr;
     if (nr < t.n_lo || n >= p.n_valid) continue;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int mr = lp.m(i, 4 * r);
-        const int m = t.m0 + mr;
-        // m_valid % 4 == 0 and tile shifts are multiples of 4: a quad is all in or all out
-        if (mr < t.m_lo || m >= p.m_valid) continue;
-        float4 v = make_float4(acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2],
-                               acc[i][j][4 * r + 3]);
-        if (p.out_f32) {
-          float4* dst = reinterpret_cast<float4*>(p.out_f32 + (int64_t)n * p.ld_f32 + m);
-          if (p.accumulate) {
-            const float4 old = *dst;
-            v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
-          }
-          *dst = v;
+    for (int i = 0; i < kBlocks; ++i) {
+      const int mr = lp.m(i, 0);
+      const int m = t.m0 + mr;
+      // m_valid % 4 == 0 and tile shifts are multiples of 4: a quad is all in or all out
+      if (mr < t.m_lo || m >= p.m_valid) continue;
+      float4 v = make_float4(acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      if (p.out_f32) {
+        float4* dst = reinterpret_cast<float4*>(p.out_f32 + (int64_t)n * p.ld_f32 + m);
+        if (p.accumulate) {
+          const float4 old = *dst;
+          v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
         }
-        if (p.out_bf16) {
-          uint2 w;
-          w.x = pack_bf16(v.x, v.y);
-          w.y = pack_bf16(v.z, v.w);
-          *reinterpret_cast<uint2*>(p.out_bf16 + (int64_t)n * p.ld_bf16 + m) = w;
-        }
+        *dst = v;
       }
+      if (p.out_bf16) {
+        uint2 w;
+        w.x = pack_bf16(v.x, v.y);
+        w.y = pack_bf16(v.z, v.w);
+        *reinterpret_cast<uint2*>(p.out_bf16 + (int64_t)n * p.ld_bf16 + m) = w;
+      }
+    }
   }
 }
 
