@@ -131,11 +131,26 @@ struct DmaLoop {
     return t;
   }
 
+  // One DMA instruction: 16 bytes per lane, LDS destination = lds + IMM + 16 * lane
+  // (wave-contiguous), memory source = base + voffset + soffset + IMM.  The instruction's immediate
+  // offset moves both sides, so four consecutive 1 KB destinations share one M0 value.
+  template <int IMM>
   __device__ static __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, int voffset, int soffset,
                                                char* lds) {
-    // LDS destination = lds + 16 * lane (wave-contiguous); memory source = base + voffset + soffset
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16,
-                                             voffset, soffset, 0, 0);
+                                             voffset, soffset, IMM, 0);
+  }
+  // instruction j of an operand tile (rows 8j .. 8j+7 of the wave's 64): lds = tile base of the wave
+  __device__ static __forceinline__ void dma_row8(__amdgpu_buffer_rsrc_t rsrc, int voffset,
+                                                  int row8_bytes, char* lds, int j) {
+    char* const l = lds + (j >> 2) * 4096;
+    const int so = j * row8_bytes - (j & 3) * 1024;
+    switch (j & 3) {
+      case 0: dma16<0>(rsrc, voffset, so, l); break;
+      case 1: dma16<1024>(rsrc, voffset, so, l); break;
+      case 2: dma16<2048>(rsrc, voffset, so, l); break;
+      default: dma16<3072>(rsrc, voffset, so, l); break;
+    }
   }
 
   __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t, AccTile& acc,
@@ -178,36 +193,36 @@ struct DmaLoop {
     const int kt_n = g.k / kBK;
     // byte offset of k-tile kt inside a row; past the end: refetches the last tile, never consumed
     auto k_byte = [&](int kt) { return min(kt, kt_n - 1) * kRowBytes; };
-    auto dma_a = [&](int slot_off, int ko, int j) {
-      dma16(ra, (j & 1) ? va_o : va_e, ko + j * step_a, dst + slot_off + j * 8 * kRowBytes);
+    // `ko` (the k-tile's byte offset inside a row) rides in the per-lane offsets, added once per tile
+    auto dma_a = [&](int slot_off, int v_even, int v_odd, int j) {
+      dma_row8(ra, (j & 1) ? v_odd : v_even, step_a, dst + slot_off, j);
     };
-    auto dma_b = [&](int slot_off, int ko, int j) {
-      dma16(rb, (j & 1) ? vb_o : vb_e, ko + j * step_b, dst + kBBase + slot_off + j * 8 * kRowBytes);
+    auto dma_b = [&](int slot_off, int v_even, int v_odd, int j) {
+      dma_row8(rb, (j & 1) ? v_odd : v_even, step_b, dst + kBBase + slot_off, j);
     };
     // One k-step of 32: 64 MFMAs on fragment set mm_set.  The sixteen fragments of the next k-step
-    // (k-step rd_kk of the slots rd_a / rd_b) are read one per four MFMAs into the other set, and
-    // NA A-operand or NB B-operand DMA instructions are issued one per eight MFMAs.  The scheduling
-    // fence after every MFMA keeps the source order: the compiler treats an LDS DMA and an LDS read
-    // as aliasing accesses and would otherwise bunch them.
-    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, int a_ko, auto na_c,
-                    int b_slot, int b_ko, auto nb_c) {
+    // (k-step rd_kk of the slots rd_a / rd_b) are read under the first half of the step, one per two
+    // MFMAs, into the other set, so that they have landed long before the barrier's wait; NA
+    // A-operand or NB B-operand DMA instructions are issued one per eight MFMAs, in slots that carry
+    // no fragment read.  The scheduling fence after every MFMA keeps the source order: the compiler
+    // treats an LDS DMA and an LDS read as aliasing accesses and would otherwise bunch them.
+    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, auto na_c, int b_slot,
+                    auto nb_c, int v_even, int v_odd, auto&& mid) {
       constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
-      constexpr int vmem = NA + NB;
+      static_assert((NA == 0 || NA == 8) && (NB == 0 || NB == 8) && NA + NB <= 8, "");
       const int rd_set = mm_set ^ 1;
 #pragma unroll
       for (int i = 0; i < kBlocks; ++i) {
 #pragma unroll
         for (int j = 0; j < kBlocks; ++j) {
           const int m = i * kBlocks + j;
-          const int before = (m * vmem) / 64, due = ((m + 1) * vmem) / 64 - before;
-#pragma unroll
-          for (int d = 0; d < due; ++d) {
-            const int idx = before + d;
-            if (idx < NB) dma_b(b_slot, b_ko, idx);
-            else dma_a(a_slot, a_ko, idx - NB);
+          if (m == 37) mid();  // index arithmetic for the coming k-tile, in a slot without other work
+          if ((m & 7) == 3) {
+            if (NB) dma_b(b_slot, v_even, v_odd, m >> 3);
+            if (NA) dma_a(a_slot, v_even, v_odd, m >> 3);
           }
-          const bool rd = (j & 3) == 0;
-          const int r = i * 2 + (j >> 2);  // A block 0, then the eight B blocks, then A blocks 1..7
+          const bool rd = (m & 1) == 0 && m < 32;
+          const int r = m >> 1;  // A block 0, then the eight B blocks, then A blocks 1..7
           if (rd && r == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk]);
           if (rd && r >= 1 && r <= 8)
             bf[rd_set][r - 1] =
@@ -225,13 +240,16 @@ struct DmaLoop {
 
     // prologue: tiles 0 and 1 whole (A slots 0, 1; B slots 0, 1)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_a(0, k_byte(0), j);
+    for (int j = 0; j < 8; ++j) dma_a(0, va_e, va_o, j);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_b(0, k_byte(0), j);
+    for (int j = 0; j < 8; ++j) dma_b(0, vb_e, vb_o, j);
+    {
+      const int ko1 = k_byte(1);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, k_byte(1), j);
+      for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, va_e + ko1, va_o + ko1, j);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_b(kOperandBytes, k_byte(1), j);
+      for (int j = 0; j < 8; ++j) dma_b(kOperandBytes, vb_e + ko1, vb_o + ko1, j);
+    }
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 has landed
     __builtin_amdgcn_s_barrier();
 #pragma unroll
@@ -241,21 +259,38 @@ struct DmaLoop {
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    int a_cur = 0, b_cur = 0;  // slots of the tile being consumed
-    for (int kt = 0; kt < kt_n; ++kt) {
-      const int a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
-      const int a_fill = (a_nxt == 2 * kOperandBytes) ? 0 : a_nxt + kOperandBytes;  // freed one barrier ago
-      const int b_nxt = b_cur ^ kOperandBytes;
+    // per-tile scalars: slots of the tile being consumed (cur), of the next one (nxt), the A slot
+    // being filled, and the per-lane source offsets of k-tile kt+2; those of the following tile are
+    // computed under the second k-step so that the loop's back edge carries no arithmetic
+    struct Tile {
+      int a_cur, a_nxt, a_fill, b_cur, b_nxt, va_e, va_o, vb_e, vb_o;
+    };
+    auto tile_vars = [&](int a_cur, int b_cur, int kt) {
+      Tile v;
+      v.a_cur = a_cur;
+      v.b_cur = b_cur;
+      v.a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
+      v.a_fill = (v.a_nxt == 2 * kOperandBytes) ? 0 : v.a_nxt + kOperandBytes;  // freed one barrier ago
+      v.b_nxt = b_cur ^ kOperandBytes;
       const int ko2 = k_byte(kt + 2);
+      v.va_e = va_e + ko2;
+      v.va_o = va_o + ko2;
+      v.vb_e = vb_e + ko2;
+      v.vb_o = vb_o + ko2;
+      return v;
+    };
+    Tile tv = tile_vars(0, 0, 0);
+    for (int kt = 0; kt < kt_n; ++kt) {
+      Tile nx;
       // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read
-      step(a_cur, b_cur, 1, 0, a_fill, ko2, I8{}, 0, 0, I0{});
+      step(tv.a_cur, tv.b_cur, 1, 0, tv.a_fill, I8{}, 0, I0{}, tv.va_e, tv.va_o, [] {});
       // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
-      step(a_nxt, b_nxt, 0, 1, 0, 0, I0{}, b_cur, ko2, I8{});
-      a_cur = a_nxt;
-      b_cur = b_nxt;
+      step(tv.a_nxt, tv.b_nxt, 0, 1, 0, I0{}, tv.b_cur, I8{}, tv.vb_e, tv.vb_o,
+           [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); });
+      tv = nx;
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
     __builtin_amdgcn_s_barrier();
