@@ -22,11 +22,12 @@ constexpr float kLn2 = 0.6931471805599453f;
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  // round-to-nearest-even; the values here are finite
-  uint32_t a = __float_as_uint(lo), b = __float_as_uint(hi);
-  a += 0x7fffu + ((a >> 16) & 1u);
-  b += 0x7fffu + ((b >> 16) & 1u);
-  return (a >> 16) | (b & 0xffff0000u);
+  // round-to-nearest-even in one instruction (v_cvt_pk_bf16_f32)
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  const bf16x2 r = __builtin_convertvector(v, bf16x2);
+  return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 // ----------------------------------------------------------------------------
@@ -264,21 +265,12 @@ __device__ __forceinline__ int stage_off(int nw, int unit) {
 
 // SOFTCAP: the recomputed logit goes through cap * tanh(. / cap) and the gradient is multiplied by
 // the derivative 1 - tanh^2 (fused_linear.py:80-83).
-template <class Loop, bool SOFTCAP>
-__device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitParams& p,
-                                            int tiles_m, int tiles_n) {
-  extern __shared__ __align__(16) char smem[];
-  int tm, tn;
-  tile_coords(tiles_m, tiles_n, tm, tn);
-  const TilePos t = Loop::place(g, tm, tn);  // t.m0 is relative to the chunk
-  AccTile acc;
-  Loop::run(g, t, acc, smem);
-  __syncthreads();  // every wave is past its last main-loop LDS access
-
-  const LanePos lp;
-  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
+// Accumulators -> bf16 dlogits in the wave's staging area.  MASKED: the tile reaches past the last
+// token or the last vocabulary row; those entries are written as zeros.
+template <bool SOFTCAP, bool MASKED>
+__device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p, const LanePos& lp,
+                                             const TilePos& t, char* stage) {
   const float c = p.inv_temp * kLog2e;
-  char* const stage = smem + lp.wave * 32768;
 #pragma unroll
   for (int j = 0; j < kBlocks; ++j) {
     const int nw = j * kBlk + lp.l16;  // token row inside the wave's sub-tile
@@ -291,13 +283,15 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
     const float g_en = (g_ok && p.dentropy) ? p.dentropy[src] : 0.f;
     const float lse2 = p.lse[nn] * kLog2e;
     const float eb = p.entropy_b[nn];
-    // dlogit = p * (a + b * x) + onehot * g / T,  x = logit / T
+    // dlogit = p * (a + b * logit) + onehot * g / T
     const float ca = (-g_lp + g_en * eb) * p.inv_temp;
-    const float cb = -g_en * p.inv_temp;
+    const float cb = -g_en * p.inv_temp * p.inv_temp;
     const float gl = g_lp * p.inv_temp;
     const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[src]
                                      : (int64_t) static_cast<const int32_t*>(p.labels)[src];
-    const int64_t lab_rel = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
+    const int64_t lab_rel64 = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
+    const int lab_rel = (lab_rel64 >= 0 && lab_rel64 < kTile) ? (int)lab_rel64 : -1;
+    const int m_end = MASKED ? (n_ok ? p.vocab - p.v_begin - t.m0 : 0) : kTile;  // rows that count
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
       float d[4];
@@ -312,13 +306,11 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
           dcap = fmaf(-th, th, 1.f);
         }
         const float pr = fast_exp2(fmaf(raw, c, -lse2));
-        const float x = raw * p.inv_temp;
-        float v = pr * fmaf(cb, x, ca);
-        if ((int64_t)mrel == lab_rel) v += gl;
+        float v = pr * fmaf(cb, raw, ca);
+        if (mrel == lab_rel) v += gl;
         if (SOFTCAP) v *= dcap;
         // rows shared with the neighbouring tile keep their (identical) values
-        const bool ok = n_ok && (p.v_begin + t.m0 + mrel < p.vocab);
-        d[r] = ok ? v : 0.f;
+        d[r] = (!MASKED || mrel < m_end) ? v : 0.f;
       }
       uint2 w;
       w.x = pack_bf16(d[0], d[1]);
@@ -326,6 +318,26 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
       *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 4 + lp.lq)) = w;
     }
   }
+}
+
+template <class Loop, bool SOFTCAP>
+__device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitParams& p,
+                                            int tiles_m, int tiles_n) {
+  extern __shared__ __align__(16) char smem[];
+  int tm, tn;
+  tile_coords(tiles_m, tiles_n, tm, tn);
+  const TilePos t = Loop::place(g, tm, tn);  // t.m0 is relative to the chunk
+  AccTile acc;
+  Loop::run(g, t, acc, smem);
+  __syncthreads();  // every wave is past its last main-loop LDS access
+
+  const LanePos lp;
+  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
+  char* const stage = smem + lp.wave * 32768;
+  if (t.n0 + kTile > p.n_tokens || p.v_begin + t.m0 + kTile > p.vocab)
+    dlogit_stage<SOFTCAP, true>(acc, p, lp, t, stage);
+  else
+    dlogit_stage<SOFTCAP, false>(acc, p, lp, t, stage);
   // the wave reads back only what it wrote itself; LDS operations of one wave complete in order
   const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
   const int n_base = t.n0 + lp.wn * kWaveTile;
