@@ -477,7 +477,9 @@ using namespace axon;
 namespace {
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
-constexpr int64_t kDefaultVocabChunk = 16384;
+// bf16 dlogits of one chunk exist in both orientations (2 x 2.1 GB at 32768 tokens); every chunk costs one
+// read-modify-write pass over the fp32 dHidden accumulator, so fewer, larger chunks are cheaper
+constexpr int64_t kDefaultVocabChunk = 32768;
 constexpr int64_t kAlign = 256;
 using SlowLoop = RegLoop<32>;
 

@@ -98,7 +98,7 @@ int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void
  *   d_hidden = dlogit @ W, d_weight = dlogit^T @ hidden, both written as bf16.
  * With softcap > 0 dlogit is additionally multiplied by 1 - tanh^2(raw logit / softcap)
  * (fused_linear.py:80-83).  dentropy may be NULL (treated as zeros).  vocab_chunk (multiple of 256, or 0
- * for the library default) bounds the bf16 dlogit scratch to
+ * for the library default, 32768) bounds the bf16 dlogit scratch to
  * 2 * n_tokens_padded * vocab_chunk * 2 bytes. */
 int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab,
                                         int64_t vocab_chunk);
