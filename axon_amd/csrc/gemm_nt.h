@@ -194,11 +194,16 @@ struct DmaLoop {
     // byte offset of k-tile kt inside a row; past the end: refetches the last tile, never consumed
     auto k_byte = [&](int kt) { return min(kt, kt_n - 1) * kRowBytes; };
     // `ko` (the k-tile's byte offset inside a row) rides in the per-lane offsets, added once per tile
-    auto dma_a = [&](int slot_off, int v_even, int v_odd, int j) {
-      dma_row8(ra, (j & 1) ? v_odd : v_even, step_a, dst + slot_off, j);
+    auto dma_a = [&](int slot_off, const __amdgpu_buffer_rsrc_t& r, int j) {
+      dma_row8(r, (j & 1) ? va_o : va_e, step_a, dst + slot_off, j);
     };
-    auto dma_b = [&](int slot_off, int v_even, int v_odd, int j) {
-      dma_row8(rb, (j & 1) ? v_odd : v_even, step_b, dst + kBBase + slot_off, j);
+    auto dma_b = [&](int slot_off, const __amdgpu_buffer_rsrc_t& r, int j) {
+      dma_row8(r, (j & 1) ? vb_o : vb_e, step_b, dst + kBBase + slot_off, j);
+    };
+    // the k-tile's byte offset inside a row rides in the buffer descriptor's base: scalar arithmetic
+    auto rsrc_at = [&](const __bf16* base, int ko) {
+      return __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(base) + ko), 0, 0x7fffffff,
+                                               0x00020000);
     };
     // One k-step of 32: 64 MFMAs on fragment set mm_set.  The sixteen fragments of the next k-step
     // (k-step rd_kk of the slots rd_a / rd_b) are read under the first half of the step, one per two
@@ -207,7 +212,7 @@ struct DmaLoop {
     // no fragment read.  The scheduling fence after every MFMA keeps the source order: the compiler
     // treats an LDS DMA and an LDS read as aliasing accesses and would otherwise bunch them.
     auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, auto na_c, int b_slot,
-                    auto nb_c, int v_even, int v_odd, auto&& mid) {
+                    auto nb_c, const __amdgpu_buffer_rsrc_t& rsrc, auto&& mid) {
       constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
       static_assert((NA == 0 || NA == 8) && (NB == 0 || NB == 8) && NA + NB <= 8, "");
       const int rd_set = mm_set ^ 1;
@@ -218,8 +223,8 @@ struct DmaLoop {
           const int m = i * kBlocks + j;
           if (m == 37) mid();  // index arithmetic for the coming k-tile, in a slot without other work
           if ((m & 7) == 3) {
-            if (NB) dma_b(b_slot, v_even, v_odd, m >> 3);
-            if (NA) dma_a(a_slot, v_even, v_odd, m >> 3);
+            if (NB) dma_b(b_slot, rsrc, m >> 3);
+            if (NA) dma_a(a_slot, rsrc, m >> 3);
           }
           const bool rd = (m & 1) == 0 && m < 32;
           const int r = m >> 1;  // A block 0, then the eight B blocks, then A blocks 1..7
@@ -240,15 +245,15 @@ struct DmaLoop {
 
     // prologue: tiles 0 and 1 whole (A slots 0, 1; B slots 0, 1)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_a(0, va_e, va_o, j);
+    for (int j = 0; j < 8; ++j) dma_a(0, ra, j);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) dma_b(0, vb_e, vb_o, j);
+    for (int j = 0; j < 8; ++j) dma_b(0, rb, j);
     {
-      const int ko1 = k_byte(1);
+      const __amdgpu_buffer_rsrc_t ra1 = rsrc_at(base_a, k_byte(1)), rb1 = rsrc_at(base_b, k_byte(1));
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, va_e + ko1, va_o + ko1, j);
+      for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, ra1, j);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) dma_b(kOperandBytes, vb_e + ko1, vb_o + ko1, j);
+      for (int j = 0; j < 8; ++j) dma_b(kOperandBytes, rb1, j);
     }
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 has landed
     __builtin_amdgcn_s_barrier();
@@ -263,7 +268,8 @@ struct DmaLoop {
     // being filled, and the per-lane source offsets of k-tile kt+2; those of the following tile are
     // computed under the second k-step so that the loop's back edge carries no arithmetic
     struct Tile {
-      int a_cur, a_nxt, a_fill, b_cur, b_nxt, va_e, va_o, vb_e, vb_o;
+      int a_cur, a_nxt, a_fill, b_cur, b_nxt;
+      __amdgpu_buffer_rsrc_t ra, rb;
     };
     auto tile_vars = [&](int a_cur, int b_cur, int kt) {
       Tile v;
@@ -273,22 +279,20 @@ struct DmaLoop {
       v.a_fill = (v.a_nxt == 2 * kOperandBytes) ? 0 : v.a_nxt + kOperandBytes;  // freed one barrier ago
       v.b_nxt = b_cur ^ kOperandBytes;
       const int ko2 = k_byte(kt + 2);
-      v.va_e = va_e + ko2;
-      v.va_o = va_o + ko2;
-      v.vb_e = vb_e + ko2;
-      v.vb_o = vb_o + ko2;
+      v.ra = rsrc_at(base_a, ko2);
+      v.rb = rsrc_at(base_b, ko2);
       return v;
     };
     Tile tv = tile_vars(0, 0, 0);
     for (int kt = 0; kt < kt_n; ++kt) {
       Tile nx;
       // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read
-      step(tv.a_cur, tv.b_cur, 1, 0, tv.a_fill, I8{}, 0, I0{}, tv.va_e, tv.va_o, [] {});
+      step(tv.a_cur, tv.b_cur, 1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [] {});
       // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
-      step(tv.a_nxt, tv.b_nxt, 0, 1, 0, I0{}, tv.b_cur, I8{}, tv.vb_e, tv.vb_o,
+      step(tv.a_nxt, tv.b_nxt, 0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb,
            [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); });
       tv = nx;
     }
