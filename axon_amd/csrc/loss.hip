@@ -222,28 +222,10 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     __syncthreads();  // the previous chunk's row window is no longer read
     rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
   }
-#pragma unroll 1
-  for (int it = 0; it < kIter; ++it) {
-    const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
-    if (i >= c1) continue;
-    float lv[4], ov[4], av[4], mv[4], wv[4] = {1.f, 1.f, 1.f, 1.f}, gv[4];
-    const bool full = (i + kVec <= n_slots);
-    if (full) {
-      load4(logp, i, lv);
-      load4(oldp, i, ov);
-      load4(adv, i, av);
-      load_mask4<MK>(mask, i, mv);
-      if (isw) load4(isw, i, wv);
-    } else {
-      for (int j = 0; j < 4; ++j) {
-        const bool ok = i + j < n_slots;
-        lv[j] = ok ? logp[i + j] : 0.f;
-        ov[j] = ok ? oldp[i + j] : 0.f;
-        av[j] = ok ? adv[i + j] : 0.f;
-        mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
-        wv[j] = (ok && isw) ? isw[i + j] : 1.f;
-      }
-    }
+  // the per-token arithmetic on one vector of four slots
+  auto process = [&](int64_t i, bool full, const float (&lv)[4], const float (&ov)[4], const float (&av)[4],
+                     const float (&mv)[4], const float (&wv)[4]) {
+    float gv[4];
     int64_t rend = -1;
     float scale = uniform_scale, sbar = 0.f;
 #pragma unroll
@@ -306,6 +288,55 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     if (full) store4(grad, i, gv);
     else
       for (int j = 0; j < 4 && i + j < n_slots; ++j) grad[i + j] = gv[j];
+  };
+  if (c1 - c0 == kChunk) {
+    // whole chunk: the loads of kB steps are issued before the first use, so that each thread has
+    // kB x (4 or 5) 16-byte requests in flight (+3 % over one step at a time at 2^26 tokens)
+    // (the sequence-level kernel keeps more state per token: two steps at a time there)
+    constexpr int kB = (KIND == 1) ? 2 : kIter;
+#pragma unroll
+    for (int b0 = 0; b0 < kIter; b0 += kB) {
+      float lv[kB][4], ov[kB][4], av[kB][4], mv[kB][4], wv[kB][4];
+#pragma unroll
+      for (int it = 0; it < kB; ++it) {
+        const int64_t i = c0 + ((int64_t)(b0 + it) * kBlock + threadIdx.x) * kVec;
+        load4(logp, i, lv[it]);
+        load4(oldp, i, ov[it]);
+        load4(adv, i, av[it]);
+        load_mask4<MK>(mask, i, mv[it]);
+        if (isw) load4(isw, i, wv[it]);
+        else wv[it][0] = wv[it][1] = wv[it][2] = wv[it][3] = 1.f;
+      }
+#pragma unroll
+      for (int it = 0; it < kB; ++it)
+        process(c0 + ((int64_t)(b0 + it) * kBlock + threadIdx.x) * kVec, true, lv[it], ov[it], av[it], mv[it],
+                wv[it]);
+    }
+  } else {
+#pragma unroll 1
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      if (i >= c1) continue;
+      float lv[4], ov[4], av[4], mv[4], wv[4] = {1.f, 1.f, 1.f, 1.f};
+      const bool full = (i + kVec <= n_slots);
+      if (full) {
+        load4(logp, i, lv);
+        load4(oldp, i, ov);
+        load4(adv, i, av);
+        load_mask4<MK>(mask, i, mv);
+        if (isw) load4(isw, i, wv);
+      } else {
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = i + j < n_slots;
+          lv[j] = ok ? logp[i + j] : 0.f;
+          ov[j] = ok ? oldp[i + j] : 0.f;
+          av[j] = ok ? adv[i + j] : 0.f;
+          mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+          wv[j] = (ok && isw) ? isw[i + j] : 1.f;
+        }
+      }
+      process(i, full, lv, ov, av, mv, wv);
+    }
   }
   }  // chunk
   if (blockIdx.x == 0 && threadIdx.x == 0) a[5] = 1.f;  // gradient factor unless post-normalised
