@@ -158,8 +158,8 @@ def hbm_kernels(n_tokens, dev):
 
 # HBM-side bytes of ONE launch of the dominant kernel at the default workload, from rocprofv3 --pmc passes
 # over `bench.py --traffic-probe` (FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0, the factors a 1 GiB
-# device copy in the same run calibrates): 6.29e9 read + 0.37e9 written.
-TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 6.65e9}
+# device copy in the same run calibrates): 12.35e9 read + 0.45e9 written, default vocabulary chunk.
+TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 12.80e9}
 
 
 def traffic_probe(workload):
@@ -282,7 +282,7 @@ def main():
         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": (dom["algorithmic_tflops"] or dom["executed_tflops"]) / MFMA_BF16_PEAK_TFLOPS,
         "avg_launch_ms": dom["avg_launch_ms"],
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if not args.tokens and "gemm_store" in dom["kernel"] else None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if not args.tokens and not args.vocab_chunk and "gemm_store" in dom["kernel"] else None,
         "kernels": kernels,
         "path_algorithmic_tflops": 6 * nhv / (ms_per_step * 1e-3) / 1e12,
         "path_frac_of_peak": 6 * nhv / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
