@@ -121,11 +121,23 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(
   float t[kPartialStride];
 #pragma unroll
   for (int k = 0; k < kPartialStride; ++k) t[k] = 0.f;
-  for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
-    const float4 lo4 = *reinterpret_cast<const float4*>(partials + (size_t)b * kPartialStride);
-    const float4 hi4 = *reinterpret_cast<const float4*>(partials + (size_t)b * kPartialStride + 4);
-    t[0] += lo4.x; t[1] += lo4.y; t[2] += lo4.z; t[3] += lo4.w;
-    t[4] += hi4.x; t[5] += hi4.y; t[6] += hi4.z; t[7] += hi4.w;
+  // four blocks per trip: eight independent 16-byte loads in flight per thread; the order in which a
+  // thread adds its blocks stays fixed, so the result is reproducible
+  for (int b0 = threadIdx.x; b0 < n_blocks; b0 += 4 * blockDim.x) {
+    float4 lo4[4], hi4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int b = b0 + u * (int)blockDim.x;
+      const int bc = b < n_blocks ? b : b0;  // a valid block; its values are dropped below
+      lo4[u] = *reinterpret_cast<const float4*>(partials + (size_t)bc * kPartialStride);
+      hi4[u] = *reinterpret_cast<const float4*>(partials + (size_t)bc * kPartialStride + 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (b0 + u * (int)blockDim.x >= n_blocks) continue;
+      t[0] += lo4[u].x; t[1] += lo4[u].y; t[2] += lo4[u].z; t[3] += lo4[u].w;
+      t[4] += hi4[u].x; t[5] += hi4[u].y; t[6] += hi4[u].z; t[7] += hi4[u].w;
+    }
   }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -160,6 +172,7 @@ __global__ __launch_bounds__(1024) void loss_row_scale_kernel(
   __shared__ float red[2 * 16];
   __shared__ float tot[2];
   float t[2] = {0.f, 0.f};
+#pragma unroll 8
   for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
     const float c = row_cnt[r];
     t[0] += c;
@@ -180,6 +193,7 @@ __global__ __launch_bounds__(1024) void loss_row_scale_kernel(
   if (valid != nullptr) bden = fmaxf((float)valid[0], 1.f);
   else if (batch_reduce == 0) bden = fmaxf(tot[0], 1.f);
   else bden = fmaxf(tot[1], 1.f);
+#pragma unroll 8
   for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
     const float c = row_cnt[r];
     float td = 1.f;
