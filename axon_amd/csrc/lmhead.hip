@@ -341,18 +341,29 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   // the wave reads back only what it wrote itself; LDS operations of one wave complete in order
   const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
   const int n_base = t.n0 + lp.wn * kWaveTile;
-  // token-major copy: 32 lanes cover one 256-byte row
+  // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
+  // destinations by running pointers (no 64-bit multiplies in the loop).
   {
     const int unit = l32;
-#pragma unroll 4
-    for (int nw = lhi; nw < kWaveTile; nw += 2) {
-      const uint2 v = *reinterpret_cast<const uint2*>(stage + stage_off(nw, unit));
-      *reinterpret_cast<uint2*>(p.dl + (int64_t)(n_base + nw) * p.ld_dl + m_base + unit * 4) = v;
+    char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
+    const int64_t dstep = p.ld_dl * 4;  // two rows of bf16
+#pragma unroll 1
+    for (int nw0 = lhi; nw0 < kWaveTile; nw0 += 16) {
+      uint2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        *reinterpret_cast<uint2*>(d) = v[u];
+        d += dstep;
+      }
     }
   }
   // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
   {
     const int nq = l32;  // token quad
+    const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
+    char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + lhi * 4) * p.ld_dlT + n_base + nq * 4);
 #pragma unroll 2
     for (int unit = lhi; unit < 32; unit += 2) {
       uint2 rws[4];
@@ -369,8 +380,8 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
       o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
       o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        *reinterpret_cast<uint2*>(p.dlT + (int64_t)(m_base + unit * 4 + e) * p.ld_dlT + n_base + nq * 4) = o[e];
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
+      d += 8 * rstep;
     }
   }
 }
