@@ -198,6 +198,49 @@ def test_aligned_packed_layout(n, h, v, lens, cap):
     assert torch.equal(hd.grad, h2.grad) and torch.equal(wd.grad, w2.grad)
 
 
+def test_forward_with_hip_backend_on_a_stub_model():
+    """The model-forward mirror (reference dense_common.py:147-235): body model -> hidden states, rolled labels,
+    fused head, output object; a config with final_logit_softcapping goes through the capped kernels."""
+    import types
+
+    from axon_amd.models.transformers.dense_common import CausalLMOutputForPPO, forward_with_hip_backend
+    n, h, v = 300, 128, 1000
+    hid, w, ids = W.lmhead_inputs(n, h, v, seed=21, label_dtype=torch.int64)
+    w = (w.float() * 8).bfloat16()
+
+    class Body(torch.nn.Module):
+        def forward(self, input_ids=None, **kw):
+            assert kw["use_cache"] is False and "return_dict" in kw
+            return (hid.to(DEV).view(1, n, h),)
+
+    class Model(torch.nn.Module):
+        def __init__(self, cap):
+            super().__init__()
+            self.model = Body()
+            self.lm_head = torch.nn.Linear(h, v, bias=False, dtype=torch.bfloat16, device=DEV)
+            self.lm_head.weight.data.copy_(w)
+            self.config = types.SimpleNamespace(output_attentions=False, output_hidden_states=False,
+                                                final_logit_softcapping=cap)
+
+    for cap in (None, 5.0):
+        model = Model(cap)
+        out = forward_with_hip_backend(model, input_ids=ids.to(DEV).view(1, n), use_cache=False, return_dict=True,
+                                       temperature=0.8)
+        assert isinstance(out, CausalLMOutputForPPO) and out.log_probs.shape == (n,)
+        ref_lp, ref_ent = OM.forward(hid, w, torch.roll(ids, -1), 0.8, softcap=cap)
+        assert (out.log_probs.cpu() - ref_lp).abs().max() < 1e-3 and (out.entropy.cpu() - ref_ent).abs().max() < 1e-3
+        out.log_probs.sum().backward()
+        assert model.lm_head.weight.grad is not None and torch.isfinite(model.lm_head.weight.grad.float()).all()
+        # the caller's pre-rolled labels win over the model's own roll
+        pre = torch.randint(0, v, (1, n)).to(DEV)
+        out2 = forward_with_hip_backend(model, input_ids=ids.to(DEV).view(1, n), use_cache=False, return_dict=True,
+                                        temperature=0.8, pre_rolled_labels=pre)
+        ref2, _ = OM.forward(hid, w, pre.cpu().view(-1), 0.8, softcap=cap)
+        assert (out2.log_probs.detach().cpu() - ref2).abs().max() < 1e-3
+    with pytest.raises(NotImplementedError):
+        forward_with_hip_backend(Model(None), input_ids=ids.to(DEV).view(1, n), use_cache=False, return_dict=False)
+
+
 @pytest.mark.parametrize("chunk", [256, 512, 0])
 def test_backward_vocab_chunks_agree(chunk):
     n, h, v = 300, 128, 1000

@@ -187,3 +187,32 @@ def test_loss_config_validation_before_any_launch():
         agg_loss(x, x, token_reduce="mean", batch_reduce="program-mean", num_program_steps=torch.ones(1))
     with pytest.raises(ValueError, match="Unknown policy loss"):
         compute_loss_fn(data, "nonexistent", {})
+
+
+def test_rolled_label_precedence_and_output_type():
+    """Label choice of the model-forward mirror (reference dense_common.py:187-196) and its output object."""
+    from axon_amd.models.transformers.dense_common import (CausalLMOutputForPPO, final_logit_softcapping,
+                                                            select_rolled_labels)
+    ids = torch.tensor([[5, 6, 7, 8]])
+    labels = torch.tensor([[1, 2, 3, 4]])
+    pre = torch.tensor([[9, 9, 9, 9]])
+    assert select_rolled_labels(pre, labels, ids) is pre
+    assert select_rolled_labels(None, labels, ids).tolist() == [[2, 3, 4, 1]]
+    assert select_rolled_labels(None, None, ids).tolist() == [[6, 7, 8, 5]]
+    with pytest.raises(RuntimeError):
+        select_rolled_labels(None, None, None)
+    out = CausalLMOutputForPPO(log_probs=torch.zeros(3), entropy=torch.ones(3))
+    assert out.log_probs.shape == (3,) and out.entropy.sum() == 3 and out.past_key_values is None
+
+    class Text:
+        final_logit_softcapping = 30.0
+
+    class Multi:
+        def get_text_config(self):
+            return Text()
+
+    class Plain:
+        pass
+
+    assert final_logit_softcapping(Multi()) == 30.0 and final_logit_softcapping(Text()) == 30.0
+    assert final_logit_softcapping(Plain()) is None
