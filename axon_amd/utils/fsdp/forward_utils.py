@@ -72,3 +72,49 @@ def packed_logprobs(hidden, weight, packed_ids, cu_seqlens, temperature: float =
 
     return linear_cross_entropy(hidden, weight, packed_ids.reshape(-1), float(temperature), "none", None,
                                 logit_softcapping, cu_seqlens)
+
+
+def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_entropy: bool = False, *,
+                       use_remove_padding: bool = True, use_fused_kernels: bool = True, ulysses_sp_size: int = 1,
+                       **_unused):
+    """Forward one micro-batch through a model whose ``forward`` is the fused-head one
+    (``forward_with_hip_backend``) and return ``(entropy, log_probs)``, both ``[batch, seq]``: position 0 is 0,
+    position t holds log P(token_t | tokens before it).  Mirror of the fused branches of ``fsdp_model_forward``
+    (forward_utils.py:185-318): with remove-padding the ids are unpadded, rolled over the packed stream and
+    handed to the model as ``pre_rolled_labels`` (:236-265), the packed outputs are scattered back and shifted
+    right (``rmpad_postprocess``, :164-182); without it the outputs are shifted right directly (:282-285).
+    Ulysses sequence parallelism (more than one GPU) and the non-fused logits path are not part of this build."""
+    if not use_fused_kernels:
+        raise NotImplementedError("only the fused-head path (use_fused_kernels=True) is built")
+    if ulysses_sp_size > 1:
+        raise NotImplementedError("Ulysses sequence parallelism needs more than one GPU")
+    input_ids = micro_batch["input_ids"]
+    batch_size, seqlen = input_ids.shape
+    attention_mask = micro_batch["attention_mask"]
+    position_ids = micro_batch["position_ids"]
+    if position_ids.dim() == 3:  # mrope layout (channels first), forward_utils.py:224-225
+        position_ids = position_ids.transpose(0, 1)
+    if use_remove_padding:
+        indices, cu_seqlens, _ = get_unpad_data(attention_mask)
+        if indices.numel() == 0:  # all-zero mask: nothing to predict (forward_utils.py:122-127, 176-177)
+            zeros = torch.zeros(batch_size, seqlen, device=input_ids.device, dtype=torch.float32)
+            return (zeros if calculate_entropy else None), zeros.clone()
+        fwd_ids = input_ids.flatten()[indices].unsqueeze(0)
+        if position_ids.dim() == 3:
+            fwd_pos = position_ids.flatten(1)[:, indices].unsqueeze(1)
+        else:
+            fwd_pos = position_ids.flatten()[indices].unsqueeze(0)
+        output = module(input_ids=fwd_ids, attention_mask=None, position_ids=fwd_pos, use_cache=False,
+                        temperature=temperature, return_dict=True, pre_rolled_labels=rolled_labels(fwd_ids))
+        log_probs = rmpad_postprocess(output.log_probs.reshape(-1), indices=indices, batch_size=batch_size,
+                                      seqlen=seqlen)
+        entropy = None
+        if calculate_entropy:
+            entropy = rmpad_postprocess(output.entropy.reshape(-1), indices=indices, batch_size=batch_size,
+                                        seqlen=seqlen)
+        return entropy, log_probs
+    output = module(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids, use_cache=False,
+                    temperature=temperature, return_dict=True)
+    log_probs = shift_to_token_positions(output.log_probs.view(batch_size, seqlen))
+    entropy = shift_to_token_positions(output.entropy.view(batch_size, seqlen)) if calculate_entropy else None
+    return entropy, log_probs

@@ -241,6 +241,54 @@ def test_forward_with_hip_backend_on_a_stub_model():
         forward_with_hip_backend(Model(None), input_ids=ids.to(DEV).view(1, n), use_cache=False, return_dict=False)
 
 
+@pytest.mark.parametrize("remove_padding", [True, False])
+def test_fsdp_model_forward_mirror(remove_padding):
+    """Padded [B, T] micro-batch -> (entropy, log_probs) [B, T] through the model-forward mirror, against the
+    oracle evaluated row by row (reference forward_utils.py:185-318: position 0 is 0, position t predicts token t)."""
+    import types
+
+    from axon_amd.models.transformers.dense_common import forward_with_hip_backend
+    from axon_amd.utils.fsdp.forward_utils import fsdp_model_forward
+    b, t, h, v = 4, 96, 128, 1000
+    g = torch.Generator().manual_seed(33)
+    lens = [96, 40, 1, 77]
+    ids = torch.randint(0, v, (b, t), generator=g)
+    mask = torch.zeros(b, t, dtype=torch.long)
+    for r, n in enumerate(lens):
+        mask[r, :n] = 1
+    emb = torch.randn(v, h, generator=g).bfloat16()      # the stub body model: an embedding lookup
+    w = (torch.randn(v, h, generator=g) * 0.3).bfloat16()
+
+    class Body(torch.nn.Module):
+        def forward(self, input_ids=None, **kw):
+            return (emb.to(DEV)[input_ids],)
+
+    model = types.SimpleNamespace(
+        model=Body(), lm_head=types.SimpleNamespace(weight=w.to(DEV).requires_grad_(True)),
+        config=types.SimpleNamespace(output_attentions=False, output_hidden_states=False))
+    module = lambda **kw: forward_with_hip_backend(model, **kw)  # noqa: E731
+    mb = {"input_ids": ids.to(DEV), "attention_mask": mask.to(DEV),
+          "position_ids": torch.arange(t).expand(b, t).to(DEV)}
+    ent, lp = fsdp_model_forward(module, mb, 0.9, True, use_remove_padding=remove_padding, use_fused_kernels=True,
+                                 ulysses_sp_size=1)
+    assert lp.shape == (b, t) and ent.shape == (b, t)
+    for r, n in enumerate(lens):
+        assert lp[r, 0].item() == 0 and ent[r, 0].item() == 0
+        if n > 1:
+            ref_lp, ref_ent = OM.forward(emb[ids[r, : n - 1]], w, ids[r, 1:n], 0.9)
+            assert (lp[r, 1:n].detach().cpu() - ref_lp).abs().max() < 1e-3
+            assert (ent[r, 1:n].detach().cpu() - ref_ent).abs().max() < 1e-3
+        if remove_padding:  # slot n holds the last token's (meaningless) prediction, as in the reference
+            assert (lp[r, n + 1:] == 0).all() and (ent[r, n + 1:] == 0).all()
+    (lp * mask.to(DEV)).sum().backward()
+    assert torch.isfinite(model.lm_head.weight.grad.float()).all()
+    zero = dict(mb, attention_mask=torch.zeros_like(mb["attention_mask"]))
+    e0, l0 = fsdp_model_forward(module, zero, 0.9, True, use_remove_padding=True, use_fused_kernels=True)
+    assert (l0 == 0).all() and (e0 == 0).all()
+    with pytest.raises(NotImplementedError):
+        fsdp_model_forward(module, mb, 0.9, use_remove_padding=True, use_fused_kernels=True, ulysses_sp_size=2)
+
+
 @pytest.mark.parametrize("chunk", [256, 512, 0])
 def test_backward_vocab_chunks_agree(chunk):
     n, h, v = 300, 128, 1000
