@@ -26,10 +26,13 @@ SIGNATURES: dict[str, tuple] = {
     "axon_lmhead_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "axon_lmhead_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
+    "axon_timer_create": (_ptr, [_ptr]),
+    "axon_timer_collect": (_i32, [_ptr, _ptr, _ptr]),
+    "axon_timer_destroy": (None, [_ptr]),
     "axon_lmhead_fwd_timed": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr,
-                                     _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr]),
+                                     _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                                     _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr, _ptr]),
+                                     _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_gemm_nt_bf16": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "axon_row_stats": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
                               _ptr, _ptr, _ptr, _ptr]),
@@ -55,7 +58,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

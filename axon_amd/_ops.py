@@ -327,30 +327,49 @@ def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_red
     return acc, agg_w, grad_kl
 
 
-# When set to a dict (benchmarks only), the LM-head autograd function routes through the
-# timed entry points and accumulates per-phase HIP-event times here.
-TIMING: dict | None = None
+# When set (benchmarks only), the LM-head autograd function routes through the timed entry points,
+# which record HIP events around every launch into this timer without synchronising.
+TIMING: "Timer | None" = None
 # vocab chunk of the LM-head backward used when the caller passes 0 (0 = library default)
 DEFAULT_VOCAB_CHUNK = 0
 
+_PHASES = ("fwd/logits_stats", "fwd/merge", "fwd/label", "fwd/unused",
+           "bwd/transpose", "bwd/dlogit", "bwd/dhidden", "bwd/dweight")
 
-def set_timing(timing: dict | None) -> None:
+
+class Timer:
+    """HIP-event timer on the current stream (``axon_timer_*``).  ``collect()`` synchronises the stream and
+    returns ``{phase: {"ms": .., "launches": ..}}`` for everything recorded since the previous collect."""
+
+    def __init__(self):
+        self._lib = _lib.load()
+        self.stream = stream_ptr()
+        self.handle = self._lib.axon_timer_create(self.stream)
+        if not self.handle:
+            raise _lib.AxonAmdError("axon_timer_create failed")
+
+    def collect(self) -> dict:
+        import ctypes
+
+        ms, cnt = (ctypes.c_float * 8)(), (ctypes.c_int32 * 8)()
+        check(self._lib.axon_timer_collect(self.handle, ms, cnt), "axon_timer_collect")
+        return {name: {"ms": float(ms[i]), "launches": int(cnt[i])} for i, name in enumerate(_PHASES) if cnt[i]}
+
+    def close(self):
+        if self.handle:
+            self._lib.axon_timer_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def set_timing(timer: "Timer | None") -> None:
     global TIMING
-    TIMING = timing
-
-
-def _phase_arrays():
-    import ctypes
-
-    return (ctypes.c_float * 4)(), (ctypes.c_int32 * 4)()
-
-
-def _add_phases(timing: dict, prefix: str, names, ms, launches):
-    for i, name in enumerate(names):
-        key = f"{prefix}/{name}"
-        t = timing.setdefault(key, {"ms": 0.0, "launches": 0})
-        t["ms"] += float(ms[i])
-        t["launches"] += int(launches[i])
+    TIMING = timer
 
 
 def seq_start_flags(cu_seqlens, n_tokens: int):
@@ -364,14 +383,14 @@ def seq_start_flags(cu_seqlens, n_tokens: int):
     return flags
 
 
-def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None = None, softcap: float = 0.0,
+def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | None" = None, softcap: float = 0.0,
                    seq_start=None):
     """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]).  ``softcap`` > 0 soft-caps the logits
     (cap * tanh(logit / cap)) before the temperature.  With ``seq_start`` (``seq_start_flags``) ``labels`` is
     the packed id stream and logprobs / entropy come back aligned to token positions.
 
-    With ``timing`` (a dict) the timed entry point is used: it synchronises and adds
-    per-phase HIP-event milliseconds and launch counts under ``fwd/...`` keys."""
+    With ``timing`` (a ``Timer``) the timed entry point is used: it records HIP events around every launch
+    into the timer and does not synchronise."""
     lib = _lib.load()
     require_device(hidden, "lmhead_forward")
     n, h = hidden.shape
@@ -388,14 +407,12 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: dict | None 
     if timing is None:
         check(lib.axon_lmhead_fwd(*args), "axon_lmhead_fwd")
     else:
-        ms, cnt = _phase_arrays()
-        check(lib.axon_lmhead_fwd_timed(*args, ms, cnt), "axon_lmhead_fwd_timed")
-        _add_phases(timing, "fwd", ("logits_stats", "merge", "label"), ms, cnt)
+        check(lib.axon_lmhead_fwd_timed(*args, timing.handle), "axon_lmhead_fwd_timed")
     return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
 
 
 def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
-                    timing: dict | None = None, softcap: float = 0.0, seq_start=None):
+                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None):
     """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``)."""
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
     lib = _lib.load()
@@ -417,9 +434,7 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     if timing is None:
         check(lib.axon_lmhead_bwd(*args), "axon_lmhead_bwd")
     else:
-        ms, cnt = _phase_arrays()
-        check(lib.axon_lmhead_bwd_timed(*args, ms, cnt), "axon_lmhead_bwd_timed")
-        _add_phases(timing, "bwd", ("transpose", "dlogit", "dhidden", "dweight"), ms, cnt)
+        check(lib.axon_lmhead_bwd_timed(*args, timing.handle), "axon_lmhead_bwd_timed")
     return d_hidden, d_weight
 
 

@@ -13,6 +13,7 @@
 // run on the same K-contiguous main loops (gemm_nt.h).
 #include "common.h"
 #include "gemm_nt.h"
+#include <vector>
 
 namespace axon {
 
@@ -578,44 +579,44 @@ BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
   return w;
 }
 
-// Optional per-phase timing with HIP events on the launch stream (used by the
-// *_timed entry points only).  A null timer costs nothing.
+// Optional per-phase timing with HIP events on the launch stream (used by the *_timed entry points
+// only).  Recording does not synchronise: the events are read when the caller collects them.  A
+// null timer costs nothing.
 struct PhaseTimer {
-  static constexpr int kMaxSpans = 256;
+  struct Rec { hipEvent_t a, b; int phase; };
   hipStream_t st;
-  hipEvent_t ev[kMaxSpans][2];
-  int phase[kMaxSpans];
-  int n = 0;
+  std::vector<Rec> recs;
+  Rec cur{};
   bool open = false;
+  int base = 0;  // added to the phase ids of the spans being recorded (0 forward, 4 backward)
   explicit PhaseTimer(hipStream_t s) : st(s) {}
   void begin(int ph) {
-    if (n >= kMaxSpans) return;
-    if (hipEventCreate(&ev[n][0]) != hipSuccess) return;
-    if (hipEventCreate(&ev[n][1]) != hipSuccess) { (void)hipEventDestroy(ev[n][0]); return; }
-    phase[n] = ph;
-    (void)hipEventRecord(ev[n][0], st);
+    if (hipEventCreate(&cur.a) != hipSuccess) return;
+    if (hipEventCreate(&cur.b) != hipSuccess) { (void)hipEventDestroy(cur.a); return; }
+    cur.phase = base + ph;
+    (void)hipEventRecord(cur.a, st);
     open = true;
   }
   void end() {
     if (!open) return;
-    (void)hipEventRecord(ev[n][1], st);
-    ++n;
+    (void)hipEventRecord(cur.b, st);
+    recs.push_back(cur);
     open = false;
   }
-  // synchronises the stream; adds elapsed ms and launch counts per phase
+  // synchronises the stream; adds elapsed ms and launch counts per phase, forgets the spans
   void collect(float* ms, int32_t* launches, int n_phases) {
     (void)hipStreamSynchronize(st);
-    for (int i = 0; i < n; ++i) {
+    for (const Rec& r : recs) {
       float t = 0.f;
-      (void)hipEventElapsedTime(&t, ev[i][0], ev[i][1]);
-      if (phase[i] < n_phases) {
-        ms[phase[i]] += t;
-        launches[phase[i]] += 1;
+      (void)hipEventElapsedTime(&t, r.a, r.b);
+      if (r.phase < n_phases) {
+        ms[r.phase] += t;
+        launches[r.phase] += 1;
       }
-      (void)hipEventDestroy(ev[i][0]);
-      (void)hipEventDestroy(ev[i][1]);
+      (void)hipEventDestroy(r.a);
+      (void)hipEventDestroy(r.b);
     }
-    n = 0;
+    recs.clear();
   }
 };
 struct Span {  // RAII: one timed span around the launches in scope
@@ -835,19 +836,34 @@ extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const voi
                   logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stream, nullptr);
 }
 
+extern "C" void* axon_timer_create(void* stream) { return new (std::nothrow) PhaseTimer((hipStream_t)stream); }
+
+extern "C" int axon_timer_collect(void* timer, float* phase_ms, int32_t* phase_launches) {
+  if (!timer || !phase_ms || !phase_launches) return AXON_ERR_ARG;
+  static_cast<PhaseTimer*>(timer)->collect(phase_ms, phase_launches, 8);
+  return AXON_OK;
+}
+
+extern "C" void axon_timer_destroy(void* timer) {
+  if (!timer) return;
+  float ms[8] = {0};
+  int32_t n[8] = {0};
+  static_cast<PhaseTimer*>(timer)->collect(ms, n, 8);  // releases the events
+  delete static_cast<PhaseTimer*>(timer);
+}
+
 extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, const void* labels,
                                      int labels_i64, int64_t n, int64_t h, int64_t v,
                                      float inv_temp, float softcap, const uint8_t* seq_start,
                                      float* logprobs, float* entropy, float* lse,
                                      float* entropy_b, void* workspace, int64_t ws_bytes,
-                                     void* stream, float* phase_ms, int32_t* phase_launches) {
-  if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
-  PhaseTimer timer((hipStream_t)stream);
-  const int rc = fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap,
-                          seq_start, logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stream,
-                          &timer);
-  timer.collect(phase_ms, phase_launches, 4);
-  return rc;
+                                     void* stream, void* timer) {
+  if (!timer) return AXON_ERR_ARG;
+  PhaseTimer* t = static_cast<PhaseTimer*>(timer);
+  if (t->st != (hipStream_t)stream) return AXON_ERR_ARG;
+  t->base = 0;
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, logprobs,
+                  entropy, lse, entropy_b, workspace, ws_bytes, stream, t);
 }
 
 extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t v,
@@ -874,15 +890,14 @@ extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentro
                                      int64_t n, int64_t h, int64_t v, float inv_temp,
                                      float softcap, const uint8_t* seq_start, void* d_hidden,
                                      void* d_weight, int64_t chunk, void* workspace,
-                                     int64_t ws_bytes, void* stream, float* phase_ms,
-                                     int32_t* phase_launches) {
-  if (!phase_ms || !phase_launches) return AXON_ERR_ARG;
-  PhaseTimer timer((hipStream_t)stream);
-  const int rc = bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n,
-                          h, v, inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace,
-                          ws_bytes, stream, &timer);
-  timer.collect(phase_ms, phase_launches, 4);
-  return rc;
+                                     int64_t ws_bytes, void* stream, void* timer) {
+  if (!timer) return AXON_ERR_ARG;
+  PhaseTimer* t = static_cast<PhaseTimer*>(timer);
+  if (t->st != (hipStream_t)stream) return AXON_ERR_ARG;
+  t->base = 4;
+  return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
+                  inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes, stream,
+                  t);
 }
 
 extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, float* out,

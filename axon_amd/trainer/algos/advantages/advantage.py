@@ -35,10 +35,13 @@ def _group_advantage(data, mode: int, eps: float, clamp_abs: float):
 
     cu = data.meta_info.get("cu_seqlens", None) if data.meta_info else None
     rows = _ops.rows_of(rewards, cu)
-    gidx = as_torch_index(uid, device=rewards.device)
-    if gidx.numel() != rows.n_rows:
-        raise ValueError(f"uid has {gidx.numel()} entries, batch has {rows.n_rows} rows")
-    n_groups = int(gidx.max().item()) + 1 if gidx.numel() else 0
+    # group ids are ranked on the host (labels are strings); the group count is read there as well, so
+    # that nothing here waits for the GPU
+    gidx_host = as_torch_index(uid, device="cpu")
+    if gidx_host.numel() != rows.n_rows:
+        raise ValueError(f"uid has {gidx_host.numel()} entries, batch has {rows.n_rows} rows")
+    n_groups = int(gidx_host.max()) + 1 if gidx_host.numel() else 0
+    gidx = gidx_host.to(rewards.device, non_blocking=True)
     _, scores, _ = _ops.row_stats(rewards, None, None, rows, want_cnt=False)
     _, _, _, scalar = _ops.group_stats(scores, gidx, n_groups, eps, norm)
     adv = _ops.row_broadcast_mask(scalar, mask, rows, clamp_abs=clamp_abs)

@@ -244,14 +244,16 @@ def main():
         step()
     torch.cuda.synchronize()
 
-    timing: dict = {}
-    _ops.set_timing(timing)  # HIP events around every LM-head launch, on the launch stream
+    timer = _ops.Timer()
+    _ops.set_timing(timer)  # HIP events around every LM-head launch, on the launch stream, no synchronisation
     t0 = time.perf_counter()
     for _ in range(args.steps):
         loss, dh, dw = step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     _ops.set_timing(None)
+    timing = timer.collect()  # events of the timed region, read after it has ended
+    timer.close()
     assert torch.isfinite(loss).item() and torch.isfinite(dh.float()).all().item()
 
     ms_per_step = 1e3 * elapsed / args.steps

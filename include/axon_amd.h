@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 7
+#define AXON_AMD_ABI_VERSION 8
 
 enum {
   AXON_OK = 0,
@@ -110,25 +110,30 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
                     int64_t vocab_chunk, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Timed variants for benchmarks: same work, plus HIP events recorded on `stream`
- * around every launch.  They SYNCHRONISE the stream before returning and create
- * and destroy events (the exception to "never synchronises").  phase_ms[4] and
- * phase_launches[4] are HOST arrays that are added to (zero them first):
- *   forward : [0] logits+statistics kernel, [1] merge, [2] label logit
- *   backward: [0] transposes, [1] dlogit recompute, [2] dHidden GEMM, [3] dWeight GEMM
+ * around every launch into a timer object.  Recording does not synchronise;
+ * axon_timer_collect synchronises the timer's stream, ADDS the elapsed milliseconds
+ * and launch counts of everything recorded since the last collect to the two HOST
+ * arrays of 8 entries (zero them first) and forgets the spans:
+ *   [0] forward logits+statistics kernel, [1] merge, [2] label logit, [3] unused,
+ *   [4] backward transposes, [5] dlogit recompute, [6] dHidden GEMM, [7] dWeight GEMM.
+ * The timer creates and destroys events and owns host memory (the exception to
+ * "never allocates"); `stream` of a timed call must be the timer's.
  * No reference counterpart (measurement only). */
+void* axon_timer_create(void* stream); /* NULL on failure */
+int axon_timer_collect(void* timer, float* phase_ms, int32_t* phase_launches);
+void axon_timer_destroy(void* timer);
 int axon_lmhead_fwd_timed(const void* hidden_bf16, const void* weight_bf16, const void* labels,
                           int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
                           float inv_temperature, float softcap, const uint8_t* seq_start,
-                          float* logprobs, float* entropy, float* lse, float* entropy_b, void* workspace, int64_t workspace_bytes,
-                          void* stream, float* phase_ms, int32_t* phase_launches);
+                          float* logprobs, float* entropy, float* lse, float* entropy_b,
+                          void* workspace, int64_t workspace_bytes, void* stream, void* timer);
 int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                           const void* weight_bf16, const void* labels, int labels_are_i64,
                           const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
                           int64_t vocab, float inv_temperature, float softcap,
                           const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
                           int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
-                          void* stream, float* phase_ms,
-                          int32_t* phase_launches);
+                          void* stream, void* timer);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
  * (fp32 accumulate, fp32 output).  No reference counterpart: it exists so tests
