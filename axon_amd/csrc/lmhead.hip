@@ -453,23 +453,46 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g
 }
 
 // out[c][r] = in[r][c] for r < rows, c < cols; zero for r in [rows, rows_pad).
-// 64x64 tiles through LDS.
+// 64x64 tiles through LDS; both sides move 16 bytes per thread and access (two per thread each
+// way) where the tile is whole, element by element at the ragged edges.  ld_in and ld_out are
+// multiples of 8 elements and both bases 16-byte aligned (checked by the launcher).
 __global__ __launch_bounds__(256) void transpose_bf16_kernel(const uint16_t* __restrict__ in,
                                                              int64_t ld_in, int rows, int cols,
                                                              uint16_t* __restrict__ out,
                                                              int64_t ld_out, int rows_pad) {
-  __shared__ uint16_t t[64][66];
+  __shared__ uint16_t t[64][66 + 6];  // 144-byte rows: 16-byte row writes stay aligned
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
-    const int r = i >> 6, c = i & 63;
-    uint16_t v = 0;
-    if (r0 + r < rows && c0 + c < cols) v = in[(int64_t)(r0 + r) * ld_in + c0 + c];
-    t[r][c] = v;
+#pragma unroll
+  for (int q = threadIdx.x; q < 512; q += 256) {
+    const int r = q >> 3, c = (q & 7) * 8;
+    union { uint4 v; uint16_t h[8]; } u;
+    u.v = make_uint4(0, 0, 0, 0);
+    if (r0 + r < rows) {
+      const uint16_t* src = in + (int64_t)(r0 + r) * ld_in + c0 + c;
+      if (c0 + c + 8 <= cols) {
+        u.v = *reinterpret_cast<const uint4*>(src);
+      } else {
+        for (int e = 0; e < 8; ++e)
+          if (c0 + c + e < cols) u.h[e] = src[e];
+      }
+    }
+    *reinterpret_cast<uint4*>(&t[r][c]) = u.v;
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < 64 * 64; i += 256) {
-    const int c = i >> 6, r = i & 63;
-    if (c0 + c < cols && r0 + r < rows_pad) out[(int64_t)(c0 + c) * ld_out + r0 + r] = t[r][c];
+#pragma unroll
+  for (int q = threadIdx.x; q < 512; q += 256) {
+    const int c = q >> 3, r = (q & 7) * 8;
+    if (c0 + c >= cols || r0 + r >= rows_pad) continue;
+    union { uint4 v; uint16_t h[8]; } u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) u.h[e] = t[r + e][c];
+    uint16_t* dst = out + (int64_t)(c0 + c) * ld_out + r0 + r;
+    if (r0 + r + 8 <= rows_pad) {
+      *reinterpret_cast<uint4*>(dst) = u.v;
+    } else {
+      for (int e = 0; e < 8; ++e)
+        if (r0 + r + e < rows_pad) dst[e] = u.h[e];
+    }
   }
 }
 
@@ -639,6 +662,9 @@ int launch_store(const GemmOperands& g, const StoreParams& sp, hipStream_t st) {
 
 int launch_transpose(const void* in, int64_t ld_in, int rows, int cols, void* out, int64_t ld_out,
                      int rows_pad, hipStream_t st) {
+  if ((ld_in | ld_out) % 8 != 0 ||
+      ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15))
+    return AXON_ERR_ARG;
   const dim3 grid((rows_pad + 63) / 64, (cols + 63) / 64);
   hipLaunchKernelGGL(transpose_bf16_kernel, grid, dim3(256), 0, st,
                      static_cast<const uint16_t*>(in), ld_in, rows, cols,
