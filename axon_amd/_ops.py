@@ -122,6 +122,76 @@ def row_broadcast_mask(row_scalar, mask, rows: Rows, clamp_abs=0.0):
     return out
 
 
+SCAN_GAE, SCAN_GAE_RESPONSE_ONLY, SCAN_DISCOUNTED, SCAN_SUFFIX_SUM = 0, 1, 2, 3
+
+
+def reverse_scan(mode, rewards, values, mask, rows: Rows, *, gamma=1.0, lam=1.0, row_baseline=None):
+    """Time recurrence from each row's last token to its first; returns ``(adv | None, ret)``.  See
+    axon_reverse_scan."""
+    lib = _lib.load()
+    require_device(rewards, "reverse_scan")
+    dev = rewards.device
+    rewards = f32(rewards)
+    values = f32(values) if values is not None else None
+    mk, kind = mask_arg(mask)
+    base = f32(row_baseline).reshape(-1) if row_baseline is not None else None
+    if base is not None and base.numel() != rows.n_rows:
+        raise ValueError(f"row_baseline has {base.numel()} entries, batch has {rows.n_rows} rows")
+    adv = None if mode == SCAN_DISCOUNTED else torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    ret = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    check(
+        lib.axon_reverse_scan(mode, ptr(rewards), ptr(values), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                              rows.uniform_len, float(gamma), float(lam), ptr(base), ptr(adv), ptr(ret),
+                              stream_ptr()),
+        "axon_reverse_scan",
+    )
+    return adv, ret
+
+
+def masked_whiten(x, mask, *, remask=False, inplace=False):
+    """``(x - mean) * rsqrt(var + 1e-8)`` with the mean and variance taken over the mask (times the mask when
+    ``remask``); returns ``(out, stats)`` with stats = device [mean, n, var, rsqrt(var + 1e-8)]."""
+    lib = _lib.load()
+    require_device(x, "masked_whiten")
+    dev = x.device
+    xf = f32(x)
+    mk, kind = mask_arg(mask)
+    n = int(xf.numel())
+    out = xf if (inplace and xf.data_ptr() == x.data_ptr()) else torch.empty_like(xf)
+    stats = _zeros(4, dev)
+    ws = torch.empty(max(lib.axon_masked_whiten_workspace_bytes(n) // 4, 8), device=dev, dtype=torch.float32)
+    check(
+        lib.axon_masked_whiten(ptr(xf), ptr(mk), kind, n, int(remask), ptr(out), ptr(stats), ptr(ws), stream_ptr()),
+        "axon_masked_whiten",
+    )
+    return out, stats
+
+
+GROUP_OPO, GROUP_MEAN_BASELINE, GROUP_PASSK, GROUP_KIMI = 0, 1, 2, 3
+
+
+def group_scalar(mode, scores, lens, members, offsets, n_groups, *, eps=1e-6, normalize=True, coef=0.0,
+                 threshold=1.0):
+    """Per-row scalar from group members in compressed form; see axon_group_scalar."""
+    lib = _lib.load()
+    require_device(scores, "group_scalar")
+    dev = scores.device
+    scores = f32(scores).reshape(-1)
+    lens = f32(lens).reshape(-1) if lens is not None else None
+    members = members.to(device=dev, dtype=torch.int32).contiguous()
+    offsets = offsets.to(device=dev, dtype=torch.int32).contiguous()
+    n = int(scores.numel())
+    if members.numel() != n or offsets.numel() != n_groups + 1:
+        raise ValueError("members / offsets do not describe the rows of scores")
+    out = torch.empty(n, device=dev, dtype=torch.float32)
+    check(
+        lib.axon_group_scalar(mode, ptr(scores), ptr(lens), ptr(members), ptr(offsets), n, int(n_groups), float(eps),
+                              int(bool(normalize)), float(coef), float(threshold), ptr(out), stream_ptr()),
+        "axon_group_scalar",
+    )
+    return out
+
+
 IS_MODES = {None: 0, "token": 1, "sequence": 2}
 RS_MODES = {None: 0, "token": 1, "sequence": 2, "geometric": 3}
 

@@ -274,6 +274,22 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
         gv[j] = -rc * A * tm * m * scale;
         continue;
       }
+      if (KIND == 4) {  // clipped value loss (loss.py:547-591): logp = vpreds, oldp = values, adv = returns,
+                        // lo = cliprange_value; the caller applies the factor 0.5
+        const float vp = lv[j], up = ov[j] + lo, dn = ov[j] - lo;
+        // clip_by_value = maximum(minimum(vp, up), dn) with tensor bounds (loss/utils.py:94-101)
+        const float g_min = (vp < up) ? 1.f : ((vp == up) ? 0.5f : 0.f);
+        const float y = fminf(vp, up);
+        const float g_clip = (y > dn) ? g_min : ((y == dn) ? 0.5f * g_min : 0.f);
+        const float vc = fmaxf(y, dn);
+        const float e1 = vp - A, e2 = vc - A;
+        const ValGrad c = vg_max(ValGrad{e1 * e1, 2.f * e1}, ValGrad{e2 * e2, 2.f * e2 * g_clip});
+        a[1] += (e2 * e2 > e1 * e1) ? m : 0.f;
+        a[2] += vp * m;
+        a[0] += c.v * m * scale;
+        gv[j] = c.g * m * scale;
+        continue;
+      }
       float x;  // exponent before the +-20 clamp
       if (KIND == 0) x = d;
       else x = (lv[j] - lv[j]) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
@@ -720,7 +736,7 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
   int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
   if (rc != AXON_OK) return rc;
   if (n_slots == 0) return AXON_OK;
-  if (kind < 0 || kind > 3) return AXON_ERR_ARG;
+  if (kind < 0 || kind > 4) return AXON_ERR_ARG;
   if (!logp || !oldp || !adv || !mask || !grad || !acc || !partials) return AXON_ERR_ARG;
   if (post_normalize && (row_scale != nullptr || kind == 1)) return AXON_ERR_ARG;
   if (kind == 1 && !row_mean) return AXON_ERR_ARG;
@@ -735,12 +751,14 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0);
     else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_F32, 1);
     else if (kind == 2) AXON_LAUNCH_PL(AXON_MASK_F32, 2);
-    else AXON_LAUNCH_PL(AXON_MASK_F32, 3);
+    else if (kind == 3) AXON_LAUNCH_PL(AXON_MASK_F32, 3);
+    else AXON_LAUNCH_PL(AXON_MASK_F32, 4);
   } else {
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_I64, 0);
     else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_I64, 1);
     else if (kind == 2) AXON_LAUNCH_PL(AXON_MASK_I64, 2);
-    else AXON_LAUNCH_PL(AXON_MASK_I64, 3);
+    else if (kind == 3) AXON_LAUNCH_PL(AXON_MASK_I64, 3);
+    else AXON_LAUNCH_PL(AXON_MASK_I64, 4);
   }
 #undef AXON_LAUNCH_PL
   AXON_CHECK_LAUNCH();

@@ -1,0 +1,428 @@
+// Return-based advantage estimators: time recurrences that run from a row's last token to its first,
+// global masked whitening, and the per-group scalars of the estimators that need more than mean/std.
+//
+// A recurrence y[t] = b[t] + a[t] * y[t+1] is a scan over pairs (a, b) under the composition
+// (a2, b2) o (a1, b1) = (a2*a1, b2 + a2*b1).  One wavefront owns one row and walks it from the end in
+// blocks of 256 tokens (four sub-blocks of one token per lane, lane 0 holding the last token), scans each
+// sub-block with shuffles and carries the boundary value from sub-block to sub-block.  The loads of the next
+// block are issued before the current one is scanned.
+#include "common.h"
+
+namespace axon {
+
+constexpr int kScanSub = 4;                      // sub-blocks per step
+constexpr int kScanStep = kScanSub * kWave;      // tokens per step
+
+struct Pair { float a, b; };
+
+// inclusive scan over lanes 0..63: lane l ends with the composition of the elements of lanes 0..l
+__device__ __forceinline__ Pair wave_scan(Pair p) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const float ap = __shfl_up(p.a, d, kWave);
+    const float bp = __shfl_up(p.b, d, kWave);
+    if (lane >= d) {
+      p.b = p.b + p.a * bp;
+      p.a = p.a * ap;
+    }
+  }
+  return p;
+}
+
+// value of the previous lane (the token after this one); lane 0 takes `carry`
+__device__ __forceinline__ float from_next_token(float incl, float carry) {
+  const float up = __shfl_up(incl, 1, kWave);
+  return (threadIdx.x & (kWave - 1)) == 0 ? carry : up;
+}
+
+enum { kScanGae = 0, kScanGaeResponseOnly = 1, kScanDiscounted = 2, kScanSuffixSum = 3 };
+
+struct ScanBlock {
+  float r[kScanSub], v[kScanSub], m[kScanSub];
+};
+
+template <int MK, int MODE>
+__device__ __forceinline__ void scan_load(ScanBlock& x, const float* __restrict__ rewards,
+                                          const float* __restrict__ values,
+                                          const void* __restrict__ mask, int64_t begin, int64_t end) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int u = 0; u < kScanSub; ++u) {
+    const int64_t p = end - 1 - (u * kWave + lane);
+    const bool ok = p >= begin;
+    x.r[u] = ok ? rewards[p] : 0.f;
+    x.v[u] = (ok && MODE <= kScanGaeResponseOnly) ? values[p] : 0.f;
+    x.m[u] = ok ? load_mask1<MK>(mask, p) : 0.f;
+    if (MODE == kScanGaeResponseOnly) x.m[u] = x.m[u] > 0.f ? 1.f : 0.f;
+  }
+}
+
+// MODE kScanGae:  nv[t] = m v + (1-m) nv[t+1];  delta = r + gamma nv[t+1] - v;
+//                 L[t] = m (delta + gamma*lam L[t+1]) + (1-m) L[t+1];  adv = L, ret = L + v.
+// MODE kScanGaeResponseOnly: the same over the tokens with mask > 0, 0 elsewhere.
+// MODE kScanDiscounted: Q[t] = m (r + gamma Q[t+1]);  ret = r + gamma Q[t+1].
+// MODE kScanSuffixSum:  ret[t] = sum_{s >= t} r m;  adv = ret - row_baseline * m.
+template <int MK, int MODE>
+__global__ __launch_bounds__(kBlock) void reverse_scan_kernel(
+    const float* __restrict__ rewards, const float* __restrict__ values,
+    const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows,
+    int64_t uniform_len, float gamma, float gamma_lam, const float* __restrict__ row_baseline,
+    float* __restrict__ adv, float* __restrict__ ret) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
+  if (row >= n_rows) return;  // whole wavefronts leave together; no workgroup barrier below
+  const int64_t begin = uniform_len > 0 ? row * uniform_len : (int64_t)cu[row];
+  const int64_t stop = uniform_len > 0 ? begin + uniform_len : (int64_t)cu[row + 1];
+  const float base = (MODE == kScanSuffixSum && row_baseline) ? row_baseline[row] : 0.f;
+  float carry0 = 0.f, carry1 = 0.f;  // the recurrences' values at the token after the current block
+  if (stop <= begin) return;
+  ScanBlock cur, nxt;
+  scan_load<MK, MODE>(cur, rewards, values, mask, begin, stop);
+  for (int64_t end = stop; end > begin; end -= kScanStep) {
+    const bool more = end - kScanStep > begin;
+    if (more) scan_load<MK, MODE>(nxt, rewards, values, mask, begin, end - kScanStep);
+    float out_adv[kScanSub], out_ret[kScanSub];
+    if (MODE <= kScanGaeResponseOnly) {
+      Pair s1[kScanSub];
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) s1[u] = wave_scan(Pair{1.f - cur.m[u], cur.m[u] * cur.v[u]});
+      Pair e2[kScanSub];
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) {
+        const float nv = s1[u].b + s1[u].a * carry0;
+        const float nv_next = from_next_token(nv, carry0);
+        carry0 = __shfl(nv, kWave - 1, kWave);
+        const float delta = cur.r[u] + gamma * nv_next - cur.v[u];
+        e2[u] = Pair{cur.m[u] * gamma_lam + (1.f - cur.m[u]), cur.m[u] * delta};
+      }
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) e2[u] = wave_scan(e2[u]);
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) {
+        const float l = e2[u].b + e2[u].a * carry1;
+        carry1 = __shfl(l, kWave - 1, kWave);
+        const bool keep = (MODE == kScanGae) || cur.m[u] > 0.f;
+        out_adv[u] = keep ? l : 0.f;
+        out_ret[u] = keep ? l + cur.v[u] : 0.f;
+      }
+    } else if (MODE == kScanDiscounted) {
+      Pair s[kScanSub];
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) s[u] = wave_scan(Pair{gamma * cur.m[u], cur.m[u] * cur.r[u]});
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) {
+        const float q = s[u].b + s[u].a * carry0;
+        const float q_next = from_next_token(q, carry0);
+        carry0 = __shfl(q, kWave - 1, kWave);
+        out_ret[u] = cur.r[u] + gamma * q_next;
+        out_adv[u] = 0.f;
+      }
+    } else {
+      Pair s[kScanSub];
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) s[u] = wave_scan(Pair{1.f, cur.r[u] * cur.m[u]});
+#pragma unroll
+      for (int u = 0; u < kScanSub; ++u) {
+        const float c = s[u].b + carry0;
+        carry0 = __shfl(c, kWave - 1, kWave);
+        out_ret[u] = c;
+        out_adv[u] = c - base * cur.m[u];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kScanSub; ++u) {
+      const int64_t p = end - 1 - (u * kWave + lane);
+      if (p >= begin) {
+        if (adv != nullptr) adv[p] = out_adv[u];
+        ret[p] = out_ret[u];
+      }
+    }
+    if (more) cur = nxt;
+  }
+}
+
+// ---- masked whitening -------------------------------------------------------------------------
+// stats[0] mean, [1] n, [2] variance (times n/(n-1) when n > 1), [3] rsqrt(variance + 1e-8)
+
+// PASS 0: sum m x, sum m.   PASS 1: sum m (x - mean)^2.
+template <int MK, int PASS>
+__global__ __launch_bounds__(kBlock) void masked_moments_kernel(const float* __restrict__ x,
+                                                                const void* __restrict__ mask,
+                                                                int64_t n_slots,
+                                                                const float* __restrict__ stats,
+                                                                float* partials) {
+  __shared__ float lds_red[2 * (kBlock / kWave)];
+  const float mean = PASS == 1 ? stats[0] : 0.f;
+  float a[2] = {0.f, 0.f};
+  const int64_t n_vec = n_slots / kVec;
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n_vec;
+       q += (int64_t)gridDim.x * kBlock) {
+    float xv[4], mv[4];
+    load4(x, q * kVec, xv);
+    load_mask4<MK>(mask, q * kVec, mv);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (PASS == 0) {
+        a[0] += (mv[j] != 0.f) ? xv[j] * mv[j] : 0.f;
+        a[1] += mv[j];
+      } else {
+        const float d = xv[j] - mean;
+        a[0] += (mv[j] != 0.f) ? d * d * mv[j] : 0.f;
+      }
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n_slots - n_vec * kVec)) {  // the ragged tail
+    const int64_t p = n_vec * kVec + threadIdx.x;
+    const float xv = x[p], m = load_mask1<MK>(mask, p);
+    if (PASS == 0) {
+      a[0] += (m != 0.f) ? xv * m : 0.f;
+      a[1] += m;
+    } else {
+      const float d = xv - mean;
+      a[0] += (m != 0.f) ? d * d * m : 0.f;
+    }
+  }
+  store_block_partials<2>(a, lds_red, partials);
+}
+
+// one workgroup adds the partials in a fixed order and finishes the statistics
+__global__ __launch_bounds__(kBlock) void masked_moments_finish_kernel(const float* __restrict__ partials,
+                                                                       int n_blocks, int pass,
+                                                                       float* __restrict__ stats) {
+  __shared__ float lds_red[2 * (kBlock / kWave)];
+  float a[2] = {0.f, 0.f};
+  for (int b = threadIdx.x; b < n_blocks; b += kBlock) {
+    a[0] += partials[(size_t)b * kPartialStride];
+    a[1] += partials[(size_t)b * kPartialStride + 1];
+  }
+  block_sum<2>(a, lds_red);
+  if (threadIdx.x == 0) {
+    if (pass == 0) {
+      stats[0] = a[0] / fmaxf(a[1], 1.f);
+      stats[1] = a[1];
+    } else {
+      const float n = stats[1];
+      float var = a[0] / fmaxf(n, 1.f);
+      if (n > 1.f) var = var * n / (n - 1.f);
+      stats[2] = var;
+      stats[3] = rsqrtf(var + 1e-8f);
+    }
+  }
+}
+
+template <int MK>
+__global__ __launch_bounds__(kBlock) void whiten_kernel(const float* __restrict__ x,
+                                                        const void* __restrict__ mask,
+                                                        int64_t n_slots,
+                                                        const float* __restrict__ stats, int remask,
+                                                        float* __restrict__ out) {
+  const float mean = stats[0], rstd = stats[3];
+  const int64_t n_vec = n_slots / kVec;
+  for (int64_t q = (int64_t)blockIdx.x * kBlock + threadIdx.x; q < n_vec;
+       q += (int64_t)gridDim.x * kBlock) {
+    float xv[4], mv[4] = {1.f, 1.f, 1.f, 1.f}, o[4];
+    load4(x, q * kVec, xv);
+    if (remask) load_mask4<MK>(mask, q * kVec, mv);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = (xv[j] - mean) * rstd * mv[j];
+    store4(out, q * kVec, o);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < (int)(n_slots - n_vec * kVec)) {
+    const int64_t p = n_vec * kVec + threadIdx.x;
+    const float m = remask ? load_mask1<MK>(mask, p) : 1.f;
+    out[p] = (x[p] - mean) * rstd * m;
+  }
+}
+
+// ---- per-group scalars --------------------------------------------------------------------------
+// One thread per group walks the group's rows in row order (members[offsets[g] .. offsets[g+1])), so sums
+// are formed in a fixed order without atomics.
+//   mode 0 (OPO): s - (n > 1 ? sum(len s) / max(sum len, 1) : 0)
+//   mode 1 (REINFORCE++ baseline): s - (n > 1 ? sum s / n : 0)
+//   mode 2 (pass@k): best row gets max - second max, divided by (unbiased std + eps) when p_norm; others 0
+//   mode 3 (Kimi k1.5): s' = s + coef-scaled length term, then the group-normalised scalar of s'
+__global__ __launch_bounds__(kBlock) void group_scalar_kernel(
+    int mode, const float* __restrict__ scores, const float* __restrict__ lens,
+    const int32_t* __restrict__ members, const int32_t* __restrict__ offsets, int64_t n_groups,
+    float eps, int p_norm, float coef, float threshold, float* __restrict__ out) {
+  const int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (g >= n_groups) return;
+  const int lo = offsets[g], hi = offsets[g + 1];
+  const float n = (float)(hi - lo);
+  if (mode == 0 || mode == 1) {
+    float s1 = 0.f, w1 = 0.f, l1 = 0.f;
+    for (int k = lo; k < hi; ++k) {
+      const int i = members[k];
+      const float s = scores[i];
+      s1 += s;
+      if (mode == 0) { w1 += lens[i] * s; l1 += lens[i]; }
+    }
+    float base = 0.f;
+    if (n > 1.f) base = (mode == 0) ? w1 / fmaxf(l1, 1.f) : s1 / fmaxf(n, 1.f);
+    for (int k = lo; k < hi; ++k) out[members[k]] = scores[members[k]] - base;
+    return;
+  }
+  if (mode == 2) {
+    float best = -INFINITY, second = -INFINITY, s1 = 0.f;
+    int arg = -1;
+    for (int k = lo; k < hi; ++k) {
+      const int i = members[k];
+      const float s = scores[i];
+      s1 += s;
+      if (arg < 0 || s > best) { second = best; best = s; arg = i; }
+      else if (s > second) second = s;
+      out[i] = 0.f;
+    }
+    if (hi - lo < 2) return;  // the caller rejects such groups before the launch
+    float a = best - second;
+    if (p_norm) {
+      const float mean = s1 / n;
+      float ss = 0.f;
+      for (int k = lo; k < hi; ++k) { const float d = scores[members[k]] - mean; ss += d * d; }
+      a = a / (sqrtf(ss / (n - 1.f)) + eps);
+    }
+    out[arg] = a;
+    return;
+  }
+  // mode 3
+  float len_lo = INFINITY, len_hi = -INFINITY;
+  for (int k = lo; k < hi; ++k) {
+    const float l = lens[members[k]];
+    len_lo = fminf(len_lo, l);
+    len_hi = fmaxf(len_hi, l);
+  }
+  const float spread = len_hi - len_lo;
+  auto shaped = [&](int i) {
+    const float s = scores[i];
+    if (!(coef > 0.f)) return s;
+    const float lam = coef * (0.5f - (lens[i] - len_lo) / fmaxf(spread, 1.f));
+    const float bonus = (s >= threshold) ? lam : fminf(lam, 0.f);
+    return s + bonus * (spread > 0.f ? 1.f : 0.f);
+  };
+  float s1 = 0.f, s2 = 0.f;
+  for (int k = lo; k < hi; ++k) { const float s = shaped(members[k]); s1 += s; s2 += s * s; }
+  const float nn = fmaxf(n, 1.f);
+  float mean = s1 / nn;
+  float sd = sqrtf(fmaxf((s2 - s1 * s1 / nn) / fmaxf(n - 1.f, 1.f), eps));
+  if (n <= 1.f) { mean = 0.f; sd = 1.f; }
+  for (int k = lo; k < hi; ++k) {
+    const int i = members[k];
+    float a = shaped(i) - mean;
+    if (p_norm) a = a / (sd + eps);
+    out[i] = (n > 1.f) ? a : 0.f;
+  }
+}
+
+}  // namespace axon
+
+using namespace axon;
+
+namespace {
+
+template <int MK>
+int launch_scan(int mode, const float* rewards, const float* values, const void* mask,
+                const int32_t* cu, int64_t n_rows, int64_t uniform_len, float gamma, float gamma_lam,
+                const float* row_baseline, float* adv, float* ret, hipStream_t st) {
+  const dim3 grid((unsigned)((n_rows + (kBlock / kWave) - 1) / (kBlock / kWave))), blk(kBlock);
+#define AXON_SCAN(M)                                                                              \
+  hipLaunchKernelGGL((reverse_scan_kernel<MK, M>), grid, blk, 0, st, rewards, values, mask, cu,   \
+                     n_rows, uniform_len, gamma, gamma_lam, row_baseline, adv, ret)
+  switch (mode) {
+    case kScanGae: AXON_SCAN(kScanGae); break;
+    case kScanGaeResponseOnly: AXON_SCAN(kScanGaeResponseOnly); break;
+    case kScanDiscounted: AXON_SCAN(kScanDiscounted); break;
+    default: AXON_SCAN(kScanSuffixSum); break;
+  }
+#undef AXON_SCAN
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+unsigned moments_grid(int64_t n_slots) {
+  const int64_t blocks = (n_slots / kVec + kBlock - 1) / kBlock;
+  const int64_t cap = 2048;  // eight workgroups per compute unit walk the tokens
+  return (unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap));
+}
+
+template <int MK>
+int launch_whiten(const float* x, const void* mask, int64_t n_slots, int remask, float* out,
+                  float* stats, float* partials, hipStream_t st) {
+  const dim3 grid(moments_grid(n_slots)), blk(kBlock);
+  hipLaunchKernelGGL((masked_moments_kernel<MK, 0>), grid, blk, 0, st, x, mask, n_slots, stats, partials);
+  hipLaunchKernelGGL(masked_moments_finish_kernel, dim3(1), blk, 0, st, partials, (int)grid.x, 0, stats);
+  hipLaunchKernelGGL((masked_moments_kernel<MK, 1>), grid, blk, 0, st, x, mask, n_slots, stats, partials);
+  hipLaunchKernelGGL(masked_moments_finish_kernel, dim3(1), blk, 0, st, partials, (int)grid.x, 1, stats);
+  AXON_CHECK_LAUNCH();
+  if (out != nullptr) {
+    hipLaunchKernelGGL((whiten_kernel<MK>), grid, blk, 0, st, x, mask, n_slots, stats, remask, out);
+    AXON_CHECK_LAUNCH();
+  }
+  return AXON_OK;
+}
+
+}  // namespace
+
+extern "C" int axon_reverse_scan(int mode, const float* rewards, const float* values,
+                                 const void* mask, int mask_kind, const int32_t* cu_seqlens,
+                                 int64_t n_rows, int64_t n_slots, int64_t uniform_len, float gamma,
+                                 float lam, const float* row_baseline, float* adv, float* ret,
+                                 void* stream) {
+  if (n_rows < 0 || n_slots < 0 || uniform_len < 0) return AXON_ERR_ARG;
+  if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
+  if (mode < kScanGae || mode > kScanSuffixSum) return AXON_ERR_ARG;
+  if (n_slots == 0 || n_rows == 0) return AXON_OK;
+  if (uniform_len == 0 && !cu_seqlens) return AXON_ERR_ARG;
+  if (!rewards || !ret) return AXON_ERR_ARG;
+  if (mode <= kScanGaeResponseOnly && (!values || !adv)) return AXON_ERR_ARG;
+  if (mode == kScanSuffixSum && !adv) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  // gamma * lam in double, rounded once: what `gamma * lam * tensor` does with Python scalars
+  const float gamma_lam = (float)((double)gamma * (double)lam);
+  float* adv_out = (mode == kScanDiscounted) ? nullptr : adv;
+  const hipStream_t st = (hipStream_t)stream;
+  if (mask_kind == AXON_MASK_F32)
+    return launch_scan<AXON_MASK_F32>(mode, rewards, values, mask, cu_seqlens, n_rows, uniform_len,
+                                      gamma, gamma_lam, row_baseline, adv_out, ret, st);
+  return launch_scan<AXON_MASK_I64>(mode, rewards, values, mask, cu_seqlens, n_rows, uniform_len,
+                                    gamma, gamma_lam, row_baseline, adv_out, ret, st);
+}
+
+extern "C" int64_t axon_masked_whiten_workspace_bytes(int64_t n_slots) {
+  if (n_slots < 0) return AXON_ERR_ARG;
+  return (int64_t)moments_grid(n_slots) * kPartialStride * (int64_t)sizeof(float);
+}
+
+extern "C" int axon_masked_whiten(const float* x, const void* mask, int mask_kind, int64_t n_slots,
+                                  int remask, float* out, float* stats, float* partials,
+                                  void* stream) {
+  if (n_slots < 0) return AXON_ERR_ARG;
+  if (n_slots >= (int64_t)INT32_MAX * 4) return AXON_ERR_SHAPE;
+  if (!stats || !partials) return AXON_ERR_ARG;
+  if (n_slots > 0 && (!x || !mask)) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(mask) |
+       reinterpret_cast<uintptr_t>(out)) & 15)
+    return AXON_ERR_ARG;
+  const hipStream_t st = (hipStream_t)stream;
+  if (mask_kind == AXON_MASK_F32)
+    return launch_whiten<AXON_MASK_F32>(x, mask, n_slots, remask, out, stats, partials, st);
+  return launch_whiten<AXON_MASK_I64>(x, mask, n_slots, remask, out, stats, partials, st);
+}
+
+extern "C" int axon_group_scalar(int mode, const float* scores, const float* lens,
+                                 const int32_t* members, const int32_t* offsets, int64_t n_rows,
+                                 int64_t n_groups, float eps, int normalize, float coef,
+                                 float threshold, float* scalar, void* stream) {
+  if (n_rows < 0 || n_groups < 0 || mode < 0 || mode > 3) return AXON_ERR_ARG;
+  if (n_rows >= (int64_t)INT32_MAX || n_groups >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (n_rows == 0 || n_groups == 0) return AXON_OK;
+  if (!scores || !members || !offsets || !scalar) return AXON_ERR_ARG;
+  if ((mode == 0 || mode == 3) && !lens) return AXON_ERR_ARG;
+  hipLaunchKernelGGL(group_scalar_kernel, dim3((unsigned)((n_groups + kBlock - 1) / kBlock)),
+                     dim3(kBlock), 0, (hipStream_t)stream, mode, scores, lens, members, offsets,
+                     n_groups, eps, normalize, coef, threshold, scalar);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}

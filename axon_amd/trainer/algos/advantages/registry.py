@@ -10,13 +10,21 @@ AdvantageRegistryEntry = FunctionRegistryEntry
 
 
 class AdvantageFn(str, Enum):
-    """Estimators this path provides (the outcome-reward, group-baseline family; the reference also
-    lists GAE and other value- or return-based estimators)."""
+    """The reference's estimator names (registry.py:44-59)."""
 
+    GAE = "gae"
     GRPO = "grpo"
     RLOO = "rloo"
     LOOP = "loop"  # alias of RLOO
+    REINFORCE_PLUS_PLUS = "reinforce_plus_plus"
+    REINFORCE_PLUS_PLUS_BASELINE = "reinforce_plus_plus_baseline"
+    REMAX = "remax"
+    OPO = "opo"
+    GRPO_PASSK = "grpo_passk"
     GPG = "gpg"
+    CHUNKED_GAE = "chunked_gae"
+    IDENTITY = "identity"
+    KIMI_K1_5 = "kimi_k1_5"
 
 
 _advantage_registry: FunctionRegistry = FunctionRegistry(name="advantage estimator")

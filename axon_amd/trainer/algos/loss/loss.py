@@ -21,7 +21,7 @@ from axon_amd import _lib, _ops
 from axon_amd.trainer.algos.constants import VALID_BATCH_REDUCE, VALID_TOKEN_REDUCE
 from axon_amd.trainer.algos.loss.registry import LossFn, register_loss
 
-_KIND_PPO, _KIND_GSPO, _KIND_REINFORCE, _KIND_CISPO = 0, 1, 2, 3
+_KIND_PPO, _KIND_GSPO, _KIND_REINFORCE, _KIND_CISPO, _KIND_VALUE = 0, 1, 2, 3, 4
 
 
 class _ClippedPolicyLoss(torch.autograd.Function):
@@ -43,20 +43,8 @@ class _ClippedPolicyLoss(torch.autograd.Function):
         return (grad * (g_loss * acc[5])).to(ctx.in_dtype), None, None, None, None
 
 
-def _run(kind: int, data, config, default_token_reduce: str):
-    b = data.batch
-    log_probs = b["log_probs"]
-    clip = config.get("clip_ratio", 0.2)
-    lo = config.get("clip_ratio_low", None)
-    hi = config.get("clip_ratio_high", None)
-    # CISPO leaves the lower side effectively unclipped unless asked to (loss.py:435-436)
-    lo = (1e10 if kind == _KIND_CISPO else clip) if lo is None else lo
-    hi = clip if hi is None else hi
-    clip_c = config.get("clip_ratio_c", 3.0)
-    if kind == _KIND_PPO:
-        assert clip_c > 1.0, f"clip_ratio_c must be > 1.0, got {clip_c}"
-    if kind == _KIND_CISPO:  # the slot carries the token_level_mask switch instead
-        clip_c = 1.0 if config.get("token_level_mask", False) else 0.0
+def _aggregation(b, config, default_token_reduce: str) -> dict:
+    """The ``agg_loss`` arguments of a loss call (loss/utils.py:120-251), validated as the reference does."""
     token_reduce = config.get("token_reduce", default_token_reduce)
     batch_reduce = config.get("batch_reduce", "token-mean")
     if token_reduce not in VALID_TOKEN_REDUCE:
@@ -75,6 +63,26 @@ def _run(kind: int, data, config, default_token_reduce: str):
     if batch_reduce == "program-mean":
         assert nps is not None, f"num_program_steps required for batch_reduce='{batch_reduce}'"
         assert valid is not None, "valid_program_count required for batch_reduce='program-mean'"
+    return dict(token_reduce=token_reduce, batch_reduce=batch_reduce,
+                per_row_token_count=b.get("per_row_token_count", None), num_program_tokens=npt,
+                num_program_steps=nps, valid_count=valid)
+
+
+def _run(kind: int, data, config, default_token_reduce: str):
+    b = data.batch
+    log_probs = b["log_probs"]
+    clip = config.get("clip_ratio", 0.2)
+    lo = config.get("clip_ratio_low", None)
+    hi = config.get("clip_ratio_high", None)
+    # CISPO leaves the lower side effectively unclipped unless asked to (loss.py:435-436)
+    lo = (1e10 if kind == _KIND_CISPO else clip) if lo is None else lo
+    hi = clip if hi is None else hi
+    clip_c = config.get("clip_ratio_c", 3.0)
+    if kind == _KIND_PPO:
+        assert clip_c > 1.0, f"clip_ratio_c must be > 1.0, got {clip_c}"
+    if kind == _KIND_CISPO:  # the slot carries the token_level_mask switch instead
+        clip_c = 1.0 if config.get("token_level_mask", False) else 0.0
+    agg = _aggregation(b, config, default_token_reduce)
 
     _lib.require_device(log_probs, "policy loss")
     rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
@@ -85,13 +93,8 @@ def _run(kind: int, data, config, default_token_reduce: str):
         # CISPO does not read the sampler weights (loss.py:421-468)
         "sampler_is_weights": None if kind == _KIND_CISPO else b.get("sampler_is_weights", None),
     }
-    hp = dict(
-        token_reduce=token_reduce, batch_reduce=batch_reduce,
-        # bounds evaluated in double and rounded once, as torch.clamp does with Python scalars
-        ratio_lo=1 - lo, ratio_hi=1 + hi, clip_c=clip_c,
-        per_row_token_count=b.get("per_row_token_count", None), num_program_tokens=npt, num_program_steps=nps,
-        valid_count=valid,
-    )
+    # bounds evaluated in double and rounded once, as torch.clamp does with Python scalars
+    hp = dict(ratio_lo=1 - lo, ratio_hi=1 + hi, clip_c=clip_c, **agg)
     loss, acc = _ClippedPolicyLoss.apply(log_probs, kind, tensors, rows, hp)
     sums = acc.tolist()  # the only host sync of the loss
     denom = max(sums[4], 1.0)
@@ -168,3 +171,23 @@ def geo_mean_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
     sums = acc.tolist()
     denom = max(sums[4], 1.0)
     return loss, {"pg_clipfrac": sums[1] / denom, "ppo_kl": sums[2] / denom, "pg_clipfrac_lower": sums[3] / denom}
+
+
+@register_loss(LossFn.VALUE)
+def value_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """Clipped value-function loss (loss.py:547-591): ``0.5 * agg_loss(max((vpreds - returns)^2,
+    (clip(vpreds, values -+ cliprange_value) - returns)^2))``, defaults sum / token-mean; the gradient flows to
+    ``vpreds``.  Metrics ``vf_loss``, ``vf_clipfrac``, ``vpred_mean``."""
+    b = data.batch
+    vpreds = b["vpreds"]
+    agg = _aggregation(b, config, "sum")
+    _lib.require_device(vpreds, "value loss")
+    rows = _ops.rows_of(vpreds, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
+    tensors = {"old_log_probs": b["values"], "advantages": b["returns"], "response_mask": b["response_mask"],
+               "sampler_is_weights": None}
+    hp = dict(ratio_lo=config.get("cliprange_value", 0.5), ratio_hi=0.0, clip_c=0.0, **agg)
+    raw, acc = _ClippedPolicyLoss.apply(vpreds, _KIND_VALUE, tensors, rows, hp)
+    loss = 0.5 * raw
+    sums = acc.tolist()
+    denom = max(sums[4], 1.0)
+    return loss, {"vf_loss": 0.5 * sums[0], "vf_clipfrac": sums[1] / denom, "vpred_mean": sums[2] / denom}

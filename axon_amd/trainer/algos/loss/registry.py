@@ -28,6 +28,7 @@ class LossFn(str, Enum):
     CISPO = "cispo"
     REINFORCE = "reinforce"
     GEO_MEAN = "geo_mean"
+    VALUE = "value"
 
 
 _loss_registry: FunctionRegistry = FunctionRegistry(name="policy loss")

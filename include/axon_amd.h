@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 8
+#define AXON_AMD_ABI_VERSION 9
 
 enum {
   AXON_OK = 0,
@@ -278,6 +278,10 @@ int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_ro
  *   kind 2: reinforce_loss_fn / gpg_loss_fn (loss.py:183-197, 471-512): -A * logp * is_weights
  *   kind 3: cispo_loss_fn (loss.py:411-468): -sg(clamp(ratio)) * A * logp; clip_c != 0 switches
  *           the optional token-level mask on; is_weights must be NULL
+ *   kind 4: value_loss_fn (loss.py:547-591) without its factor 0.5: logp carries vpreds, old_logp the
+ *           old values, adv the returns, ratio_lo the cliprange_value; max((vpreds - returns)^2,
+ *           (clip_by_value(vpreds, values -+ cliprange) - returns)^2) with torch's tie rules for the
+ *           gradient; acc[1] = sum mask*(clipped term larger), acc[2] = sum mask*vpreds
  * ratio_lo / ratio_hi: the clamp bounds 1 - clip_ratio_low and 1 + clip_ratio_high,
  * evaluated in double by the caller and rounded to fp32 (what torch.clamp does
  * with Python scalars).  clip_c: dual-clip constant (> 1), PPO only.
@@ -301,6 +305,49 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
                      float uniform_scale, int post_normalize, const int64_t* valid_count,
                      float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                      float* partials, void* stream);
+
+/* Time recurrences of the return-based advantage estimators, run from each row's last token to its
+ * first (axon/trainer/algos/advantages/advantage.py), before any whitening:
+ *   mode 0: gae_advantage_fn :57-73.  nextvalues and lastgaelam skip tokens with mask 0 (a fractional
+ *           mask blends as in the reference); adv = lastgaelam, ret = adv + values.
+ *   mode 1: chunked_gae_advantage_fn :480-537 (_chunked_gae_core :374-477): the same recurrence over the
+ *           tokens with mask > 0 only, V past the last response token = 0; adv = ret = 0 elsewhere.
+ *   mode 2: reinforce_plus_plus_advantage_fn :163-171: ret[t] = r[t] + gamma * mask[t+1] * ret[t+1];
+ *           adv is not written (may be NULL).
+ *   mode 3: remax_advantage_fn :234-238: ret[t] = sum_{s>=t} r[s]*mask[s];
+ *           adv = ret - row_baseline[row] * mask.
+ * values is read by modes 0 and 1, lam by modes 0 and 1, row_baseline [n_rows] by mode 3.
+ * Rows as in axon_row_stats (uniform_len > 0: padded [n_rows, uniform_len]; else cu_seqlens). */
+int axon_reverse_scan(int mode, const float* rewards, const float* values, const void* mask,
+                      int mask_kind, const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                      int64_t uniform_len, float gamma, float lam, const float* row_baseline,
+                      float* adv, float* ret, void* stream);
+
+/* masked_whiten (axon/utils/rl/advantage.py:153-190): mean and variance over the mask (variance times
+ * n/(n-1) when n > 1), out = (x - mean) * rsqrt(var + 1e-8), times the mask when remask != 0 (the
+ * `* response_mask` of advantage.py:174,215).  out may equal x, or be NULL for the statistics alone.
+ * stats[4] (device): mean, n, variance, rsqrt(variance + 1e-8).  partials: workspace of
+ * axon_masked_whiten_workspace_bytes(n_slots) bytes; the sums are formed in a fixed order.
+ * x, mask and out 16-byte aligned. */
+int64_t axon_masked_whiten_workspace_bytes(int64_t n_slots);
+int axon_masked_whiten(const float* x, const void* mask, int mask_kind, int64_t n_slots, int remask,
+                       float* out, float* stats, float* partials, void* stream);
+
+/* Per-row scalars of the group-based estimators that need more than a group mean and deviation
+ * (advantage.py).  The caller passes the groups in compressed form: members[n_rows] = row indices ordered
+ * by group (row order kept within a group), offsets[n_groups + 1] into members.
+ *   mode 0: opo_advantage_fn :260-277: score - (n > 1 ? sum(len*score)/max(sum len, 1) : 0)
+ *   mode 1: reinforce_plus_plus_baseline_advantage_fn :197-210: score - (n > 1 ? group mean : 0)
+ *   mode 2: grpo_passk_advantage_fn :304-330: the best row of a group gets max - second max, divided by
+ *           (unbiased std + eps) when normalize != 0; every other row 0 (groups of one row: the caller
+ *           raises before the launch, as the reference does)
+ *   mode 3: kimi_k1_5_advantage_fn :586-623: score + length term (coef = the scheduled length_coef,
+ *           threshold = correct_threshold, min/max length over the whole group, off when coef <= 0),
+ *           then (shaped - mean)/(std + eps) or shaped - mean, 0 for groups of one row
+ * lens [n_rows] (sum of the response mask per row) is read by modes 0 and 3. */
+int axon_group_scalar(int mode, const float* scores, const float* lens, const int32_t* members,
+                      const int32_t* offsets, int64_t n_rows, int64_t n_groups, float eps,
+                      int normalize, float coef, float threshold, float* scalar, void* stream);
 
 /* Per-token KL penalty against a reference policy, kl_penalty / kl_penalty_forward
  * (axon/utils/rl/kl.py:154-245): kl_type 1 "kl"/"k1", 2 "abs", 3 "mse"/"k2", 4 "low_var_kl"/"k3";
