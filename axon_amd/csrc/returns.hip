@@ -3,17 +3,22 @@
 //
 // A recurrence y[t] = b[t] + a[t] * y[t+1] is a scan over pairs (a, b) under the composition
 // (a2, b2) o (a1, b1) = (a2*a1, b2 + a2*b1).  One wavefront owns one row and walks it from the end in
-// blocks of 256 tokens (four sub-blocks of one token per lane, lane 0 holding the last token), scans each
-// sub-block with shuffles and carries the boundary value from sub-block to sub-block.  The loads of the next
-// block are issued before the current one is scanned.
+// windows of 256 tokens that are 4-aligned in the token array: a lane holds four consecutive tokens (one
+// 16-byte access where the vector lies inside the row, guarded scalar accesses at the row's edges), lane 0
+// the last ones.  A lane composes its four elements, the wavefront scans the 64 composites with shuffles,
+// and each lane then replays its four tokens from the value that enters it.  The loads of the next window
+// are issued before the current one is scanned.
 #include "common.h"
 
 namespace axon {
 
-constexpr int kScanSub = 4;                      // sub-blocks per step
-constexpr int kScanStep = kScanSub * kWave;      // tokens per step
+constexpr int kScanVec = 4;                      // tokens per lane
+constexpr int kScanStep = kScanVec * kWave;      // tokens per window
 
 struct Pair { float a, b; };
+
+// p after q: y -> p.b + p.a * (q.b + q.a * y)
+__device__ __forceinline__ Pair after(Pair p, Pair q) { return Pair{p.a * q.a, p.b + p.a * q.b}; }
 
 // inclusive scan over lanes 0..63: lane l ends with the composition of the elements of lanes 0..l
 __device__ __forceinline__ Pair wave_scan(Pair p) {
@@ -22,39 +27,59 @@ __device__ __forceinline__ Pair wave_scan(Pair p) {
   for (int d = 1; d < kWave; d <<= 1) {
     const float ap = __shfl_up(p.a, d, kWave);
     const float bp = __shfl_up(p.b, d, kWave);
-    if (lane >= d) {
-      p.b = p.b + p.a * bp;
-      p.a = p.a * ap;
-    }
+    if (lane >= d) p = after(p, Pair{ap, bp});
   }
   return p;
 }
 
-// value of the previous lane (the token after this one); lane 0 takes `carry`
-__device__ __forceinline__ float from_next_token(float incl, float carry) {
-  const float up = __shfl_up(incl, 1, kWave);
-  return (threadIdx.x & (kWave - 1)) == 0 ? carry : up;
+// Scans the lanes' composites; returns the value that enters this lane (the recurrence at the token after the
+// lane's last one) and moves `carry` to the value that leaves lane 63.
+__device__ __forceinline__ float scan_enter(Pair lane_total, float& carry) {
+  const Pair s = wave_scan(lane_total);
+  const float leaves = s.b + s.a * carry;
+  const float up = __shfl_up(leaves, 1, kWave);
+  const float enters = (threadIdx.x & (kWave - 1)) == 0 ? carry : up;
+  carry = __shfl(leaves, kWave - 1, kWave);
+  return enters;
 }
 
 enum { kScanGae = 0, kScanGaeResponseOnly = 1, kScanDiscounted = 2, kScanSuffixSum = 3 };
 
 struct ScanBlock {
-  float r[kScanSub], v[kScanSub], m[kScanSub];
+  float r[kScanVec], v[kScanVec], m[kScanVec];
+  int ok;  // bit j: token p0 + j lies inside the row
 };
 
+// window [end - 256, end), end a multiple of 4; this lane's tokens are p0 .. p0 + 3
 template <int MK, int MODE>
 __device__ __forceinline__ void scan_load(ScanBlock& x, const float* __restrict__ rewards,
                                           const float* __restrict__ values,
-                                          const void* __restrict__ mask, int64_t begin, int64_t end) {
+                                          const void* __restrict__ mask, int64_t begin, int64_t stop,
+                                          int64_t end, bool vec_ok) {
   const int lane = threadIdx.x & (kWave - 1);
+  const int64_t p0 = end - kScanVec * (lane + 1);
+  constexpr bool kValues = MODE <= kScanGaeResponseOnly;
+  if (vec_ok && p0 >= begin && p0 + kScanVec <= stop) {
+    load4(rewards, p0, x.r);
+    if (kValues) load4(values, p0, x.v);
+    load_mask4<MK>(mask, p0, x.m);
+    x.ok = 15;
+  } else {
+    x.ok = 0;
 #pragma unroll
-  for (int u = 0; u < kScanSub; ++u) {
-    const int64_t p = end - 1 - (u * kWave + lane);
-    const bool ok = p >= begin;
-    x.r[u] = ok ? rewards[p] : 0.f;
-    x.v[u] = (ok && MODE <= kScanGaeResponseOnly) ? values[p] : 0.f;
-    x.m[u] = ok ? load_mask1<MK>(mask, p) : 0.f;
-    if (MODE == kScanGaeResponseOnly) x.m[u] = x.m[u] > 0.f ? 1.f : 0.f;
+    for (int j = 0; j < kScanVec; ++j) {
+      const int64_t p = p0 + j;
+      const bool ok = p >= begin && p < stop;
+      x.r[j] = ok ? rewards[p] : 0.f;
+      x.v[j] = (ok && kValues) ? values[p] : 0.f;
+      x.m[j] = ok ? load_mask1<MK>(mask, p) : 0.f;
+      x.ok |= ok ? (1 << j) : 0;
+    }
+  }
+  if (!kValues) x.v[0] = x.v[1] = x.v[2] = x.v[3] = 0.f;
+  if (MODE == kScanGaeResponseOnly) {
+#pragma unroll
+    for (int j = 0; j < kScanVec; ++j) x.m[j] = x.m[j] > 0.f ? 1.f : 0.f;
   }
 }
 
@@ -68,74 +93,74 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(
     const float* __restrict__ rewards, const float* __restrict__ values,
     const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows,
     int64_t uniform_len, float gamma, float gamma_lam, const float* __restrict__ row_baseline,
-    float* __restrict__ adv, float* __restrict__ ret) {
+    float* __restrict__ adv, float* __restrict__ ret, int vec_ok) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
   if (row >= n_rows) return;  // whole wavefronts leave together; no workgroup barrier below
   const int64_t begin = uniform_len > 0 ? row * uniform_len : (int64_t)cu[row];
   const int64_t stop = uniform_len > 0 ? begin + uniform_len : (int64_t)cu[row + 1];
-  const float base = (MODE == kScanSuffixSum && row_baseline) ? row_baseline[row] : 0.f;
-  float carry0 = 0.f, carry1 = 0.f;  // the recurrences' values at the token after the current block
   if (stop <= begin) return;
+  const float base = (MODE == kScanSuffixSum && row_baseline) ? row_baseline[row] : 0.f;
+  float carry0 = 0.f, carry1 = 0.f;  // the recurrences' values at the token after the current window
+  const int64_t last = (stop + kScanVec - 1) & ~(int64_t)(kScanVec - 1);
   ScanBlock cur, nxt;
-  scan_load<MK, MODE>(cur, rewards, values, mask, begin, stop);
-  for (int64_t end = stop; end > begin; end -= kScanStep) {
+  scan_load<MK, MODE>(cur, rewards, values, mask, begin, stop, last, vec_ok);
+  for (int64_t end = last; end > begin; end -= kScanStep) {
     const bool more = end - kScanStep > begin;
-    if (more) scan_load<MK, MODE>(nxt, rewards, values, mask, begin, end - kScanStep);
-    float out_adv[kScanSub], out_ret[kScanSub];
+    if (more) scan_load<MK, MODE>(nxt, rewards, values, mask, begin, stop, end - kScanStep, vec_ok);
+    float out_adv[kScanVec], out_ret[kScanVec];
     if (MODE <= kScanGaeResponseOnly) {
-      Pair s1[kScanSub];
+      Pair e[kScanVec];
 #pragma unroll
-      for (int u = 0; u < kScanSub; ++u) s1[u] = wave_scan(Pair{1.f - cur.m[u], cur.m[u] * cur.v[u]});
-      Pair e2[kScanSub];
+      for (int j = 0; j < kScanVec; ++j) e[j] = Pair{1.f - cur.m[j], cur.m[j] * cur.v[j]};
+      float nv = scan_enter(after(e[0], after(e[1], after(e[2], e[3]))), carry0);
 #pragma unroll
-      for (int u = 0; u < kScanSub; ++u) {
-        const float nv = s1[u].b + s1[u].a * carry0;
-        const float nv_next = from_next_token(nv, carry0);
-        carry0 = __shfl(nv, kWave - 1, kWave);
-        const float delta = cur.r[u] + gamma * nv_next - cur.v[u];
-        e2[u] = Pair{cur.m[u] * gamma_lam + (1.f - cur.m[u]), cur.m[u] * delta};
+      for (int j = kScanVec - 1; j >= 0; --j) {
+        const float delta = cur.r[j] + gamma * nv - cur.v[j];
+        nv = e[j].b + e[j].a * nv;
+        e[j] = Pair{cur.m[j] * gamma_lam + (1.f - cur.m[j]), cur.m[j] * delta};
       }
+      float l = scan_enter(after(e[0], after(e[1], after(e[2], e[3]))), carry1);
 #pragma unroll
-      for (int u = 0; u < kScanSub; ++u) e2[u] = wave_scan(e2[u]);
-#pragma unroll
-      for (int u = 0; u < kScanSub; ++u) {
-        const float l = e2[u].b + e2[u].a * carry1;
-        carry1 = __shfl(l, kWave - 1, kWave);
-        const bool keep = (MODE == kScanGae) || cur.m[u] > 0.f;
-        out_adv[u] = keep ? l : 0.f;
-        out_ret[u] = keep ? l + cur.v[u] : 0.f;
-      }
-    } else if (MODE == kScanDiscounted) {
-      Pair s[kScanSub];
-#pragma unroll
-      for (int u = 0; u < kScanSub; ++u) s[u] = wave_scan(Pair{gamma * cur.m[u], cur.m[u] * cur.r[u]});
-#pragma unroll
-      for (int u = 0; u < kScanSub; ++u) {
-        const float q = s[u].b + s[u].a * carry0;
-        const float q_next = from_next_token(q, carry0);
-        carry0 = __shfl(q, kWave - 1, kWave);
-        out_ret[u] = cur.r[u] + gamma * q_next;
-        out_adv[u] = 0.f;
+      for (int j = kScanVec - 1; j >= 0; --j) {
+        l = e[j].b + e[j].a * l;
+        const bool keep = (MODE == kScanGae) || cur.m[j] > 0.f;
+        out_adv[j] = keep ? l : 0.f;
+        out_ret[j] = keep ? l + cur.v[j] : 0.f;
       }
     } else {
-      Pair s[kScanSub];
+      Pair e[kScanVec];
 #pragma unroll
-      for (int u = 0; u < kScanSub; ++u) s[u] = wave_scan(Pair{1.f, cur.r[u] * cur.m[u]});
+      for (int j = 0; j < kScanVec; ++j) {
+        const bool ok = (cur.ok >> j) & 1;
+        if (MODE == kScanDiscounted) e[j] = Pair{ok ? gamma * cur.m[j] : 1.f, cur.m[j] * cur.r[j]};
+        else e[j] = Pair{1.f, cur.r[j] * cur.m[j]};
+      }
+      float q = scan_enter(after(e[0], after(e[1], after(e[2], e[3]))), carry0);
 #pragma unroll
-      for (int u = 0; u < kScanSub; ++u) {
-        const float c = s[u].b + carry0;
-        carry0 = __shfl(c, kWave - 1, kWave);
-        out_ret[u] = c;
-        out_adv[u] = c - base * cur.m[u];
+      for (int j = kScanVec - 1; j >= 0; --j) {
+        if (MODE == kScanDiscounted) {
+          out_ret[j] = cur.r[j] + gamma * q;
+          out_adv[j] = 0.f;
+          q = e[j].b + e[j].a * q;
+        } else {
+          q = e[j].b + q;
+          out_ret[j] = q;
+          out_adv[j] = q - base * cur.m[j];
+        }
       }
     }
+    const int64_t p0 = end - kScanVec * (lane + 1);
+    if (cur.ok == 15 && vec_ok) {
+      if (adv != nullptr) store4(adv, p0, out_adv);
+      store4(ret, p0, out_ret);
+    } else {
 #pragma unroll
-    for (int u = 0; u < kScanSub; ++u) {
-      const int64_t p = end - 1 - (u * kWave + lane);
-      if (p >= begin) {
-        if (adv != nullptr) adv[p] = out_adv[u];
-        ret[p] = out_ret[u];
+      for (int j = 0; j < kScanVec; ++j) {
+        if ((cur.ok >> j) & 1) {
+          if (adv != nullptr) adv[p0 + j] = out_adv[j];
+          ret[p0 + j] = out_ret[j];
+        }
       }
     }
     if (more) cur = nxt;
@@ -324,10 +349,14 @@ template <int MK>
 int launch_scan(int mode, const float* rewards, const float* values, const void* mask,
                 const int32_t* cu, int64_t n_rows, int64_t uniform_len, float gamma, float gamma_lam,
                 const float* row_baseline, float* adv, float* ret, hipStream_t st) {
+  // 16-byte accesses need every array on a 16-byte boundary (an int64 mask then is on 32)
+  const int vec_ok = ((reinterpret_cast<uintptr_t>(rewards) | reinterpret_cast<uintptr_t>(values) |
+                       reinterpret_cast<uintptr_t>(mask) | reinterpret_cast<uintptr_t>(adv) |
+                       reinterpret_cast<uintptr_t>(ret)) & 15) == 0;
   const dim3 grid((unsigned)((n_rows + (kBlock / kWave) - 1) / (kBlock / kWave))), blk(kBlock);
 #define AXON_SCAN(M)                                                                              \
   hipLaunchKernelGGL((reverse_scan_kernel<MK, M>), grid, blk, 0, st, rewards, values, mask, cu,   \
-                     n_rows, uniform_len, gamma, gamma_lam, row_baseline, adv, ret)
+                     n_rows, uniform_len, gamma, gamma_lam, row_baseline, adv, ret, vec_ok)
   switch (mode) {
     case kScanGae: AXON_SCAN(kScanGae); break;
     case kScanGaeResponseOnly: AXON_SCAN(kScanGaeResponseOnly); break;

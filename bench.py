@@ -146,6 +146,13 @@ def hbm_kernels(n_tokens, dev):
                                    log_rs_hi=math.log(2.0))),
         ("row_broadcast_kernel: GRPO advantage = per-sequence scalar * mask", 8,
          lambda: _ops.row_broadcast_mask(seq_scalar, mask, rows)),
+        ("reverse_scan_kernel: GAE time recurrence per sequence (rewards, values, mask -> advantages, returns)", 20,
+         lambda: _ops.reverse_scan(_ops.SCAN_GAE, adv, new, mask, rows, gamma=0.99, lam=0.95)),
+        ("masked_whiten kernels: mean pass + variance pass + normalise (three reads of x, two of mask, one write)",
+         24, lambda: _ops.masked_whiten(adv, mask)),
+        ("policy_loss_kernel: clipped value loss + gradient, sum/token-mean (one pass)", 20,
+         lambda: _ops.policy_loss(4, new, old, adv, mask, None, rows, token_reduce="sum", batch_reduce="token-mean",
+                                  ratio_lo=0.5, ratio_hi=0.0, clip_c=0.0)),
     ]
     out = []
     for name, bpt, fn in cases:
