@@ -50,6 +50,12 @@ SIGNATURES: dict[str, tuple] = {
     "axon_reduce_partials_bytes": (_i64, [_i64]),
     "axon_gmpo_loss": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr,
                               _ptr, _ptr]),
+    "axon_cov_select_state_bytes": (_i64, []),
+    "axon_cov_select_workspace_bytes": (_i64, [_i64]),
+    "axon_cov_select": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _i64, ctypes.c_double, _f32, _f32, _f32, _f32,
+                               ctypes.c_uint32, _ptr, _ptr, _ptr, _ptr]),
+    "axon_cov_policy_loss": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64, _ptr, _f32,
+                                    _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_kl_penalty": (_i32, [_ptr, _ptr, _i64, _i32, _i32, _ptr, _ptr, _ptr]),
     "axon_side_terms": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _ptr, _f32, _i32, _ptr, _i32,
                                _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
@@ -63,7 +69,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

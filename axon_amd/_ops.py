@@ -310,6 +310,56 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     return acc, grad
 
 
+def cov_policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows, *, select_ratio,
+                    ratio_lo=0.0, ratio_hi=0.0, cov_lb=0.0, cov_ub=0.0, kl_coef=1.0, seed=0, token_reduce,
+                    batch_reduce, per_row_token_count=None, num_program_tokens=None, num_program_steps=None,
+                    valid_count=None):
+    """KL-Cov (kind 0) / Clip-Cov (kind 1): token selection (axon_cov_select) + loss and gradient
+    (axon_cov_policy_loss).  Returns ``(acc[8], grad, keys, state)``; acc as in ``policy_loss`` with
+    acc[1] = number of selected tokens (mask-weighted)."""
+    lib = _lib.load()
+    require_device(log_probs, "cov_policy_loss")
+    dev = log_probs.device
+    lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
+    mk, mkind = mask_arg(mask)
+    isw = f32(is_weights) if is_weights is not None else None
+    tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
+    n = rows.n_slots
+    keys = torch.empty(max(n, 4), device=dev, dtype=torch.int32)
+    state = torch.zeros((int(lib.axon_cov_select_state_bytes()) + 7) // 8, device=dev, dtype=torch.int64)
+    ws = torch.empty(max(int(lib.axon_cov_select_workspace_bytes(n)), 16), device=dev, dtype=torch.uint8)
+    check(
+        lib.axon_cov_select(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, n, float(select_ratio), float(cov_lb),
+                            float(cov_ub), float(ratio_lo), float(ratio_hi), int(seed) & 0xFFFFFFFF, ptr(keys),
+                            ptr(state), ptr(ws), stream_ptr()),
+        "axon_cov_select",
+    )
+    valid = _i64_dev(valid_count, dev)
+    grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    acc = _acc8(n, dev)
+    one_pass = tr == 0 and br == 0
+    row_scale = None
+    if not one_pass:
+        cnt, _, _ = row_stats(lp, None, mk, rows, want_sum=False)
+        row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
+        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        check(
+            lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
+                                    ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),
+            "axon_loss_row_scale",
+        )
+    check(
+        lib.axon_cov_policy_loss(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
+                                 n, rows.uniform_len, ptr(row_scale), 1.0, int(one_pass),
+                                 ptr(valid if one_pass else None), float(ratio_lo), float(ratio_hi), float(kl_coef),
+                                 ptr(keys), ptr(state), ptr(grad), ptr(acc), ptr(_partials(n, dev)), stream_ptr()),
+        "axon_cov_policy_loss",
+    )
+    return acc, grad, keys, state
+
+
 def gmpo_loss(log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows, *, clip_low, clip_high):
     """GMPO loss and gradient; returns (acc[8], grad).  See axon_gmpo_loss."""
     lib = _lib.load()

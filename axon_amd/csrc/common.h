@@ -19,6 +19,31 @@ constexpr int kLdsRows = 2048;        // cu_seqlens window cached in LDS per wor
     if (hipGetLastError() != hipSuccess) return AXON_ERR_LAUNCH; \
   } while (0)
 
+constexpr float kSafetyBound = 20.0f;  // axon/utils/rl/sampler.py:27, loss.py:77
+
+__device__ __forceinline__ float clampf(float x, float lo, float hi) {
+  // torch.clamp semantics: NaN propagates
+  return (x != x) ? x : fminf(fmaxf(x, lo), hi);
+}
+
+// State of a top-k selection over 32-bit keys (largest keys win; key 0 never wins).  A token i is
+// selected when key > threshold, or key == threshold and i < index_limit (ties go to the lowest indices).
+struct SelectState {
+  uint32_t threshold;    // key of the k-th largest element, built 11 + 11 + 10 bits at a time
+  uint32_t remaining;    // how many elements with the current prefix are still to be taken
+  uint32_t candidates;   // non-zero keys
+  uint32_t ties;         // elements equal to the threshold
+  int64_t index_limit;   // -1 while a tie pass still has to find it
+  float mean_a, mean_b;  // the centring constants of the covariance
+  float count;           // sum of the mask (weighted) or number of tokens with mask > 0
+  uint32_t k;            // elements to select
+};
+
+__device__ __forceinline__ bool select_hit(const SelectState& s, uint32_t key, int64_t i) {
+  if (s.k == 0 || key == 0) return false;
+  return key > s.threshold || (key == s.threshold && i < s.index_limit);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, kWave);

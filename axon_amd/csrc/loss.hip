@@ -5,13 +5,6 @@
 
 namespace axon {
 
-constexpr float kSafetyBound = 20.0f;  // axon/utils/rl/sampler.py:27, loss.py:77
-
-__device__ __forceinline__ float clampf(float x, float lo, float hi) {
-  // torch.clamp semantics: NaN propagates
-  return (x != x) ? x : fminf(fmaxf(x, lo), hi);
-}
-
 template <int MK>
 __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
     const float* __restrict__ oldp, const float* __restrict__ samp, const void* __restrict__ mask,
@@ -221,10 +214,13 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     const void* __restrict__ mask, const float* __restrict__ isw, const int32_t* __restrict__ cu,
     int64_t n_rows, int64_t n_slots, int64_t uniform_len, const float* __restrict__ row_scale,
     const float* __restrict__ row_mean, float uniform_scale, float lo, float hi, float clip_c,
+    const uint32_t* __restrict__ sel_keys, const SelectState* __restrict__ sel_state,
     float* __restrict__ grad, float* partials) {
   __shared__ int32_t lds_cu[kLdsRows];
   __shared__ float lds_red[6 * (kBlock / kWave)];
   const bool need_row = (row_scale != nullptr) || (KIND == 1);
+  SelectState sel{};
+  if (KIND >= 5) sel = *sel_state;
   const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
@@ -290,8 +286,23 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
         gv[j] = c.g * m * scale;
         continue;
       }
+      if (KIND == 5) {  // KL-Cov (loss.py:283-352): -A*ratio, plus clip_c * |log ratio| on the selected tokens
+        const bool pass = (d >= -kSafetyBound && d <= kSafetyBound);
+        const float xc = clampf(d, -kSafetyBound, kSafetyBound);
+        const float r_ = expf(xc);
+        float v = -A * r_, g = -A * r_;
+        if (select_hit(sel, sel_keys[p], p)) {
+          v += clip_c * fabsf(xc);
+          g += clip_c * ((xc > 0.f) ? 1.f : ((xc < 0.f) ? -1.f : 0.f));
+          a[1] += m;
+        }
+        a[2] += fabsf(xc) * m;
+        a[0] += (v * w) * m * scale;
+        gv[j] = (pass ? g : 0.f) * w * m * scale;
+        continue;
+      }
       float x;  // exponent before the +-20 clamp
-      if (KIND == 0) x = d;
+      if (KIND == 0 || KIND == 6) x = d;
       else x = (lv[j] - lv[j]) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
       const bool pass = (x >= -kSafetyBound && x <= kSafetyBound);  // clamp passes grad inclusively
       const float xc = clampf(x, -kSafetyBound, kSafetyBound);
@@ -301,8 +312,14 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
       const bool rin = (r_ >= lo && r_ <= hi);
       const ValGrad p2{-A * rc, rin ? -A * r_ : 0.f};
       ValGrad c = vg_max(p1, p2);
-      a[1] += (p2.v > p1.v) ? m : 0.f;
-      a[2] += (KIND == 0 ? -xc : -d) * m;  // ppo_kl: clamped for PPO (loss.py:77-79), raw for GSPO (loss.py:173)
+      if (KIND == 6) {  // Clip-Cov (loss.py:198-280): the selected tokens drop out of the loss
+        const bool hit = select_hit(sel, sel_keys[p], p);
+        if (hit) c = ValGrad{c.v * 0.f, 0.f};
+        a[1] += hit ? m : 0.f;
+      } else {
+        a[1] += (p2.v > p1.v) ? m : 0.f;
+      }
+      a[2] += (KIND == 1 ? -d : -xc) * m;  // ppo_kl: raw for GSPO (loss.py:173), clamped otherwise (loss.py:77-79)
       if (KIND == 0) {
         const float pg3 = -A * clip_c;
         a[3] += (c.v > pg3 && A < 0.f) ? m : 0.f;
@@ -746,7 +763,8 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
 #define AXON_LAUNCH_PL(MK, KD)                                                                   \
   hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
                      n_rows, n_slots, uniform_len, row_scale, row_mean, uniform_scale, ratio_lo, \
-                     ratio_hi, clip_c, grad, partials)
+                     ratio_hi, clip_c, (const uint32_t*)nullptr, (const SelectState*)nullptr, grad,  \
+                     partials)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0);
     else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_F32, 1);
@@ -761,6 +779,45 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
     else AXON_LAUNCH_PL(AXON_MASK_I64, 4);
   }
 #undef AXON_LAUNCH_PL
+  AXON_CHECK_LAUNCH();
+  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
+                     post_normalize ? 1 : 0, valid, acc);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_cov_policy_loss(int kind, const float* logp, const float* oldp, const float* adv,
+                                    const void* mask, int mask_kind, const float* isw,
+                                    const int32_t* cu, int64_t n_rows, int64_t n_slots,
+                                    int64_t uniform_len, const float* row_scale, float uniform_scale,
+                                    int post_normalize, const int64_t* valid, float ratio_lo,
+                                    float ratio_hi, float kl_coef, const uint32_t* keys,
+                                    const void* state, float* grad, float* acc, float* partials,
+                                    void* stream) {
+  const bool need_row = (row_scale != nullptr);
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0) return AXON_OK;
+  if (kind < 0 || kind > 1) return AXON_ERR_ARG;
+  if (!logp || !oldp || !adv || !mask || !grad || !acc || !partials || !keys || !state)
+    return AXON_ERR_ARG;
+  if (post_normalize && row_scale != nullptr) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
+  const hipStream_t st = (hipStream_t)stream;
+  const SelectState* sel = static_cast<const SelectState*>(state);
+#define AXON_LAUNCH_CV(MK, KD)                                                                    \
+  hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
+                     n_rows, n_slots, uniform_len, row_scale, (const float*)nullptr,              \
+                     uniform_scale, ratio_lo, ratio_hi, kl_coef, keys, sel, grad, partials)
+  if (mask_kind == AXON_MASK_F32) {
+    if (kind == 0) AXON_LAUNCH_CV(AXON_MASK_F32, 5);
+    else AXON_LAUNCH_CV(AXON_MASK_F32, 6);
+  } else {
+    if (kind == 0) AXON_LAUNCH_CV(AXON_MASK_I64, 5);
+    else AXON_LAUNCH_CV(AXON_MASK_I64, 6);
+  }
+#undef AXON_LAUNCH_CV
   AXON_CHECK_LAUNCH();
   hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
                      post_normalize ? 1 : 0, valid, acc);

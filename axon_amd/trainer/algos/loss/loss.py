@@ -191,3 +191,66 @@ def value_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
     sums = acc.tolist()
     denom = max(sums[4], 1.0)
     return loss, {"vf_loss": 0.5 * sums[0], "vf_clipfrac": sums[1] / denom, "vpred_mean": sums[2] / denom}
+
+
+class _CovPolicyLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, kind, batch, rows, hp):
+        acc, grad, _, _ = _ops.cov_policy_loss(
+            kind, log_probs, batch["old_log_probs"], batch["advantages"], batch["response_mask"],
+            batch["sampler_is_weights"], rows, **hp,
+        )
+        ctx.save_for_backward(grad, acc)
+        ctx.in_dtype = log_probs.dtype
+        ctx.mark_non_differentiable(acc)
+        return acc[0].clone(), acc
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_acc):
+        grad, acc = ctx.saved_tensors
+        return (grad * (g_loss * acc[5])).to(ctx.in_dtype), None, None, None, None
+
+
+def _run_cov(kind: int, data, config, hp: dict, default_token_reduce: str):
+    b = data.batch
+    log_probs = b["log_probs"]
+    agg = _aggregation(b, config, default_token_reduce)
+    _lib.require_device(log_probs, "policy loss")
+    rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
+    tensors = {"old_log_probs": b["old_log_probs"], "advantages": b["advantages"],
+               "response_mask": b["response_mask"], "sampler_is_weights": b.get("sampler_is_weights", None)}
+    loss, acc = _CovPolicyLoss.apply(log_probs, kind, tensors, rows, dict(**hp, **agg))
+    sums = acc.tolist()
+    return loss, sums, max(sums[4], 1.0)
+
+
+@register_loss(LossFn.KL_COV)
+def kl_cov_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """KL-Cov (loss.py:283-352): ``-A * ratio`` everywhere, plus ``ppo_kl_coef * |log ratio|`` on the
+    ``kl_cov_ratio`` share of response tokens with the largest advantage / log-prob covariance.  The reference
+    takes that top-k on the host; here a radix select finds it on the device.  Defaults sum / token-mean."""
+    ratio = config.get("kl_cov_ratio", 0.0002)
+    assert ratio > 0, "kl_cov_ratio must be > 0"
+    loss, sums, denom = _run_cov(0, data, config, dict(select_ratio=ratio, kl_coef=config.get("ppo_kl_coef", 1.0)),
+                                 "sum")
+    return loss, {"ppo_kl": sums[2] / denom}
+
+
+@register_loss(LossFn.CLIP_COV)
+def clip_cov_loss_fn(data, config) -> tuple[torch.Tensor, dict[str, Any]]:
+    """Clip-Cov (loss.py:198-280): the PPO clipped surrogate with a random ``clip_cov_ratio`` share of the
+    unclipped tokens whose covariance lies in ``(clip_cov_lb, clip_cov_ub)`` dropped from the loss.  The draw
+    takes its seed from torch's CPU generator, so ``torch.manual_seed`` makes it repeatable, as it does the
+    reference's ``randperm``.  Code defaults mean / token-mean (:265)."""
+    clip = config.get("clip_ratio", 0.2)
+    lo = config.get("clip_ratio_low", None)
+    hi = config.get("clip_ratio_high", None)
+    lo = clip if lo is None else lo
+    hi = clip if hi is None else hi
+    ratio = config.get("clip_cov_ratio", 0.0002)
+    assert ratio > 0, "clip_cov_ratio must be > 0"
+    seed = int(torch.randint(0, 2**31 - 1, (1,)).item())
+    hp = dict(select_ratio=ratio, ratio_lo=1 - lo, ratio_hi=1 + hi, cov_lb=config.get("clip_cov_lb", 1.0),
+              cov_ub=config.get("clip_cov_ub", 5.0), seed=seed)
+    loss, sums, denom = _run_cov(1, data, config, hp, "mean")
+    return loss, {"pg_clipfrac": sums[1] / denom, "ppo_kl": sums[2] / denom}

@@ -25,6 +25,8 @@ class LossFn(str, Enum):
     PPO = "ppo"
     GSPO = "gspo"
     GPG = "gpg"
+    CLIP_COV = "clip_cov"
+    KL_COV = "kl_cov"
     CISPO = "cispo"
     REINFORCE = "reinforce"
     GEO_MEAN = "geo_mean"

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 9
+#define AXON_AMD_ABI_VERSION 10
 
 enum {
   AXON_OK = 0,
@@ -348,6 +348,42 @@ int axon_masked_whiten(const float* x, const void* mask, int mask_kind, int64_t 
 int axon_group_scalar(int mode, const float* scores, const float* lens, const int32_t* members,
                       const int32_t* offsets, int64_t n_rows, int64_t n_groups, float eps,
                       int normalize, float coef, float threshold, float* scalar, void* stream);
+
+/* Token selection of the covariance-based losses (axon/trainer/algos/loss/loss.py):
+ *   kind 0: kl_cov_loss_fn :311-330.  Over the tokens with mask > 0: covariance
+ *           (A - mean A) * (logp - mean logp) with plain means; the k = max(1, int(count * ratio)) largest
+ *           are selected (torch.topk there).
+ *   kind 1: clip_cov_loss_fn :238-261.  Means are masked_mean; candidates are the tokens with mask > 0 that
+ *           the PPO clip leaves alone (pg_losses2 <= pg_losses1, bounds ratio_lo / ratio_hi as in
+ *           axon_policy_loss) and whose covariance lies in (cov_lb, cov_ub);
+ *           k = min(max(int(ratio * sum mask), 1), candidates) of them are selected uniformly at random
+ *           (torch.randperm there; here the k largest of a hash of (token index, seed)).
+ * keys [n_slots] (uint32) and state (axon_cov_select_state_bytes() bytes, 8-byte aligned) are outputs that
+ * axon_cov_policy_loss reads; state starts with uint32 threshold, remaining, candidates, ties, then
+ * int64 index_limit, float mean_a, mean_b, count, uint32 k.  Equal keys at the threshold go to the lowest
+ * token indices (the reference leaves that order to the library).  workspace:
+ * axon_cov_select_workspace_bytes(n_slots) bytes.  All arrays 16-byte aligned.  The histograms use integer
+ * atomics only: the selection is reproducible. */
+int64_t axon_cov_select_state_bytes(void);
+int64_t axon_cov_select_workspace_bytes(int64_t n_slots);
+int axon_cov_select(int kind, const float* logp, const float* old_logp, const float* adv,
+                    const void* mask, int mask_kind, int64_t n_slots, double ratio, float cov_lb,
+                    float cov_ub, float ratio_lo, float ratio_hi, uint32_t seed, uint32_t* keys,
+                    void* state, void* workspace, void* stream);
+
+/* The loss and gradient that go with axon_cov_select, aggregated as in axon_policy_loss (same row_scale /
+ * uniform_scale / post_normalize / valid_count / acc / partials conventions):
+ *   kind 0: kl_cov_loss_fn :303-345: -A*ratio, plus kl_coef * |clamped log ratio| on the selected tokens;
+ *           acc[1] = sum mask*selected, acc[2] = sum mask*|clamped log ratio|
+ *   kind 1: clip_cov_loss_fn :229-266: max(-A*ratio, -A*clamp(ratio)) with the selected tokens zeroed;
+ *           acc[1] = sum mask*selected, acc[2] = sum mask*(-(clamped log ratio)) */
+int axon_cov_policy_loss(int kind, const float* logp, const float* old_logp, const float* adv,
+                         const void* mask, int mask_kind, const float* is_weights,
+                         const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                         int64_t uniform_len, const float* row_scale, float uniform_scale,
+                         int post_normalize, const int64_t* valid_count, float ratio_lo,
+                         float ratio_hi, float kl_coef, const uint32_t* keys, const void* state,
+                         float* grad, float* acc, float* partials, void* stream);
 
 /* Per-token KL penalty against a reference policy, kl_penalty / kl_penalty_forward
  * (axon/utils/rl/kl.py:154-245): kl_type 1 "kl"/"k1", 2 "abs", 3 "mse"/"k2", 4 "low_var_kl"/"k3";

@@ -1,7 +1,8 @@
 """Oracle: loss aggregation and the PPO / GSPO clipped losses in plain torch (CPU, autograd).
 
 Restates axon/trainer/algos/loss/utils.py:88-251 (``masked_mean``, ``agg_loss``) and
-axon/trainer/algos/loss/loss.py:47-180 (``ppo_loss_fn``, ``gspo_loss_fn``) on plain
+axon/trainer/algos/loss/loss.py:47-180 (``ppo_loss_fn``, ``gspo_loss_fn``; further down ``clip_cov_loss_fn``
+:198-280 and ``kl_cov_loss_fn`` :283-352) on plain
 tensors (no DataProto), keeping the order of operations so autograd reproduces the
 reference's gradient conventions (clamp passes gradient at the bound, maximum/min
 split ties evenly).
@@ -206,3 +207,80 @@ def geo_mean_loss(log_prob, old_log_prob, advantages, response_mask, *, clip_rat
     return loss, {"pg_clipfrac": masked_mean((clipped * (advantages > 0)).float(), response_mask).item(),
                   "ppo_kl": masked_mean(-nak, response_mask).item(),
                   "pg_clipfrac_lower": masked_mean((clipped * (advantages < 0)).float(), response_mask).item()}
+
+
+def kl_cov_loss(log_prob, old_log_prob, advantages, response_mask, *, kl_cov_ratio=0.0002, ppo_kl_coef=1.0,
+                sampler_is_weights=None, token_reduce="sum", batch_reduce="token-mean", **agg_kwargs):
+    """loss.py:283-352.  ``(loss, metrics, selected)``; selected = flat indices that carry the KL term."""
+    nak = torch.clamp(log_prob - old_log_prob, -20.0, 20.0)
+    abs_kl = nak.abs()
+    ratio = torch.exp(nak)
+    pg1 = -advantages * ratio
+    pg_kl = -advantages * ratio + ppo_kl_coef * abs_kl
+    losses = pg1.clone()
+    valid = response_mask > 0
+    valid_idx = torch.nonzero(valid.reshape(-1), as_tuple=True)[0]
+    v_adv = advantages[valid].detach().reshape(-1)
+    v_lp = log_prob[valid].detach().reshape(-1)
+    picked = torch.empty(0, dtype=torch.long)
+    if min(kl_cov_ratio, len(v_adv)) != 0 and len(v_adv) > 0:
+        cov = (v_adv - v_adv.mean()) * (v_lp - v_lp.mean())
+        k = max(1, int(len(cov) * kl_cov_ratio))
+        picked = valid_idx[torch.topk(cov, k, largest=True).indices]
+        t = advantages.shape[1]
+        losses[picked // t, picked % t] = pg_kl[picked // t, picked % t]
+    if sampler_is_weights is not None:
+        losses = losses * sampler_is_weights
+    loss = agg_loss(losses, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    return loss, {"ppo_kl": float(masked_mean(abs_kl, response_mask).detach())}, picked
+
+
+def clip_cov_candidates(log_prob, old_log_prob, advantages, response_mask, *, clip_ratio=0.2, clip_ratio_low=None,
+                        clip_ratio_high=None, clip_cov_ratio=0.0002, clip_cov_lb=1.0, clip_cov_ub=5.0):
+    """loss.py:226-252: ``(candidate mask, clip_num)``: the tokens the random pick draws from and how many it may
+    take."""
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    ratio = torch.exp(torch.clamp(log_prob - old_log_prob, -20.0, 20.0)).detach()
+    pg1 = -advantages * ratio
+    pg2 = -advantages * torch.clamp(ratio, 1 - lo, 1 + hi)
+    clip_by_origin = (pg2 > pg1) & (response_mask > 0)
+    cov = (advantages - masked_mean(advantages, response_mask)) * (
+        log_prob.detach() - masked_mean(log_prob.detach(), response_mask))
+    cov = cov.clone()
+    cov[response_mask == 0] = -torch.inf
+    cov[clip_by_origin] = -torch.inf
+    clip_num = max(int(clip_cov_ratio * response_mask.sum().item()), 1)
+    return (cov < clip_cov_ub) & (cov > clip_cov_lb) & (response_mask > 0), clip_num
+
+
+def clip_cov_loss(log_prob, old_log_prob, advantages, response_mask, *, selected=None, clip_ratio=0.2,
+                  clip_ratio_low=None, clip_ratio_high=None, clip_cov_ratio=0.0002, clip_cov_lb=1.0, clip_cov_ub=5.0,
+                  sampler_is_weights=None, token_reduce="mean", batch_reduce="token-mean", **agg_kwargs):
+    """loss.py:198-280.  The reference draws the zeroed tokens with ``torch.randperm``; ``selected`` (a boolean
+    mask of the drawn tokens) replaces that draw so that two implementations can be compared on one draw."""
+    lo = clip_ratio if clip_ratio_low is None else clip_ratio_low
+    hi = clip_ratio if clip_ratio_high is None else clip_ratio_high
+    nak = torch.clamp(log_prob - old_log_prob, -20.0, 20.0)
+    ratio = torch.exp(nak)
+    pg1 = -advantages * ratio
+    pg2 = -advantages * torch.clamp(ratio, 1 - lo, 1 + hi)
+    if selected is None:
+        cand, clip_num = clip_cov_candidates(log_prob, old_log_prob, advantages, response_mask, clip_ratio=clip_ratio,
+                                             clip_ratio_low=clip_ratio_low, clip_ratio_high=clip_ratio_high,
+                                             clip_cov_ratio=clip_cov_ratio, clip_cov_lb=clip_cov_lb,
+                                             clip_cov_ub=clip_cov_ub)
+        idx = torch.nonzero(cand.reshape(-1)).flatten()
+        idx = idx[torch.randperm(len(idx))[: min(clip_num, len(idx))]]
+        selected = torch.zeros(cand.numel(), dtype=torch.bool)
+        selected[idx] = True
+        selected = selected.view_as(cand)
+    corr = torch.ones_like(advantages)
+    corr[selected] = 0
+    losses = torch.maximum(pg1, pg2) * corr
+    if sampler_is_weights is not None:
+        losses = losses * sampler_is_weights
+    loss = agg_loss(losses, response_mask, token_reduce=token_reduce, batch_reduce=batch_reduce, **agg_kwargs)
+    metrics = {"pg_clipfrac": float(masked_mean((corr == 0).float(), response_mask)),
+               "ppo_kl": float(masked_mean(-nak, response_mask).detach())}
+    return loss, metrics

@@ -299,3 +299,161 @@ def test_value_loss_known_answers_gpu():
     assert loss.item() == pytest.approx(0.5 * (0.64 + 0.16 + 2.25 + 4.0) / 4, rel=1e-6)
     assert torch.allclose(vp.grad.cpu(), T([[-0.8, 0.4, 0.0, -2.0]]) / 4, atol=1e-6)
     assert m["vf_clipfrac"] == pytest.approx(0.25)
+
+
+# ---- KL-Cov / Clip-Cov -----------------------------------------------------------------------------------
+from oracle import loss as OL  # noqa: E402
+
+
+def _selected(keys, state, n):
+    """The selection rule of the library, replayed on the host from its outputs."""
+    raw = state.cpu().numpy().tobytes()
+    thr, k = np.frombuffer(raw[0:4], np.uint32)[0], np.frombuffer(raw[36:40], np.uint32)[0]
+    limit = np.frombuffer(raw[16:24], np.int64)[0]
+    key = keys.cpu().numpy()[:n].view(np.uint32)
+    idx = np.arange(n)
+    hit = (key != 0) & ((key > thr) | ((key == thr) & (idx < limit)))
+    return torch.from_numpy(hit if k > 0 else np.zeros(n, bool))
+
+
+def _cov_batch(b=16, t=512, seed=41):
+    g = torch.Generator().manual_seed(seed)
+    old = -torch.empty(b, t).exponential_(1.0, generator=g)
+    lp = old + 0.1 * torch.randn(b, t, generator=g)
+    adv = torch.randn(b, 1, generator=g).expand(b, t).contiguous() + 0.1 * torch.randn(b, t, generator=g)
+    mask = (torch.rand(b, t, generator=g) > 0.3).float()
+    mask[3] = 0
+    isw = torch.rand(b, t, generator=g) + 0.5
+    return lp, old, adv, mask, isw
+
+
+@pytest.mark.parametrize("tr,br", [("sum", "token-mean"), ("mean", "step-mean")])
+@pytest.mark.parametrize("ratio,with_isw", [(0.002, False), (0.05, True)])
+def test_kl_cov_vs_oracle(ratio, with_isw, tr, br):
+    lp, old, adv, mask, isw = _cov_batch()
+    ref_in = lp.clone().requires_grad_(True)
+    ref_loss, ref_m, picked = OL.kl_cov_loss(ref_in, old, adv, mask, kl_cov_ratio=ratio, ppo_kl_coef=0.7,
+                                             sampler_is_weights=isw if with_isw else None, token_reduce=tr,
+                                             batch_reduce=br)
+    ref_loss.backward()
+    # the selected token indices, bit-exact
+    rows = _ops.rows_of(lp.to(DEV))
+    _, _, keys, state = _ops.cov_policy_loss(0, lp.to(DEV), old.to(DEV), adv.to(DEV), mask.to(DEV), None, rows,
+                                             select_ratio=ratio, kl_coef=0.7, token_reduce=tr, batch_reduce=br)
+    got = torch.nonzero(_selected(keys, state, lp.numel())).flatten()
+    assert got.tolist() == sorted(picked.tolist())
+    # loss, gradient and metric through the registry
+    x = lp.to(DEV).requires_grad_(True)
+    tensors = {"old_log_probs": old, "advantages": adv, "response_mask": mask}
+    if with_isw:
+        tensors["sampler_is_weights"] = isw
+    data = _proto(tensors)
+    data.batch["log_probs"] = x
+    loss, m = compute_loss_fn(data, "kl_cov", {"kl_cov_ratio": ratio, "ppo_kl_coef": 0.7, "token_reduce": tr,
+                                               "batch_reduce": br})
+    loss.backward()
+    assert loss.item() == pytest.approx(ref_loss.item(), rel=1e-4)
+    assert rel_l2(x.grad, ref_in.grad) < 1e-5
+    assert m["ppo_kl"] == pytest.approx(ref_m["ppo_kl"], rel=1e-4)
+
+
+def test_kl_cov_worked_example_ties_and_errors_gpu():
+    adv = T([[1.0, -1.0, 2.0, 0.0]])
+    lp = T([[-1.0, -2.0, -0.5, -3.0]])
+    old = lp - T([[0.1, -0.2, 0.3, 0.0]])
+    data = _proto({"log_probs": lp, "old_log_probs": old, "advantages": adv, "response_mask": torch.ones(1, 4)})
+    loss, m = compute_loss_fn(data, "kl_cov", {"kl_cov_ratio": 0.25, "ppo_kl_coef": 2.0})
+    import math
+    base = -1.0 * math.exp(0.1) + 1.0 * math.exp(-0.2) - 2.0 * math.exp(0.3)
+    assert loss.item() == pytest.approx((base + 2.0 * 0.3) / 4, rel=1e-5)
+    assert m["ppo_kl"] == pytest.approx(0.15, rel=1e-5)
+    with pytest.raises(AssertionError, match="kl_cov_ratio must be > 0"):
+        compute_loss_fn(data, "kl_cov", {"kl_cov_ratio": 0})
+    # every covariance equal (constant advantage): the k lowest-index response tokens are taken
+    lp2, old2, _, mask, _ = _cov_batch(4, 300, seed=43)
+    adv2 = torch.full_like(lp2, 0.5)
+    rows = _ops.rows_of(lp2.to(DEV))
+    acc, _, keys, state = _ops.cov_policy_loss(0, lp2.to(DEV), old2.to(DEV), adv2.to(DEV), mask.to(DEV), None, rows,
+                                               select_ratio=0.01, kl_coef=1.0, token_reduce="sum",
+                                               batch_reduce="token-mean")
+    k = max(1, int(int(mask.sum()) * 0.01))
+    got = torch.nonzero(_selected(keys, state, lp2.numel())).flatten()
+    assert got.tolist() == torch.nonzero(mask.flatten() > 0).flatten()[:k].tolist()
+    nak = (lp2 - old2).flatten()
+    per_tok = -0.5 * torch.exp(nak)
+    per_tok[got] += nak[got].abs()
+    assert acc[0].item() == pytest.approx(float((per_tok * mask.flatten()).sum() / mask.sum()), rel=1e-4)
+    # an all-zero mask selects nothing and gives a zero loss
+    acc, grad, keys, state = _ops.cov_policy_loss(0, lp2.to(DEV), old2.to(DEV), adv2.to(DEV),
+                                                  torch.zeros_like(mask).to(DEV), None, rows, select_ratio=0.01,
+                                                  token_reduce="sum", batch_reduce="token-mean")
+    assert acc[0].item() == 0.0 and not _selected(keys, state, lp2.numel()).any() and (grad == 0).all()
+
+
+@pytest.mark.parametrize("tr,br", [("mean", "token-mean"), ("sum", "step-mean")])
+@pytest.mark.parametrize("ratio", [0.002, 0.5])
+def test_clip_cov_vs_oracle_on_the_same_draw(ratio, tr, br):
+    lp, old, adv, mask, isw = _cov_batch(seed=47)
+    adv = adv * 2
+    kw = dict(clip_ratio_low=0.2, clip_ratio_high=0.28, clip_cov_ratio=ratio, clip_cov_lb=0.5, clip_cov_ub=5.0)
+    cand, clip_num = OL.clip_cov_candidates(lp, old, adv, mask, **kw)
+    rows = _ops.rows_of(lp.to(DEV))
+    draws = []
+    for seed in (1, 2):
+        acc, grad, keys, state = _ops.cov_policy_loss(
+            1, lp.to(DEV), old.to(DEV), adv.to(DEV), mask.to(DEV), isw.to(DEV), rows, select_ratio=ratio,
+            ratio_lo=1 - 0.2, ratio_hi=1 + 0.28, cov_lb=0.5, cov_ub=5.0, seed=seed, token_reduce=tr, batch_reduce=br)
+        sel = _selected(keys, state, lp.numel()).view_as(cand)
+        # the draw: exactly min(clip_num, candidates) tokens, every one a candidate
+        assert int(sel.sum()) == min(clip_num, int(cand.sum())) and not (sel & ~cand).any()
+        draws.append(sel)
+        ref_in = lp.clone().requires_grad_(True)
+        ref_loss, ref_m = OL.clip_cov_loss(ref_in, old, adv, mask, selected=sel, sampler_is_weights=isw,
+                                           token_reduce=tr, batch_reduce=br, **kw)
+        ref_loss.backward()
+        sums = acc.tolist()
+        assert sums[0] == pytest.approx(ref_loss.item(), rel=1e-4)
+        assert rel_l2(grad * sums[5], ref_in.grad) < 1e-5
+        assert sums[1] / max(sums[4], 1) == pytest.approx(ref_m["pg_clipfrac"], rel=1e-5)
+        assert sums[2] / max(sums[4], 1) == pytest.approx(ref_m["ppo_kl"], rel=1e-4, abs=1e-7)
+    if clip_num < int(cand.sum()):
+        assert not torch.equal(draws[0], draws[1])  # another seed, another draw
+    else:
+        assert torch.equal(draws[0], cand)  # more wanted than there are: every candidate goes
+
+
+def test_clip_cov_registry_seed_and_errors():
+    lp, old, adv, mask, _ = _cov_batch(seed=49)
+    data = _proto({"log_probs": lp, "old_log_probs": old, "advantages": adv * 2, "response_mask": mask})
+    args = {"clip_cov_ratio": 0.01, "clip_cov_lb": 0.5}
+    torch.manual_seed(5)
+    l1, m1 = compute_loss_fn(data, "clip_cov", args)
+    torch.manual_seed(5)
+    l2, m2 = compute_loss_fn(data, "clip_cov", args)
+    assert l1.item() == l2.item() and m1 == m2 and set(m1) == {"pg_clipfrac", "ppo_kl"}
+    want = max(int(0.01 * float(mask.sum())), 1)
+    assert m1["pg_clipfrac"] == pytest.approx(want / float(mask.sum()), rel=1e-5)
+    with pytest.raises(AssertionError, match="clip_cov_ratio must be > 0"):
+        compute_loss_fn(data, "clip_cov", {"clip_cov_ratio": 0})
+
+
+def test_cov_losses_packed_layout():
+    lens = [700, 33, 1, 1200, 64, 257]
+    n = sum(lens)
+    g = torch.Generator().manual_seed(53)
+    old = -torch.empty(n).exponential_(1.0, generator=g)
+    lp = old + 0.1 * torch.randn(n, generator=g)
+    adv = torch.randn(n, generator=g)
+    mask = (torch.rand(n, generator=g) > 0.2).float()
+    cu = W.cu_from_lengths(lens)
+    tmax = max(lens)
+    pad = lambda x: torch.stack([torch.nn.functional.pad(x[s:e], (0, tmax - (e - s)))  # noqa: E731
+                                 for s, e in zip(cu[:-1].tolist(), cu[1:].tolist())])
+    ref_loss, ref_m, _ = OL.kl_cov_loss(pad(lp), pad(old), pad(adv), pad(mask), kl_cov_ratio=0.01,
+                                        token_reduce="mean", batch_reduce="step-mean")
+    data = _proto({"log_probs": lp, "old_log_probs": old, "advantages": adv, "response_mask": mask},
+                  meta={"cu_seqlens": cu})
+    loss, m = compute_loss_fn(data, "kl_cov", {"kl_cov_ratio": 0.01, "token_reduce": "mean",
+                                               "batch_reduce": "step-mean"})
+    assert loss.item() == pytest.approx(ref_loss.item(), rel=1e-4)
+    assert m["ppo_kl"] == pytest.approx(ref_m["ppo_kl"], rel=1e-4)

@@ -287,3 +287,52 @@ def test_oracle_geo_mean_known_answer_and_by_hand():
     r1 = math.exp((-0.2 + 0.1) / 2)
     assert loss2.item() == pytest.approx((-1.0 * r0 + 1.0 * r1) / 2, rel=1e-6)
     assert met2["pg_clipfrac"] == pytest.approx(0.5) and met2["pg_clipfrac_lower"] == pytest.approx(0.25)
+
+
+# ---- KL-Cov / Clip-Cov (loss.py:198-352).  The reference's own tests (tests/trainer/algos/loss/test_loss.py:
+# 270-365) check shapes, metric keys and the ratio assertion only; the numbers below are worked by hand. ----
+def test_kl_cov_worked_example():
+    adv = torch.tensor([[1.0, -1.0, 2.0, 0.0]])
+    lp = torch.tensor([[-1.0, -2.0, -0.5, -3.0]], requires_grad=True)
+    d = torch.tensor([[0.1, -0.2, 0.3, 0.0]])
+    old = lp.detach() - d
+    # means 0.5 and -1.625: covariances .3125, .5625, 1.6875, .6875 -> k = max(1, int(4 * .25)) = 1 picks token 2
+    loss, m, picked = O.kl_cov_loss(lp, old, adv, torch.ones(1, 4), kl_cov_ratio=0.25, ppo_kl_coef=2.0)
+    assert picked.tolist() == [2]
+    base = [-1.0 * math.exp(0.1), 1.0 * math.exp(-0.2), -2.0 * math.exp(0.3), 0.0]
+    assert loss.item() == pytest.approx((sum(base) + 2.0 * 0.3) / 4, rel=1e-6)
+    assert m["ppo_kl"] == pytest.approx((0.1 + 0.2 + 0.3) / 4, rel=1e-6)
+    loss.backward()
+    expect = torch.tensor([[base[0], base[1], base[2] + 2.0, 0.0]]) / 4  # d/dlogp of -A e^d is itself; +coef*sign(d)
+    assert torch.allclose(lp.grad, expect, atol=1e-6)
+    # masked tokens neither enter the means nor get picked; half the tokens -> k = max(1, int(2 * .25)) = 1
+    mask = torch.tensor([[1.0, 1.0, 0.0, 0.0]])
+    _, _, picked = O.kl_cov_loss(lp.detach(), old, adv, mask, kl_cov_ratio=0.25)
+    assert picked.tolist() == [0]  # means 0 and -1.5: covariances .5 and .5 ... the first of two equal values
+    # a larger share picks more tokens: k = int(4 * .75) = 3 -> all but the smallest covariance
+    _, _, picked = O.kl_cov_loss(lp.detach(), old, adv, torch.ones(1, 4), kl_cov_ratio=0.75)
+    assert sorted(picked.tolist()) == [1, 2, 3]
+
+
+def test_clip_cov_worked_example():
+    adv = torch.tensor([[2.0, -1.0, 1.0, 3.0]])
+    lp = torch.tensor([[-1.0, -2.0, -0.5, -3.0]], requires_grad=True)
+    d = torch.tensor([[0.5, 0.1, -0.5, 0.0]])
+    old = lp.detach() - d
+    ones = torch.ones(1, 4)
+    # clip 0.2: ratios 1.649 (A>0: clipped at 1.2, pg2 > pg1 -> clipped by origin), 1.105, .607 (A>0: pg1 wins), 1
+    cand, clip_num = O.clip_cov_candidates(lp.detach(), old, adv, ones, clip_cov_ratio=0.3, clip_cov_lb=-1.0,
+                                            clip_cov_ub=10.0)
+    # means 1.25 and -1.625: covariances .46875, .84375, -.28125, -2.40625; token 0 clipped, token 3 below the band
+    assert cand.tolist() == [[False, True, True, False]] and clip_num == 1
+    sel = torch.tensor([[False, False, True, False]])
+    loss, m = O.clip_cov_loss(lp, old, adv, ones, selected=sel, token_reduce="sum")
+    terms = [-2.0 * 1.2, 1.0 * math.exp(0.1), 0.0, -3.0]
+    assert loss.item() == pytest.approx(sum(terms) / 4, rel=1e-6)
+    assert m["pg_clipfrac"] == pytest.approx(0.25) and m["ppo_kl"] == pytest.approx(-0.1 / 4, abs=1e-7)
+    loss.backward()
+    assert torch.allclose(lp.grad, torch.tensor([[0.0, math.exp(0.1), 0.0, -3.0]]) / 4, atol=1e-6)
+    # the random draw takes min(clip_num, candidates) tokens, all of them candidates
+    torch.manual_seed(0)
+    _, m = O.clip_cov_loss(lp.detach(), old, adv, ones, clip_cov_ratio=0.9, clip_cov_lb=-1.0, clip_cov_ub=10.0)
+    assert m["pg_clipfrac"] == pytest.approx(0.5)  # clip_num = int(.9 * 4) = 3, two candidates
