@@ -113,3 +113,78 @@ def test_qwen3_8b_shape_properties():
     assert rel_l2(dh[idx.to(DEV)], ref_dh) < 2e-2
     dh2, dw2 = _ops.lmhead_backward(2 * g, None, hd, wd, ld, lse, eb, 1.0)
     assert rel_l2(dh2, 2 * dh.float()) < 1e-2 and rel_l2(dw2, 2 * dw.float()) < 1e-2
+
+
+def test_micro_batched_dapo_chain_vs_whole_batch_oracle():
+    """The GPT-OSS-style configuration at reduced size (hidden 2880 kept: K not a multiple of 128): advantages and
+    dynamic sampling over all sequences, then head + DAPO loss per micro-batch of whole sequences with the
+    mini-batch-global ``valid_token_count``, dHidden per micro-batch and dWeight accumulated over them.  The
+    oracle evaluates the kept sequences as ONE batch: the micro-batch losses must add up to its loss and the
+    accumulated gradients must be its gradients."""
+    from axon_amd.utils.rl.utils import filter_zero_advantage_samples
+    h, v, groups, samples, tmax = 2880, 3000, 4, 3, 80
+    g = torch.Generator().manual_seed(61)
+    n_seq = groups * samples
+    lens = torch.randint(20, tmax + 1, (n_seq,), generator=g).tolist()
+    uid = W.uids_for(n_seq, samples)
+    score = (torch.rand(n_seq, generator=g) < 0.3).float()
+    score[0:3] = 1.0                      # group 0: all equal -> zero advantage -> dropped
+    score[3:6] = T_([1.0, 0.0, 0.0])      # the others mixed
+    score[6:9] = T_([0.0, 1.0, 1.0])
+    score[9:12] = T_([1.0, 0.0, 1.0])
+    rewards, mask = torch.zeros(n_seq, tmax), torch.zeros(n_seq, tmax)
+    for i, l in enumerate(lens):
+        mask[i, 1:l] = 1                   # position 0 is the prompt token
+        rewards[i, l - 1] = score[i]
+    # 1. advantages over every sequence, then dynamic sampling (row indices bit-exact against the oracle)
+    data = DataProto.from_dict(tensors={"token_level_rewards": rewards.to(DEV), "response_mask": mask.to(DEV),
+                                        "row": torch.arange(n_seq).to(DEV)})
+    data.non_tensor_batch["uid"] = uid
+    data = compute_advantage(data, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}})
+    gidx = torch.tensor(np.unique(uid, return_inverse=True)[1])
+    ref_adv = OA.grpo_advantage(rewards, mask, gidx, 1e-6)
+    kept = filter_zero_advantage_samples(data).batch["row"].tolist()
+    assert kept == OA.zero_advantage_keep_rows(ref_adv) == list(range(3, 12))
+    # 2. the kept sequences, packed, in micro-batches of three sequences
+    lens_k = [lens[i] for i in kept]
+    n = sum(lens_k)
+    hid, w, ids = W.lmhead_inputs(n, h, v, seed=62)
+    w = (w.float() * 6).bfloat16()
+    cu = W.cu_from_lengths(lens_k).long()
+    pack = lambda x: torch.cat([x[i, :lens[i]] for i in kept])  # noqa: E731
+    adv_p, mask_p = pack(data.batch["advantages"].cpu()), pack(mask)
+    labels = torch.roll(ids, -1)
+    old = OM.forward(hid, w, labels)[0]
+    old_tok = torch.zeros_like(old)
+    old_tok[1:] = old[:-1]
+    old_tok = old_tok - 0.05 * torch.randn(n, generator=g)
+    valid = int(mask_p.sum())
+    wd = w.to(DEV).requires_grad_(True)
+    total, dh_parts = 0.0, []
+    for first in range(0, len(kept), 3):
+        a, b = int(cu[first]), int(cu[min(first + 3, len(kept))])
+        cu_mb = (cu[first:first + 4] - a).int().to(DEV)
+        hd = hid[a:b].to(DEV).requires_grad_(True)
+        from axon_amd.utils.fsdp.forward_utils import packed_logprobs
+        lp, _ = packed_logprobs(hd, wd, ids[a:b].to(DEV), cu_mb)
+        mb = DataProto.from_dict(
+            tensors={"log_probs": lp, "old_log_probs": old_tok[a:b].to(DEV), "advantages": adv_p[a:b].to(DEV),
+                     "response_mask": mask_p[a:b].to(DEV),
+                     "valid_token_count": torch.full((b - a,), valid, dtype=torch.int64, device=DEV)},
+            meta_info={"cu_seqlens": cu_mb})
+        loss, _ = compute_loss_fn(mb, "ppo", {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28})
+        loss.backward()
+        total += loss.item()
+        dh_parts.append(hd.grad)
+    # 3. the oracle on the whole kept batch
+    rl = {"cu_seqlens": cu.int(), "token_level_rewards": pack(rewards), "response_mask": mask_p,
+          "uid": uid[kept]}
+    # every kept group is complete, so the group statistics of the kept rows equal those of the full batch
+    ref = oracle_chain(hid, w, labels, rl, old_tok)
+    assert total == pytest.approx(ref[0].item(), rel=1e-4, abs=1e-8)
+    assert rel_l2(torch.cat(dh_parts), ref[3]) < 2e-2
+    assert rel_l2(wd.grad, ref[4]) < 2e-2
+
+
+def T_(x):
+    return torch.tensor(x)
