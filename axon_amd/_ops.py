@@ -57,6 +57,14 @@ def mask_arg(mask: torch.Tensor):
     return mask.contiguous(), MASK_F32
 
 
+def _same_len(what: str, n: int, **tensors) -> None:
+    """The kernels index every operand with the same token (or row) index: a shorter operand would be read
+    out of bounds, so the lengths are checked here, on the host."""
+    for name, t in tensors.items():
+        if t is not None and int(t.numel()) != n:
+            raise ValueError(f"{what}: {name} has {int(t.numel())} elements, expected {n}")
+
+
 def _zeros(n, device, dtype=torch.float32):
     return torch.zeros(n, device=device, dtype=dtype)
 
@@ -76,6 +84,7 @@ def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=Tr
     """Per-row (count, sum of (a-b)*mask, any-flag); see axon_row_stats."""
     lib = _lib.load()
     require_device(a, "row_stats")
+    _same_len("row_stats", rows.n_slots, a=a, b=b, mask=mask)
     dev = a.device
     a = f32(a)
     b = f32(b) if b is not None else None
@@ -100,6 +109,7 @@ def group_stats(scores, gidx, n_groups, eps, norm_by_std=True, want_scalar=True)
     gidx = gidx.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
     n = int(scores.numel())
     stats = _zeros(3 * max(n_groups, 1), dev).view(3, -1)
+    _same_len("group_stats", n, gidx=gidx)
     scalar = torch.empty(n, device=dev, dtype=torch.float32) if want_scalar else None
     check(
         lib.axon_group_stats(ptr(scores), ptr(gidx), n, int(n_groups), float(eps), int(norm_by_std),
@@ -112,6 +122,8 @@ def group_stats(scores, gidx, n_groups, eps, norm_by_std=True, want_scalar=True)
 def row_broadcast_mask(row_scalar, mask, rows: Rows, clamp_abs=0.0):
     lib = _lib.load()
     require_device(row_scalar, "row_broadcast_mask")
+    _same_len("row_broadcast_mask", rows.n_slots, mask=mask)
+    _same_len("row_broadcast_mask", rows.n_rows, row_scalar=row_scalar)
     mk, kind = mask_arg(mask)
     out = torch.empty(rows.shape, device=row_scalar.device, dtype=torch.float32)
     check(
@@ -130,6 +142,7 @@ def reverse_scan(mode, rewards, values, mask, rows: Rows, *, gamma=1.0, lam=1.0,
     axon_reverse_scan."""
     lib = _lib.load()
     require_device(rewards, "reverse_scan")
+    _same_len("reverse_scan", rows.n_slots, rewards=rewards, values=values, mask=mask)
     dev = rewards.device
     rewards = f32(rewards)
     values = f32(values) if values is not None else None
@@ -153,6 +166,7 @@ def masked_whiten(x, mask, *, remask=False, inplace=False):
     ``remask``); returns ``(out, stats)`` with stats = device [mean, n, var, rsqrt(var + 1e-8)]."""
     lib = _lib.load()
     require_device(x, "masked_whiten")
+    _same_len("masked_whiten", int(x.numel()), mask=mask)
     dev = x.device
     xf = f32(x)
     mk, kind = mask_arg(mask)
@@ -204,6 +218,7 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
     """
     lib = _lib.load()
     require_device(old_lp, "sampler_correction")
+    _same_len("sampler_correction", rows.n_slots, old_log_probs=old_lp, sampler_log_probs=samp_lp, mask=mask)
     dev = old_lp.device
     old_lp, samp_lp = f32(old_lp), f32(samp_lp)
     mk, kind = mask_arg(mask)
@@ -236,6 +251,7 @@ def sampler_diag(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_lo, is_hi, rs
     (layout: axon_sampler_diag in include/axon_amd.h).  No host synchronisation."""
     lib = _lib.load()
     require_device(old_lp, "sampler_diag")
+    _same_len("sampler_diag", rows.n_slots, old_log_probs=old_lp, sampler_log_probs=samp_lp, mask=mask)
     dev = old_lp.device
     old_lp, samp_lp = f32(old_lp), f32(samp_lp)
     mk, kind = mask_arg(mask)
@@ -257,9 +273,11 @@ TOKEN_REDUCE = {"sum": 0, "mean": 1, "mean-norm": 2, "mean-program": 3}
 BATCH_REDUCE = {"token-mean": 0, "step-mean": 1, "program-mean": 2}
 
 
-def _i64_dev(x, dev):
+def _i64_dev(x, dev, n=None, what="count"):
     if x is None:
         return None
+    if n is not None and int(x.numel()) != n:
+        raise ValueError(f"{what} has {int(x.numel())} entries, expected one per row ({n})")
     t = torch.as_tensor(x)
     return t.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
 
@@ -274,6 +292,8 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     """
     lib = _lib.load()
     require_device(log_probs, "policy_loss")
+    _same_len("policy_loss", rows.n_slots, log_probs=log_probs, old_log_probs=old_log_probs, advantages=advantages,
+              mask=mask, is_weights=is_weights)
     dev = log_probs.device
     lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
     mk, mkind = mask_arg(mask)
@@ -291,9 +311,9 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
         cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
         row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
         row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
-        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
             lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr,
                                     br, ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
@@ -319,6 +339,8 @@ def cov_policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights
     acc[1] = number of selected tokens (mask-weighted)."""
     lib = _lib.load()
     require_device(log_probs, "cov_policy_loss")
+    _same_len("cov_policy_loss", rows.n_slots, log_probs=log_probs, old_log_probs=old_log_probs,
+              advantages=advantages, mask=mask, is_weights=is_weights)
     dev = log_probs.device
     lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
     mk, mkind = mask_arg(mask)
@@ -342,9 +364,9 @@ def cov_policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights
     if not one_pass:
         cnt, _, _ = row_stats(lp, None, mk, rows, want_sum=False)
         row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
             lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
                                     ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),
@@ -364,6 +386,8 @@ def gmpo_loss(log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows
     """GMPO loss and gradient; returns (acc[8], grad).  See axon_gmpo_loss."""
     lib = _lib.load()
     require_device(log_probs, "gmpo_loss")
+    _same_len("gmpo_loss", rows.n_slots, log_probs=log_probs, old_log_probs=old_log_probs, advantages=advantages,
+              mask=mask, is_weights=is_weights)
     dev = log_probs.device
     lp, old, adv = f32(log_probs), f32(old_log_probs), f32(advantages)
     mk, mkind = mask_arg(mask)
@@ -399,6 +423,7 @@ def kl_penalty(logprob, ref_logprob, kl_type: int, kl_plus: int):
     """Per-token estimate and its derivative w.r.t. logprob (both fp32, shape of logprob)."""
     lib = _lib.load()
     require_device(logprob, "kl_penalty")
+    _same_len("kl_penalty", int(logprob.numel()), ref_logprob=ref_logprob)
     lp, ref = f32(logprob), f32(ref_logprob)
     out, grad = torch.empty_like(lp), torch.empty_like(lp)
     check(lib.axon_kl_penalty(ptr(lp), ptr(ref), lp.numel(), kl_type, kl_plus, ptr(out), ptr(grad), stream_ptr()),
@@ -414,6 +439,8 @@ def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_red
     lib = _lib.load()
     anchor = entropy if entropy is not None else log_probs
     require_device(anchor, "side_terms")
+    _same_len("side_terms", rows.n_slots, entropy=entropy, log_probs=log_probs if kl_type else None,
+              ref_log_probs=ref_log_probs if kl_type else None, mask=mask)
     dev = anchor.device
     ent = f32(entropy) if entropy is not None else None
     lp = f32(log_probs) if kl_type else None
@@ -426,9 +453,9 @@ def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_red
     if not one_pass:
         cnt, _, _ = row_stats(anchor, None, mk, rows, want_sum=False)
         row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        prtc = _i64_dev(per_row_token_count, dev) if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev) if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev) if br == 2 else None
+        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
             lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
                                     ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),
@@ -503,6 +530,25 @@ def seq_start_flags(cu_seqlens, n_tokens: int):
     return flags
 
 
+def _head_operands(what, hidden, weight, labels, seq_start):
+    """Shapes and types the head's kernels assume; returns (tokens, hidden size, vocabulary)."""
+    if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
+        raise ValueError(f"{what}: hidden {tuple(hidden.shape)} and weight {tuple(weight.shape)} do not match")
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError(f"{what}: hidden and weight must be bf16")
+    if labels.dtype not in (torch.int32, torch.int64):
+        raise ValueError(f"{what}: labels must be int32 or int64")
+    if not (hidden.is_contiguous() and weight.is_contiguous() and labels.is_contiguous()):
+        raise ValueError(f"{what}: operands must be contiguous")
+    if weight.device != hidden.device or labels.device != hidden.device:
+        raise ValueError(f"{what}: operands live on different devices")
+    n = int(hidden.shape[0])
+    _same_len(what, n, labels=labels)
+    if seq_start is not None and int(seq_start.numel()) < n:
+        raise ValueError(f"{what}: seq_start has {int(seq_start.numel())} flags for {n} tokens")
+    return n, int(hidden.shape[1]), int(weight.shape[0])
+
+
 def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | None" = None, softcap: float = 0.0,
                    seq_start=None):
     """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]).  ``softcap`` > 0 soft-caps the logits
@@ -513,8 +559,7 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | Non
     into the timer and does not synchronise."""
     lib = _lib.load()
     require_device(hidden, "lmhead_forward")
-    n, h = hidden.shape
-    v = weight.shape[0]
+    n, h, v = _head_operands("lmhead_forward", hidden, weight, labels, seq_start)
     dev = hidden.device
     out = torch.empty(4, max(n, 1), device=dev, dtype=torch.float32)
     ws_bytes = lib.axon_lmhead_fwd_workspace_bytes(n, h, v)
@@ -537,8 +582,8 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
     lib = _lib.load()
     require_device(hidden, "lmhead_backward")
-    n, h = hidden.shape
-    v = weight.shape[0]
+    n, h, v = _head_operands("lmhead_backward", hidden, weight, labels, seq_start)
+    _same_len("lmhead_backward", n, dlogprobs=dlogprobs, dentropy=dentropy, lse=lse, entropy_b=entropy_b)
     dev = hidden.device
     d_hidden = torch.empty_like(hidden)
     d_weight = torch.empty_like(weight)

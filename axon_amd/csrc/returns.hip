@@ -91,14 +91,16 @@ __device__ __forceinline__ void scan_load(ScanBlock& x, const float* __restrict_
 template <int MK, int MODE>
 __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(
     const float* __restrict__ rewards, const float* __restrict__ values,
-    const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows,
+    const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots,
     int64_t uniform_len, float gamma, float gamma_lam, const float* __restrict__ row_baseline,
     float* __restrict__ adv, float* __restrict__ ret, int vec_ok) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row = (int64_t)blockIdx.x * (kBlock / kWave) + (threadIdx.x / kWave);
   if (row >= n_rows) return;  // whole wavefronts leave together; no workgroup barrier below
-  const int64_t begin = uniform_len > 0 ? row * uniform_len : (int64_t)cu[row];
-  const int64_t stop = uniform_len > 0 ? begin + uniform_len : (int64_t)cu[row + 1];
+  int64_t begin = uniform_len > 0 ? row * uniform_len : (int64_t)cu[row];
+  int64_t stop = uniform_len > 0 ? begin + uniform_len : (int64_t)cu[row + 1];
+  begin = begin < 0 ? 0 : begin;              // offsets outside the arrays (caller error) touch nothing
+  stop = stop > n_slots ? n_slots : stop;
   if (stop <= begin) return;
   const float base = (MODE == kScanSuffixSum && row_baseline) ? row_baseline[row] : 0.f;
   float carry0 = 0.f, carry1 = 0.f;  // the recurrences' values at the token after the current window
@@ -347,8 +349,8 @@ namespace {
 
 template <int MK>
 int launch_scan(int mode, const float* rewards, const float* values, const void* mask,
-                const int32_t* cu, int64_t n_rows, int64_t uniform_len, float gamma, float gamma_lam,
-                const float* row_baseline, float* adv, float* ret, hipStream_t st) {
+                const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len, float gamma,
+                float gamma_lam, const float* row_baseline, float* adv, float* ret, hipStream_t st) {
   // 16-byte accesses need every array on a 16-byte boundary (an int64 mask then is on 32)
   const int vec_ok = ((reinterpret_cast<uintptr_t>(rewards) | reinterpret_cast<uintptr_t>(values) |
                        reinterpret_cast<uintptr_t>(mask) | reinterpret_cast<uintptr_t>(adv) |
@@ -356,7 +358,7 @@ int launch_scan(int mode, const float* rewards, const float* values, const void*
   const dim3 grid((unsigned)((n_rows + (kBlock / kWave) - 1) / (kBlock / kWave))), blk(kBlock);
 #define AXON_SCAN(M)                                                                              \
   hipLaunchKernelGGL((reverse_scan_kernel<MK, M>), grid, blk, 0, st, rewards, values, mask, cu,   \
-                     n_rows, uniform_len, gamma, gamma_lam, row_baseline, adv, ret, vec_ok)
+                     n_rows, n_slots, uniform_len, gamma, gamma_lam, row_baseline, adv, ret, vec_ok)
   switch (mode) {
     case kScanGae: AXON_SCAN(kScanGae); break;
     case kScanGaeResponseOnly: AXON_SCAN(kScanGaeResponseOnly); break;
@@ -412,9 +414,9 @@ extern "C" int axon_reverse_scan(int mode, const float* rewards, const float* va
   float* adv_out = (mode == kScanDiscounted) ? nullptr : adv;
   const hipStream_t st = (hipStream_t)stream;
   if (mask_kind == AXON_MASK_F32)
-    return launch_scan<AXON_MASK_F32>(mode, rewards, values, mask, cu_seqlens, n_rows, uniform_len,
+    return launch_scan<AXON_MASK_F32>(mode, rewards, values, mask, cu_seqlens, n_rows, n_slots, uniform_len,
                                       gamma, gamma_lam, row_baseline, adv_out, ret, st);
-  return launch_scan<AXON_MASK_I64>(mode, rewards, values, mask, cu_seqlens, n_rows, uniform_len,
+  return launch_scan<AXON_MASK_I64>(mode, rewards, values, mask, cu_seqlens, n_rows, n_slots, uniform_len,
                                     gamma, gamma_lam, row_baseline, adv_out, ret, st);
 }
 

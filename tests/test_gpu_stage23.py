@@ -726,3 +726,30 @@ def test_geo_mean_known_answer_and_packed_gpu():
     l_pad, _ = compute_loss_fn(_loss_proto(d), "geo_mean", {})
     # the mean of +-O(1) row terms cancels to ~3e-4: compare on the scale of the terms
     assert l_pk.item() == pytest.approx(l_pad.item(), abs=1e-6)
+
+
+# ---- operand checks on the host: a short operand never reaches a kernel ------------------------------------
+def test_operand_length_mismatch_raises():
+    x = torch.zeros(4, 64, device=DEV)
+    short = torch.zeros(4, 32, device=DEV)
+    rows = _ops.rows_of(x)
+    with pytest.raises(ValueError, match="advantages has 128 elements, expected 256"):
+        _ops.policy_loss(0, x, x, short, x, None, rows, token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8,
+                         ratio_hi=1.2, clip_c=3.0)
+    with pytest.raises(ValueError, match="mask has 128"):
+        _ops.row_stats(x, None, short, rows)
+    with pytest.raises(ValueError, match="sampler_log_probs has 128"):
+        _ops.sampler_correction(x, short, x, rows, is_mode=1, is_threshold=2.0, rs_mode=0, rs_lr_lo=0.0, rs_lr_hi=0.0,
+                                log_veto=None)
+    with pytest.raises(ValueError, match="values has 128"):
+        _ops.reverse_scan(_ops.SCAN_GAE, x, short, x, rows)
+    with pytest.raises(ValueError, match="one per row"):
+        _ops.policy_loss(0, x, x, x, x, None, rows, token_reduce="mean-program", batch_reduce="token-mean",
+                         ratio_lo=0.8, ratio_hi=1.2, clip_c=3.0, num_program_tokens=torch.ones(3, dtype=torch.int64))
+    hid = torch.zeros(8, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(100, 32, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="do not match"):
+        _ops.lmhead_forward(hid, w, torch.zeros(8, dtype=torch.int32, device=DEV), 1.0)
+    with pytest.raises(ValueError, match="labels has 7"):
+        _ops.lmhead_forward(hid, torch.zeros(100, 64, device=DEV, dtype=torch.bfloat16),
+                            torch.zeros(7, dtype=torch.int32, device=DEV), 1.0)
