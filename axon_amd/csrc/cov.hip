@@ -60,20 +60,27 @@ __global__ __launch_bounds__(kBlock) void cov_moments_finish_kernel(const float*
                                                                     int n_blocks, int kind, double ratio,
                                                                     SelectState* st, uint32_t* hist) {
   __shared__ float lds_red[3 * (kBlock / kWave)];
+  __shared__ double lds_cnt[kBlock / kWave];
   float a[3] = {0.f, 0.f, 0.f};
+  double cnt = 0.0;  // a workgroup's count is exact in fp32; their total may not be
   for (int b = threadIdx.x; b < n_blocks; b += kBlock) {
     a[0] += partials[(size_t)b * kPartialStride];
     a[1] += partials[(size_t)b * kPartialStride + 1];
     a[2] += partials[(size_t)b * kPartialStride + 2];
+    cnt += (double)partials[(size_t)b * kPartialStride + 2];
   }
-  block_sum<3>(a, lds_red);
+  for (int off = 32; off > 0; off >>= 1) cnt += __shfl_down(cnt, off, kWave);
+  if ((threadIdx.x & (kWave - 1)) == 0) lds_cnt[threadIdx.x / kWave] = cnt;
+  block_sum<3>(a, lds_red);  // has a workgroup barrier: lds_cnt is visible after it
   for (int b = threadIdx.x; b < kBins; b += kBlock) hist[b] = 0;
   if (threadIdx.x == 0) {
+    double total = 0.0;
+    for (int w = 0; w < kBlock / kWave; ++w) total += lds_cnt[w];
     const float den = (kind == 0) ? a[2] : fmaxf(a[2], 1.f);
     st->mean_a = a[2] > 0.f || kind == 1 ? a[0] / den : 0.f;
     st->mean_b = a[2] > 0.f || kind == 1 ? a[1] / den : 0.f;
     st->count = a[2];
-    const long long want = (long long)((double)a[2] * ratio);
+    const long long want = (long long)(total * ratio);
     uint32_t k = (uint32_t)(want < 1 ? 1 : (want > 0x7fffffffLL ? 0x7fffffffLL : want));
     if (kind == 0 && !(a[2] > 0.f)) k = 0;
     st->k = k;

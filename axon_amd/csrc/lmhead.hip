@@ -171,22 +171,49 @@ __global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restric
   if (s0 >= 0 && s0 < n_tokens && cu[i + 1] > s0) is_start[s0] = 1;  // empty sequences own no position
 }
 
-// Merge partials: lse, entropy_b, entropy.  One thread per token.
-__global__ __launch_bounds__(256) void lmhead_merge_kernel(
+// Merge partials: lse, entropy_b, entropy.  A workgroup owns kMergeTokens consecutive tokens; its
+// kMergeGroups thread groups each fold every kMergeGroups-th partial of a token (four loads ahead of the
+// fold), then the first group folds the groups' results in group order.
+constexpr int kMergeTokens = 32;
+constexpr int kMergeGroups = 8;
+
+__global__ __launch_bounds__(kMergeTokens * kMergeGroups) void lmhead_merge_kernel(
     const float* __restrict__ pm, const float* __restrict__ ps, const float* __restrict__ pe,
     int parts, int n_tokens, float* __restrict__ lse, float* __restrict__ entropy_b,
     float* __restrict__ entropy, float* __restrict__ fin_max, float* __restrict__ fin_log2s,
     const uint8_t* __restrict__ is_start) {
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
-  if (n >= n_tokens) return;
-  float M = pm[n], s = ps[n], e = pe[n];
-  for (int q = 1; q < parts; ++q) {
-    const int64_t o = (int64_t)q * n_tokens + n;
-    const float M2 = pm[o], s2 = ps[o], e2 = pe[o];
+  __shared__ float red[3][kMergeGroups][kMergeTokens];
+  const int tok = threadIdx.x % kMergeTokens, grp = threadIdx.x / kMergeTokens;
+  const int n = blockIdx.x * kMergeTokens + tok;
+  const int nc = n < n_tokens ? n : n_tokens - 1;  // a valid token; its result is dropped below
+  float M = 0.f, s = 0.f, e = 0.f;
+  bool any = false;  // a group beyond the number of partials folds nothing
+  auto fold = [&](float M2, float s2, float e2) {
+    if (!any) { M = M2; s = s2; e = e2; any = true; return; }
     const float Mn = fmaxf(M, M2);
     merge_stats(M, s, e, M2, s2, e2, Mn);
     M = Mn;
+  };
+  int q = grp;
+  for (; q + 3 * kMergeGroups < parts; q += 4 * kMergeGroups) {
+    float M2[4], s2[4], e2[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t o = (int64_t)(q + u * kMergeGroups) * n_tokens + nc;
+      M2[u] = pm[o]; s2[u] = ps[o]; e2[u] = pe[o];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) fold(M2[u], s2[u], e2[u]);
   }
+  for (; q < parts; q += kMergeGroups) {
+    const int64_t o = (int64_t)q * n_tokens + nc;
+    fold(pm[o], ps[o], pe[o]);
+  }
+  red[0][grp][tok] = M; red[1][grp][tok] = s; red[2][grp][tok] = e;
+  __syncthreads();
+  if (grp != 0 || n >= n_tokens) return;
+  for (int g2 = 1; g2 < kMergeGroups && g2 < parts; ++g2)
+    fold(red[0][g2][tok], red[1][g2][tok], red[2][g2][tok]);
   // log2 units: logsumexp = M + L, sum softmax*logit = M + e/s; differences are taken
   // before adding M so that large logits do not cancel
   const float L = __log2f(s);
@@ -716,7 +743,8 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
   }
   {
     Span span(timer, 1);
-    hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + kMergeTokens - 1) / kMergeTokens)),
+                       dim3(kMergeTokens * kMergeGroups), 0, st,
                        w.pm, w.ps, w.pe, w.parts, (int)n, lse, entropy_b, entropy, w.fin_max,
                        w.fin_log2s, is_start);
   }
