@@ -5,7 +5,7 @@
 // (a2, b2) o (a1, b1) = (a2*a1, b2 + a2*b1).  One wavefront owns one row and walks it from the end in
 // windows of 256 tokens that are 4-aligned in the token array: a lane holds four consecutive tokens (one
 // 16-byte access where the vector lies inside the row, guarded scalar accesses at the row's edges), lane 0
-// the last ones.  A lane composes its four elements, the wavefront scans the 64 composites with shuffles,
+// the last ones.  A lane composes its four elements, the wavefront scans the 64 composites with DPP row shifts and broadcasts,
 // and each lane then replays its four tokens from the value that enters it.  The loads of the next window
 // are issued before the current one is scanned.
 #include "common.h"
@@ -20,15 +20,32 @@ struct Pair { float a, b; };
 // p after q: y -> p.b + p.a * (q.b + q.a * y)
 __device__ __forceinline__ Pair after(Pair p, Pair q) { return Pair{p.a * q.a, p.b + p.a * q.b}; }
 
-// inclusive scan over lanes 0..63: lane l ends with the composition of the elements of lanes 0..l
+// Data-parallel-primitive moves (GFX9 DPP): `row_shr:n` hands lane i the value of lane i-n inside its row
+// of 16 lanes, `row_bcast:15` / `row_bcast:31` hand the last lane of a row / of the lower half to the rows
+// selected by ROW_MASK, `wave_shr:1` shifts across the whole wavefront.  A lane without a source keeps `old`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float old, float src) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                               __builtin_bit_cast(int, src), CTRL,
+                                                               ROW_MASK, 0xf, false));
+}
+
+// inclusive scan over lanes 0..63: lane l ends with the composition of the elements of lanes 0..l.
+// Lanes without a partner compose with the identity (1, 0).
 __device__ __forceinline__ Pair wave_scan(Pair p) {
-  const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const float ap = __shfl_up(p.a, d, kWave);
-    const float bp = __shfl_up(p.b, d, kWave);
-    if (lane >= d) p = after(p, Pair{ap, bp});
+#define AXON_SCAN_STEP(CTRL, ROW_MASK)                                  \
+  {                                                                     \
+    const float ap = dpp_move<CTRL, ROW_MASK>(1.f, p.a);                \
+    const float bp = dpp_move<CTRL, ROW_MASK>(0.f, p.b);                \
+    p = after(p, Pair{ap, bp});                                         \
   }
+  AXON_SCAN_STEP(0x111, 0xf)  // row_shr:1
+  AXON_SCAN_STEP(0x112, 0xf)  // row_shr:2
+  AXON_SCAN_STEP(0x114, 0xf)  // row_shr:4
+  AXON_SCAN_STEP(0x118, 0xf)  // row_shr:8
+  AXON_SCAN_STEP(0x142, 0xa)  // row_bcast:15 into rows 1 and 3
+  AXON_SCAN_STEP(0x143, 0xc)  // row_bcast:31 into rows 2 and 3
+#undef AXON_SCAN_STEP
   return p;
 }
 
@@ -37,9 +54,8 @@ __device__ __forceinline__ Pair wave_scan(Pair p) {
 __device__ __forceinline__ float scan_enter(Pair lane_total, float& carry) {
   const Pair s = wave_scan(lane_total);
   const float leaves = s.b + s.a * carry;
-  const float up = __shfl_up(leaves, 1, kWave);
-  const float enters = (threadIdx.x & (kWave - 1)) == 0 ? carry : up;
-  carry = __shfl(leaves, kWave - 1, kWave);
+  const float enters = dpp_move<0x138, 0xf>(carry, leaves);  // wave_shr:1; lane 0 keeps the carry
+  carry = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, leaves), kWave - 1));
   return enters;
 }
 
