@@ -78,6 +78,19 @@ def test_gae_other_mask_types_and_defaults(mask_dtype):
     assert rel_l2(ret, ref_ret) < 2e-5 and rel_l2(adv, ref_adv) < 1e-4
 
 
+def test_fractional_masks_blend_like_the_reference():
+    """The reference blends with the mask value (``x * m + (1 - m) * carried``); a weight of 0.5 must do so here."""
+    r, v, m = _value_batch(5, 300, seed=8)
+    g = torch.Generator().manual_seed(9)
+    m = m * torch.where(torch.rand(5, 300, generator=g) > 0.5, 1.0, 0.5)
+    rows = _ops.rows_of(r.to(DEV))
+    adv, ret = _ops.reverse_scan(_ops.SCAN_GAE, r.to(DEV), v.to(DEV), m.to(DEV), rows, gamma=0.99, lam=0.95)
+    ref_adv, ref_ret = OR.gae_raw(r, v, m, 0.99, 0.95)
+    assert rel_l2(adv, ref_adv) < 2e-5 and rel_l2(ret, ref_ret) < 2e-5
+    _, ret = _ops.reverse_scan(_ops.SCAN_DISCOUNTED, r.to(DEV), None, m.to(DEV), rows, gamma=0.9)
+    assert rel_l2(ret, OR.reinforce_plus_plus_raw(r, m, 0.9)) < 2e-5
+
+
 def test_gae_closed_forms_on_the_gpu():
     """Independent of the oracle: lam = gamma = 1 gives reward-to-go minus value; lam = 0 the TD error."""
     g = torch.Generator().manual_seed(11)
