@@ -43,18 +43,23 @@ def rows_of(t: torch.Tensor, cu_seqlens: torch.Tensor | None = None) -> Rows:
     return Rows(int(b), int(b * s), int(s), None, tuple(t.shape))
 
 
+def _on_16_bytes(t: torch.Tensor) -> torch.Tensor:
+    """The kernels move four values per access: a view that starts off a 16-byte boundary is copied."""
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def f32(t: torch.Tensor) -> torch.Tensor:
-    return t.detach().to(torch.float32).contiguous()
+    return _on_16_bytes(t.detach().to(torch.float32).contiguous())
 
 
 def mask_arg(mask: torch.Tensor):
     """Normalise a response mask once: fp32 and int64 are read natively by the kernels."""
     mask = mask.detach()
     if mask.dtype == torch.int64:
-        return mask.contiguous(), MASK_I64
+        return _on_16_bytes(mask.contiguous()), MASK_I64
     if mask.dtype != torch.float32:
         mask = mask.to(torch.float32)
-    return mask.contiguous(), MASK_F32
+    return _on_16_bytes(mask.contiguous()), MASK_F32
 
 
 def _same_len(what: str, n: int, **tensors) -> None:

@@ -753,3 +753,20 @@ def test_operand_length_mismatch_raises():
     with pytest.raises(ValueError, match="labels has 7"):
         _ops.lmhead_forward(hid, torch.zeros(100, 64, device=DEV, dtype=torch.bfloat16),
                             torch.zeros(7, dtype=torch.int32, device=DEV), 1.0)
+
+
+def test_views_off_a_16_byte_boundary():
+    g = torch.Generator().manual_seed(3)
+    big = torch.randn(4 * 64 + 1, generator=g).to(DEV)
+    x = big[1:].view(4, 64)  # contiguous, 4 bytes past a 16-byte boundary
+    mask = (torch.rand(4 * 64 + 1, generator=g) > 0.3).float().to(DEV)[1:].view(4, 64)
+    assert x.data_ptr() % 16 == 4
+    out, stats = _ops.masked_whiten(x, mask)
+    ref, _ = _ops.masked_whiten(x.clone(), mask.clone())
+    assert torch.equal(out, ref)
+    rows = _ops.rows_of(x)
+    a1, g1 = _ops.policy_loss(0, x, x * 0.9, x, mask, None, rows, token_reduce="sum", batch_reduce="token-mean",
+                              ratio_lo=0.8, ratio_hi=1.2, clip_c=3.0)
+    a2, g2 = _ops.policy_loss(0, x.clone(), x.clone() * 0.9, x.clone(), mask.clone(), None, rows, token_reduce="sum",
+                              batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.2, clip_c=3.0)
+    assert torch.equal(a1[:5], a2[:5]) and torch.equal(g1, g2)
