@@ -166,7 +166,7 @@ def reverse_scan(mode, rewards, values, mask, rows: Rows, *, gamma=1.0, lam=1.0,
     return adv, ret
 
 
-def masked_whiten(x, mask, *, remask=False, inplace=False):
+def masked_whiten(x, mask, *, remask=False, inplace=False, stats_only=False):
     """``(x - mean) * rsqrt(var + 1e-8)`` with the mean and variance taken over the mask (times the mask when
     ``remask``); returns ``(out, stats)`` with stats = device [mean, n, var, rsqrt(var + 1e-8)]."""
     lib = _lib.load()
@@ -176,7 +176,10 @@ def masked_whiten(x, mask, *, remask=False, inplace=False):
     xf = f32(x)
     mk, kind = mask_arg(mask)
     n = int(xf.numel())
-    out = xf if (inplace and xf.data_ptr() == x.data_ptr()) else torch.empty_like(xf)
+    if stats_only:
+        out = None
+    else:
+        out = xf if (inplace and xf.data_ptr() == x.data_ptr()) else torch.empty_like(xf)
     stats = _zeros(4, dev)
     ws = torch.empty(max(lib.axon_masked_whiten_workspace_bytes(n) // 4, 8), device=dev, dtype=torch.float32)
     check(

@@ -1,8 +1,9 @@
-"""Group helpers: ``as_torch_index`` and ``group_mean_std``.
+"""Group helpers ``as_torch_index`` and ``group_mean_std``, and the masked moments ``masked_mean``,
+``masked_var``, ``masked_whiten``.
 
-Same behaviour as axon/utils/rl/advantage.py:46-150.  ``as_torch_index`` is host
-logic (``np.unique`` over arbitrary labels); ``group_mean_std`` runs in
-libaxon_amd.so (``axon_group_stats``).
+Same behaviour as axon/utils/rl/advantage.py:46-190.  ``as_torch_index`` is host logic (``np.unique`` over
+arbitrary labels); ``group_mean_std`` runs in libaxon_amd.so (``axon_group_stats``), the masked moments in
+``axon_masked_whiten`` (sums in a fixed order, statistics left on the device).
 """
 
 from __future__ import annotations
@@ -14,7 +15,7 @@ import torch
 
 from axon_amd import _lib, _ops
 
-__all__ = ["as_torch_index", "group_mean_std"]
+__all__ = ["as_torch_index", "group_mean_std", "masked_mean", "masked_var", "masked_whiten"]
 
 _INT_DTYPES = (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool)
 _FLOAT_DTYPES = (torch.float16, torch.float32, torch.float64, torch.bfloat16)
@@ -82,3 +83,29 @@ def group_mean_std(scores: torch.Tensor, gidx: torch.Tensor, eps: float = 1e-6, 
     n_groups = int(gidx.max().item()) + 1
     mean, std, count, _ = _ops.group_stats(scores, gidx, n_groups, eps, want_scalar=False)
     return mean, std, count
+
+
+@torch.no_grad()
+def masked_mean(values: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+    """``sum(values * mask) / max(sum(mask), 1)`` as a 0-d device tensor (advantage.py:153-157)."""
+    _, stats = _ops.masked_whiten(values, mask, stats_only=True)
+    return stats[0]
+
+
+@torch.no_grad()
+def masked_var(values: torch.Tensor, mask: torch.Tensor, bessel_correction: bool = True) -> torch.Tensor:
+    """Masked variance about the masked mean, times n/(n-1) when n > 1 (advantage.py:160-170)."""
+    _, stats = _ops.masked_whiten(values, mask, stats_only=True)
+    if bessel_correction:
+        return stats[2]
+    n = stats[1]
+    return torch.where(n > 1, stats[2] * (n - 1) / n.clamp_min(1.0), stats[2])
+
+
+@torch.no_grad()
+def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True) -> torch.Tensor:
+    """``(values - mean) * rsqrt(var + 1e-8)`` with the moments taken over the mask; the mean is added back when
+    ``shift_mean`` is False (advantage.py:173-190)."""
+    out, stats = _ops.masked_whiten(values, mask)
+    out = out.view(values.shape)
+    return out if shift_mean else out + stats[0]

@@ -470,3 +470,18 @@ def test_cov_losses_packed_layout():
                                                "batch_reduce": "step-mean"})
     assert loss.item() == pytest.approx(ref_loss.item(), rel=1e-4)
     assert m["ppo_kl"] == pytest.approx(ref_m["ppo_kl"], rel=1e-4)
+
+
+def test_masked_moment_helpers():
+    from axon_amd.utils.rl.advantage import masked_mean, masked_var, masked_whiten
+    g = torch.Generator().manual_seed(17)
+    x = torch.randn(6, 301, generator=g) * 2 + 1
+    m = (torch.rand(6, 301, generator=g) > 0.5).float()
+    xd, md = x.to(DEV), m.to(DEV)
+    assert masked_mean(xd, md).item() == pytest.approx(float(OL.masked_mean(x, m)), rel=1e-5)
+    assert masked_var(xd, md).item() == pytest.approx(float(OR.masked_var(x, m)), rel=1e-5)
+    assert masked_var(xd, md, False).item() == pytest.approx(float(OR.masked_var(x, m, False)), rel=1e-5)
+    assert torch.allclose(masked_whiten(xd, md).cpu(), OR.masked_whiten(x, m), rtol=2e-5, atol=2e-5)
+    assert torch.allclose(masked_whiten(xd, md, shift_mean=False).cpu(), OR.masked_whiten(x, m, False), rtol=2e-5,
+                          atol=2e-5)
+    assert float(masked_var(T([1.0, 3.0]).to(DEV), T([1.0, 1.0]).to(DEV))) == pytest.approx(2.0)
