@@ -39,6 +39,8 @@ SIGNATURES: dict[str, tuple] = {
     "axon_group_stats": (_i32, [_ptr, _ptr, _i64, _i64, _f32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_row_broadcast_mask": (_i32, [_ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _f32, _ptr, _ptr]),
     "axon_fill_zero": (_i32, [_ptr, _i64, _ptr]),
+    "axon_logits_fwd": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i32, _ptr, _ptr, _ptr, _ptr]),
+    "axon_logits_bwd": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "axon_reverse_scan": (_i32, [_i32, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr,
                                  _ptr]),
     "axon_masked_whiten_workspace_bytes": (_i64, [_i64]),
@@ -69,7 +71,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -611,6 +611,60 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     return d_hidden, d_weight
 
 
+_LOGITS_DTYPES = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _logits_operands(what, logits, labels):
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise ValueError(f"{what}: logits must be [tokens, vocab] with unit stride over the vocabulary")
+    if logits.dtype not in _LOGITS_DTYPES:
+        raise ValueError(f"{what}: logits must be fp32 or bf16, got {logits.dtype}")
+    n, v = int(logits.shape[0]), int(logits.shape[1])
+    if labels is not None:
+        if labels.dtype not in (torch.int32, torch.int64) or not labels.is_contiguous():
+            raise ValueError(f"{what}: labels must be contiguous int32 or int64")
+        if labels.device != logits.device:
+            raise ValueError(f"{what}: operands live on different devices")
+        _same_len(what, n, labels=labels)
+    return n, v, int(logits.stride(0)) if n > 1 else v
+
+
+def logits_forward(logits, labels=None, want_entropy=True):
+    """``(logprob | None, entropy | None, lse)`` fp32 [tokens] from materialised logits; see axon_logits_fwd."""
+    lib = _lib.load()
+    require_device(logits, "logits_forward")
+    n, v, ld = _logits_operands("logits_forward", logits, labels)
+    dev = logits.device
+    out = torch.empty(3, max(n, 1), device=dev, dtype=torch.float32)
+    check(
+        lib.axon_logits_fwd(ptr(logits), _LOGITS_DTYPES[logits.dtype], ld, n, v, ptr(labels),
+                            int(labels is not None and labels.dtype == torch.int64),
+                            ptr(out[0]) if labels is not None else None, ptr(out[1]) if want_entropy else None,
+                            ptr(out[2]), stream_ptr()),
+        "axon_logits_fwd",
+    )
+    return (out[0][:n] if labels is not None else None), (out[1][:n] if want_entropy else None), out[2][:n]
+
+
+def logits_backward(logits, labels, lse, entropy, g_logprob, g_entropy, inplace=False):
+    """d loss / d logits in the logits' dtype (written over the logits when ``inplace``); see axon_logits_bwd."""
+    lib = _lib.load()
+    require_device(logits, "logits_backward")
+    n, v, ld = _logits_operands("logits_backward", logits, labels)
+    g_lp = f32(g_logprob) if g_logprob is not None else None
+    g_en = f32(g_entropy) if g_entropy is not None else None
+    _same_len("logits_backward", n, lse=lse, entropy=entropy, g_logprob=g_lp, g_entropy=g_en)
+    out = logits if inplace else torch.empty_like(logits, memory_format=torch.contiguous_format)
+    ld_d = int(out.stride(0)) if n > 1 else v
+    check(
+        lib.axon_logits_bwd(ptr(logits), _LOGITS_DTYPES[logits.dtype], ld, n, v, ptr(labels),
+                            int(labels is not None and labels.dtype == torch.int64), ptr(lse), ptr(entropy),
+                            ptr(g_lp), ptr(g_en), ptr(out), ld_d, stream_ptr()),
+        "axon_logits_bwd",
+    )
+    return out
+
+
 def gemm_nt(a, b):
     """out[n][m] = sum_k a[m][k] * b[n][k]; bf16 in, fp32 out.  Test/benchmark helper."""
     lib = _lib.load()

@@ -74,6 +74,17 @@ def packed_logprobs(hidden, weight, packed_ids, cu_seqlens, temperature: float =
                                 logit_softcapping, cu_seqlens)
 
 
+def _from_logits(logits, labels, temperature: float, calculate_entropy: bool):
+    """The non-fused head (forward_utils.py:287-304): divide the logits by the temperature in place, then
+    log-probability and entropy from one pass over them."""
+    from axon_amd.utils.torch.ops import logprobs_and_entropy_from_logits, logprobs_from_logits
+
+    logits.div_(temperature)
+    if calculate_entropy:
+        return logprobs_and_entropy_from_logits(logits, labels)
+    return logprobs_from_logits(logits, labels, inplace_backward=True), None
+
+
 def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_entropy: bool = False, *,
                        use_remove_padding: bool = True, use_fused_kernels: bool = True, ulysses_sp_size: int = 1,
                        **_unused):
@@ -83,9 +94,9 @@ def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_
     (forward_utils.py:185-318): with remove-padding the ids are unpadded, rolled over the packed stream and
     handed to the model as ``pre_rolled_labels`` (:236-265), the packed outputs are scattered back and shifted
     right (``rmpad_postprocess``, :164-182); without it the outputs are shifted right directly (:282-285).
-    Ulysses sequence parallelism (more than one GPU) and the non-fused logits path are not part of this build."""
-    if not use_fused_kernels:
-        raise NotImplementedError("only the fused-head path (use_fused_kernels=True) is built")
+    With ``use_fused_kernels=False`` the model writes the logits and ``axon_amd.utils.torch.ops`` turns them into
+    log-probabilities and entropy (:287-304).  Ulysses sequence parallelism (more than one GPU) is not part of
+    this build."""
     if ulysses_sp_size > 1:
         raise NotImplementedError("Ulysses sequence parallelism needs more than one GPU")
     input_ids = micro_batch["input_ids"]
@@ -104,17 +115,30 @@ def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_
             fwd_pos = position_ids.flatten(1)[:, indices].unsqueeze(1)
         else:
             fwd_pos = position_ids.flatten()[indices].unsqueeze(0)
-        output = module(input_ids=fwd_ids, attention_mask=None, position_ids=fwd_pos, use_cache=False,
-                        temperature=temperature, return_dict=True, pre_rolled_labels=rolled_labels(fwd_ids))
-        log_probs = rmpad_postprocess(output.log_probs.reshape(-1), indices=indices, batch_size=batch_size,
-                                      seqlen=seqlen)
+        labels = rolled_labels(fwd_ids)
+        if use_fused_kernels:
+            output = module(input_ids=fwd_ids, attention_mask=None, position_ids=fwd_pos, use_cache=False,
+                            temperature=temperature, return_dict=True, pre_rolled_labels=labels)
+            lp_packed = output.log_probs.reshape(-1)
+            ent_packed = output.entropy.reshape(-1) if calculate_entropy else None
+        else:  # the model writes the logits (forward_utils.py:287-292)
+            output = module(input_ids=fwd_ids, attention_mask=None, position_ids=fwd_pos, use_cache=False)
+            lp_packed, ent_packed = _from_logits(output.logits.squeeze(0), labels.reshape(-1), temperature,
+                                                 calculate_entropy)
+        log_probs = rmpad_postprocess(lp_packed, indices=indices, batch_size=batch_size, seqlen=seqlen)
         entropy = None
         if calculate_entropy:
-            entropy = rmpad_postprocess(output.entropy.reshape(-1), indices=indices, batch_size=batch_size,
-                                        seqlen=seqlen)
+            entropy = rmpad_postprocess(ent_packed, indices=indices, batch_size=batch_size, seqlen=seqlen)
         return entropy, log_probs
-    output = module(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids, use_cache=False,
-                    temperature=temperature, return_dict=True)
-    log_probs = shift_to_token_positions(output.log_probs.view(batch_size, seqlen))
-    entropy = shift_to_token_positions(output.entropy.view(batch_size, seqlen)) if calculate_entropy else None
+    if use_fused_kernels:
+        output = module(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids,
+                        use_cache=False, temperature=temperature, return_dict=True)
+        log_probs = shift_to_token_positions(output.log_probs.view(batch_size, seqlen))
+        entropy = shift_to_token_positions(output.entropy.view(batch_size, seqlen)) if calculate_entropy else None
+        return entropy, log_probs
+    # padded, non-fused (forward_utils.py:294-304): logits[:, t] predicts token t + 1
+    output = module(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids, use_cache=False)
+    lp, ent = _from_logits(output.logits[:, :-1, :], input_ids[:, 1:], temperature, calculate_entropy)
+    log_probs = F.pad(lp, (1, 0), value=0.0)
+    entropy = F.pad(ent, (1, 0), value=0.0) if calculate_entropy else None
     return entropy, log_probs

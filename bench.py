@@ -160,6 +160,28 @@ def hbm_kernels(n_tokens, dev):
         gbs = n_tokens * bpt / (ms * 1e-3) / 1e9
         out.append({"kernel": name, "bytes_per_token": bpt, "ms": ms, "achieved": gbs, "peak": HBM_PEAK_GBS,
                     "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS})
+    # the materialised-logits path (use_fused_kernels off): bf16 logits of 8192 tokens at the Qwen vocabulary
+    del old, new, samp, adv, x
+    ln, lv = min(8192, max(n_tokens // 1024, 64)), 151936
+    logits = torch.randn(ln, lv, device=dev, dtype=torch.bfloat16, generator=gd)
+    labels = torch.randint(0, lv, (ln,), device=dev, generator=gd)
+    lp, ent, lse = _ops.logits_forward(logits, labels, True)
+    g1, g2 = torch.randn(ln, device=dev, generator=gd), torch.randn(ln, device=dev, generator=gd)
+    dl = torch.empty_like(logits)
+
+    def bwd():
+        lib_out = _ops.logits_backward(logits, labels, lse, ent, g1, g2, inplace=False)
+        return lib_out
+
+    for name, nbytes, fn in (
+            ("logits_stats_kernel: bf16 logits [8192 x 151936] -> log-prob, entropy (one read)", ln * lv * 2,
+             lambda: _ops.logits_forward(logits, labels, True)),
+            ("logits_grad_kernel: d logits from both gradients (one read, one write)", ln * lv * 4, bwd)):
+        ms = median_ms(fn, iters=10, warm=2)
+        gbs = nbytes / (ms * 1e-3) / 1e9
+        out.append({"kernel": name, "bytes_per_token": nbytes // ln, "ms": ms, "achieved": gbs, "peak": HBM_PEAK_GBS,
+                    "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS})
+    del dl
     return {"tokens": n_tokens, "sequences": len(lens), "bound": "hbm", "kernels": out}
 
 

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 10
+#define AXON_AMD_ABI_VERSION 11
 
 enum {
   AXON_OK = 0,
@@ -305,6 +305,28 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
                      float uniform_scale, int post_normalize, const int64_t* valid_count,
                      float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                      float* partials, void* stream);
+
+/* The non-fused branch of fsdp_model_forward (axon/utils/fsdp/forward_utils.py:287-304): the model has
+ * written logits [n, vocab] (row stride ld elements; dtype AXON_LOGITS_F32 or AXON_LOGITS_BF16, already
+ * divided by the temperature).  One read of each row gives
+ *   logprob[t] = log_softmax(logits[t])[labels[t]]    (logprobs_from_logits, axon/utils/torch/ops.py:39-102)
+ *   entropy[t] = logsumexp(logits[t]) - sum softmax*logits   (entropy_from_logits, ops.py:105-120)
+ *   lse[t]     = logsumexp(logits[t])                 (kept for the backward)
+ * in fp32.  logprob (with labels) or entropy may be NULL.  A label outside [0, vocab) gives logprob 0. */
+enum { AXON_LOGITS_F32 = 0, AXON_LOGITS_BF16 = 1 };
+int axon_logits_fwd(const void* logits, int dtype, int64_t ld, int64_t n, int64_t vocab,
+                    const void* labels, int labels_are_i64, float* logprob, float* entropy, float* lse,
+                    void* stream);
+
+/* Backward of the above in one read and one write of the rows:
+ *   dlogits[t][j] = g_logprob[t] (onehot - p) - g_entropy[t] p (log p + entropy[t]),  p = exp(logits - lse)
+ * in the logits' dtype.  g_logprob or g_entropy may be NULL (that output had no gradient).  dlogits may be
+ * the logits' own storage (the in-place backward of the reference's flash-attn cross entropy,
+ * ops.py:70-75, inplace_backward). */
+int axon_logits_bwd(const void* logits, int dtype, int64_t ld, int64_t n, int64_t vocab,
+                    const void* labels, int labels_are_i64, const float* lse, const float* entropy,
+                    const float* g_logprob, const float* g_entropy, void* dlogits, int64_t ld_dlogits,
+                    void* stream);
 
 /* Time recurrences of the return-based advantage estimators, run from each row's last token to its
  * first (axon/trainer/algos/advantages/advantage.py), before any whitening:

@@ -114,3 +114,16 @@ def backward_bf16_torch_path(dlogp, hidden, weight, labels, temperature: float =
         d_h[s:e] += dl @ weight
         d_w += dl.t() @ hidden[s:e]
     return d_h, d_w
+
+
+def logprobs_from_logits(logits, labels):
+    """axon/utils/torch/ops.py:39-102 in fp32: ``log_softmax(logits)[labels]`` (the definition the reference's own
+    test uses, tests/utils/torch/test_ops.py:36-42)."""
+    lp = torch.log_softmax(logits.float(), dim=-1)
+    return lp.gather(-1, labels.long().unsqueeze(-1)).squeeze(-1)
+
+
+def entropy_from_logits(logits):
+    """axon/utils/torch/ops.py:105-120 in fp32: ``logsumexp - sum softmax * logits``."""
+    z = logits.float()
+    return torch.logsumexp(z, dim=-1) - (torch.softmax(z, dim=-1) * z).sum(-1)

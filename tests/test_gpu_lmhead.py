@@ -334,3 +334,94 @@ def test_config2_shape_forward():
     ref_lp, ref_ent = OM.forward(hid[idx], w, lab[idx])
     assert (lp.cpu()[idx] - ref_lp).abs().max() < 1e-3 and (ent.cpu()[idx] - ref_ent).abs().max() < 1e-3
     assert torch.isfinite(lp).all() and torch.isfinite(ent).all()
+
+
+# ---- materialised-logits path (use_fused_kernels off) --------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,v", [(5, 37), (64, 1000), (33, 4099), (3, 151936)])
+def test_logits_path_vs_oracle(dtype, n, v):
+    from axon_amd.utils.torch.ops import (entropy_from_logits, logprobs_and_entropy_from_logits,
+                                          logprobs_from_logits)
+    g = torch.Generator().manual_seed(n * 7 + v)
+    logits = (torch.randn(n, v, generator=g) * 3).to(dtype)
+    labels = torch.randint(0, v, (n,), generator=g)
+    ref_in = logits.float().clone().requires_grad_(True)
+    ref_lp, ref_en = OM.logprobs_from_logits(ref_in, labels), OM.entropy_from_logits(ref_in)
+    g_lp, g_en = torch.randn(n, generator=g), torch.randn(n, generator=g)
+    (ref_lp * g_lp + ref_en * g_en).sum().backward()
+    x = logits.to(DEV).requires_grad_(True)
+    lp, en = logprobs_and_entropy_from_logits(x, labels.to(DEV))
+    assert lp.dtype == torch.float32 and lp.shape == (n,)
+    assert (lp.cpu() - ref_lp.detach()).abs().max() < 1e-3 and (en.cpu() - ref_en.detach()).abs().max() < 1e-3
+    (lp * g_lp.to(DEV) + en * g_en.to(DEV)).sum().backward()
+    # fp32: p = exp(z - lse) carries the rounding of lse (about 1e-6 relative at |lse| = 16) and of the fast exp
+    tol = 2e-2 if dtype == torch.bfloat16 else 5e-5
+    assert rel_l2(x.grad, ref_in.grad) < tol
+    # each function on its own
+    x2 = logits.to(DEV).requires_grad_(True)
+    lp2 = logprobs_from_logits(x2, labels.to(DEV), inplace_backward=False)
+    assert torch.equal(lp2, lp)
+    (lp2 * g_lp.to(DEV)).sum().backward()
+    ref2 = logits.float().clone().requires_grad_(True)
+    (OM.logprobs_from_logits(ref2, labels) * g_lp).sum().backward()
+    assert rel_l2(x2.grad, ref2.grad) < tol
+    assert torch.equal(entropy_from_logits(logits.to(DEV)), en.detach())
+
+
+def test_logits_path_inplace_backward_shapes_and_strides():
+    from axon_amd.utils.torch.ops import entropy_from_logits_with_chunking, logprobs_from_logits
+    g = torch.Generator().manual_seed(5)
+    b, t, v = 3, 9, 515
+    logits = torch.randn(b, t, v, generator=g)
+    labels = torch.randint(0, v, (b, t), generator=g)
+    ref_in = logits.clone().requires_grad_(True)
+    OM.logprobs_from_logits(ref_in, labels).sum().backward()
+    # in-place backward: the gradient is written over the logits' storage (the leaf is a product, as in a model)
+    w = torch.ones((), device=DEV, requires_grad=True)
+    z = logits.to(DEV) * w
+    lp = logprobs_from_logits(z, labels.to(DEV), inplace_backward=True)
+    assert lp.shape == (b, t)
+    lp.sum().backward()
+    assert rel_l2(z, ref_in.grad) < 5e-5  # z now holds d loss / d logits
+    # a row stride larger than the vocabulary (a column slice) and rows off a 16-byte boundary
+    wide = torch.randn(6, v + 5, generator=g)
+    x = wide.to(DEV)[:, 1:v + 1]
+    lab = torch.randint(0, v, (6,), generator=g)
+    got = logprobs_from_logits(x, lab.to(DEV), inplace_backward=False)
+    assert (got.cpu() - OM.logprobs_from_logits(wide[:, 1:v + 1], lab)).abs().max() < 1e-5
+    ent = entropy_from_logits_with_chunking(x, chunk_size=2)
+    assert (ent.cpu() - OM.entropy_from_logits(wide[:, 1:v + 1])).abs().max() < 1e-5
+    with pytest.raises(ValueError, match="fp32 or bf16"):
+        logprobs_from_logits(x.half(), lab.to(DEV))
+
+
+@pytest.mark.parametrize("remove_padding", [True, False])
+def test_fsdp_model_forward_non_fused(remove_padding):
+    """The model returns logits; log-probabilities and entropy must equal those of the fused branch."""
+    from types import SimpleNamespace
+    from axon_amd.utils.fsdp.forward_utils import fsdp_model_forward
+    g = torch.Generator().manual_seed(9)
+    b, t, h, v = 3, 12, 64, 300
+    emb = (torch.randn(v, h, generator=g) * 0.5).to(DEV)
+    w = (torch.randn(v, h, generator=g) * 0.3).to(torch.bfloat16).to(DEV)
+
+    class LogitsModel(torch.nn.Module):
+        def forward(self, input_ids=None, attention_mask=None, position_ids=None, use_cache=False):
+            hidden = emb[input_ids].to(torch.bfloat16)
+            return SimpleNamespace(logits=(hidden.float() @ w.float().t()))
+
+    ids = torch.randint(0, v, (b, t), generator=g)
+    mask = torch.ones(b, t, dtype=torch.int64)
+    mask[1, 8:] = 0
+    mask[2, 5:] = 0
+    batch = {"input_ids": ids.to(DEV), "attention_mask": mask.to(DEV),
+             "position_ids": torch.arange(t).expand(b, t).to(DEV)}
+    ent, lp = fsdp_model_forward(LogitsModel(), batch, 0.7, True, use_remove_padding=remove_padding,
+                                 use_fused_kernels=False)
+    assert lp.shape == (b, t) and ent.shape == (b, t) and (lp[:, 0] == 0).all() and (ent[:, 0] == 0).all()
+    logits = (emb[ids.to(DEV)].to(torch.bfloat16).float() @ w.float().t()).cpu() / 0.7
+    ref_lp = OM.logprobs_from_logits(logits[:, :-1], ids[:, 1:])
+    ref_en = OM.entropy_from_logits(logits[:, :-1])
+    valid = (mask[:, 1:] > 0) if remove_padding else torch.ones(b, t - 1, dtype=torch.bool)
+    assert ((lp.cpu()[:, 1:] - ref_lp).abs() * valid).max() < 1e-3
+    assert ((ent.cpu()[:, 1:] - ref_en).abs() * valid).max() < 1e-3

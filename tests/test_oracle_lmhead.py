@@ -183,3 +183,23 @@ def test_softcap_backward_matches_autograd_and_finite_differences():
         d = torch.zeros_like(wd); d[j, k] = eps
         fd = (f(hd, wd + d) - f(hd, wd - d)).item() / (2 * eps)
         assert dw[j, k].item() == pytest.approx(fd, abs=2e-4)
+
+
+# ---- materialised-logits path (ops.py:39-120): closed forms and the textbook definitions ---------------------
+def test_logits_oracle_closed_forms():
+    v = 37
+    z = torch.zeros(3, v)
+    lab = torch.tensor([0, 5, 36])
+    assert torch.allclose(M.logprobs_from_logits(z, lab), torch.full((3,), -math.log(v)), atol=1e-6)
+    assert torch.allclose(M.entropy_from_logits(z), torch.full((3,), math.log(v)), atol=1e-6)
+    peak = torch.full((1, v), -50.0)
+    peak[0, 7] = 50.0
+    assert abs(float(M.logprobs_from_logits(peak, torch.tensor([7])))) < 1e-6
+    assert abs(float(M.entropy_from_logits(peak))) < 1e-6
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(4, v, generator=g, dtype=torch.float64)
+    lab = torch.randint(0, v, (4,), generator=g)
+    p = torch.softmax(x, -1)
+    assert torch.allclose(M.entropy_from_logits(x.float()).double(), -(p * p.log()).sum(-1), atol=1e-6)
+    assert torch.allclose(M.logprobs_from_logits(x.float(), lab).double(), p.log()[torch.arange(4), lab], atol=1e-6)
+    assert torch.allclose(M.entropy_from_logits(x.float() + 3.0), M.entropy_from_logits(x.float()), atol=1e-5)
