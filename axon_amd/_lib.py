@@ -59,6 +59,7 @@ SIGNATURES: dict[str, tuple] = {
     "axon_cov_policy_loss": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64, _ptr, _f32,
                                     _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_kl_penalty": (_i32, [_ptr, _ptr, _i64, _i32, _i32, _ptr, _ptr, _ptr]),
+    "axon_kl_reward": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32, _ptr, _ptr, _ptr]),
     "axon_side_terms": (_i32, [_ptr, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _ptr, _f32, _i32, _ptr, _i32,
                                _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_sampler_diag_workspace_bytes": (_i64, [_i64, _i64]),
@@ -71,7 +72,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

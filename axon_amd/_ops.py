@@ -439,6 +439,25 @@ def kl_penalty(logprob, ref_logprob, kl_type: int, kl_plus: int):
     return out, grad
 
 
+def kl_reward(scores, old_log_probs, ref_log_probs, mask, rows: Rows, *, kl_type: int, beta: float):
+    """``(rewards, row mask sums, row kld sums)``; see axon_kl_reward."""
+    lib = _lib.load()
+    require_device(scores, "kl_reward")
+    _same_len("kl_reward", rows.n_slots, scores=scores, old_log_probs=old_log_probs, ref_log_probs=ref_log_probs,
+              mask=mask)
+    dev = scores.device
+    sc, old, ref = f32(scores), f32(old_log_probs), f32(ref_log_probs)
+    mk, kind = mask_arg(mask)
+    rewards = torch.empty(rows.shape, device=dev, dtype=torch.float32)
+    row_vals = _zeros(2 * max(rows.n_rows, 1), dev).view(2, -1)
+    check(
+        lib.axon_kl_reward(ptr(sc), ptr(old), ptr(ref), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
+                           rows.uniform_len, int(kl_type), float(beta), ptr(rewards), ptr(row_vals), stream_ptr()),
+        "axon_kl_reward",
+    )
+    return rewards, row_vals[0][: rows.n_rows], row_vals[1][: rows.n_rows]
+
+
 def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_reduce, batch_reduce, kl_type=0,
                kl_plus=0, per_row_token_count=None, num_program_tokens=None, num_program_steps=None,
                valid_count=None):

@@ -432,6 +432,73 @@ __global__ __launch_bounds__(kBlock) void kl_penalty_kernel(const float* __restr
 // policy.  partial slots: [0] sum entropy*w  [1] sum kld*w  [2] sum entropy*mask  [4] sum mask,
 // w = mask * scale.  Outputs agg_w[t] = w (the gradient of slot 0 w.r.t. entropy) and
 // grad_kl[t] = w * d kld / d log_prob.
+// KL penalty inside the reward (axon/utils/rl/kl.py:276-322): kld = kl_penalty(old, ref) * mask,
+// rewards = scores - beta * kld, and per row sum mask -> row_vals[0][r], sum kld -> row_vals[1][r].
+template <int MK>
+__global__ __launch_bounds__(kBlock) void kl_reward_kernel(
+    const float* __restrict__ scores, const float* __restrict__ oldp, const float* __restrict__ refp,
+    const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots,
+    int64_t uniform_len, int kl_type, float beta, float* __restrict__ rewards, float* row_vals) {
+  __shared__ int32_t lds_cu[kLdsRows];
+  const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
+#pragma unroll 1
+  for (int64_t chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const int64_t c0 = chunk * kChunk;
+    const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
+    __syncthreads();
+    RowFinder rf;
+    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+#pragma unroll 1
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      RowSeg<2> s;
+      s.row = -1;
+      s.v[0] = s.v[1] = 0.f;
+      if (i < c1) {
+        float sv[4], ov[4], rv[4], mv[4], out[4];
+        const bool full = (i + kVec <= n_slots);
+        if (full) {
+          load4(scores, i, sv);
+          load4(oldp, i, ov);
+          load4(refp, i, rv);
+          load_mask4<MK>(mask, i, mv);
+        } else {
+          for (int j = 0; j < 4; ++j) {
+            const bool ok = i + j < n_slots;
+            sv[j] = ok ? scores[i + j] : 0.f;
+            ov[j] = ok ? oldp[i + j] : 0.f;
+            rv[j] = ok ? refp[i + j] : 0.f;
+            mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+          }
+        }
+        int r = rf.row(i);
+        int64_t rend = rf.row_end(r);
+        s.row = r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int64_t p = i + j;
+          if (p >= n_slots) { out[j] = 0.f; continue; }
+          if (p >= rend) {
+            row_seg_flush(s, row_vals, n_rows);
+            r = rf.row(p);
+            rend = rf.row_end(r);
+            s.row = r;
+            s.v[0] = s.v[1] = 0.f;
+          }
+          const float kld = kl_term(ov[j], rv[j], kl_type, 0).v * mv[j];
+          out[j] = sv[j] - beta * kld;
+          s.v[0] += mv[j];
+          s.v[1] += kld;
+        }
+        if (full) store4(rewards, i, out);
+        else
+          for (int j = 0; j < 4 && i + j < n_slots; ++j) rewards[i + j] = out[j];
+      }
+      row_seg_wave_reduce_flush(s, row_vals, n_rows);
+    }
+  }
+}
+
 template <int MK>
 __global__ __launch_bounds__(kBlock) void side_terms_kernel(
     const float* __restrict__ entropy, const float* __restrict__ logp, const float* __restrict__ ref,
@@ -835,6 +902,27 @@ extern "C" int axon_kl_penalty(const float* logp, const float* ref_logp, int64_t
   const int grid = (int)(nb < 8192 ? nb : 8192);
   hipLaunchKernelGGL(kl_penalty_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, logp,
                      ref_logp, n, kl_type, kl_plus, out, grad);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_kl_reward(const float* scores, const float* old_logp, const float* ref_logp,
+                              const void* mask, int mask_kind, const int32_t* cu, int64_t n_rows,
+                              int64_t n_slots, int64_t uniform_len, int kl_type, float beta,
+                              float* rewards, float* row_vals, void* stream) {
+  int rc = check_rows2(cu, n_rows, n_slots, uniform_len, true);
+  if (rc != AXON_OK) return rc;
+  if (n_slots == 0) return AXON_OK;
+  if (!scores || !old_logp || !ref_logp || !mask || !rewards || !row_vals) return AXON_ERR_ARG;
+  if (kl_type < 1 || kl_type > 4) return AXON_ERR_ARG;
+  if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  const dim3 g(stream_grid(n_slots)), blk(kBlock);
+  if (mask_kind == AXON_MASK_F32)
+    hipLaunchKernelGGL(kl_reward_kernel<AXON_MASK_F32>, g, blk, 0, (hipStream_t)stream, scores, old_logp,
+                       ref_logp, mask, cu, n_rows, n_slots, uniform_len, kl_type, beta, rewards, row_vals);
+  else
+    hipLaunchKernelGGL(kl_reward_kernel<AXON_MASK_I64>, g, blk, 0, (hipStream_t)stream, scores, old_logp,
+                       ref_logp, mask, cu, n_rows, n_slots, uniform_len, kl_type, beta, rewards, row_vals);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 11
+#define AXON_AMD_ABI_VERSION 12
 
 enum {
   AXON_OK = 0,
@@ -327,6 +327,17 @@ int axon_logits_bwd(const void* logits, int dtype, int64_t ld, int64_t n, int64_
                     const void* labels, int labels_are_i64, const float* lse, const float* entropy,
                     const float* g_logprob, const float* g_entropy, void* dlogits, int64_t ld_dlogits,
                     void* stream);
+
+/* KL penalty inside the reward, the tensor part of apply_kl_penalty (axon/utils/rl/kl.py:276-322):
+ *   kld = kl_penalty(old_logp, ref_logp, kl_type) * mask      (types as in axon_kl_penalty)
+ *   rewards = scores - beta * kld
+ *   row_vals[0][r] = sum_t mask,  row_vals[1][r] = sum_t kld  (row_vals [2][n_rows], zero-filled by the caller)
+ * from which the caller forms current_kl = mean_r(row_vals[1][r] / max(row_vals[0][r], 1)) for its KL
+ * controller. */
+int axon_kl_reward(const float* scores, const float* old_logp, const float* ref_logp, const void* mask,
+                   int mask_kind, const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                   int64_t uniform_len, int kl_type, float beta, float* rewards, float* row_vals,
+                   void* stream);
 
 /* Time recurrences of the return-based advantage estimators, run from each row's last token to its
  * first (axon/trainer/algos/advantages/advantage.py), before any whitening:

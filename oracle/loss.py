@@ -284,3 +284,11 @@ def clip_cov_loss(log_prob, old_log_prob, advantages, response_mask, *, selected
     metrics = {"pg_clipfrac": float(masked_mean((corr == 0).float(), response_mask)),
                "ppo_kl": float(masked_mean(-nak, response_mask).detach())}
     return loss, metrics
+
+
+def apply_kl_penalty(token_level_scores, old_log_probs, ref_log_prob, response_mask, beta, kl_penalty_type="kl"):
+    """axon/utils/rl/kl.py:276-322 without the controller: ``(token_level_rewards, current_kl)``."""
+    kld = kl_penalty(old_log_probs, ref_log_prob, kl_penalty_type) * response_mask
+    rewards = token_level_scores - beta * kld
+    lengths = response_mask.sum(dim=-1).clamp(min=1)
+    return rewards, float((kld.sum(dim=-1) / lengths).mean())

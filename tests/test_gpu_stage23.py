@@ -770,3 +770,49 @@ def test_views_off_a_16_byte_boundary():
     a2, g2 = _ops.policy_loss(0, x.clone(), x.clone() * 0.9, x.clone(), mask.clone(), None, rows, token_reduce="sum",
                               batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.2, clip_c=3.0)
     assert torch.equal(a1[:5], a2[:5]) and torch.equal(g1, g2)
+
+
+# ---- KL penalty inside the reward (kl.py:248-322) -----------------------------------------------------------
+@pytest.mark.parametrize("ktype", ["kl", "abs", "mse", "low_var_kl"])
+@pytest.mark.parametrize("where", ["gpu", "cpu"])
+def test_apply_kl_penalty_vs_oracle(ktype, where):
+    from axon_amd.utils.rl.kl import AdaptiveKLController, apply_kl_penalty, compute_rewards_with_kl
+    g = torch.Generator().manual_seed(71)
+    b, t = 7, 333
+    scores = torch.randn(b, t, generator=g)
+    old = -torch.empty(b, t).exponential_(1.0, generator=g)
+    ref = old + 0.3 * torch.randn(b, t, generator=g)
+    mask = (torch.rand(b, t, generator=g) > 0.3).float()
+    mask[2] = 0
+    dev = DEV if where == "gpu" else "cpu"
+    ctrl = AdaptiveKLController(init_kl_coef=0.2, target_kl=0.01, horizon=100)
+    rewards, m = apply_kl_penalty(scores.to(dev), old.to(dev), ref.to(dev), mask.to(dev), ctrl, ktype)
+    ref_rewards, ref_kl = OL.apply_kl_penalty(scores, old, ref, mask, 0.2, ktype)
+    assert rewards.device.type == ("cuda" if where == "gpu" else "cpu")
+    assert torch.allclose(rewards.cpu(), ref_rewards, rtol=1e-5, atol=1e-6)
+    assert m["actor/reward_kl_penalty"] == pytest.approx(ref_kl, rel=1e-4, abs=1e-7)
+    assert m["actor/reward_kl_penalty_coeff"] == 0.2
+    expect = AdaptiveKLController(0.2, 0.01, 100)
+    expect.update(ref_kl, b)
+    assert ctrl.value == pytest.approx(expect.value, rel=1e-6)  # the controller saw n_steps = number of sequences
+    plain = compute_rewards_with_kl(scores.to(dev), old.to(dev), ref.to(dev), 0.05)
+    assert torch.allclose(plain.cpu(), scores - (old - ref) * 0.05, rtol=1e-5, atol=1e-6)
+
+
+def test_apply_kl_penalty_packed_layout():
+    from axon_amd.utils.rl.kl import FixedKLController, apply_kl_penalty
+    lens = [700, 33, 1, 1200, 64, 257]
+    n = sum(lens)
+    g = torch.Generator().manual_seed(73)
+    scores, old = torch.randn(n, generator=g), -torch.empty(n).exponential_(1.0, generator=g)
+    ref = old + 0.2 * torch.randn(n, generator=g)
+    mask = (torch.rand(n, generator=g) > 0.2).float()
+    cu = W.cu_from_lengths(lens)
+    rewards, m = apply_kl_penalty(scores.to(DEV), old.to(DEV), ref.to(DEV), mask.to(DEV), FixedKLController(0.1),
+                                  "low_var_kl", cu_seqlens=cu)
+    tmax = max(lens)
+    pad = lambda x: torch.stack([torch.nn.functional.pad(x[s:e], (0, tmax - (e - s)))  # noqa: E731
+                                 for s, e in zip(cu[:-1].tolist(), cu[1:].tolist())])
+    ref_rewards, ref_kl = OL.apply_kl_penalty(pad(scores), pad(old), pad(ref), pad(mask), 0.1, "low_var_kl")
+    assert torch.allclose(rewards.cpu(), pad_to_packed(ref_rewards, lens), rtol=1e-5, atol=1e-6)
+    assert m["actor/reward_kl_penalty"] == pytest.approx(ref_kl, rel=1e-4)

@@ -216,3 +216,38 @@ def test_rolled_label_precedence_and_output_type():
 
     assert final_logit_softcapping(Multi()) == 30.0 and final_logit_softcapping(Text()) == 30.0
     assert final_logit_softcapping(Plain()) is None
+
+
+# ---- KL controllers: known answers of the reference's tests/utils/test_kl.py:26-150 ----------------------------
+def test_kl_controllers_known_answers():
+    import math
+    from types import SimpleNamespace
+    from axon_amd.utils.rl.kl import AdaptiveKLController, FixedKLController, get_kl_controller
+    c = AdaptiveKLController(init_kl_coef=0.5, target_kl=4.0, horizon=1000)
+    c.update(current_kl=8.0, n_steps=10)  # error 1.0 clipped to 0.2
+    assert c.value == pytest.approx(0.5 * (1 + 0.2 * 10 / 1000))
+    c = AdaptiveKLController(1.0, 10.0, 100)
+    c.update(current_kl=0.001, n_steps=10)  # clipped to -0.2
+    assert c.value == pytest.approx(1 - 0.2 * 10 / 100)
+    c = AdaptiveKLController(1.0, 5.0, 100)
+    for _ in range(3):
+        c.update(10.0, 10)
+    assert c.value == pytest.approx(1.02 ** 3)
+    c = AdaptiveKLController(0.1, 6.0, 10000)
+    c.update(6.0, 32)
+    assert c.value == 0.1  # at the target: unchanged
+    c.update(100.0, 0)
+    assert c.value == 0.1  # no steps: unchanged
+    z = AdaptiveKLController(0.1, 0.0, 10)
+    z.update(0.5, 1)  # a zero target does not divide by zero
+    assert z.value == pytest.approx(0.1 * (1 + 0.2 / 10)) and math.isfinite(z.value)
+    f = FixedKLController(kl_coef=0.05)
+    f.update(100.0, 32)
+    assert f.value == 0.05
+    assert isinstance(get_kl_controller(SimpleNamespace(type="fixed", kl_coef=0.1)), FixedKLController)
+    a = get_kl_controller(SimpleNamespace(type="adaptive", kl_coef=0.2, target_kl=6.0, horizon=100))
+    assert isinstance(a, AdaptiveKLController) and (a.value, a.target, a.horizon) == (0.2, 6.0, 100)
+    with pytest.raises(AssertionError, match="horizon must be larger than 0"):
+        get_kl_controller(SimpleNamespace(type="adaptive", kl_coef=0.2, target_kl=6.0, horizon=0))
+    with pytest.raises(NotImplementedError):
+        get_kl_controller(SimpleNamespace(type="bogus", kl_coef=0.2))
