@@ -816,3 +816,32 @@ def test_apply_kl_penalty_packed_layout():
     ref_rewards, ref_kl = OL.apply_kl_penalty(pad(scores), pad(old), pad(ref), pad(mask), 0.1, "low_var_kl")
     assert torch.allclose(rewards.cpu(), pad_to_packed(ref_rewards, lens), rtol=1e-5, atol=1e-6)
     assert m["actor/reward_kl_penalty"] == pytest.approx(ref_kl, rel=1e-4)
+
+
+# ---- reward statistics and pass metrics: known answers of the reference's tests/utils/test_rl_utils.py:107-263 --
+def test_reward_statistics_and_pass_metrics_known_answers():
+    from axon_amd.utils.rl.utils import compute_pass_metrics, compute_reward_statistics
+
+    def proto(scores, **nt):
+        return DataProto.from_dict(tensors={"token_level_scores": T(scores).to(DEV)},
+                                   non_tensors={k: np.array(v) for k, v in nt.items()})
+    s = compute_reward_statistics(proto([[0.0, 1.0], [0.0, 2.0], [0.0, 100.0]], is_padding=[False, False, True],
+                                        is_last_step=[True, True, True]))
+    assert (s["batch/reward/mean"], s["batch/reward/max"], s["batch/reward/min"]) == (1.5, 2.0, 1.0)
+    s = compute_reward_statistics(proto([[0.0, 1.0], [0.0, 2.0], [0.0, 3.0]], is_padding=[False] * 3,
+                                        is_last_step=[True, False, True]))
+    assert (s["batch/reward/mean"], s["batch/reward/max"], s["batch/reward/min"]) == (2.0, 3.0, 1.0)
+    s = compute_reward_statistics(proto([[0.0, 1.0]], is_padding=[True]))
+    assert s == {"reward_mean": 0.0, "reward_max": 0.0, "reward_min": 0.0}
+    s = compute_reward_statistics(proto([[-1.0, 0.0], [-2.0, -3.0], [-3.0, 0.0]]))
+    assert (s["batch/reward/mean"], s["batch/reward/max"], s["batch/reward/min"]) == (-3.0, -1.0, -5.0)
+    m, rates = compute_pass_metrics(proto([[0.0, 1.0], [0.0, 0.0], [0.0, 2.0], [0.0, 1.0]], uid=["a", "a", "b", "b"]))
+    assert m == {"batch/solve/none": 0, "batch/solve/all": 1, "batch/solve/partial": 1}
+    assert rates["a"] == 0.5 and rates["b"] == 1.0
+    m, rates = compute_pass_metrics(proto([[0.0, 100.0], [0.0, 1.0], [0.0, 0.0], [0.0, 2.0]], uid=["a", "a", "b", "b"],
+                                          is_last_step=[False, True, False, True]))
+    assert rates == {"a": 1.0, "b": 1.0} and m["batch/solve/all"] == 2
+    m, rates = compute_pass_metrics(proto([[0.0, 0.0], [0.0, 0.0], [0.0, -1.0]], uid=["a", "a", "b"]))
+    assert m == {"batch/solve/none": 2, "batch/solve/all": 0, "batch/solve/partial": 0}
+    assert compute_pass_metrics(proto([[0.0, 1.0]], uid=["x"]))[1]["x"] == 1.0
+    assert compute_pass_metrics(proto([[0.0, 0.999]], uid=["x"]))[1]["x"] == 0.0
