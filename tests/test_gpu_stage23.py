@@ -845,3 +845,45 @@ def test_reward_statistics_and_pass_metrics_known_answers():
     assert m == {"batch/solve/none": 2, "batch/solve/all": 0, "batch/solve/partial": 0}
     assert compute_pass_metrics(proto([[0.0, 1.0]], uid=["x"]))[1]["x"] == 1.0
     assert compute_pass_metrics(proto([[0.0, 0.999]], uid=["x"]))[1]["x"] == 0.0
+
+
+# ---- the operators make no host synchronisation and can be captured into a HIP graph ---------------------------
+def test_loss_and_correction_in_a_hip_graph():
+    """Captured once, replayed several times with other inputs and with eager work and synchronisations between
+    the replays: every replay must equal the eager result bit for bit."""
+    g = torch.Generator(device=DEV).manual_seed(1)
+    b, t = 32, 777
+    old = -torch.empty(b, t, device=DEV).exponential_(1.0, generator=g)
+    new = old + 0.05 * torch.randn(b, t, device=DEV, generator=g)
+    samp = old + 0.01 * torch.randn(b, t, device=DEV, generator=g)
+    adv = torch.randn(b, t, device=DEV, generator=g)
+    mask = (torch.rand(b, t, device=DEV, generator=g) > 0.3).float()
+    rows = _ops.rows_of(new)
+    kw = dict(token_reduce="mean", batch_reduce="step-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
+    # token-level weights and rejection, the veto (an integer flag per row) and the PPO loss with per-row token
+    # counts: none of these adds floats atomically, so two runs agree bit for bit (the sequence-level modes and
+    # GSPO add per-row float sums in whatever order the wavefronts arrive and agree to rounding only)
+    ckw = dict(is_mode=1, is_threshold=2.0, rs_mode=1, rs_lr_lo=-math.log(2.0), rs_lr_hi=math.log(2.0),
+               log_veto=math.log(1e-4))
+
+    def chain():
+        isw, new_mask, cacc = _ops.sampler_correction(old, samp, mask, rows, **ckw)
+        acc, grad = _ops.policy_loss(0, new, old, adv, new_mask, isw, rows, **kw)
+        return cacc, acc, grad
+
+    side = torch.cuda.Stream()  # warm-up off the capture stream, as torch asks for
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_cacc, g_acc, g_grad = chain()
+    for _ in range(4):
+        new.copy_(old + 0.05 * torch.randn(b, t, device=DEV, generator=g))
+        samp.copy_(old + 0.01 * torch.randn(b, t, device=DEV, generator=g))
+        e_cacc, e_acc, e_grad = chain()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_acc[:6], e_acc[:6]) and torch.equal(g_grad, e_grad) and torch.equal(g_cacc[:6], e_cacc[:6])
