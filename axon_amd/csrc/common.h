@@ -50,6 +50,23 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Sum over the wavefront by DPP row shifts and broadcasts (no LDS traffic); the total lands in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  const float moved = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+  return v + moved;
+}
+__device__ __forceinline__ float wave_sum_to_last(float v) {
+  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);  // row_shr:8
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Sum NV values over the workgroup; the total lands in thread 0.
 template <int NV>
 __device__ __forceinline__ void block_sum(float (&v)[NV], float* lds /* [NV * 4] */) {
@@ -189,14 +206,36 @@ struct RowFinder {
     return lo;
   }
 
+  // the same count with three probes per step (their loads are independent): half as many dependent loads
+  __device__ static int upper4(const int32_t* cu, int lo, int hi, int64_t pos) {
+    while (hi - lo >= 4) {
+      const int q = (hi - lo) >> 2;
+      const int m1 = lo + q, m2 = lo + 2 * q, m3 = lo + 3 * q;
+      const bool b1 = (int64_t)cu[m1] <= pos, b2 = (int64_t)cu[m2] <= pos, b3 = (int64_t)cu[m3] <= pos;
+      if (b3) lo = m3;
+      else if (b2) { lo = m2; hi = m3 - 1; }
+      else if (b1) { lo = m1; hi = m2 - 1; }
+      else hi = m1 - 1;
+    }
+    return upper(cu, lo, hi, pos);
+  }
+
   __device__ void init(const int32_t* cu_, int64_t n_rows, int64_t uniform_len, int64_t c0,
                        int64_t c1, int32_t* lds) {
     cu = cu_;
     uniform = uniform_len;
     win = nullptr;
     if (uniform_len > 0) return;
-    lo = upper(cu, 0, (int)n_rows, c0);
-    hi = upper(cu, lo, (int)n_rows, c1 - 1);
+    lo = upper4(cu, 0, (int)n_rows, c0);
+    // the chunk's last row is a few rows on: gallop from lo, then search the bracket
+    int step = 1, top = lo;
+    while (top < (int)n_rows) {
+      const int probe = min(top + step, (int)n_rows);
+      if ((int64_t)cu[probe] > c1 - 1) { hi = upper(cu, top, probe - 1, c1 - 1); break; }
+      top = probe;
+      step *= 2;
+    }
+    if (top >= (int)n_rows) hi = (int)n_rows;
     if (lo >= n_rows) lo = (int)n_rows - 1;  // slots past cu[n_rows] (caller error) stay in range
     if (hi >= n_rows) hi = (int)n_rows - 1;
     const int n = hi - lo + 2;

@@ -27,6 +27,17 @@ __device__ __forceinline__ void seg_flush(const Seg& s, float* cnt, float* sum, 
 __device__ __forceinline__ void seg_wave_reduce_flush(Seg s, float* cnt, float* sum,
                                                       int32_t* flag) {
   const int lane = threadIdx.x & (kWave - 1);
+  // the common case: the whole wavefront sits in one row (rows are mostly longer than 256 slots)
+  const int first = __builtin_amdgcn_readfirstlane(s.row);
+  if (first >= 0 && __builtin_amdgcn_readlane(s.row, kWave - 1) == first) {  // rows are sorted across lanes
+    Seg t;
+    t.row = first;
+    t.cnt = wave_sum_to_last(s.cnt);
+    t.sum = wave_sum_to_last(s.sum);
+    t.flag = (flag != nullptr) ? (__ballot(s.flag != 0) != 0) : 0;
+    if (lane == kWave - 1) seg_flush(t, cnt, sum, flag);
+    return;
+  }
 #pragma unroll
   for (int off = 1; off < kWave; off <<= 1) {
     const int r2 = __shfl_down(s.row, off, kWave);
