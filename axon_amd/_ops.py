@@ -94,9 +94,13 @@ def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=Tr
     a = f32(a)
     b = f32(b) if b is not None else None
     mk = (None, MASK_F32) if mask is None else mask_arg(mask)
-    cnt = _zeros(rows.n_rows, dev) if want_cnt else None
-    ssum = _zeros(rows.n_rows, dev) if want_sum else None
-    flag = _zeros(rows.n_rows, dev, torch.int32) if flag_mode else None
+    # one zero-filled buffer (one fill launch) carries the up to three per-row outputs
+    parts = [want_cnt, want_sum, bool(flag_mode)]
+    buf = _zeros(sum(parts) * max(rows.n_rows, 1), dev).view(sum(parts), -1) if any(parts) else None
+    slots = iter(range(sum(parts)))
+    cnt = buf[next(slots)][: rows.n_rows] if want_cnt else None
+    ssum = buf[next(slots)][: rows.n_rows] if want_sum else None
+    flag = buf[next(slots)][: rows.n_rows].view(torch.int32) if flag_mode else None
     check(
         lib.axon_row_stats(ptr(a), ptr(b), ptr(mk[0]), mk[1], rows.cu_ptr, rows.n_rows, rows.n_slots,
                            rows.uniform_len, flag_mode, float(threshold), ptr(cnt), ptr(ssum), ptr(flag),
