@@ -170,6 +170,14 @@ __device__ __forceinline__ void row_seg_flush(const RowSeg<NV>& s, float* row_va
 template <int NV>
 __device__ __forceinline__ void row_seg_wave_reduce_flush(RowSeg<NV> s, float* row_vals, int64_t n_rows) {
   const int lane = threadIdx.x & (kWave - 1);
+  // the common case: the whole wavefront sits in one row (rows are sorted across lanes)
+  const int first = __builtin_amdgcn_readfirstlane(s.row);
+  if (first >= 0 && __builtin_amdgcn_readlane(s.row, kWave - 1) == first) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) s.v[k] = wave_sum_to_last(s.v[k]);
+    if (lane == kWave - 1) row_seg_flush(s, row_vals, n_rows);
+    return;
+  }
 #pragma unroll
   for (int off = 1; off < kWave; off <<= 1) {
     const int r2 = __shfl_down(s.row, off, kWave);
