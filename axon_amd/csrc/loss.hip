@@ -186,8 +186,11 @@ __global__ __launch_bounds__(1024) void loss_row_scale_kernel(
   if (valid != nullptr) bden = fmaxf((float)valid[0], 1.f);
   else if (batch_reduce == 0) bden = fmaxf(tot[0], 1.f);
   else bden = fmaxf(tot[1], 1.f);
+  // every workgroup has formed the same totals in the same order; each writes its own slice of the rows
+  const int64_t per = (n_rows + gridDim.x - 1) / gridDim.x;
+  const int64_t r_begin = (int64_t)blockIdx.x * per, r_end = min(r_begin + per, n_rows);
 #pragma unroll 8
-  for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) {
+  for (int64_t r = r_begin + threadIdx.x; r < r_end; r += blockDim.x) {
     const float c = row_cnt[r];
     float td = 1.f;
     if (token_reduce == 1) td = fmaxf(prtc ? (float)prtc[r] : c, 1.f);
@@ -802,7 +805,10 @@ extern "C" int axon_loss_row_scale(const float* row_cnt, const float* row_sum, i
   if (token_reduce == 3 && !npt) return AXON_ERR_ARG;
   if (token_reduce == 2 && row_len <= 0) return AXON_ERR_ARG;
   if (batch_reduce == 2 && (!nps || !valid)) return AXON_ERR_ARG;
-  hipLaunchKernelGGL(loss_row_scale_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, row_cnt,
+  // the pass over the counts is repeated by every workgroup (cheap: 4 bytes per row from L2); the per-row
+  // pass is shared out
+  const unsigned blocks = (unsigned)((n_rows + 2047) / 2048 < 64 ? (n_rows + 2047) / 2048 : 64);
+  hipLaunchKernelGGL(loss_row_scale_kernel, dim3(blocks), dim3(1024), 0, (hipStream_t)stream, row_cnt,
                      row_sum, n_rows, row_len, token_reduce, batch_reduce, prtc, npt, nps, valid,
                      row_scale, row_mean);
   AXON_CHECK_LAUNCH();

@@ -265,7 +265,7 @@ int axon_sampler_diag(const float* old_logp, const float* sampler_logp, const vo
  *   int64 [n_rows]; valid_count: optional int64 pointer whose element [0] is
  *   the mini-batch-wide denominator (utils.py:224-229), else computed locally.
  * Outputs row_scale[n_rows], row_mean[n_rows] (= row_sum / max(row_cnt,1)).
- * Single workgroup. */
+ * Up to 64 workgroups: each repeats the pass over the counts (same order, same totals) and writes its share of the rows. */
 int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_rows,
                         int64_t row_len_for_norm, int token_reduce, int batch_reduce,
                         const int64_t* per_row_token_count, const int64_t* num_program_tokens,
