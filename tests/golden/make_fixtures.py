@@ -20,6 +20,10 @@ tensors are stored as their 16-bit patterns (``int16``).
   sampler_boundaries.npz      log-ratios within 20 ulps of +-ln 2 and ln 1e-4: rejection mask,
                               veto mask, truncated IS weights
   grpo_groups.npz             GRPO advantages for group sizes 1/2/3/8 incl. an all-equal group
+  gae_returns.npz             GAE, chunked GAE, REINFORCE++ and ReMax on 6 rows of 300 tokens with
+                              observation gaps in the response: advantages and returns
+  value_kl_cov.npz            clipped value loss and KL-Cov loss on 8 x 257 tokens: loss, gradient,
+                              metrics, the tokens KL-Cov picks
 """
 
 from __future__ import annotations
@@ -39,6 +43,7 @@ if ROOT not in sys.path:
 from oracle import advantage as OA  # noqa: E402
 from oracle import lmhead as OM  # noqa: E402
 from oracle import loss as OL  # noqa: E402
+from oracle import returns as OR  # noqa: E402
 from oracle import sampler as OS  # noqa: E402
 
 
@@ -162,6 +167,48 @@ def grpo_groups():
          std=std, count=cnt, **out)
 
 
+def gae_returns():
+    g = torch.Generator().manual_seed(6)
+    b, t = 6, 300
+    rewards = torch.randn(b, t, generator=g) * (torch.rand(b, t, generator=g) > 0.8)
+    values = torch.randn(b, t, generator=g)
+    lens = torch.tensor([300, 1, 64, 257, 150, 299])
+    mask = (torch.arange(t)[None] < lens[:, None]).float() * (torch.rand(b, t, generator=g) > 0.2)
+    mask[1, 0] = 1
+    base = torch.randn(b, generator=g)
+    gae_adv, gae_ret = OR.gae_advantage(rewards, values, mask, 0.99, 0.95)
+    raw_adv, _ = OR.gae_raw(rewards, values, mask, 0.99, 0.95)
+    ch_adv, ch_ret = OR.chunked_gae_advantage(rewards, values, mask, 0.99, 0.95)
+    rpp_adv, rpp_ret = OR.reinforce_plus_plus_advantage(rewards, mask, 0.97)
+    rm_adv, rm_ret = OR.remax_advantage(rewards, mask, base)
+    save("gae_returns.npz", rewards=rewards, values=values, response_mask=mask, reward_baselines=base,
+         gae_raw=raw_adv, gae_adv=gae_adv, gae_ret=gae_ret, chunked_adv=ch_adv, chunked_ret=ch_ret, rpp_adv=rpp_adv,
+         rpp_ret=rpp_ret, remax_adv=rm_adv, remax_ret=rm_ret)
+
+
+def value_kl_cov():
+    g = torch.Generator().manual_seed(8)
+    b, t = 8, 257
+    values = torch.randn(b, t, generator=g)
+    vpreds = values + 0.4 * torch.randn(b, t, generator=g)
+    returns = values + torch.randn(b, t, generator=g)
+    mask = (torch.rand(b, t, generator=g) > 0.3).float()
+    mask[5] = 0
+    vp = vpreds.clone().requires_grad_(True)
+    vloss, vm = OR.value_loss(vp, values, returns, mask, cliprange_value=0.3)
+    vloss.backward()
+    old = -torch.empty(b, t).exponential_(1.0, generator=g)
+    lp = (old + 0.1 * torch.randn(b, t, generator=g)).requires_grad_(True)
+    adv = torch.randn(b, 1, generator=g).expand(b, t).contiguous() + 0.1 * torch.randn(b, t, generator=g)
+    kloss, km, picked = OL.kl_cov_loss(lp, old, adv, mask, kl_cov_ratio=0.01, ppo_kl_coef=1.0)
+    kloss.backward()
+    save("value_kl_cov.npz", values=values, vpreds=vpreds, returns=returns, response_mask=mask,
+         value_loss=vloss.detach(), value_grad=vp.grad, vf_clipfrac=np.float32(vm["vf_clipfrac"]),
+         vpred_mean=np.float32(vm["vpred_mean"]), old_log_probs=old, log_probs=lp.detach(), advantages=adv,
+         kl_cov_loss=kloss.detach(), kl_cov_grad=lp.grad, kl_cov_ppo_kl=np.float32(km["ppo_kl"]),
+         kl_cov_picked=torch.sort(picked).values)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)  # summation order of the CPU reductions independent of the machine
     lmhead()
@@ -169,3 +216,5 @@ if __name__ == "__main__":
     gspo_ragged()
     sampler_boundaries()
     grpo_groups()
+    gae_returns()
+    value_kl_cov()

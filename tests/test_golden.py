@@ -16,6 +16,7 @@ import torch
 from oracle import advantage as OA
 from oracle import lmhead as OM
 from oracle import loss as OL
+from oracle import returns as OR
 from oracle import sampler as OS
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
@@ -167,6 +168,69 @@ def test_fixture_grpo_groups():
         assert torch.allclose(got, f[f"adv_norm{int(norm)}"], atol=1e-7)
 
 
+def test_fixture_gae_returns():
+    f = load("gae_returns.npz")
+    r, v, m = f["rewards"], f["values"], f["response_mask"]
+    # the oracle reproduces what is stored
+    adv, ret = OR.gae_advantage(r, v, m, 0.99, 0.95)
+    assert torch.allclose(adv, f["gae_adv"], atol=1e-6) and torch.allclose(ret, f["gae_ret"], atol=1e-6)
+    cadv, cret = OR.chunked_gae_advantage(r, v, m, 0.99, 0.95)
+    assert torch.allclose(cadv, f["chunked_adv"], atol=1e-6) and torch.allclose(cret, f["chunked_ret"], atol=1e-6)
+    # facts that do not come from the oracle: the fp64 recurrence over the gathered response tokens of each row
+    for b in range(r.shape[0]):
+        idx = torch.nonzero(m[b] > 0).flatten().tolist()
+        s, nextv = 0.0, 0.0
+        for i in reversed(idx):
+            delta = float(r[b, i]) + 0.99 * nextv - float(v[b, i])
+            s = delta + 0.99 * 0.95 * s
+            nextv = float(v[b, i])
+            assert f["gae_raw"][b, i].item() == pytest.approx(s, abs=2e-5)
+            assert f["chunked_ret"][b, i].item() == pytest.approx(s + float(v[b, i]), abs=2e-5)
+    assert (f["chunked_ret"][m == 0] == 0).all()
+    n = m.sum()
+    white = f["gae_adv"]
+    mean = (white * m).sum() / n
+    assert abs(float(mean)) < 1e-5 and float((((white - mean) ** 2) * m).sum() / (n - 1)) == pytest.approx(1.0, abs=1e-4)
+    # REINFORCE++: ret[t] = r[t] + gamma * mask[t+1] * ret[t+1];  ReMax: suffix sums of the masked rewards
+    ret = f["rpp_ret"].double()
+    nxt = torch.cat([(ret * m.double())[:, 1:], torch.zeros(r.shape[0], 1, dtype=torch.float64)], 1)
+    assert torch.allclose(ret, r.double() + 0.97 * nxt, atol=1e-5)
+    assert (f["rpp_adv"][m == 0] == 0).all()
+    togo = (r.double() * m.double()).flip(-1).cumsum(-1).flip(-1)
+    assert torch.allclose(f["remax_ret"].double(), togo, atol=1e-5)
+    assert torch.allclose(f["remax_adv"].double(), togo - f["reward_baselines"].double()[:, None] * m.double(), atol=1e-5)
+
+
+def test_fixture_value_kl_cov():
+    f = load("value_kl_cov.npz")
+    v, vp, ret, m = f["values"].double(), f["vpreds"].double(), f["returns"].double(), f["response_mask"].double()
+    clipped = torch.maximum(torch.minimum(vp, v + 0.3), v - 0.3)
+    l1, l2 = (vp - ret) ** 2, (clipped - ret) ** 2
+    n = m.sum()
+    assert f["value_loss"].item() == pytest.approx(float(0.5 * (torch.maximum(l1, l2) * m).sum() / n), rel=1e-5)
+    inside = (vp >= v - 0.3) & (vp <= v + 0.3)
+    g = torch.where(inside | (l1 > l2), vp - ret, torch.zeros_like(vp)) * m / n  # the clipped branch has no gradient
+    assert torch.allclose(f["value_grad"].double(), g, atol=1e-7)
+    assert f["vf_clipfrac"].item() == pytest.approx(float(((l2 > l1).double() * m).sum() / n), rel=1e-5)
+    # KL-Cov: the picked tokens are the k = max(1, int(n * 0.01)) largest covariances among the response tokens
+    lp, old, adv = f["log_probs"].double(), f["old_log_probs"].double(), f["advantages"].double()
+    valid = m.flatten() > 0
+    a, l = adv.flatten()[valid], lp.flatten()[valid]
+    cov = (a - a.mean()) * (l - l.mean())
+    k = max(1, int(int(valid.sum()) * 0.01))
+    want = torch.nonzero(valid).flatten()[torch.topk(cov, k).indices]
+    assert sorted(want.tolist()) == f["kl_cov_picked"].tolist()
+    nak = lp - old
+    per = -adv * torch.exp(nak)
+    per.view(-1)[f["kl_cov_picked"]] += nak.abs().view(-1)[f["kl_cov_picked"]]
+    assert f["kl_cov_loss"].item() == pytest.approx(float((per * m).sum() / n), rel=1e-5)
+    assert f["kl_cov_ppo_kl"].item() == pytest.approx(float((nak.abs() * m).sum() / n), rel=1e-5)
+    # and the oracle reproduces what is stored
+    x = f["vpreds"].clone().requires_grad_(True)
+    loss, _ = OR.value_loss(x, f["values"], f["returns"], f["response_mask"], cliprange_value=0.3)
+    assert loss.item() == pytest.approx(f["value_loss"].item(), rel=1e-6)
+
+
 # ---------------------------------------------------------------------------------------------
 # GPU: HIP path vs fixtures
 # ---------------------------------------------------------------------------------------------
@@ -260,3 +324,67 @@ def test_gpu_grpo_groups_match_fixture(norm):
     got = out.batch["advantages"].cpu()
     assert torch.allclose(got, want, atol=2e-6, rtol=1e-5)
     assert (got[f["response_mask"] == 0] == 0).all()
+
+
+@pytest.mark.gpu
+def test_gpu_gae_returns_match_fixture():
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.advantages import compute_advantage
+    f = load("gae_returns.npz")
+
+    def run(name, args, extra=()):
+        keys = ("rewards", "values", "response_mask") + tuple(extra)
+        names = {"rewards": "token_level_rewards"}
+        data = DataProto.from_dict(tensors={names.get(k, k): f[k].to(DEV) for k in keys})
+        out = compute_advantage(data, {"advantage": name, "advantage_args": args})
+        return out.batch["advantages"].cpu(), out.batch["returns"].cpu()
+
+    adv, ret = run("gae", {"gamma": 0.99, "lam": 0.95})
+    assert rel_l2(ret, f["gae_ret"]) < 2e-5 and rel_l2(adv, f["gae_adv"]) < 1e-4
+    adv, ret = run("chunked_gae", {"gamma": 0.99, "lam": 0.95})
+    assert rel_l2(ret, f["chunked_ret"]) < 2e-5 and rel_l2(adv, f["chunked_adv"]) < 1e-4
+    assert (ret[f["response_mask"] == 0] == 0).all()
+    adv, ret = run("reinforce_plus_plus", {"gamma": 0.97})
+    assert rel_l2(ret, f["rpp_ret"]) < 2e-5 and rel_l2(adv, f["rpp_adv"]) < 1e-4
+    adv, ret = run("remax", {}, extra=("reward_baselines",))
+    assert rel_l2(ret, f["remax_ret"]) < 2e-5 and rel_l2(adv, f["remax_adv"]) < 2e-5
+
+
+@pytest.mark.gpu
+def test_gpu_value_and_kl_cov_match_fixture():
+    from axon_amd import _ops
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    f = load("value_kl_cov.npz")
+    vp = f["vpreds"].to(DEV).requires_grad_(True)
+    data = DataProto.from_dict(tensors={"values": f["values"].to(DEV), "returns": f["returns"].to(DEV),
+                                        "response_mask": f["response_mask"].to(DEV)})
+    data.batch["vpreds"] = vp
+    loss, m = compute_loss_fn(data, "value", {"cliprange_value": 0.3})
+    loss.backward()
+    assert loss.item() == pytest.approx(f["value_loss"].item(), rel=1e-4)
+    assert rel_l2(vp.grad, f["value_grad"]) < 1e-5
+    assert m["vf_clipfrac"] == pytest.approx(f["vf_clipfrac"].item(), rel=1e-5)
+    assert m["vpred_mean"] == pytest.approx(f["vpred_mean"].item(), rel=1e-4, abs=1e-6)
+    lp = f["log_probs"].to(DEV).requires_grad_(True)
+    data = DataProto.from_dict(tensors={"old_log_probs": f["old_log_probs"].to(DEV),
+                                        "advantages": f["advantages"].to(DEV),
+                                        "response_mask": f["response_mask"].to(DEV)})
+    data.batch["log_probs"] = lp
+    loss, m = compute_loss_fn(data, "kl_cov", {"kl_cov_ratio": 0.01, "ppo_kl_coef": 1.0})
+    loss.backward()
+    assert loss.item() == pytest.approx(f["kl_cov_loss"].item(), rel=1e-4)
+    assert rel_l2(lp.grad, f["kl_cov_grad"]) < 1e-5
+    assert m["ppo_kl"] == pytest.approx(f["kl_cov_ppo_kl"].item(), rel=1e-4)
+    # the picked token indices, bit-exact
+    rows = _ops.rows_of(f["log_probs"].to(DEV))
+    _, _, keys, state = _ops.cov_policy_loss(0, f["log_probs"].to(DEV), f["old_log_probs"].to(DEV),
+                                             f["advantages"].to(DEV), f["response_mask"].to(DEV), None, rows,
+                                             select_ratio=0.01, kl_coef=1.0, token_reduce="sum",
+                                             batch_reduce="token-mean")
+    raw = state.cpu().numpy().tobytes()
+    thr = np.frombuffer(raw[0:4], np.uint32)[0]
+    limit = np.frombuffer(raw[16:24], np.int64)[0]
+    key = keys.cpu().numpy()[: f["log_probs"].numel()].view(np.uint32)
+    hit = (key != 0) & ((key > thr) | ((key == thr) & (np.arange(key.size) < limit)))
+    assert np.nonzero(hit)[0].tolist() == f["kl_cov_picked"].tolist()
