@@ -404,9 +404,11 @@ struct RegLoop {
 // different XCDs (round-robin over 8), so ids are first regrouped so that each
 // XCD walks a contiguous range, and inside that range tiles are visited in
 // bands of `kBand` n-tiles so that concurrently resident workgroups of one XCD
-// share A and B tiles in its L2.
+// share A and B tiles in its L2 (32 workgroups per XCD: 8 x 4 tiles at kBand = 4, 4 x 8 at kBand = 8; the
+// forward, whose A operand is the weight, is 1.7 % faster with 8, the output GEMMs 2.3 % faster with 4).
+template <int kBand = 4>
 __device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, int& tn) {
-  constexpr int kXcd = 8, kBand = 4;
+  constexpr int kXcd = 8;
   const int total = tiles_m * tiles_n;
   int pid = blockIdx.x;
   const int per = total / kXcd;  // ids beyond kXcd*per keep their natural position

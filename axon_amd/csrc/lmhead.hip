@@ -119,7 +119,7 @@ __device__ __forceinline__ void fwd_body(const GemmOperands& g, const FwdParams&
                                          int tiles_n) {
   extern __shared__ __align__(16) char smem[];
   int tm, tn;
-  tile_coords(tiles_m, tiles_n, tm, tn);
+  tile_coords<8>(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);
   AccTile acc;
   Loop::run(g, t, acc, smem);
