@@ -196,6 +196,70 @@ def hbm_kernels(n_tokens, dev):
     return {"tokens": n_tokens, "sequences": len(lens), "bound": "hbm", "kernels": out}
 
 
+def baseline_sizes_cold(dev):
+    """The loss and correction operators at the two small published sizes (padded 128 x 1024 PPO;
+    65536 packed tokens of correction + GSPO), each timed twice: on one set of buffers (inputs
+    sit in L2 / Infinity Cache) and rotating through more than 512 MB of distinct input sets, so
+    every call reads its inputs from HBM.  Microseconds per call of the whole operator, every
+    launch included; at these sizes launches, not bandwidth, set the time."""
+    import math
+
+    import torch
+
+    from axon_amd import _ops, workloads as W
+
+    def per_call_us(fn, sets, rounds):
+        for k in range(min(sets, 8)):
+            fn(k)
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(rounds):
+            for k in range(sets):
+                fn(k)
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) * 1e3 / (rounds * sets)
+
+    def stack(t, sets):  # `sets` copies at distinct addresses
+        return t.to(dev).unsqueeze(0).repeat(sets, *([1] * t.dim())).contiguous()
+
+    out = []
+    c1 = W.c1_loss_only()
+    sets = 288  # x 4 inputs x 512 KiB = 576 MiB
+    new, old, mask = (stack(c1[k], sets) for k in ("log_probs", "old_log_probs", "response_mask"))
+    adv = stack(torch.randn(c1["log_probs"].shape, generator=torch.Generator().manual_seed(5)), sets) * mask
+    rows = _ops.rows_of(new[0])
+    ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
+    f = lambda k: _ops.policy_loss(0, new[k], old[k], adv[k], mask[k], None, rows, **ppo)
+    n_slots = rows.n_slots
+    for label, s_, r_ in (("cold", sets, 2), ("cached", 1, 400)):
+        us = per_call_us(f, s_, r_)
+        out.append({"case": "PPO loss + gradient, padded 128 x 1024, sum/token-mean", "inputs": label,
+                    "bytes": n_slots * 20, "us_per_call": us, "achieved_GBps": n_slots * 20 / us / 1e3})
+    del new, old, mask, adv
+
+    c4 = W.c4_correction()
+    sets = 520  # x 4 inputs x 256 KiB = 520 MiB
+    old, samp, new, mask = (stack(c4[k], sets) for k in ("old_log_probs", "sampler_log_probs", "log_probs",
+                                                           "response_mask"))
+    advs = stack(torch.randn(old.shape[1], generator=torch.Generator().manual_seed(6)), sets)
+    rows = _ops.rows_of(new[0], c4["cu_seqlens"].to(dev))
+    n_slots = rows.n_slots
+    corr = dict(is_mode=1, is_threshold=2.0, rs_mode=1, rs_lr_lo=-math.log(2.0), rs_lr_hi=math.log(2.0),
+                log_veto=math.log(1e-4))
+    gspo = dict(token_reduce="mean", batch_reduce="step-mean", ratio_lo=1 - 3e-4, ratio_hi=1 + 4e-4, clip_c=3.0)
+    fc = lambda k: _ops.sampler_correction(old[k], samp[k], mask[k], rows, **corr)
+    fg = lambda k: _ops.policy_loss(1, new[k], old[k], advs[k], mask[k], None, rows, **gspo)
+    for case, fn, nbytes in (("sampler correction (token IS, token rejection, veto), 65536 packed tokens", fc, 20),
+                             ("GSPO loss + gradient, 65536 packed tokens, mean/step-mean", fg, 20)):
+        for label, s_, r_ in (("cold", sets, 1), ("cached", 1, 400)):
+            us = per_call_us(fn, s_, r_)
+            out.append({"case": case, "inputs": label, "bytes": n_slots * nbytes, "us_per_call": us,
+                        "achieved_GBps": n_slots * nbytes / us / 1e3})
+    return out
+
+
 # HBM-side bytes of ONE launch of the dominant kernel at the default workload, from rocprofv3 --pmc passes
 # over `bench.py --traffic-probe` (FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0, the factors a 1 GiB
 # device copy in the same run calibrates): 12.35e9 read + 0.45e9 written, default vocabulary chunk.
@@ -343,6 +407,7 @@ def main():
         del hd, wd, dh, dw
         torch.cuda.empty_cache()
         out["hbm_kernels"] = hbm_kernels(args.hbm_tokens, dev)
+        out["hbm_kernels"]["baseline_sizes"] = baseline_sizes_cold(dev)
     if args.cpu_seconds > 0:
         out["cpu_baseline"] = cpu_baseline(hid, w, lab, args.cpu_seconds, check=(idx, lp_subset))
     print(json.dumps(out))
