@@ -33,6 +33,10 @@ SIGNATURES: dict[str, tuple] = {
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                      _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_active_rows": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
+    "axon_lmhead_gather_rows": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64,
+                                       _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
+    "axon_lmhead_scatter_rows": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr]),
     "axon_gemm_nt_bf16": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "axon_row_stats": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
                               _ptr, _ptr, _ptr, _ptr]),
@@ -72,7 +76,7 @@ SIGNATURES: dict[str, tuple] = {
                                 _ptr]),
 }
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -607,15 +607,57 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | Non
     return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
 
 
+# The backward runs over the rows with an upstream gradient only when they are at most this share of all rows
+# (below that the two row copies cost more than the skipped work saves).
+SKIP_ROWS_BELOW = 0.97
+
+
+def _active_rows(g_lp, g_en, seq_start, n):
+    """(row_index, row_rank, number of rows whose upstream gradient is not zero); one readback."""
+    lib = _lib.load()
+    idx = torch.empty(2, n, device=g_lp.device, dtype=torch.int32)
+    cnt = torch.empty(1, device=g_lp.device, dtype=torch.int32)
+    check(lib.axon_lmhead_active_rows(ptr(g_lp), ptr(g_en), ptr(seq_start), n, ptr(idx[0]), ptr(idx[1]), ptr(cnt),
+                                      stream_ptr()), "axon_lmhead_active_rows")
+    return idx[0], idx[1], int(cnt.item())
+
+
 def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
-                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None):
-    """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``)."""
+                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=True):
+    """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``).
+
+    With ``skip_zero_rows`` the rows whose upstream gradients are both exactly zero (prompt positions that
+    the trainer slices away, masked or clipped tokens) are left out of the three GEMMs: they contribute
+    nothing to ``d_weight`` and their ``d_hidden`` rows are zero.  Finding them costs one readback, so it
+    is not done while the stream is being captured into a graph."""
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
     lib = _lib.load()
     require_device(hidden, "lmhead_backward")
     n, h, v = _head_operands("lmhead_backward", hidden, weight, labels, seq_start)
     _same_len("lmhead_backward", n, dlogprobs=dlogprobs, dentropy=dentropy, lse=lse, entropy_b=entropy_b)
     dev = hidden.device
+    if skip_zero_rows and n > 0 and h % 8 == 0 and not torch.cuda.is_current_stream_capturing():
+        g_lp = f32(dlogprobs)
+        g_en = f32(dentropy) if dentropy is not None else None
+        row_index, row_rank, n_act = _active_rows(g_lp, g_en, seq_start, n)
+        if n_act == 0:
+            return torch.zeros_like(hidden), torch.zeros_like(weight)
+        if n_act <= SKIP_ROWS_BELOW * n:
+            hidden_c = torch.empty(n_act, h, device=dev, dtype=hidden.dtype)
+            labels_c = torch.empty(n_act, device=dev, dtype=labels.dtype)
+            f = torch.empty(4, n_act, device=dev, dtype=torch.float32)
+            check(lib.axon_lmhead_gather_rows(ptr(hidden), ptr(labels), int(labels.dtype == torch.int64), ptr(lse),
+                                              ptr(entropy_b), ptr(g_lp), ptr(g_en), ptr(seq_start), n, h,
+                                              ptr(row_index), n_act, ptr(hidden_c), ptr(labels_c), ptr(f[0]),
+                                              ptr(f[1]), ptr(f[2]), ptr(f[3] if g_en is not None else None),
+                                              stream_ptr()), "axon_lmhead_gather_rows")
+            dh_c, d_weight = lmhead_backward(f[2], f[3] if g_en is not None else None, hidden_c, weight, labels_c,
+                                             f[0], f[1], inv_temperature, vocab_chunk, timing, softcap, None,
+                                             skip_zero_rows=False)
+            d_hidden = torch.empty_like(hidden)
+            check(lib.axon_lmhead_scatter_rows(ptr(dh_c), ptr(row_rank), n, h, ptr(d_hidden), stream_ptr()),
+                  "axon_lmhead_scatter_rows")
+            return d_hidden, d_weight
     d_hidden = torch.empty_like(hidden)
     d_weight = torch.empty_like(weight)
     ws_bytes = lib.axon_lmhead_bwd_workspace_bytes(n, h, v, int(vocab_chunk))

@@ -532,6 +532,87 @@ __global__ __launch_bounds__(256) void zero_cols_bf16_kernel(uint16_t* p, int64_
     p[(i / ncols) * ld + col0 + (i % ncols)] = 0;
 }
 
+
+// ----------------------------------------------------------------------------
+// Rows without an upstream gradient (prompt positions, masked or clipped tokens)
+// ----------------------------------------------------------------------------
+// One workgroup walks the rows in blocks of 1024 and numbers the active ones in ascending order
+// (ballot + popcount inside a wave, wave totals through LDS): the list is the same on every run.
+__global__ __launch_bounds__(1024) void active_rows_kernel(
+    const float* __restrict__ dlogprobs, const float* __restrict__ dentropy,
+    const uint8_t* __restrict__ is_start, int n_tokens, int32_t* __restrict__ row_index,
+    int32_t* __restrict__ row_rank, int32_t* __restrict__ count) {
+  __shared__ int wave_total[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int base = 0;
+  for (int n0 = 0; n0 < n_tokens; n0 += 1024) {
+    const int n = n0 + (int)threadIdx.x;
+    bool act = false;
+    if (n < n_tokens) {
+      const int src = aligned_pos(n, n_tokens, is_start);
+      if (!(is_start && is_start[src]))
+        act = dlogprobs[src] != 0.f || (dentropy && dentropy[src] != 0.f);  // NaN counts as active
+    }
+    const unsigned long long b = __ballot(act);
+    if (lane == 0) wave_total[wave] = __popcll(b);
+    __syncthreads();
+    int before = base, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+      if (w < wave) before += wave_total[w];
+      total += wave_total[w];
+    }
+    if (n < n_tokens) {
+      const int r = before + __popcll(b & ((1ull << lane) - 1ull));
+      if (act) row_index[r] = n;
+      row_rank[n] = act ? r : -1;
+    }
+    base += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) count[0] = base;
+}
+
+// One workgroup per active row: its hidden vector (16-byte accesses) and its scalars, the label and the
+// gradients taken from the aligned position.
+template <typename LabelT>
+__global__ __launch_bounds__(256) void gather_rows_kernel(
+    const uint4* __restrict__ hidden, int row_vec, const LabelT* __restrict__ labels,
+    const float* __restrict__ lse, const float* __restrict__ entropy_b,
+    const float* __restrict__ dlogprobs, const float* __restrict__ dentropy,
+    const uint8_t* __restrict__ is_start, int n_tokens, const int32_t* __restrict__ row_index,
+    uint4* __restrict__ hidden_c, LabelT* __restrict__ labels_c, float* __restrict__ lse_c,
+    float* __restrict__ entropy_b_c, float* __restrict__ dlogprobs_c, float* __restrict__ dentropy_c) {
+  const int r = blockIdx.x;
+  const int n = row_index[r];
+  const uint4* src_row = hidden + (int64_t)n * row_vec;
+  uint4* dst_row = hidden_c + (int64_t)r * row_vec;
+  for (int c = threadIdx.x; c < row_vec; c += 256) dst_row[c] = src_row[c];
+  if (threadIdx.x == 0) {
+    const int src = aligned_pos(n, n_tokens, is_start);
+    labels_c[r] = labels[src];
+    lse_c[r] = lse[n];
+    entropy_b_c[r] = entropy_b[n];
+    dlogprobs_c[r] = dlogprobs[src];
+    if (dentropy_c) dentropy_c[r] = dentropy ? dentropy[src] : 0.f;
+  }
+}
+
+// One workgroup per row of d_hidden: the compact row, or zeros.
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const uint4* __restrict__ d_hidden_c,
+                                                           const int32_t* __restrict__ row_rank,
+                                                           int row_vec, uint4* __restrict__ d_hidden) {
+  const int n = blockIdx.x;
+  const int r = row_rank[n];
+  uint4* dst_row = d_hidden + (int64_t)n * row_vec;
+  if (r < 0) {
+    for (int c = threadIdx.x; c < row_vec; c += 256) dst_row[c] = make_uint4(0, 0, 0, 0);
+    return;
+  }
+  const uint4* src_row = d_hidden_c + (int64_t)r * row_vec;
+  for (int c = threadIdx.x; c < row_vec; c += 256) dst_row[c] = src_row[c];
+}
+
 }  // namespace axon
 
 using namespace axon;
@@ -872,6 +953,66 @@ extern "C" int axon_seq_start_flags(const int32_t* cu_seqlens, int64_t n_seqs, i
   if (n_seqs == 0) return AXON_OK;
   hipLaunchKernelGGL(seq_start_kernel, dim3((unsigned)((n_seqs + 255) / 256)), dim3(256), 0,
                      (hipStream_t)stream, cu_seqlens, (int)n_seqs, (int)n_tokens, flags);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_lmhead_active_rows(const float* dlogprobs, const float* dentropy,
+                                       const uint8_t* seq_start, int64_t n, int32_t* row_index,
+                                       int32_t* row_rank, int32_t* count, void* stream) {
+  if (n < 0 || n >= (int64_t)INT32_MAX - 1024) return AXON_ERR_SHAPE;  // the walk steps by 1024
+  if (!count) return AXON_ERR_ARG;
+  if (n > 0 && (!dlogprobs || !row_index || !row_rank)) return AXON_ERR_ARG;
+  hipLaunchKernelGGL(active_rows_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, dlogprobs,
+                     dentropy, seq_start, (int)n, row_index, row_rank, count);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_lmhead_gather_rows(const void* hidden, const void* labels, int labels_i64,
+                                       const float* lse, const float* entropy_b,
+                                       const float* dlogprobs, const float* dentropy,
+                                       const uint8_t* seq_start, int64_t n, int64_t h,
+                                       const int32_t* row_index, int64_t n_active, void* hidden_c,
+                                       void* labels_c, float* lse_c, float* entropy_b_c,
+                                       float* dlogprobs_c, float* dentropy_c, void* stream) {
+  if (n < 0 || n >= (int64_t)INT32_MAX || n_active < 0 || n_active > n) return AXON_ERR_SHAPE;
+  if (h < 8 || h % 8 != 0 || h / 8 >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (n_active == 0) return AXON_OK;
+  if (!hidden || !labels || !lse || !entropy_b || !dlogprobs || !row_index || !hidden_c ||
+      !labels_c || !lse_c || !entropy_b_c || !dlogprobs_c)
+    return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(hidden_c)) & 15)
+    return AXON_ERR_ARG;
+  const dim3 grid((unsigned)n_active), block(256);
+  const hipStream_t st = (hipStream_t)stream;
+  if (labels_i64)
+    hipLaunchKernelGGL(gather_rows_kernel<int64_t>, grid, block, 0, st,
+                       static_cast<const uint4*>(hidden), (int)(h / 8),
+                       static_cast<const int64_t*>(labels), lse, entropy_b, dlogprobs, dentropy,
+                       seq_start, (int)n, row_index, static_cast<uint4*>(hidden_c),
+                       static_cast<int64_t*>(labels_c), lse_c, entropy_b_c, dlogprobs_c, dentropy_c);
+  else
+    hipLaunchKernelGGL(gather_rows_kernel<int32_t>, grid, block, 0, st,
+                       static_cast<const uint4*>(hidden), (int)(h / 8),
+                       static_cast<const int32_t*>(labels), lse, entropy_b, dlogprobs, dentropy,
+                       seq_start, (int)n, row_index, static_cast<uint4*>(hidden_c),
+                       static_cast<int32_t*>(labels_c), lse_c, entropy_b_c, dlogprobs_c, dentropy_c);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
+extern "C" int axon_lmhead_scatter_rows(const void* d_hidden_c, const int32_t* row_rank, int64_t n,
+                                        int64_t h, void* d_hidden, void* stream) {
+  if (n < 0 || n >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (h < 8 || h % 8 != 0 || h / 8 >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
+  if (n == 0) return AXON_OK;
+  if (!row_rank || !d_hidden) return AXON_ERR_ARG;  // d_hidden_c may be NULL when no row is active
+  if ((reinterpret_cast<uintptr_t>(d_hidden_c) | reinterpret_cast<uintptr_t>(d_hidden)) & 15)
+    return AXON_ERR_ARG;
+  hipLaunchKernelGGL(scatter_rows_kernel, dim3((unsigned)n), dim3(256), 0, (hipStream_t)stream,
+                     static_cast<const uint4*>(d_hidden_c), row_rank, (int)(h / 8),
+                     static_cast<uint4*>(d_hidden));
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

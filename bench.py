@@ -43,6 +43,9 @@ def parse_args():
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (debugging)")
     ap.add_argument("--vocab-chunk", type=int, default=0)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
+    ap.add_argument("--prompt-fraction", type=float, default=1 / 3,
+                    help="after the headline, time the step again with this leading share of every sequence "
+                         "masked as prompt; 0 disables it")
     ap.add_argument("--hbm-tokens", type=int, default=1 << 26,
                     help="token count for the HBM-bound stage-2/3 kernels' bandwidth figures; 0 disables them")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -327,7 +330,7 @@ def main():
 
     loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
 
-    def step():
+    def step(mask=mask):
         hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
         lp_tok, _ent = packed_logprobs(hg, wg, ld, cu)
         adv_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
@@ -359,6 +362,27 @@ def main():
 
     ms_per_step = 1e3 * elapsed / args.steps
     tokens_per_s = n * args.steps / elapsed
+
+    # Not the headline: the same step when the first third of every sequence is prompt (response_mask 0), as in
+    # the trainer's batches.  Those positions send exact zeros back into the head, whose backward leaves their
+    # rows out of its GEMMs; the forward still covers every token, as the reference's does.
+    prompt_variant = None
+    if args.prompt_fraction > 0:
+        pos = torch.arange(n, device=dev)
+        row = torch.searchsorted(cu.long(), pos, right=True) - 1
+        start, length = cu.long()[row], (cu.long()[1:] - cu.long()[:-1])[row]
+        mask_p = mask * (pos - start >= (length.float() * args.prompt_fraction).long()).to(mask.dtype)
+        step(mask_p)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(3):
+            loss_p, dh_p, _ = step(mask_p)
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        assert torch.isfinite(loss_p).item() and torch.isfinite(dh_p.float()).all().item()
+        prompt_variant = {"prompt_fraction_of_tokens": 1.0 - mask_p.sum().item() / n, "steps": 3,
+                          "ms_per_step": 1e3 * el / 3, "tokens_per_s": 3 * n / el}
+        del loss_p, dh_p
     nhv = float(n) * h * v
 
     # kernel classes: (label, timing keys, algorithmic flops per step, executed flops per step)
@@ -403,6 +427,8 @@ def main():
                    "vocab_chunk": args.vocab_chunk or "default"},
         "roofline": roofline,
     }
+    if prompt_variant:
+        out["prompt_rows_variant"] = prompt_variant
     if args.hbm_tokens > 0:
         del hd, wd, dh, dw
         torch.cuda.empty_cache()

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 12
+#define AXON_AMD_ABI_VERSION 13
 
 enum {
   AXON_OK = 0,
@@ -108,6 +108,37 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
                     int64_t vocab, float inv_temperature, float softcap,
                     const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
                     int64_t vocab_chunk, void* workspace, int64_t workspace_bytes, void* stream);
+
+/* Rows of the backward without an upstream gradient.  The reference's trainer runs the head over every
+ * packed token, prompt included, and slices the prompt positions away afterwards
+ * (rmpad_postprocess, axon/utils/fsdp/forward_utils.py:164-182; the response slice,
+ * forward_utils.py:306-316): their dlogprobs / dentropy arrive as exact zeros, and so do those of
+ * tokens that the loss masks or clips.  Such a row's dlogit is zero: it adds nothing to d_weight and
+ * its d_hidden row is zero (efficient_entropy_backward, axon/utils/kernel/kernels.py:1377-1585,
+ * computes them all the same).  These three calls let the host run axon_lmhead_bwd over the other
+ * rows only.
+ *   axon_lmhead_active_rows: row_index[r] = the r-th hidden row (ascending) whose dlogprobs or
+ *        dentropy is not zero (NaN counts as not zero); with seq_start both are read at the aligned
+ *        position n + 1 and sequence starts never count.  row_rank[n] = r for such a row, -1 for the
+ *        others; count[0] = their number.  row_index and row_rank hold n_tokens entries.  One
+ *        workgroup; the numbering is the same on every run.
+ *   axon_lmhead_gather_rows: the operands of those rows, compact: hidden_c[r] = hidden[row_index[r]],
+ *        lse_c, entropy_b_c likewise; labels_c (same integer type as labels), dlogprobs_c, dentropy_c
+ *        (may be NULL; zeros where dentropy is NULL) from the aligned position.  They are operands of
+ *        axon_lmhead_bwd with n_tokens = n_active and seq_start = NULL.
+ *   axon_lmhead_scatter_rows: d_hidden[n] = d_hidden_c[row_rank[n]], or zeros where row_rank[n] < 0.
+ * hidden % 8 == 0; hidden, hidden_c, d_hidden, d_hidden_c on 16-byte boundaries. */
+int axon_lmhead_active_rows(const float* dlogprobs, const float* dentropy, const uint8_t* seq_start,
+                            int64_t n_tokens, int32_t* row_index, int32_t* row_rank, int32_t* count,
+                            void* stream);
+int axon_lmhead_gather_rows(const void* hidden_bf16, const void* labels, int labels_are_i64,
+                            const float* lse, const float* entropy_b, const float* dlogprobs,
+                            const float* dentropy, const uint8_t* seq_start, int64_t n_tokens,
+                            int64_t hidden, const int32_t* row_index, int64_t n_active,
+                            void* hidden_c_bf16, void* labels_c, float* lse_c, float* entropy_b_c,
+                            float* dlogprobs_c, float* dentropy_c, void* stream);
+int axon_lmhead_scatter_rows(const void* d_hidden_c_bf16, const int32_t* row_rank, int64_t n_tokens,
+                             int64_t hidden, void* d_hidden_bf16, void* stream);
 
 /* Timed variants for benchmarks: same work, plus HIP events recorded on `stream`
  * around every launch into a timer object.  Recording does not synchronise;

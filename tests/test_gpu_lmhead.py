@@ -425,3 +425,92 @@ def test_fsdp_model_forward_non_fused(remove_padding):
     valid = (mask[:, 1:] > 0) if remove_padding else torch.ones(b, t - 1, dtype=torch.bool)
     assert ((lp.cpu()[:, 1:] - ref_lp).abs() * valid).max() < 1e-3
     assert ((ent.cpu()[:, 1:] - ref_en).abs() * valid).max() < 1e-3
+
+
+# ---- rows without an upstream gradient are left out of the backward's GEMMs --------------------------------
+def _head_state(n, h, v, seed, ldt=torch.int32):
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=seed, label_dtype=ldt)
+    w = (w.float() * 8).bfloat16()
+    hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
+    _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    return hid, w, lab, hd, wd, ld, lse, eb
+
+
+def test_active_rows_index_known_answers():
+    """The C entry point against a list written by hand and against numpy on a ragged case."""
+    from axon_amd import _lib
+    g_lp = torch.tensor([0.0, 1.0, 0.0, -0.0, 2.0, 0.0, float("nan"), 0.0], device=DEV)
+    g_en = torch.tensor([0.0, 0.0, 3.0, 0.0, 0.0, 0.0, 0.0, 0.0], device=DEV)
+    idx, rank, cnt = _ops._active_rows(g_lp, g_en, None, 8)
+    assert cnt == 4 and idx[:4].tolist() == [1, 2, 4, 6]
+    assert rank.tolist() == [-1, 0, 1, -1, 2, -1, 3, -1]
+    idx, rank, cnt = _ops._active_rows(g_lp, None, None, 8)
+    assert cnt == 3 and idx[:3].tolist() == [1, 4, 6]
+    # aligned layout: hidden row n owns position n + 1 (the last row owns position 0); starts never count
+    starts = torch.tensor([1, 0, 0, 0, 1, 0, 0, 0], dtype=torch.uint8, device=DEV)
+    g = torch.tensor([5.0, 1.0, 0.0, 1.0, 7.0, 0.0, 1.0, 1.0], device=DEV)
+    idx, rank, cnt = _ops._active_rows(g, None, starts, 8)
+    assert cnt == 4 and idx[:4].tolist() == [0, 2, 5, 6]  # rows 3 and 7 point at starts, 1 and 4 at zeros
+    # more rows than one walk of the workgroup, ragged tail
+    n = 5000
+    gen = torch.Generator().manual_seed(3)
+    big = torch.randn(n, generator=gen) * (torch.rand(n, generator=gen) < 0.4)
+    idx, rank, cnt = _ops._active_rows(big.to(DEV), None, None, n)
+    want = torch.nonzero(big).flatten()
+    assert cnt == len(want) and torch.equal(idx[:cnt].cpu().long(), want)
+    inv = torch.full((n,), -1, dtype=torch.int32)
+    inv[want] = torch.arange(len(want), dtype=torch.int32)
+    assert torch.equal(rank.cpu(), inv)
+    assert _lib.load().axon_lmhead_active_rows(None, None, None, 4, None, None, None, None) != 0  # no count pointer
+
+
+@pytest.mark.parametrize("n,h,v,ldt,with_entropy", [(700, 256, 1500, torch.int32, True),
+                                                    (300, 96, 777, torch.int64, False),
+                                                    (1030, 128, 2000, torch.int32, True)])
+def test_backward_skips_rows_without_gradient(n, h, v, ldt, with_entropy):
+    hid, w, lab, hd, wd, ld, lse, eb = _head_state(n, h, v, n + v, ldt)
+    gen = torch.Generator().manual_seed(n)
+    live = torch.rand(n, generator=gen) < 0.45  # the rest are prompt-like rows: exact zeros
+    g_lp = torch.randn(n, generator=gen) / n * live
+    g_en = torch.randn(n, generator=gen) / n * live if with_entropy else None
+    args = (g_lp.to(DEV), None if g_en is None else g_en.to(DEV), hd, wd, ld, lse, eb, 1.0)
+    dh, dw = _ops.lmhead_backward(*args)
+    dh_all, dw_all = _ops.lmhead_backward(*args, skip_zero_rows=False)
+    assert (dh[~live.to(DEV)] == 0).all() and (dh_all[~live.to(DEV)] == 0).all()
+    # a d_hidden row is a sum over the vocabulary only: the row set does not change it
+    assert torch.equal(dh, dh_all)
+    assert rel_l2(dw, dw_all) < 1e-3  # d_weight sums over fewer rows, in another order
+    ref_dh, ref_dw = OM.backward(g_lp, g_en, hid, w, lab, 1.0)
+    assert rel_l2(dh, ref_dh) < 2e-2 and rel_l2(dw, ref_dw) < 2e-2
+
+
+def test_backward_row_skipping_in_the_aligned_layout_and_all_zero():
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs
+    n, h, v, lens = 600, 128, 1200, [200, 1, 150, 249]
+    hid, w, ids = W.lmhead_inputs(n, h, v, seed=77, label_dtype=torch.int64)
+    w = (w.float() * 8).bfloat16()
+    cu = W.cu_from_lengths(lens).to(DEV)
+    # prompt positions (the first 60 % of every sequence) carry no gradient
+    pos = torch.arange(n)
+    resp = torch.zeros(n, dtype=torch.bool)
+    for a, b in zip(cu.tolist()[:-1], cu.tolist()[1:]):
+        resp |= (pos >= a + int(0.6 * (b - a))) & (pos < b)
+    gen = torch.Generator().manual_seed(8)
+    g_lp = (torch.randn(n, generator=gen) / n * resp).to(DEV)
+    grads = []
+    for skip in (True, False):
+        hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        lp, _ = packed_logprobs(hd, wd, ids.to(DEV).view(1, -1), cu, 0.9)
+        old = _ops.SKIP_ROWS_BELOW
+        _ops.SKIP_ROWS_BELOW = old if skip else -1.0
+        try:
+            (lp * g_lp).sum().backward()
+        finally:
+            _ops.SKIP_ROWS_BELOW = old
+        grads.append((hd.grad, wd.grad))
+    assert torch.equal(grads[0][0], grads[1][0]) and rel_l2(grads[0][1], grads[1][1]) < 1e-3
+    assert (grads[0][0].abs().sum(1) > 0).sum().item() <= int(resp.sum())  # only rows that predict a response token
+    # nothing to do at all: exact zeros, no GEMM
+    _, _, lab, hd, wd, ld, lse, eb = _head_state(64, 64, 500, 5)
+    dh, dw = _ops.lmhead_backward(torch.zeros(64, device=DEV), None, hd, wd, ld, lse, eb, 1.0)
+    assert not dh.any() and not dw.any() and dh.dtype == torch.bfloat16 and dw.shape == wd.shape
