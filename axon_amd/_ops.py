@@ -626,8 +626,8 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
                     timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=True):
     """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``).
 
-    With ``skip_zero_rows`` the rows whose upstream gradients are both exactly zero (prompt positions that
-    the trainer slices away, masked or clipped tokens) are left out of the three GEMMs: they contribute
+    With ``skip_zero_rows`` the rows whose upstream gradients are both exactly zero (prompt positions, where the
+    response mask is zero, rejected or clipped tokens) are left out of the three GEMMs: they contribute
     nothing to ``d_weight`` and their ``d_hidden`` rows are zero.  Finding them costs one readback, so it
     is not done while the stream is being captured into a graph."""
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK

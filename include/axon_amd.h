@@ -110,10 +110,10 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
                     int64_t vocab_chunk, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* Rows of the backward without an upstream gradient.  The reference's trainer runs the head over every
- * packed token, prompt included, and slices the prompt positions away afterwards
- * (rmpad_postprocess, axon/utils/fsdp/forward_utils.py:164-182; the response slice,
- * forward_utils.py:306-316): their dlogprobs / dentropy arrive as exact zeros, and so do those of
- * tokens that the loss masks or clips.  Such a row's dlogit is zero: it adds nothing to d_weight and
+ * packed token, prompt included (fsdp_model_forward, axon/utils/fsdp/forward_utils.py:236-265), and the
+ * loss weighs every token with response_mask, which is zero on the prompt (agg_loss,
+ * axon/trainer/algos/loss/utils.py:120-251): the dlogprobs / dentropy of those positions arrive as exact
+ * zeros, and so do those of tokens that the correction rejects or the loss clips.  Such a row's dlogit is zero: it adds nothing to d_weight and
  * its d_hidden row is zero (efficient_entropy_backward, axon/utils/kernel/kernels.py:1377-1585,
  * computes them all the same).  These three calls let the host run axon_lmhead_bwd over the other
  * rows only.
