@@ -63,15 +63,37 @@ def shift_packed(values: torch.Tensor, cu_seqlens: torch.Tensor) -> torch.Tensor
     return out
 
 
-def packed_logprobs(hidden, weight, packed_ids, cu_seqlens, temperature: float = 1.0, logit_softcapping=None):
+def packed_logprobs(hidden, weight, packed_ids, cu_seqlens, temperature: float = 1.0, logit_softcapping=None,
+                    response_mask=None):
     """Head of the remove-padding path in one call: packed hidden states ``[N, H]`` and the packed token ids
     ``[N]`` (or ``[1, N]``) in, ``(log_probs, entropy)`` ``[N]`` aligned to token positions out — what
     ``rolled_labels`` + the fused head + ``shift_packed`` produce, without the roll and shift passes
-    (forward_utils.py:131,164-182 in packed form)."""
+    (forward_utils.py:131,164-182 in packed form).
+
+    ``response_mask`` ``[N]`` (optional; the reference has no such argument and runs the head over every
+    token): the positions where it is zero — the prompt — come back as 0 and their rows stay out of the
+    head, forward and backward.  Every consumer of these values weighs them with the same mask (``agg_loss``,
+    axon/trainer/algos/loss/utils.py:120-251), so losses, gradients and masked metrics do not change.  Costs
+    one readback (the number of response positions)."""
     from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
 
-    return linear_cross_entropy(hidden, weight, packed_ids.reshape(-1), float(temperature), "none", None,
-                                logit_softcapping, cu_seqlens)
+    ids = packed_ids.reshape(-1)
+    if response_mask is None:
+        return linear_cross_entropy(hidden, weight, ids, float(temperature), "none", None, logit_softcapping,
+                                    cu_seqlens)
+    n = ids.numel()
+    wanted = response_mask.reshape(-1) != 0
+    if wanted.numel() != n:
+        raise ValueError(f"response_mask has {wanted.numel()} entries for {n} packed tokens")
+    starts = cu_seqlens[:-1].long()
+    wanted[starts[starts < n]] = False  # a sequence's first token has no prediction (comparison made a new tensor)
+    wanted[:1] = False
+    pos = torch.nonzero(wanted).flatten()  # position p is predicted from the hidden state at p - 1
+    lp_c, ent_c = linear_cross_entropy(hidden.reshape(n, -1).index_select(0, pos - 1), weight,
+                                       ids.index_select(0, pos), float(temperature), "none", None,
+                                       logit_softcapping)
+    zeros = torch.zeros(n, device=lp_c.device, dtype=lp_c.dtype)
+    return zeros.index_copy(0, pos, lp_c), zeros.index_copy(0, pos, ent_c)
 
 
 def _from_logits(logits, labels, temperature: float, calculate_entropy: bool):

@@ -330,9 +330,9 @@ def main():
 
     loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
 
-    def step(mask=mask):
+    def step(mask=mask, head_mask=None):
         hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
-        lp_tok, _ent = packed_logprobs(hg, wg, ld, cu)
+        lp_tok, _ent = packed_logprobs(hg, wg, ld, cu, response_mask=head_mask)
         adv_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
                                      meta_info={"cu_seqlens": cu})
         adv_in.non_tensor_batch["uid"] = uid
@@ -365,24 +365,27 @@ def main():
 
     # Not the headline: the same step when the first third of every sequence is prompt (response_mask 0), as in
     # the trainer's batches.  Those positions send exact zeros back into the head, whose backward leaves their
-    # rows out of its GEMMs; the forward still covers every token, as the reference's does.
+    # rows out of its GEMMs while the forward still covers every token, as the reference's does ("backward");
+    # with the mask handed to the head as well, the forward leaves them out too ("forward_and_backward").
     prompt_variant = None
     if args.prompt_fraction > 0:
         pos = torch.arange(n, device=dev)
         row = torch.searchsorted(cu.long(), pos, right=True) - 1
         start, length = cu.long()[row], (cu.long()[1:] - cu.long()[:-1])[row]
         mask_p = mask * (pos - start >= (length.float() * args.prompt_fraction).long()).to(mask.dtype)
-        step(mask_p)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(3):
-            loss_p, dh_p, _ = step(mask_p)
-        torch.cuda.synchronize()
-        el = time.perf_counter() - t0
-        assert torch.isfinite(loss_p).item() and torch.isfinite(dh_p.float()).all().item()
-        prompt_variant = {"prompt_fraction_of_tokens": 1.0 - mask_p.sum().item() / n, "steps": 3,
-                          "ms_per_step": 1e3 * el / 3, "tokens_per_s": 3 * n / el}
+        prompt_variant = {"prompt_fraction_of_tokens": 1.0 - mask_p.sum().item() / n, "steps": 3}
+        for name, head_mask in (("backward", None), ("forward_and_backward", mask_p)):
+            step(mask_p, head_mask)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                loss_p, dh_p, _ = step(mask_p, head_mask)
+            torch.cuda.synchronize()
+            el = time.perf_counter() - t0
+            assert torch.isfinite(loss_p).item() and torch.isfinite(dh_p.float()).all().item()
+            prompt_variant[name] = {"ms_per_step": 1e3 * el / 3, "tokens_per_s": 3 * n / el, "loss": loss_p.item()}
         del loss_p, dh_p
+
     nhv = float(n) * h * v
 
     # kernel classes: (label, timing keys, algorithmic flops per step, executed flops per step)

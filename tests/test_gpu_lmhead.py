@@ -514,3 +514,42 @@ def test_backward_row_skipping_in_the_aligned_layout_and_all_zero():
     _, _, lab, hd, wd, ld, lse, eb = _head_state(64, 64, 500, 5)
     dh, dw = _ops.lmhead_backward(torch.zeros(64, device=DEV), None, hd, wd, ld, lse, eb, 1.0)
     assert not dh.any() and not dw.any() and dh.dtype == torch.bfloat16 and dw.shape == wd.shape
+
+
+def test_packed_logprobs_with_response_mask_leaves_prompt_rows_out():
+    """Optional response mask: prompt positions come back as 0, everything the loss can see is unchanged."""
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs
+    n, h, v, lens = 700, 128, 1300, [300, 1, 0, 250, 149]
+    hid, w, ids = W.lmhead_inputs(n, h, v, seed=21, label_dtype=torch.int64)
+    w = (w.float() * 8).bfloat16()
+    cu = W.cu_from_lengths(lens).to(DEV)
+    pos = torch.arange(n)
+    resp = torch.zeros(n)
+    for a, b in zip(cu.tolist()[:-1], cu.tolist()[1:]):
+        resp[(pos >= a + (b - a) // 2) & (pos < b)] = 1  # second half of every sequence (a one-token sequence whole)
+    resp_d = resp.to(DEV)
+    gen = torch.Generator().manual_seed(2)
+    g_lp, g_en = (torch.randn(n, generator=gen) / n).to(DEV), (torch.randn(n, generator=gen) / n).to(DEV)
+    outs = []
+    for m in (None, resp_d):
+        hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+        lp, ent = packed_logprobs(hd, wd, ids.to(DEV), cu, 0.8, None, response_mask=m)
+        ((lp * g_lp * resp_d).sum() + (ent * g_en * resp_d).sum()).backward()
+        outs.append((lp.detach(), ent.detach(), hd.grad, wd.grad))
+    (lp0, ent0, dh0, dw0), (lp1, ent1, dh1, dw1) = outs
+    starts = cu[:-1].long()[cu[:-1] < n]
+    seen = resp_d.clone()
+    seen[starts] = 0
+    assert (lp1[seen == 0] == 0).all() and (ent1[seen == 0] == 0).all()
+    assert torch.equal(lp1[seen > 0], lp0[seen > 0]) and torch.equal(ent1[seen > 0], ent0[seen > 0])
+    assert torch.equal(dh1, dh0) and rel_l2(dw1, dw0) < 1e-3
+    ref_lp, ref_ent, _ = _aligned_reference(hid, w, ids, lens, 0.8)
+    assert ((lp1.cpu() - ref_lp) * seen.cpu()).abs().max() < 1e-3
+    assert ((ent1.cpu() - ref_ent) * seen.cpu()).abs().max() < 1e-3
+    # an all-zero mask: nothing runs, zeros come back and the gradients are zero
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = packed_logprobs(hd, wd, ids.to(DEV), cu, 0.8, None, response_mask=torch.zeros(n, device=DEV))
+    (lp.sum() + ent.sum()).backward()
+    assert not lp.any() and not ent.any() and not hd.grad.any() and not wd.grad.any()
+    with pytest.raises(ValueError):
+        packed_logprobs(hd, wd, ids.to(DEV), cu, 0.8, None, response_mask=torch.zeros(n - 1, device=DEV))
