@@ -15,7 +15,7 @@ from typing import Any
 
 import torch
 
-from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+from axon_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy, linear_cross_entropy_rows
 
 try:  # the reference's output type extends the Hugging Face one (dense_common.py:23-26)
     from transformers.modeling_outputs import CausalLMOutputWithPast as _Base
@@ -93,10 +93,18 @@ def forward_with_hip_backend(
         raise NotImplementedError("forward_with_hip_backend has to return_dict")
 
     rolled_labels = select_rolled_labels(loss_kwargs.pop("pre_rolled_labels", None), labels, input_ids)
-    log_probs, entropy = linear_cross_entropy(
-        hidden_states.contiguous(), self.lm_head.weight, rolled_labels.contiguous(), float(temperature), "none",
-        None, final_logit_softcapping(self.config),
-    )
+    # optional, no counterpart in the reference: rows (positions of hidden_states) the caller will not look at
+    head_row_mask = loss_kwargs.pop("head_row_mask", None)
+    if head_row_mask is not None:
+        log_probs, entropy = linear_cross_entropy_rows(
+            hidden_states, self.lm_head.weight, rolled_labels, head_row_mask, float(temperature),
+            final_logit_softcapping(self.config),
+        )
+    else:
+        log_probs, entropy = linear_cross_entropy(
+            hidden_states.contiguous(), self.lm_head.weight, rolled_labels.contiguous(), float(temperature), "none",
+            None, final_logit_softcapping(self.config),
+        )
     return CausalLMOutputForPPO(
         log_probs=log_probs,
         entropy=entropy,

@@ -109,7 +109,7 @@ def _from_logits(logits, labels, temperature: float, calculate_entropy: bool):
 
 def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_entropy: bool = False, *,
                        use_remove_padding: bool = True, use_fused_kernels: bool = True, ulysses_sp_size: int = 1,
-                       **_unused):
+                       skip_prompt_rows: bool = False, **_unused):
     """Forward one micro-batch through a model whose ``forward`` is the fused-head one
     (``forward_with_hip_backend``) and return ``(entropy, log_probs)``, both ``[batch, seq]``: position 0 is 0,
     position t holds log P(token_t | tokens before it).  Mirror of the fused branches of ``fsdp_model_forward``
@@ -118,7 +118,14 @@ def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_
     right (``rmpad_postprocess``, :164-182); without it the outputs are shifted right directly (:282-285).
     With ``use_fused_kernels=False`` the model writes the logits and ``axon_amd.utils.torch.ops`` turns them into
     log-probabilities and entropy (:287-304).  Ulysses sequence parallelism (more than one GPU) is not part of
-    this build."""
+    this build.
+
+    ``skip_prompt_rows`` (no counterpart in the reference, off by default; fused branches only): positions where
+    ``micro_batch["response_mask"]`` ``[batch, seq]`` is zero come back as 0 and their rows stay out of the head."""
+    head_kwargs = {}
+    if skip_prompt_rows and use_fused_kernels and "response_mask" in micro_batch:
+        # hidden position t predicts token t + 1: keep it when the response mask covers t + 1
+        keep = F.pad(micro_batch["response_mask"][:, 1:] != 0, (0, 1), value=False)
     if ulysses_sp_size > 1:
         raise NotImplementedError("Ulysses sequence parallelism needs more than one GPU")
     input_ids = micro_batch["input_ids"]
@@ -139,8 +146,10 @@ def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_
             fwd_pos = position_ids.flatten()[indices].unsqueeze(0)
         labels = rolled_labels(fwd_ids)
         if use_fused_kernels:
+            if skip_prompt_rows and "response_mask" in micro_batch:
+                head_kwargs["head_row_mask"] = keep.flatten()[indices].unsqueeze(0)
             output = module(input_ids=fwd_ids, attention_mask=None, position_ids=fwd_pos, use_cache=False,
-                            temperature=temperature, return_dict=True, pre_rolled_labels=labels)
+                            temperature=temperature, return_dict=True, pre_rolled_labels=labels, **head_kwargs)
             lp_packed = output.log_probs.reshape(-1)
             ent_packed = output.entropy.reshape(-1) if calculate_entropy else None
         else:  # the model writes the logits (forward_utils.py:287-292)
@@ -153,8 +162,10 @@ def fsdp_model_forward(module, micro_batch: dict, temperature: float, calculate_
             entropy = rmpad_postprocess(ent_packed, indices=indices, batch_size=batch_size, seqlen=seqlen)
         return entropy, log_probs
     if use_fused_kernels:
+        if skip_prompt_rows and "response_mask" in micro_batch:
+            head_kwargs["head_row_mask"] = keep
         output = module(input_ids=input_ids, attention_mask=attention_mask, position_ids=position_ids,
-                        use_cache=False, temperature=temperature, return_dict=True)
+                        use_cache=False, temperature=temperature, return_dict=True, **head_kwargs)
         log_probs = shift_to_token_positions(output.log_probs.view(batch_size, seqlen))
         entropy = shift_to_token_positions(output.entropy.view(batch_size, seqlen)) if calculate_entropy else None
         return entropy, log_probs

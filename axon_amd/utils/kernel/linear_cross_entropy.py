@@ -89,3 +89,19 @@ class LinearCrossEntropy(torch.autograd.Function):
 
 
 linear_cross_entropy = LinearCrossEntropy.apply
+
+
+def linear_cross_entropy_rows(hidden, weight, labels, row_mask, temperature=1.0, logit_softcapping=None):
+    """``linear_cross_entropy(..., "none")`` over the rows where ``row_mask`` is not zero only; the other rows
+    come back as 0 and receive a zero gradient.  For callers that know which rows nobody will look at (prompt
+    positions under a response mask): the reference runs the head over all of them.  One readback."""
+    shape = labels.shape
+    h2 = hidden.reshape(-1, hidden.shape[-1])
+    rows = torch.nonzero(row_mask.reshape(-1)).flatten()
+    if row_mask.numel() != h2.shape[0]:
+        raise ValueError(f"row_mask has {row_mask.numel()} entries for {h2.shape[0]} rows")
+    lp_c, ent_c = linear_cross_entropy(h2.index_select(0, rows), weight, labels.reshape(-1).index_select(0, rows),
+                                       float(temperature), "none", None, logit_softcapping)
+    zeros = torch.zeros(h2.shape[0], device=lp_c.device, dtype=lp_c.dtype)
+    return zeros.index_copy(0, rows, lp_c).view(shape), zeros.index_copy(0, rows, ent_c).view(shape)
+

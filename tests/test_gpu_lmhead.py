@@ -553,3 +553,50 @@ def test_packed_logprobs_with_response_mask_leaves_prompt_rows_out():
     assert not lp.any() and not ent.any() and not hd.grad.any() and not wd.grad.any()
     with pytest.raises(ValueError):
         packed_logprobs(hd, wd, ids.to(DEV), cu, 0.8, None, response_mask=torch.zeros(n - 1, device=DEV))
+
+
+@pytest.mark.parametrize("remove_padding", [True, False])
+def test_fsdp_model_forward_skip_prompt_rows(remove_padding):
+    """Opt-in: positions outside the response mask come back as 0; inside it nothing changes, values or gradients."""
+    import types
+
+    from axon_amd.models.transformers.dense_common import forward_with_hip_backend
+    from axon_amd.utils.fsdp.forward_utils import fsdp_model_forward
+    b, t, h, v = 4, 96, 128, 1000
+    g = torch.Generator().manual_seed(35)
+    lens, prompts = [96, 40, 1, 77], [30, 39, 0, 20]  # valid tokens and leading prompt tokens per row
+    ids = torch.randint(0, v, (b, t), generator=g)
+    att, resp = torch.zeros(b, t, dtype=torch.long), torch.zeros(b, t)
+    for r, (n, p) in enumerate(zip(lens, prompts)):
+        att[r, :n] = 1
+        resp[r, p:n] = 1
+    emb = torch.randn(v, h, generator=g).bfloat16()
+    w = (torch.randn(v, h, generator=g) * 0.3).bfloat16()
+
+    class Body(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = torch.nn.Parameter(emb.to(DEV))
+
+        def forward(self, input_ids=None, **kw):
+            return (self.emb[input_ids],)
+
+    res = []
+    for skip in (False, True):
+        model = types.SimpleNamespace(
+            model=Body(), lm_head=types.SimpleNamespace(weight=w.to(DEV).requires_grad_(True)),
+            config=types.SimpleNamespace(output_attentions=False, output_hidden_states=False))
+        module = lambda **kw: forward_with_hip_backend(model, **kw)  # noqa: E731
+        mb = {"input_ids": ids.to(DEV), "attention_mask": att.to(DEV), "response_mask": resp.to(DEV),
+              "position_ids": torch.arange(t).expand(b, t).to(DEV)}
+        ent, lp = fsdp_model_forward(module, mb, 0.9, True, use_remove_padding=remove_padding,
+                                     use_fused_kernels=True, skip_prompt_rows=skip)
+        ((lp * resp.to(DEV)).sum() + 0.3 * (ent * resp.to(DEV)).sum()).backward()
+        res.append((lp.detach(), ent.detach(), model.lm_head.weight.grad, model.model.emb.grad))
+    (lp0, ent0, dw0, de0), (lp1, ent1, dw1, de1) = res
+    seen = resp.to(DEV).clone()
+    seen[:, 0] = 0  # position 0 has no prediction
+    assert (lp1[seen == 0] == 0).all() and (ent1[seen == 0] == 0).all()
+    # fewer rows can put the head on its other main loop (another summation order over the hidden size)
+    assert (lp1 - lp0)[seen > 0].abs().max() < 1e-5 and (ent1 - ent0)[seen > 0].abs().max() < 1e-5
+    assert rel_l2(dw1, dw0) < 1e-3 and rel_l2(de1, de0) < 1e-3
