@@ -536,36 +536,51 @@ __global__ __launch_bounds__(256) void zero_cols_bf16_kernel(uint16_t* p, int64_
 // ----------------------------------------------------------------------------
 // Rows without an upstream gradient (prompt positions, masked or clipped tokens)
 // ----------------------------------------------------------------------------
-// One workgroup walks the rows in blocks of 1024 and numbers the active ones in ascending order
-// (ballot + popcount inside a wave, wave totals through LDS): the list is the same on every run.
+// One workgroup walks the rows in blocks of 4096 (four consecutive rows per thread) and numbers the
+// active ones in ascending order (ballots + popcounts inside a wave, wave totals through LDS): the
+// list is the same on every run.
 __global__ __launch_bounds__(1024) void active_rows_kernel(
     const float* __restrict__ dlogprobs, const float* __restrict__ dentropy,
     const uint8_t* __restrict__ is_start, int n_tokens, int32_t* __restrict__ row_index,
     int32_t* __restrict__ row_rank, int32_t* __restrict__ count) {
   __shared__ int wave_total[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const unsigned long long below = (1ull << lane) - 1ull;
   int base = 0;
-  for (int n0 = 0; n0 < n_tokens; n0 += 1024) {
-    const int n = n0 + (int)threadIdx.x;
-    bool act = false;
-    if (n < n_tokens) {
-      const int src = aligned_pos(n, n_tokens, is_start);
-      if (!(is_start && is_start[src]))
-        act = dlogprobs[src] != 0.f || (dentropy && dentropy[src] != 0.f);  // NaN counts as active
+  for (int n0 = 0; n0 < n_tokens; n0 += 4096) {
+    const int first = n0 + (int)threadIdx.x * 4;
+    bool act[4];
+    int before = 0, mine = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = first + j;
+      act[j] = false;
+      if (n < n_tokens) {
+        const int src = aligned_pos(n, n_tokens, is_start);
+        if (!(is_start && is_start[src]))
+          act[j] = dlogprobs[src] != 0.f || (dentropy && dentropy[src] != 0.f);  // NaN counts as active
+      }
+      const unsigned long long b = __ballot(act[j]);
+      before += __popcll(b & below);  // active rows of the lanes below, this j
+      mine += __popcll(b);
     }
-    const unsigned long long b = __ballot(act);
-    if (lane == 0) wave_total[wave] = __popcll(b);
+    if (lane == 0) wave_total[wave] = mine;
     __syncthreads();
-    int before = base, total = 0;
+    int total = 0;
 #pragma unroll
     for (int w = 0; w < 16; ++w) {
       if (w < wave) before += wave_total[w];
       total += wave_total[w];
     }
-    if (n < n_tokens) {
-      const int r = before + __popcll(b & ((1ull << lane) - 1ull));
-      if (act) row_index[r] = n;
-      row_rank[n] = act ? r : -1;
+    int r = base + before;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = first + j;
+      if (n < n_tokens) {
+        if (act[j]) row_index[r] = n;
+        row_rank[n] = act[j] ? r : -1;
+        r += act[j] ? 1 : 0;
+      }
     }
     base += total;
     __syncthreads();
@@ -960,7 +975,7 @@ extern "C" int axon_seq_start_flags(const int32_t* cu_seqlens, int64_t n_seqs, i
 extern "C" int axon_lmhead_active_rows(const float* dlogprobs, const float* dentropy,
                                        const uint8_t* seq_start, int64_t n, int32_t* row_index,
                                        int32_t* row_rank, int32_t* count, void* stream) {
-  if (n < 0 || n >= (int64_t)INT32_MAX - 1024) return AXON_ERR_SHAPE;  // the walk steps by 1024
+  if (n < 0 || n >= (int64_t)INT32_MAX - 8192) return AXON_ERR_SHAPE;  // the walk steps by 4096
   if (!count) return AXON_ERR_ARG;
   if (n > 0 && (!dlogprobs || !row_index || !row_rank)) return AXON_ERR_ARG;
   hipLaunchKernelGGL(active_rows_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, dlogprobs,
