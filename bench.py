@@ -89,6 +89,7 @@ def cpu_baseline(hid, w, lab, budget_s, check=None):
         "value": n / t, "unit": "tokens/s", "cores": cores, "kind": "port",
         "sample": f"{n} of the workload's tokens, full hidden and vocab, fwd+loss+bwd, {t:.1f} s; linear in tokens",
     }
+    out["config1"] = config1_cpu_vs_gpu()
     if check is not None:
         idx, got = check
         ref_lp, _ = OM.forward(hid[idx - 1], w, lab[idx])
@@ -96,6 +97,68 @@ def cpu_baseline(hid, w, lab, budget_s, check=None):
         assert err < 1e-3, f"log-prob parity failed: {err}"
         out["logprob_max_abs_err_subset"] = err
     return out
+
+
+def config1_cpu_vs_gpu():
+    """The small published configuration (padded 128 x 1024, 16 groups of 8; GRPO advantage, PPO loss and its
+    gradient): the CPU port beside the GPU path on the same inputs, with the errors between the two."""
+    import numpy as np
+    import torch
+
+    from axon_amd import workloads as W
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.advantages import compute_advantage
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    from oracle import advantage as OA
+    from oracle import loss as OL
+
+    d = W.c1_loss_only()
+    args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "clip_ratio_c": 3.0, "token_reduce": "sum",
+            "batch_reduce": "token-mean"}
+    gidx = torch.as_tensor(np.unique(d["uid"], return_inverse=True)[1])
+
+    def cpu():
+        adv = OA.grpo_advantage(d["token_level_rewards"], d["response_mask"], gidx, 1e-6, True)
+        lp = d["log_probs"].clone().requires_grad_(True)
+        loss, _ = OL.ppo_loss(lp, d["old_log_probs"], adv, d["response_mask"], **args)
+        loss.backward()
+        return loss.detach(), lp.grad
+
+    dev = "cuda:0"
+    gpu_in = {k: d[k].to(dev) for k in ("token_level_rewards", "response_mask", "log_probs", "old_log_probs")}
+
+    def gpu():
+        a = DataProto.from_dict(tensors={"token_level_rewards": gpu_in["token_level_rewards"],
+                                         "response_mask": gpu_in["response_mask"]})
+        a.non_tensor_batch["uid"] = d["uid"]
+        adv = compute_advantage(a, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}).batch["advantages"]
+        lp = gpu_in["log_probs"].detach().requires_grad_(True)
+        data = DataProto.from_dict(tensors={"log_probs": lp, "old_log_probs": gpu_in["old_log_probs"],
+                                            "advantages": adv, "response_mask": gpu_in["response_mask"]})
+        loss, _ = compute_loss_fn(data, "ppo", args)
+        loss.backward()
+        return loss.detach(), lp.grad
+
+    def timed(fn, reps, sync):
+        fn()
+        if sync:
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            r = fn()
+        if sync:
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps, r
+
+    t_cpu, (l_cpu, g_cpu) = timed(cpu, 20, False)
+    t_gpu, (l_gpu, g_gpu) = timed(gpu, 50, True)
+    g_gpu = g_gpu.cpu().double()
+    return {
+        "workload": "128 x 1024 padded, GRPO advantage + PPO loss (0.2 / 0.28 / 3.0, sum / token-mean) + gradient",
+        "cpu_ms": 1e3 * t_cpu, "cpu_cores": torch.get_num_threads(), "gpu_ms": 1e3 * t_gpu,
+        "loss_rel_err": abs(l_gpu.item() - l_cpu.item()) / abs(l_cpu.item()),
+        "grad_rel_l2": ((g_gpu - g_cpu.double()).norm() / g_cpu.double().norm()).item(),
+    }
 
 
 def hbm_kernels(n_tokens, dev):
