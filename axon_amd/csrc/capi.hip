@@ -11,6 +11,7 @@ extern "C" const char* axon_amd_error_string(int code) {
     case AXON_ERR_WORKSPACE: return "workspace too small";
     case AXON_ERR_LAUNCH: return "kernel launch failed";
     case AXON_ERR_DEVICE: return "device is not gfx950";
+    case AXON_ERR_TOO_LARGE: return "input larger than the fixed capacity of the no-allocation entry point";
     default: return "unknown error code";
   }
 }

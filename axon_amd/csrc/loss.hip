@@ -2,6 +2,7 @@
 // loss with its gradient.  One read of every input, one write of every output;
 // scalar sums leave through per-workgroup partials that the last workgroup adds up.
 #include "common.h"
+#include <mutex>
 
 namespace axon {
 
@@ -815,13 +816,13 @@ extern "C" int axon_loss_row_scale(const float* row_cnt, const float* row_sum, i
   return AXON_OK;
 }
 
-extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, const float* adv,
-                                const void* mask, int mask_kind, const float* isw,
-                                const int32_t* cu, int64_t n_rows, int64_t n_slots,
-                                int64_t uniform_len, const float* row_scale, const float* row_mean,
-                                float uniform_scale, int post_normalize, const int64_t* valid,
-                                float ratio_lo, float ratio_hi, float clip_c, float* grad,
-                                float* acc, float* partials, void* stream) {
+static int policy_loss_impl(int kind, const float* logp, const float* oldp, const float* adv,
+                            const void* mask, int mask_kind, const float* isw, const int32_t* cu,
+                            int64_t n_rows, int64_t n_slots, int64_t uniform_len,
+                            const float* row_scale, const float* row_mean, float uniform_scale,
+                            int post_normalize, const int64_t* valid, float ratio_lo,
+                            float ratio_hi, float clip_c, float* grad, float* acc, float* partials,
+                            void* stream) {
   const bool need_row = (row_scale != nullptr) || (kind == 1);
   int rc = check_rows2(cu, n_rows, n_slots, uniform_len, need_row);
   if (rc != AXON_OK) return rc;
@@ -857,6 +858,67 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
                      post_normalize ? 1 : 0, valid, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
+}
+
+extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, const float* adv,
+                                const void* mask, int mask_kind, const float* isw,
+                                const int32_t* cu, int64_t n_rows, int64_t n_slots,
+                                int64_t uniform_len, const float* row_scale, const float* row_mean,
+                                float uniform_scale, int post_normalize, const int64_t* valid,
+                                float ratio_lo, float ratio_hi, float clip_c, float* grad,
+                                float* acc, float* partials, void* stream) {
+  return policy_loss_impl(kind, logp, oldp, adv, mask, mask_kind, isw, cu, n_rows, n_slots,
+                          uniform_len, row_scale, row_mean, uniform_scale, post_normalize, valid,
+                          ratio_lo, ratio_hi, clip_c, grad, acc, partials, stream);
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Same kernels as axon_policy_loss; the per-workgroup partial sums go to a fixed array in device
+// memory instead of a caller-provided workspace.  The array is sized for kNoAllocBlocks workgroups
+// of one chunk each (128 KB); every GPU the library runs on holds its own copy until the process
+// ends.  In host code the array's name is only a handle: its device address is looked up once per
+// device (with that device current) and kept, and only that address is handed to kernels.
+namespace {
+constexpr int kNoAllocBlocks = 4096;
+constexpr int64_t kNoAllocMaxSlots = (int64_t)kNoAllocBlocks * kChunk;  // 2^24 tokens
+constexpr int kNoAllocMaxDevices = 64;
+}  // namespace
+static __device__ __align__(256) float scratch[kNoAllocBlocks * kPartialStride];
+static float* g_scratch_addr[kNoAllocMaxDevices];  // per device; null until the first call there
+static std::mutex g_scratch_mutex;
+
+static int scratch_of_current_device(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return AXON_ERR_LAUNCH;
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return AXON_ERR_DEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_addr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr)
+      return AXON_ERR_LAUNCH;
+    g_scratch_addr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_addr[dev];
+  return AXON_OK;
+}
+
+extern "C" int axon_policy_loss_noalloc(int kind, const float* logp, const float* oldp,
+                                        const float* adv, const void* mask, int mask_kind,
+                                        const float* isw, const int32_t* cu, int64_t n_rows,
+                                        int64_t n_slots, int64_t uniform_len,
+                                        const float* row_scale, const float* row_mean,
+                                        float uniform_scale, int post_normalize,
+                                        const int64_t* valid, float ratio_lo, float ratio_hi,
+                                        float clip_c, float* grad, float* acc, void* stream) {
+  if (n_slots > kNoAllocMaxSlots) return AXON_ERR_TOO_LARGE;
+  float* partials = nullptr;
+  const int rc = scratch_of_current_device(&partials);
+  if (rc != AXON_OK) return rc;
+  // every workgroup overwrites its whole row of the array and the reduction reads only the rows of
+  // this launch, so nothing left by an earlier call is read and nothing has to be cleared
+  return policy_loss_impl(kind, logp, oldp, adv, mask, mask_kind, isw, cu, n_rows, n_slots,
+                          uniform_len, row_scale, row_mean, uniform_scale, post_normalize, valid,
+                          ratio_lo, ratio_hi, clip_c, grad, acc, partials, stream);
 }
 
 extern "C" int axon_cov_policy_loss(int kind, const float* logp, const float* oldp, const float* adv,

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 13
+#define AXON_AMD_ABI_VERSION 14
 
 enum {
   AXON_OK = 0,
@@ -37,7 +37,8 @@ enum {
   AXON_ERR_SHAPE = -2,     /* size constraint violated (see each function)    */
   AXON_ERR_WORKSPACE = -3, /* workspace too small or misaligned               */
   AXON_ERR_LAUNCH = -4,    /* hipGetLastError() after a launch was not success */
-  AXON_ERR_DEVICE = -5     /* not a gfx950 device                             */
+  AXON_ERR_DEVICE = -5,    /* not a gfx950 device                             */
+  AXON_ERR_TOO_LARGE = -6  /* beyond the fixed capacity of a no-allocation entry point */
 };
 
 /* mask element types accepted by stage-2/3 kernels (response_mask is int64 in
@@ -336,6 +337,27 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
                      float uniform_scale, int post_normalize, const int64_t* valid_count,
                      float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                      float* partials, void* stream);
+
+/* axon_policy_loss for callers that cannot allocate.  No counterpart in the reference: it is
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid
+ * hipMalloc, which cannot obtain the `partials` workspace.  Arguments, outputs and results
+ * are those of axon_policy_loss (same kernels) without `partials`: the per-workgroup partial
+ * sums go to a fixed 128 KB array in device memory that the library holds on every GPU it
+ * runs on until the process ends.  Calls no hipMalloc / hipFree and no allocating routine.
+ *   n_slots <= 16 777 216 (2^24 tokens: one 4096-token chunk for each of the array's 4096
+ *   rows); larger inputs return AXON_ERR_TOO_LARGE and launch nothing.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress, with that
+ * device current) and must therefore happen outside stream capture; later calls on that
+ * device only launch.  All calls on one GPU share the array: calls that overlap in time on
+ * one GPU (different streams) race on it; calls ordered on one stream, or by events, do not.
+ * Nothing in the array has to start at zero, so nothing is cleared between calls. */
+int axon_policy_loss_noalloc(int kind, const float* logp, const float* old_logp, const float* adv,
+                             const void* mask, int mask_kind, const float* is_weights,
+                             const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                             int64_t uniform_len, const float* row_scale, const float* row_mean,
+                             float uniform_scale, int post_normalize, const int64_t* valid_count,
+                             float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
+                             void* stream);
 
 /* The non-fused branch of fsdp_model_forward (axon/utils/fsdp/forward_utils.py:287-304): the model has
  * written logits [n, vocab] (row stride ld elements; dtype AXON_LOGITS_F32 or AXON_LOGITS_BF16, already
