@@ -607,7 +607,12 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | Non
     return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
 
 
-# The backward runs over the rows with an upstream gradient only when they are at most this share of all rows
+# Opt-in: let the LM-head backward look for rows without an upstream gradient and leave them out.  Finding
+# them costs a device-to-host readback (a host synchronisation per backward), which the reference's backward
+# does not have, so the default backward never does it; a caller that knows its response mask hands it to
+# ``packed_logprobs(..., response_mask=)`` instead, which keeps those rows out of forward and backward alike.
+SKIP_ZERO_GRAD_ROWS = False
+# With the search on, the backward runs over the active rows only when they are at most this share of all rows
 # (below that the two row copies cost more than the skipped work saves).
 SKIP_ROWS_BELOW = 0.97
 
@@ -623,20 +628,25 @@ def _active_rows(g_lp, g_en, seq_start, n):
 
 
 def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
-                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=True):
-    """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``).
+                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=None):
+    """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``).  By default the
+    call only enqueues launches: no readback, no host synchronisation, and it can be captured into a HIP graph.
 
-    With ``skip_zero_rows`` the rows whose upstream gradients are both exactly zero (prompt positions, where the
-    response mask is zero, rejected or clipped tokens) are left out of the three GEMMs: they contribute
-    nothing to ``d_weight`` and their ``d_hidden`` rows are zero.  Finding them costs one readback, so it
-    is not done while the stream is being captured into a graph."""
+    With ``skip_zero_rows`` (default: the module switch ``SKIP_ZERO_GRAD_ROWS``, off) the rows whose upstream
+    gradients are both exactly zero (prompt positions, where the response mask is zero, rejected or clipped
+    tokens) are left out of the three GEMMs: they contribute nothing to ``d_weight`` and their ``d_hidden`` rows
+    are zero.  Finding them costs one readback, so it cannot be used while the stream is being captured."""
     vocab_chunk = vocab_chunk or DEFAULT_VOCAB_CHUNK
+    if skip_zero_rows is None:
+        skip_zero_rows = SKIP_ZERO_GRAD_ROWS
     lib = _lib.load()
     require_device(hidden, "lmhead_backward")
     n, h, v = _head_operands("lmhead_backward", hidden, weight, labels, seq_start)
     _same_len("lmhead_backward", n, dlogprobs=dlogprobs, dentropy=dentropy, lse=lse, entropy_b=entropy_b)
     dev = hidden.device
-    if skip_zero_rows and n > 0 and h % 8 == 0 and not torch.cuda.is_current_stream_capturing():
+    if skip_zero_rows and torch.cuda.is_current_stream_capturing():
+        raise _lib.AxonAmdError("lmhead_backward: skip_zero_rows reads a count back and cannot run under stream capture")
+    if skip_zero_rows and n > 0 and h % 8 == 0:
         g_lp = f32(dlogprobs)
         g_en = f32(dentropy) if dentropy is not None else None
         row_index, row_rank, n_act = _active_rows(g_lp, g_en, seq_start, n)

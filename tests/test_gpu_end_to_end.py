@@ -115,6 +115,98 @@ def test_qwen3_8b_shape_properties():
     assert rel_l2(dh2, 2 * dh.float()) < 1e-2 and rel_l2(dw2, 2 * dw.float()) < 1e-2
 
 
+def _fp32_torch_head_reference(hd, wd, ld, g_lp, g_en, rows, token_block=2048):
+    """The head in plain fp32 torch on the GPU, block of tokens by block of tokens (library matmul,
+    logsumexp, softmax: nothing of the HIP kernels): log-prob and entropy of every token, and d_weight for
+    the vocabulary rows ``rows`` under upstream gradients ``g_lp`` (log-prob) and ``g_en`` (entropy),
+    dlogit = g_lp (onehot - p) - g_en p (logit - sum p logit), d_weight[r] = sum_n dlogit[n, r] hidden[n]."""
+    n = hd.shape[0]
+    w32 = wd.float()
+    lp = torch.empty(n, device=hd.device)
+    ent = torch.empty(n, device=hd.device)
+    dw_rows = torch.zeros(len(rows), hd.shape[1], device=hd.device, dtype=torch.float64)
+    rows_d = rows.to(hd.device)
+    for a in range(0, n, token_block):
+        b = min(a + token_block, n)
+        h32 = hd[a:b].float()
+        logits = h32 @ w32.t()
+        lse = torch.logsumexp(logits, -1)
+        p = torch.softmax(logits, -1)
+        eb = (p * logits).sum(-1)
+        lab = ld[a:b].long()
+        lp[a:b] = logits.gather(1, lab[:, None])[:, 0] - lse
+        ent[a:b] = lse - eb
+        pr = p[:, rows_d]
+        dl = -g_lp[a:b, None] * pr + g_lp[a:b, None] * (lab[:, None] == rows_d[None, :]).float()
+        if g_en is not None:
+            dl = dl - g_en[a:b, None] * pr * (logits[:, rows_d] - eb[:, None])
+        dw_rows += (dl.t().double() @ h32.double())
+        del logits, p
+    return lp, ent, dw_rows
+
+
+def _spread_rows(v, chunk=32768):
+    """Vocabulary rows spread over every chunk of the backward, with the edges of the chunks and of the last
+    (partial) 256-row tile among them."""
+    rows = set(range(0, v, 1571)) | {0, 255, 256, v - 1, v - 2, v - 128, v - 129, v - 256, v - 257}
+    for c in range(chunk, v, chunk):
+        rows |= {c - 1, c, c + 255, c + 256}
+    return torch.tensor(sorted(r for r in rows if 0 <= r < v))
+
+
+def test_qwen3_8b_dweight_rows_vs_fp32_torch():
+    """Config 3 at full size: d_weight on ~120 vocabulary rows spread over all five vocabulary chunks of the
+    backward (rows >= 131072 and the last tile included), log-prob and entropy of every token, against an
+    fp32 torch reference computed on the GPU.  Tolerances: 1e-3 absolute, 2e-2 relative L2."""
+    n, h, v = 32768, 4096, 151936
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=3)
+    hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
+    from axon_amd import _ops
+    lp, ent, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    gen = torch.Generator().manual_seed(33)
+    g_lp = (torch.randn(n, generator=gen) / n).to(DEV)
+    g_en = (0.3 * torch.randn(n, generator=gen) / n).to(DEV)
+    dh, dw = _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0)
+    rows = _spread_rows(v)
+    assert (rows >= 131072).sum() >= 10 and len(rows) >= 64
+    ref_lp, ref_ent, ref_dw = _fp32_torch_head_reference(hd, wd, ld, g_lp, g_en, rows)
+    assert (lp - ref_lp).abs().max().item() < 1e-3
+    assert (ent - ref_ent).abs().max().item() < 1e-3
+    got = dw[rows.to(DEV)].double()
+    assert rel_l2(got, ref_dw) < 2e-2
+    per_row = (got - ref_dw).norm(dim=1) / ref_dw.norm(dim=1).clamp_min(1e-30)
+    assert per_row.max().item() < 5e-2, (per_row.argmax().item(), per_row.max().item())  # no single row is off
+
+
+def test_gpt_oss_head_full_shape():
+    """Config 5's head at its full shape (16384 x 2880 x 201088; hidden size not a multiple of 128): forward
+    on every token and d_weight on spread rows against the fp32 torch reference on the GPU, a token subset of
+    forward and d_hidden against the CPU oracle, and linearity of the backward."""
+    import math
+    n, h, v = 16384, 2880, 201088
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=5)
+    hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
+    from axon_amd import _ops
+    lp, ent, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+    assert torch.isfinite(lp).all() and (lp <= 1e-4).all()
+    assert (ent >= -1e-4).all() and (ent <= math.log(v) + 1e-3).all()
+    idx = torch.arange(0, n, 497)
+    o_lp, o_ent = OM.forward(hid[idx], w, lab[idx])
+    assert (lp.cpu()[idx] - o_lp).abs().max() < 1e-3 and (ent.cpu()[idx] - o_ent).abs().max() < 1e-3
+    gen = torch.Generator().manual_seed(55)
+    g_lp = (torch.randn(n, generator=gen) / n).to(DEV)
+    dh, dw = _ops.lmhead_backward(g_lp, None, hd, wd, ld, lse, eb, 1.0)
+    assert torch.isfinite(dh.float()).all() and torch.isfinite(dw.float()).all()
+    rows = _spread_rows(v)
+    ref_lp, ref_ent, ref_dw = _fp32_torch_head_reference(hd, wd, ld, g_lp, None, rows)
+    assert (lp - ref_lp).abs().max().item() < 1e-3 and (ent - ref_ent).abs().max().item() < 1e-3
+    assert rel_l2(dw[rows.to(DEV)].double(), ref_dw) < 2e-2
+    o_dh, _ = OM.backward(g_lp.cpu()[idx], None, hid[idx], w, lab[idx])
+    assert rel_l2(dh[idx.to(DEV)], o_dh) < 2e-2
+    dh2, dw2 = _ops.lmhead_backward(2 * g_lp, None, hd, wd, ld, lse, eb, 1.0)
+    assert rel_l2(dh2, 2 * dh.float()) < 1e-2 and rel_l2(dw2, 2 * dw.float()) < 1e-2
+
+
 def test_micro_batched_dapo_chain_vs_whole_batch_oracle():
     """The GPT-OSS-style configuration at reduced size (hidden 2880 kept: K not a multiple of 128): advantages and
     dynamic sampling over all sequences, then head + DAPO loss per micro-batch of whole sequences with the

@@ -474,8 +474,8 @@ def test_backward_skips_rows_without_gradient(n, h, v, ldt, with_entropy):
     g_lp = torch.randn(n, generator=gen) / n * live
     g_en = torch.randn(n, generator=gen) / n * live if with_entropy else None
     args = (g_lp.to(DEV), None if g_en is None else g_en.to(DEV), hd, wd, ld, lse, eb, 1.0)
-    dh, dw = _ops.lmhead_backward(*args)
-    dh_all, dw_all = _ops.lmhead_backward(*args, skip_zero_rows=False)
+    dh, dw = _ops.lmhead_backward(*args, skip_zero_rows=True)
+    dh_all, dw_all = _ops.lmhead_backward(*args)  # the default: every row, no readback
     assert (dh[~live.to(DEV)] == 0).all() and (dh_all[~live.to(DEV)] == 0).all()
     # a d_hidden row is a sum over the vocabulary only: the row set does not change it
     assert torch.equal(dh, dh_all)
@@ -501,18 +501,17 @@ def test_backward_row_skipping_in_the_aligned_layout_and_all_zero():
     for skip in (True, False):
         hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
         lp, _ = packed_logprobs(hd, wd, ids.to(DEV).view(1, -1), cu, 0.9)
-        old = _ops.SKIP_ROWS_BELOW
-        _ops.SKIP_ROWS_BELOW = old if skip else -1.0
+        _ops.SKIP_ZERO_GRAD_ROWS = skip
         try:
             (lp * g_lp).sum().backward()
         finally:
-            _ops.SKIP_ROWS_BELOW = old
+            _ops.SKIP_ZERO_GRAD_ROWS = False
         grads.append((hd.grad, wd.grad))
     assert torch.equal(grads[0][0], grads[1][0]) and rel_l2(grads[0][1], grads[1][1]) < 1e-3
     assert (grads[0][0].abs().sum(1) > 0).sum().item() <= int(resp.sum())  # only rows that predict a response token
     # nothing to do at all: exact zeros, no GEMM
     _, _, lab, hd, wd, ld, lse, eb = _head_state(64, 64, 500, 5)
-    dh, dw = _ops.lmhead_backward(torch.zeros(64, device=DEV), None, hd, wd, ld, lse, eb, 1.0)
+    dh, dw = _ops.lmhead_backward(torch.zeros(64, device=DEV), None, hd, wd, ld, lse, eb, 1.0, skip_zero_rows=True)
     assert not dh.any() and not dw.any() and dh.dtype == torch.bfloat16 and dw.shape == wd.shape
 
 
@@ -600,3 +599,35 @@ def test_fsdp_model_forward_skip_prompt_rows(remove_padding):
     # fewer rows can put the head on its other main loop (another summation order over the hidden size)
     assert (lp1 - lp0)[seen > 0].abs().max() < 1e-5 and (ent1 - ent0)[seen > 0].abs().max() < 1e-5
     assert rel_l2(dw1, dw0) < 1e-3 and rel_l2(de1, de0) < 1e-3
+
+
+def test_default_backward_has_no_readback_and_replays_in_a_hip_graph():
+    """The default backward only enqueues launches: it can be captured into a HIP graph, and every replay is
+    bit-identical to the eager call (eager work and synchronisations between the replays)."""
+    n, h, v = 1024, 256, 2048
+    hid, w, lab, hd, wd, ld, lse, eb = _head_state(n, h, v, 91)
+    gen = torch.Generator().manual_seed(9)
+    g_lp = (torch.randn(n, generator=gen) / n).to(DEV)
+    g_en = (torch.randn(n, generator=gen) / n).to(DEV)
+    dh_e, dw_e = _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0, vocab_chunk=1024)  # two chunks
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            dh_g, dw_g = _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0, vocab_chunk=1024)
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        dh_g.zero_(); dw_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(dh_g, dh_e) and torch.equal(dw_g, dw_e)
+        again = _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0, vocab_chunk=1024)  # eager work in between
+        torch.cuda.synchronize()
+        assert torch.equal(again[0], dh_e) and torch.equal(again[1], dw_e)
+    with torch.cuda.stream(side):
+        with pytest.raises(Exception):
+            with torch.cuda.graph(torch.cuda.CUDAGraph(), stream=side):
+                _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, lse, eb, 1.0, skip_zero_rows=True)
+    torch.cuda.synchronize()

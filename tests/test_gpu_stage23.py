@@ -308,8 +308,9 @@ def test_ppo_clip_regions_table_gpu():
         assert data.batch["log_probs"].grad[0, k].item() == pytest.approx(g / n, rel=1e-5, abs=1e-9), REGIONS[k]
 
 
-def test_gspo_packed_config4_vs_oracle():
-    d = W.c4_correction(n_tokens=20000)
+@pytest.mark.parametrize("n_tokens", [20000, 65536])  # 65536 is the full size of the configuration
+def test_gspo_packed_config4_vs_oracle(n_tokens):
+    d = W.c4_correction(n_tokens=n_tokens)
     s = len(d["lengths"])
     gidx = T(np.unique(d["uid"], return_inverse=True)[1])
     tmax = max(d["lengths"])
