@@ -14,7 +14,7 @@ import tempfile
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libaxon_amd.so")
-SOURCES = ("capi.hip", "rows.hip", "loss.hip", "diag.hip", "returns.hip", "cov.hip", "logits.hip", "lmhead.hip")
+SOURCES = ("capi.hip", "rows.hip", "loss.hip", "owned.hip", "diag.hip", "returns.hip", "cov.hip", "logits.hip", "lmhead.hip")
 
 HIPCC_FLAGS = (
     "--offload-arch=gfx950",

@@ -74,11 +74,16 @@ SIGNATURES: dict[str, tuple] = {
     "axon_policy_loss": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                 _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr,
                                 _ptr]),
+    "axon_policy_loss_rows": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64, _i32, _i32,
+                                     _ptr, _ptr, _ptr, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr, _ptr]),
+    "axon_sampler_correction_rows": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32, _i32,
+                                            _f32, _f32, _i32, _f32, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                            _ptr]),
     "axon_policy_loss_noalloc": (_i32, [_i32, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                         _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
 }
 
-ABI_VERSION = 14
+ABI_VERSION = 16
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -79,10 +79,20 @@ def _acc8(n_slots, device):
     return _zeros(8, device) if n_slots == 0 else torch.empty(8, device=device, dtype=torch.float32)
 
 
+_PARTIALS: dict = {}
+
+
 def _partials(n_slots, device):
-    """Uninitialised workspace for the per-workgroup partial sums of the elementwise kernels."""
-    nbytes = _lib.load().axon_reduce_partials_bytes(int(n_slots))
-    return torch.empty(max(nbytes // 4, 8), device=device, dtype=torch.float32)
+    """Workspace of the per-workgroup partial sums (and the ticket counter behind them) of the elementwise
+    kernels.  The counter has to be zero before the first launch and every launch leaves it zero, so one
+    zero-filled buffer per (device, stream) is kept and reused: launches on one stream are ordered."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr())
+    ws = _PARTIALS.get(key)
+    if ws is None:
+        nbytes = _lib.load().axon_reduce_partials_bytes(int(n_slots))
+        ws = torch.zeros(nbytes // 4, device=device, dtype=torch.float32)
+        _PARTIALS[key] = ws
+    return ws
 
 
 def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=True, want_sum=True):
@@ -236,18 +246,23 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
     mk, kind = mask_arg(mask)
     has_veto = log_veto is not None
     need_row = is_mode == 2 or rs_mode >= 2 or has_veto
-    cnt = ssum = flag = None
-    if need_row:
-        cnt, ssum, flag = row_stats(old_lp, samp_lp, mk, rows, flag_mode=1 if has_veto else 0,
-                                    threshold=log_veto if has_veto else 0.0)
     isw = torch.empty(rows.shape, device=dev, dtype=torch.float32) if is_mode else None
     new_mask = torch.empty(rows.shape, device=dev, dtype=torch.float32)
     acc = _acc8(rows.n_slots, dev)
+    if need_row:  # a workgroup owns whole rows: one pass over the tokens, row sums in a fixed order
+        check(
+            lib.axon_sampler_correction_rows(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows,
+                                             rows.n_slots, rows.uniform_len, is_mode, float(is_threshold), rs_mode,
+                                             float(rs_lr_lo), float(rs_lr_hi), int(has_veto),
+                                             float(log_veto if has_veto else 0.0), ptr(isw), ptr(new_mask), None,
+                                             None, None, ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
+            "axon_sampler_correction_rows",
+        )
+        return isw, new_mask, acc
     check(
         lib.axon_sampler_correction(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
                                     rows.uniform_len, is_mode, float(is_threshold), rs_mode, float(rs_lr_lo),
-                                    float(rs_lr_hi), int(has_veto), float(log_veto if has_veto else 0.0), ptr(cnt),
-                                    ptr(ssum), ptr(flag), ptr(isw), ptr(new_mask), ptr(acc),
+                                    float(rs_lr_hi), 0, 0.0, None, None, None, ptr(isw), ptr(new_mask), ptr(acc),
                                     ptr(_partials(rows.n_slots, dev)), stream_ptr()),
         "axon_sampler_correction",
     )
@@ -285,13 +300,15 @@ TOKEN_REDUCE = {"sum": 0, "mean": 1, "mean-norm": 2, "mean-program": 3}
 BATCH_REDUCE = {"token-mean": 0, "step-mean": 1, "program-mean": 2}
 
 
-def _i64_dev(x, dev, n=None, what="count"):
+def _count_dev(x, dev, n=None, what="count"):
+    """A count (or one count per row) as float64 on the device: the reference divides by the value as it is
+    (loss/utils.py:224-229), so a fractional count, e.g. one averaged over ranks, is not truncated."""
     if x is None:
         return None
     if n is not None and int(x.numel()) != n:
         raise ValueError(f"{what} has {int(x.numel())} entries, expected one per row ({n})")
     t = torch.as_tensor(x)
-    return t.to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
+    return t.to(device=dev, dtype=torch.float64).reshape(-1).contiguous()
 
 
 def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, rows: Rows, *, token_reduce,
@@ -312,31 +329,31 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     isw = f32(is_weights) if is_weights is not None else None
     tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
 
-    valid = _i64_dev(valid_count, dev)
+    valid = _count_dev(valid_count, dev)
     grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
     acc = _acc8(rows.n_slots, dev)
     # PPO with sum / token-mean needs no per-row quantity: one pass over the tokens, the
     # division by the token count happens when the last workgroup has the total.
     one_pass = kind != 1 and tr == 0 and br == 0
-    row_scale = row_mean = None
-    if not one_pass:
-        cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
-        row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
-        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
+    if not one_pass:  # a workgroup owns whole rows: still one pass over the tokens
+        if tr == 2 and not rows.uniform_len:
+            raise ValueError("token_reduce='mean-norm' divides by the padded row length: needs a [batch, seq] layout")
+        prtc = _count_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _count_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
-            lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr,
-                                    br, ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
-                                    stream_ptr()),
-            "axon_loss_row_scale",
+            lib.axon_policy_loss_rows(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr,
+                                      rows.n_rows, rows.n_slots, rows.uniform_len, tr, br, ptr(prtc), ptr(npt),
+                                      ptr(nps), ptr(valid), float(ratio_lo), float(ratio_hi), float(clip_c),
+                                      ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
+            "axon_policy_loss_rows",
         )
+        return acc, grad
     check(
         lib.axon_policy_loss(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
-                             rows.n_slots, rows.uniform_len, ptr(row_scale), ptr(row_mean), 1.0, int(one_pass),
-                             ptr(valid if one_pass else None), float(ratio_lo), float(ratio_hi), float(clip_c),
-                             ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
+                             rows.n_slots, rows.uniform_len, None, None, 1.0, 1, ptr(valid), float(ratio_lo),
+                             float(ratio_hi), float(clip_c), ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)),
+                             stream_ptr()),
         "axon_policy_loss",
     )
     return acc, grad
@@ -368,7 +385,7 @@ def cov_policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights
                             ptr(state), ptr(ws), stream_ptr()),
         "axon_cov_select",
     )
-    valid = _i64_dev(valid_count, dev)
+    valid = _count_dev(valid_count, dev)
     grad = torch.empty(rows.shape, device=dev, dtype=torch.float32)
     acc = _acc8(n, dev)
     one_pass = tr == 0 and br == 0
@@ -376,9 +393,9 @@ def cov_policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights
     if not one_pass:
         cnt, _, _ = row_stats(lp, None, mk, rows, want_sum=False)
         row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
+        prtc = _count_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _count_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
             lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
                                     ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),
@@ -478,15 +495,15 @@ def side_terms(entropy, log_probs, ref_log_probs, mask, rows: Rows, *, token_red
     ref = f32(ref_log_probs) if kl_type else None
     mk, mkind = mask_arg(mask)
     tr, br = TOKEN_REDUCE[token_reduce], BATCH_REDUCE[batch_reduce]
-    valid = _i64_dev(valid_count, dev)
+    valid = _count_dev(valid_count, dev)
     one_pass = tr == 0 and br == 0
     row_scale = None
     if not one_pass:
         cnt, _, _ = row_stats(anchor, None, mk, rows, want_sum=False)
         row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
-        prtc = _i64_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
-        npt = _i64_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
-        nps = _i64_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
+        prtc = _count_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+        npt = _count_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+        nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
         check(
             lib.axon_loss_row_scale(ptr(cnt), None, rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr, br,
                                     ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), None, stream_ptr()),

@@ -91,10 +91,18 @@ __device__ __forceinline__ void block_sum(float (&v)[NV], float* lds /* [NV * 4]
 
 // Grid-wide sums without same-address atomics: a streaming kernel runs at most kMaxStreamBlocks
 // workgroups, each walking chunks blockIdx.x, blockIdx.x + gridDim.x, ... and leaving its NV
-// partial sums in partials[blockIdx.x][8]; reduce_partials_kernel (one workgroup, launched
-// next on the same stream) adds them in a fixed order, so results are reproducible.
+// partial sums in partials[blockIdx.x][8].  They are added in a fixed order, so results are
+// reproducible: either inside the launch (grid_finish below) or by a small kernel launched next on
+// the same stream (store_block_partials + a finishing kernel).
 constexpr int kMaxStreamBlocks = 16384;  // one chunk per workgroup up to 2^26 tokens
 constexpr int kPartialStride = 8;
+constexpr int kFinishGroup = 64;         // workgroups whose rows one wavefront adds
+constexpr int kMaxFinishGroups = kMaxStreamBlocks / kFinishGroup;  // 256: one workgroup adds the group rows
+// workspace of grid_finish: rows, group rows, then the ticket counters (one per group, one for the grid)
+constexpr int64_t kGroupRowsOffset = (int64_t)kMaxStreamBlocks * kPartialStride;                    // in floats
+constexpr int64_t kTicketsOffset = kGroupRowsOffset + (int64_t)kMaxFinishGroups * kPartialStride;  // in floats
+constexpr int64_t kTicketBytes = 2048;  // 257 counters
+constexpr int64_t kPartialsBytes = kTicketsOffset * 4 + kTicketBytes;
 
 template <int NV>
 __device__ __forceinline__ void store_block_partials(float (&v)[NV], float* lds /* [NV * 4] */,
@@ -108,9 +116,88 @@ __device__ __forceinline__ void store_block_partials(float (&v)[NV], float* lds 
   }
 }
 
+// One row of eight floats to the level all XCDs share, then a ticket: true for the caller that draws
+// the last of `n` tickets.  The row goes out with agent-scope stores, which write through; waiting
+// for their acknowledgement orders them before the ticket.  (A release fence would also write back
+// every dirty line of this XCD's L2, the kernel's own output stream included, once per workgroup:
+// +35 % kernel time at 2^26 tokens.)
+__device__ __forceinline__ bool publish_row_take_ticket(float* row, const float (&v)[kPartialStride],
+                                                        unsigned* ticket, unsigned n) {
+#pragma unroll
+  for (int k = 0; k < kPartialStride; ++k)
+    __hip_atomic_store(row + k, v[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+  const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (t != n - 1) return false;
+  __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+  return true;
+}
+
+// The sums finished inside the launch, in two levels.  Every workgroup publishes its row and takes a
+// ticket of its group of kFinishGroup workgroups; the workgroup that draws a group's last ticket adds
+// the group's rows (one wavefront: lane l takes row l, then the fixed tree of wave_sum), publishes
+// the group row and takes a ticket of the grid; the workgroup that draws the last of those adds the
+// group rows (thread t takes group t, then the fixed tree of block_sum) and hands the eight totals
+// to `fin` in its thread 0.  The order of every addition is fixed by the grid size alone.  The
+// counters must be zero when the kernel starts and are zero again when it ends.
+template <int NV, class Fin>
+__device__ __forceinline__ void grid_finish(float (&v)[NV], float* lds /* [8 * 4] */, float* ws,
+                                            Fin&& fin) {
+  static_assert(NV <= kPartialStride, "partials row too small");
+  __shared__ int s_stage;
+  unsigned* tickets = reinterpret_cast<unsigned*>(ws + kTicketsOffset);
+  const unsigned group = blockIdx.x / kFinishGroup;
+  const unsigned n_groups = (gridDim.x + kFinishGroup - 1) / kFinishGroup;
+  const unsigned first = group * kFinishGroup;
+  const unsigned in_group = min((unsigned)kFinishGroup, gridDim.x - first);
+  block_sum<NV>(v, lds);
+  if (threadIdx.x == 0) {
+    float row[kPartialStride];
+#pragma unroll
+    for (int k = 0; k < kPartialStride; ++k) row[k] = (k < NV) ? v[k < NV ? k : 0] : 0.f;
+    s_stage = publish_row_take_ticket(ws + (size_t)blockIdx.x * kPartialStride, row, tickets + 1 + group,
+                                      in_group) ? 1 : 0;
+  }
+  __syncthreads();
+  if (s_stage == 0) return;
+  // every row of the group was acknowledged at the shared level before its ticket was drawn; drop
+  // what this XCD's caches may still hold of those addresses (an earlier launch), then read them
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  if (threadIdx.x < kWave) {
+    float t[kPartialStride];
+    const bool ok = threadIdx.x < in_group;
+    const float* row = ws + (size_t)(first + (ok ? threadIdx.x : 0)) * kPartialStride;
+    const float4 lo4 = *reinterpret_cast<const float4*>(row), hi4 = *reinterpret_cast<const float4*>(row + 4);
+    t[0] = ok ? lo4.x : 0.f; t[1] = ok ? lo4.y : 0.f; t[2] = ok ? lo4.z : 0.f; t[3] = ok ? lo4.w : 0.f;
+    t[4] = ok ? hi4.x : 0.f; t[5] = ok ? hi4.y : 0.f; t[6] = ok ? hi4.z : 0.f; t[7] = ok ? hi4.w : 0.f;
+#pragma unroll
+    for (int k = 0; k < kPartialStride; ++k) t[k] = wave_sum(t[k]);
+    if (threadIdx.x == 0)
+      s_stage = publish_row_take_ticket(ws + kGroupRowsOffset + (size_t)group * kPartialStride, t, tickets,
+                                        n_groups) ? 2 : 1;
+  }
+  __syncthreads();
+  if (s_stage != 2) return;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  float t[kPartialStride];
+  {
+    const bool ok = threadIdx.x < n_groups;  // n_groups <= kBlock
+    const float* row = ws + kGroupRowsOffset + (size_t)(ok ? threadIdx.x : 0) * kPartialStride;
+    const float4 lo4 = *reinterpret_cast<const float4*>(row), hi4 = *reinterpret_cast<const float4*>(row + 4);
+    t[0] = ok ? lo4.x : 0.f; t[1] = ok ? lo4.y : 0.f; t[2] = ok ? lo4.z : 0.f; t[3] = ok ? lo4.w : 0.f;
+    t[4] = ok ? hi4.x : 0.f; t[5] = ok ? hi4.y : 0.f; t[6] = ok ? hi4.z : 0.f; t[7] = ok ? hi4.w : 0.f;
+  }
+  block_sum<kPartialStride>(t, lds);  // the barriers above separate this use of `lds` from the first
+  if (threadIdx.x == 0) fin(t);
+}
+
+#ifndef AXON_EXP_GRIDCAP
+#define AXON_EXP_GRIDCAP 6144
+#endif
+constexpr int kStreamGridCap = AXON_EXP_GRIDCAP;
 inline unsigned stream_grid(int64_t n_slots) {
   const int64_t chunks = (n_slots + kChunk - 1) / kChunk;
-  return (unsigned)(chunks < kMaxStreamBlocks ? chunks : kMaxStreamBlocks);
+  return (unsigned)(chunks < kStreamGridCap ? chunks : kStreamGridCap);
 }
 
 // 16-byte streaming accesses.  Every input of these kernels is read once and every output

@@ -2,9 +2,23 @@
 // loss with its gradient.  One read of every input, one write of every output;
 // scalar sums leave through per-workgroup partials that the last workgroup adds up.
 #include "common.h"
+#include "token_math.h"
 #include <mutex>
 
 namespace axon {
+
+// acc[0..7] from the eight totals.  norm_slots != 0: the slots in that bit mask (plain masked sums)
+// become token-means, acc[5] the factor 1/denominator.
+__device__ __forceinline__ void write_acc(float (&tot)[kPartialStride], int norm_slots,
+                                          const double* valid, float* acc) {
+  if (norm_slots) {  // token-mean over a plain sum: the denominator is known only now
+    const float den = fmaxf(valid != nullptr ? (float)valid[0] : tot[4], 1.f);
+    for (int k = 0; k < kPartialStride; ++k)
+      if ((norm_slots >> k) & 1) tot[k] = tot[k] / den;
+    tot[5] = 1.f / den;
+  }
+  for (int k = 0; k < kPartialStride; ++k) acc[k] = tot[k];
+}
 
 template <int MK>
 __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
@@ -13,10 +27,11 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
     int is_mode, float is_thr, int rs_mode, float rs_lo, float rs_hi, int has_veto, float log_veto,
     const float* __restrict__ row_cnt, const float* __restrict__ row_sum,
     const int32_t* __restrict__ row_flag, float* __restrict__ isw, float* __restrict__ new_mask,
-    float* partials) {
+    float* partials, float* __restrict__ acc) {
   __shared__ int32_t lds_cu[kLdsRows];
-  __shared__ float lds_red[6 * (kBlock / kWave)];
+  __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   const bool need_row = (is_mode == 2) || (rs_mode >= 2) || has_veto;
+  const CorrCfg cfg{is_mode, is_thr, rs_mode, rs_lo, rs_hi, has_veto, log_veto};
   const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
@@ -46,48 +61,19 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
         mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
       }
     }
-    int r = -1;
     int64_t rend = -1;
-    float row_w = 0.f, row_keep = 1.f, row_veto_keep = 1.f;
+    CorrRow row{0.f, 1.f, 1.f};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t p = i + j;
       if (p >= n_slots) { wv[j] = 0.f; nm[j] = 0.f; continue; }
       if (need_row && p >= rend) {
-        r = rf.row(p);
+        const int r = rf.row(p);
         rend = rf.row_end(r);
-        const float rsum = row_sum ? row_sum[r] : 0.f;
-        const float rcnt = row_cnt ? row_cnt[r] : 0.f;
-        if (is_mode == 2) row_w = expf(clampf(rsum, -kSafetyBound, kSafetyBound));
-        row_keep = 1.f;
-        if (rs_mode == 2) row_keep = (rsum >= rs_lo && rsum <= rs_hi) ? 1.f : 0.f;
-        if (rs_mode == 3) {
-          const float g = rsum / (rcnt + 1e-8f);
-          row_keep = (g >= rs_lo && g <= rs_hi) ? 1.f : 0.f;
-        }
-        row_veto_keep = (has_veto && row_flag[r]) ? 0.f : 1.f;
+        row = corr_row(cfg, row_sum ? row_sum[r] : 0.f, row_cnt ? row_cnt[r] : 0.f,
+                       has_veto && row_flag[r] != 0);
       }
-      const float lr = ov[j] - sv[j];
-      const float m = mv[j];
-      const bool on = (m != 0.f);
-      // importance weight
-      float w = 0.f;
-      if (is_mode == 1) w = expf(clampf(lr, -kSafetyBound, kSafetyBound)) * m;
-      if (is_mode == 2) w = row_w * m;
-      a[1] += on ? w * m : 0.f;
-      w = (w != w) ? w : fminf(w, is_thr);  // clamp(max=thr), NaN propagates
-      wv[j] = w;
-      a[5] += on ? w * m : 0.f;
-      // rejection
-      float keep = 1.f;
-      if (rs_mode == 1) keep = (lr >= rs_lo && lr <= rs_hi) ? 1.f : 0.f;
-      if (rs_mode >= 2) keep = row_keep;
-      const float veto_keep = row_veto_keep;
-      a[2] += on ? (1.f - keep) * m : 0.f;
-      const bool cat = has_veto && on && (lr < log_veto);
-      a[3] += cat ? m : 0.f;
-      a[0] += m;
-      nm[j] = m * keep * veto_keep;
+      corr_token(cfg, row, ov[j], sv[j], mv[j], wv[j], nm[j], a);
     }
     if (full) {
       if (isw) store4(isw, i, wv);
@@ -103,14 +89,14 @@ __global__ __launch_bounds__(kBlock) void sampler_correction_kernel(
   if (blockIdx.x == 0 && has_veto) {
     for (int64_t r = threadIdx.x; r < n_rows; r += blockDim.x) a[4] += row_flag[r] ? 1.f : 0.f;
   }
-  store_block_partials<6>(a, lds_red, partials);
+  grid_finish<6>(a, lds_red, partials,
+                 [&](float (&tot)[kPartialStride]) { write_acc(tot, 0, nullptr, acc); });
 }
 
-// Adds the per-workgroup partial sums in a fixed order and writes acc[0..7].  norm_slots != 0:
-// the slots in that bit mask (plain masked sums) become token-means, acc[5] the factor 1/denominator.
+// Adds the per-workgroup partial sums in a fixed order and writes acc[0..7] (write_acc).
 __global__ __launch_bounds__(1024) void reduce_partials_kernel(
     const float* __restrict__ partials, int n_blocks, int norm_slots,
-    const int64_t* __restrict__ valid, float* __restrict__ acc) {
+    const double* __restrict__ valid, float* __restrict__ acc) {
   __shared__ float red[16][kPartialStride];
   float t[kPartialStride];
 #pragma unroll
@@ -147,21 +133,15 @@ __global__ __launch_bounds__(1024) void reduce_partials_kernel(
       for (int w = 0; w < (int)(blockDim.x >> 6); ++w) s += red[w][k];
       tot[k] = s;
     }
-    if (norm_slots) {  // token-mean over a plain sum: the denominator is known only now
-      const float den = fmaxf(valid != nullptr ? (float)valid[0] : tot[4], 1.f);
-      for (int k = 0; k < kPartialStride; ++k)
-        if ((norm_slots >> k) & 1) tot[k] = tot[k] / den;
-      tot[5] = 1.f / den;
-    }
-    for (int k = 0; k < kPartialStride; ++k) acc[k] = tot[k];
+    write_acc(tot, norm_slots, valid, acc);
   }
 }
 
 __global__ __launch_bounds__(1024) void loss_row_scale_kernel(
     const float* __restrict__ row_cnt, const float* __restrict__ row_sum, int64_t n_rows,
-    int64_t row_len, int token_reduce, int batch_reduce, const int64_t* __restrict__ prtc,
-    const int64_t* __restrict__ npt, const int64_t* __restrict__ nps,
-    const int64_t* __restrict__ valid, float* __restrict__ row_scale,
+    int64_t row_len, int token_reduce, int batch_reduce, const double* __restrict__ prtc,
+    const double* __restrict__ npt, const double* __restrict__ nps,
+    const double* __restrict__ valid, float* __restrict__ row_scale,
     float* __restrict__ row_mean) {
   __shared__ float red[2 * 16];
   __shared__ float tot[2];
@@ -203,15 +183,6 @@ __global__ __launch_bounds__(1024) void loss_row_scale_kernel(
   }
 }
 
-// max/min with PyTorch's gradient convention: ties split the gradient evenly.
-struct ValGrad { float v, g; };
-__device__ __forceinline__ ValGrad vg_max(ValGrad a, ValGrad b) {
-  if (a.v > b.v) return a;
-  if (a.v < b.v) return b;
-  if (a.v == b.v) return ValGrad{a.v, 0.5f * (a.g + b.g)};
-  return ValGrad{a.v + b.v, 0.f};  // NaN operand: propagate
-}
-
 template <int MK, int KIND>
 __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     const float* __restrict__ logp, const float* __restrict__ oldp, const float* __restrict__ adv,
@@ -219,9 +190,10 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     int64_t n_rows, int64_t n_slots, int64_t uniform_len, const float* __restrict__ row_scale,
     const float* __restrict__ row_mean, float uniform_scale, float lo, float hi, float clip_c,
     const uint32_t* __restrict__ sel_keys, const SelectState* __restrict__ sel_state,
-    float* __restrict__ grad, float* partials) {
+    float* __restrict__ grad, float* partials, int norm_slots, const double* __restrict__ valid,
+    float* __restrict__ acc) {
   __shared__ int32_t lds_cu[kLdsRows];
-  __shared__ float lds_red[6 * (kBlock / kWave)];
+  __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   const bool need_row = (row_scale != nullptr) || (KIND == 1);
   SelectState sel{};
   if (KIND >= 5) sel = *sel_state;
@@ -252,89 +224,10 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
         if (row_scale) scale = row_scale[r];
         if (KIND == 1) sbar = row_mean[r];
       }
-      const float A = av[j], m = mv[j];
-      const float d = lv[j] - ov[j];
-      const float w = wv[j];
-      a[4] += m;
-      if (KIND == 2) {  // REINFORCE / GPG (loss.py:471-512): -A * log_prob * w
-        a[2] += -d * m;
-        a[0] += (-A * lv[j] * w) * m * scale;
-        gv[j] = -A * w * m * scale;
-        continue;
-      }
-      if (KIND == 3) {  // CISPO (loss.py:411-468): -sg(clip(r)) * A * log_prob, IS weights not used
-        const float xc = clampf(d, -kSafetyBound, kSafetyBound);
-        const float r_ = expf(xc);
-        const float rc = clampf(r_, lo, hi);
-        float tm = 1.f;  // optional token-level mask of the unified formulation (clip_c != 0)
-        if (clip_c != 0.f && ((A > 0.f && r_ > hi) || (A < 0.f && r_ < lo))) tm = 0.f;
-        a[1] += (r_ > hi || r_ < lo) ? m : 0.f;
-        a[2] += -xc * m;
-        a[0] += (-rc * A * lv[j] * tm) * m * scale;
-        gv[j] = -rc * A * tm * m * scale;
-        continue;
-      }
-      if (KIND == 4) {  // clipped value loss (loss.py:547-591): logp = vpreds, oldp = values, adv = returns,
-                        // lo = cliprange_value; the caller applies the factor 0.5
-        const float vp = lv[j], up = ov[j] + lo, dn = ov[j] - lo;
-        // clip_by_value = maximum(minimum(vp, up), dn) with tensor bounds (loss/utils.py:94-101)
-        const float g_min = (vp < up) ? 1.f : ((vp == up) ? 0.5f : 0.f);
-        const float y = fminf(vp, up);
-        const float g_clip = (y > dn) ? g_min : ((y == dn) ? 0.5f * g_min : 0.f);
-        const float vc = fmaxf(y, dn);
-        const float e1 = vp - A, e2 = vc - A;
-        const ValGrad c = vg_max(ValGrad{e1 * e1, 2.f * e1}, ValGrad{e2 * e2, 2.f * e2 * g_clip});
-        a[1] += (e2 * e2 > e1 * e1) ? m : 0.f;
-        a[2] += vp * m;
-        a[0] += c.v * m * scale;
-        gv[j] = c.g * m * scale;
-        continue;
-      }
-      if (KIND == 5) {  // KL-Cov (loss.py:283-352): -A*ratio, plus clip_c * |log ratio| on the selected tokens
-        const bool pass = (d >= -kSafetyBound && d <= kSafetyBound);
-        const float xc = clampf(d, -kSafetyBound, kSafetyBound);
-        const float r_ = expf(xc);
-        float v = -A * r_, g = -A * r_;
-        if (select_hit(sel, sel_keys[p], p)) {
-          v += clip_c * fabsf(xc);
-          g += clip_c * ((xc > 0.f) ? 1.f : ((xc < 0.f) ? -1.f : 0.f));
-          a[1] += m;
-        }
-        a[2] += fabsf(xc) * m;
-        a[0] += (v * w) * m * scale;
-        gv[j] = (pass ? g : 0.f) * w * m * scale;
-        continue;
-      }
-      float x;  // exponent before the +-20 clamp
-      if (KIND == 0 || KIND == 6) x = d;
-      else x = (lv[j] - lv[j]) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
-      const bool pass = (x >= -kSafetyBound && x <= kSafetyBound);  // clamp passes grad inclusively
-      const float xc = clampf(x, -kSafetyBound, kSafetyBound);
-      const float r_ = expf(xc);
-      const ValGrad p1{-A * r_, -A * r_};
-      const float rc = clampf(r_, lo, hi);
-      const bool rin = (r_ >= lo && r_ <= hi);
-      const ValGrad p2{-A * rc, rin ? -A * r_ : 0.f};
-      ValGrad c = vg_max(p1, p2);
-      if (KIND == 6) {  // Clip-Cov (loss.py:198-280): the selected tokens drop out of the loss
-        const bool hit = select_hit(sel, sel_keys[p], p);
-        if (hit) c = ValGrad{c.v * 0.f, 0.f};
-        a[1] += hit ? m : 0.f;
-      } else {
-        a[1] += (p2.v > p1.v) ? m : 0.f;
-      }
-      a[2] += (KIND == 1 ? -d : -xc) * m;  // ppo_kl: raw for GSPO (loss.py:173), clamped otherwise (loss.py:77-79)
-      if (KIND == 0) {
-        const float pg3 = -A * clip_c;
-        a[3] += (c.v > pg3 && A < 0.f) ? m : 0.f;
-        if (A < 0.f) {  // torch.min(pg3, c1), pg3 carries no gradient
-          if (pg3 < c.v) c = ValGrad{pg3, 0.f};
-          else if (pg3 == c.v) c = ValGrad{c.v, 0.5f * c.g};
-          else if (!(pg3 > c.v)) c = ValGrad{pg3 + c.v, 0.f};
-        }
-      }
-      a[0] += (c.v * w) * m * scale;
-      gv[j] = (pass ? c.g : 0.f) * w * m * scale;
+      const float m = mv[j];
+      const bool hit = (KIND >= 5) ? select_hit(sel, sel_keys[p], p) : false;
+      const TokenTerm t = policy_token<KIND>(lv[j], ov[j], av[j], wv[j], sbar, lo, hi, clip_c, hit);
+      gv[j] = accumulate_token(t, m, scale, a);
     }
     if (full) store4(grad, i, gv);
     else
@@ -391,7 +284,8 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
   }
   }  // chunk
   if (blockIdx.x == 0 && threadIdx.x == 0) a[5] = 1.f;  // gradient factor unless post-normalised
-  store_block_partials<6>(a, lds_red, partials);
+  grid_finish<6>(a, lds_red, partials,
+                 [&](float (&tot)[kPartialStride]) { write_acc(tot, norm_slots, valid, acc); });
 }
 
 // KL penalty estimators of axon/utils/rl/kl.py:154-245 with PyTorch's gradient conventions.
@@ -508,9 +402,10 @@ __global__ __launch_bounds__(kBlock) void side_terms_kernel(
     const float* __restrict__ entropy, const float* __restrict__ logp, const float* __restrict__ ref,
     const void* __restrict__ mask, const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots,
     int64_t uniform_len, const float* __restrict__ row_scale, float uniform_scale, int kl_type,
-    int kl_plus, float* __restrict__ agg_w, float* __restrict__ grad_kl, float* partials) {
+    int kl_plus, float* __restrict__ agg_w, float* __restrict__ grad_kl, float* partials,
+    int norm_slots, const double* __restrict__ valid, float* __restrict__ acc) {
   __shared__ int32_t lds_cu[kLdsRows];
-  __shared__ float lds_red[6 * (kBlock / kWave)];
+  __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   const bool need_row = (row_scale != nullptr);
   const int64_t n_chunks = (n_slots + kChunk - 1) / kChunk;
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -582,7 +477,8 @@ __global__ __launch_bounds__(kBlock) void side_terms_kernel(
     }
   }
   if (blockIdx.x == 0 && threadIdx.x == 0) a[5] = 1.f;
-  store_block_partials<6>(a, lds_red, partials);
+  grid_finish<6>(a, lds_red, partials,
+                 [&](float (&tot)[kPartialStride]) { write_acc(tot, norm_slots, valid, acc); });
 }
 
 // ---- GMPO (geo_mean_loss_fn, axon/trainer/algos/loss/loss.py:355-408) ------------------------------
@@ -746,8 +642,7 @@ using namespace axon;
 
 extern "C" int64_t axon_reduce_partials_bytes(int64_t n_slots) {
   if (n_slots < 0) return AXON_ERR_ARG;
-  const int64_t blocks = n_slots > 0 ? (int64_t)stream_grid(n_slots) : 1;
-  return blocks * kPartialStride * (int64_t)sizeof(float);
+  return kPartialsBytes;  // rows for the largest grid plus the ticket counter
 }
 
 static int check_rows2(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
@@ -756,6 +651,8 @@ static int check_rows2(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64
   if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
   if (need_row && uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
+  // tokens that belong to no row: the row lookup would read in front of cu_seqlens
+  if (need_row && uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;
   return AXON_OK;
 }
 
@@ -780,23 +677,20 @@ extern "C" int axon_sampler_correction(
     hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_F32>, g, blk, 0, (hipStream_t)stream,
                        oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
                        rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
-                       partials);
+                       partials, acc);
   else
     hipLaunchKernelGGL(sampler_correction_kernel<AXON_MASK_I64>, g, blk, 0, (hipStream_t)stream,
                        oldp, samp, mask, cu, n_rows, n_slots, uniform_len, is_mode, is_thr, rs_mode,
                        rs_lo, rs_hi, has_veto, log_veto, row_cnt, row_sum, row_flag, isw, new_mask,
-                       partials);
-  AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, partials,
-                     (int)g.x, 0, (const int64_t*)nullptr, acc);
+                       partials, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
 
 extern "C" int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_rows,
                                    int64_t row_len, int token_reduce, int batch_reduce,
-                                   const int64_t* prtc, const int64_t* npt, const int64_t* nps,
-                                   const int64_t* valid, float* row_scale, float* row_mean,
+                                   const double* prtc, const double* npt, const double* nps,
+                                   const double* valid, float* row_scale, float* row_mean,
                                    void* stream) {
   if (n_rows < 0) return AXON_ERR_ARG;
   if (n_rows == 0) return AXON_OK;
@@ -820,7 +714,7 @@ static int policy_loss_impl(int kind, const float* logp, const float* oldp, cons
                             const void* mask, int mask_kind, const float* isw, const int32_t* cu,
                             int64_t n_rows, int64_t n_slots, int64_t uniform_len,
                             const float* row_scale, const float* row_mean, float uniform_scale,
-                            int post_normalize, const int64_t* valid, float ratio_lo,
+                            int post_normalize, const double* valid, float ratio_lo,
                             float ratio_hi, float clip_c, float* grad, float* acc, float* partials,
                             void* stream) {
   const bool need_row = (row_scale != nullptr) || (kind == 1);
@@ -838,7 +732,7 @@ static int policy_loss_impl(int kind, const float* logp, const float* oldp, cons
   hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
                      n_rows, n_slots, uniform_len, row_scale, row_mean, uniform_scale, ratio_lo, \
                      ratio_hi, clip_c, (const uint32_t*)nullptr, (const SelectState*)nullptr, grad,  \
-                     partials)
+                     partials, post_normalize ? 1 : 0, valid, acc)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_PL(AXON_MASK_F32, 0);
     else if (kind == 1) AXON_LAUNCH_PL(AXON_MASK_F32, 1);
@@ -854,9 +748,6 @@ static int policy_loss_impl(int kind, const float* logp, const float* oldp, cons
   }
 #undef AXON_LAUNCH_PL
   AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
-                     post_normalize ? 1 : 0, valid, acc);
-  AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
 
@@ -864,7 +755,7 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
                                 const void* mask, int mask_kind, const float* isw,
                                 const int32_t* cu, int64_t n_rows, int64_t n_slots,
                                 int64_t uniform_len, const float* row_scale, const float* row_mean,
-                                float uniform_scale, int post_normalize, const int64_t* valid,
+                                float uniform_scale, int post_normalize, const double* valid,
                                 float ratio_lo, float ratio_hi, float clip_c, float* grad,
                                 float* acc, float* partials, void* stream) {
   return policy_loss_impl(kind, logp, oldp, adv, mask, mask_kind, isw, cu, n_rows, n_slots,
@@ -873,17 +764,16 @@ extern "C" int axon_policy_loss(int kind, const float* logp, const float* oldp, 
 }
 
 // ---- the entry point that allocates nothing ---------------------------------------------------
-// Same kernels as axon_policy_loss; the per-workgroup partial sums go to a fixed array in device
-// memory instead of a caller-provided workspace.  The array is sized for kNoAllocBlocks workgroups
-// of one chunk each (128 KB); every GPU the library runs on holds its own copy until the process
-// ends.  In host code the array's name is only a handle: its device address is looked up once per
-// device (with that device current) and kept, and only that address is handed to kernels.
+// Same kernels as axon_policy_loss; the per-workgroup partial sums and the ticket counter live in a
+// fixed array in device memory instead of a caller-provided workspace (522 KB; every
+// GPU the library runs on holds its own copy until the process ends).  In host code the array's
+// name is only a handle: its device address is looked up once per device (with that device
+// current) and kept, and only that address is handed to kernels.
 namespace {
-constexpr int kNoAllocBlocks = 4096;
-constexpr int64_t kNoAllocMaxSlots = (int64_t)kNoAllocBlocks * kChunk;  // 2^24 tokens
+constexpr int64_t kNoAllocMaxSlots = (int64_t)1 << 24;  // the stated capacity of the entry point
 constexpr int kNoAllocMaxDevices = 64;
 }  // namespace
-static __device__ __align__(256) float scratch[kNoAllocBlocks * kPartialStride];
+static __device__ __align__(256) float scratch[kPartialsBytes / 4];
 static float* g_scratch_addr[kNoAllocMaxDevices];  // per device; null until the first call there
 static std::mutex g_scratch_mutex;
 
@@ -908,14 +798,15 @@ extern "C" int axon_policy_loss_noalloc(int kind, const float* logp, const float
                                         int64_t n_slots, int64_t uniform_len,
                                         const float* row_scale, const float* row_mean,
                                         float uniform_scale, int post_normalize,
-                                        const int64_t* valid, float ratio_lo, float ratio_hi,
+                                        const double* valid, float ratio_lo, float ratio_hi,
                                         float clip_c, float* grad, float* acc, void* stream) {
   if (n_slots > kNoAllocMaxSlots) return AXON_ERR_TOO_LARGE;
   float* partials = nullptr;
   const int rc = scratch_of_current_device(&partials);
   if (rc != AXON_OK) return rc;
   // every workgroup overwrites its whole row of the array and the reduction reads only the rows of
-  // this launch, so nothing left by an earlier call is read and nothing has to be cleared
+  // this launch; the ticket counter starts at zero (static storage) and the kernel's last workgroup
+  // puts it back to zero, so nothing left by an earlier call is read and nothing is cleared here
   return policy_loss_impl(kind, logp, oldp, adv, mask, mask_kind, isw, cu, n_rows, n_slots,
                           uniform_len, row_scale, row_mean, uniform_scale, post_normalize, valid,
                           ratio_lo, ratio_hi, clip_c, grad, acc, partials, stream);
@@ -925,7 +816,7 @@ extern "C" int axon_cov_policy_loss(int kind, const float* logp, const float* ol
                                     const void* mask, int mask_kind, const float* isw,
                                     const int32_t* cu, int64_t n_rows, int64_t n_slots,
                                     int64_t uniform_len, const float* row_scale, float uniform_scale,
-                                    int post_normalize, const int64_t* valid, float ratio_lo,
+                                    int post_normalize, const double* valid, float ratio_lo,
                                     float ratio_hi, float kl_coef, const uint32_t* keys,
                                     const void* state, float* grad, float* acc, float* partials,
                                     void* stream) {
@@ -944,7 +835,8 @@ extern "C" int axon_cov_policy_loss(int kind, const float* logp, const float* ol
 #define AXON_LAUNCH_CV(MK, KD)                                                                    \
   hipLaunchKernelGGL((policy_loss_kernel<MK, KD>), g, blk, 0, st, logp, oldp, adv, mask, isw, cu, \
                      n_rows, n_slots, uniform_len, row_scale, (const float*)nullptr,              \
-                     uniform_scale, ratio_lo, ratio_hi, kl_coef, keys, sel, grad, partials)
+                     uniform_scale, ratio_lo, ratio_hi, kl_coef, keys, sel, grad, partials,           \
+                     post_normalize ? 1 : 0, valid, acc)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_CV(AXON_MASK_F32, 5);
     else AXON_LAUNCH_CV(AXON_MASK_F32, 6);
@@ -953,9 +845,6 @@ extern "C" int axon_cov_policy_loss(int kind, const float* logp, const float* ol
     else AXON_LAUNCH_CV(AXON_MASK_I64, 6);
   }
 #undef AXON_LAUNCH_CV
-  AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
-                     post_normalize ? 1 : 0, valid, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
@@ -998,7 +887,7 @@ extern "C" int axon_kl_reward(const float* scores, const float* old_logp, const 
 extern "C" int axon_side_terms(const float* entropy, const float* logp, const float* ref_logp,
                                const void* mask, int mask_kind, const int32_t* cu, int64_t n_rows,
                                int64_t n_slots, int64_t uniform_len, const float* row_scale,
-                               float uniform_scale, int post_normalize, const int64_t* valid,
+                               float uniform_scale, int post_normalize, const double* valid,
                                int kl_type, int kl_plus, float* agg_w, float* grad_kl, float* acc,
                                float* partials, void* stream) {
   const bool need_row = (row_scale != nullptr);
@@ -1016,14 +905,11 @@ extern "C" int axon_side_terms(const float* entropy, const float* logp, const fl
   if (mask_kind == AXON_MASK_F32)
     hipLaunchKernelGGL(side_terms_kernel<AXON_MASK_F32>, g, blk, 0, st, entropy, logp, ref_logp, mask,
                        cu, n_rows, n_slots, uniform_len, row_scale, uniform_scale, kl_type, kl_plus,
-                       agg_w, grad_kl, partials);
+                       agg_w, grad_kl, partials, post_normalize ? 3 : 0, valid, acc);
   else
     hipLaunchKernelGGL(side_terms_kernel<AXON_MASK_I64>, g, blk, 0, st, entropy, logp, ref_logp, mask,
                        cu, n_rows, n_slots, uniform_len, row_scale, uniform_scale, kl_type, kl_plus,
-                       agg_w, grad_kl, partials);
-  AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x,
-                     post_normalize ? 3 : 0, valid, acc);
+                       agg_w, grad_kl, partials, post_normalize ? 3 : 0, valid, acc);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
@@ -1047,7 +933,7 @@ extern "C" int axon_gmpo_loss(const float* logp, const float* oldp, const float*
   if (mask_kind == AXON_MASK_F32) AXON_LAUNCH_GMPO(AXON_MASK_F32, 0); else AXON_LAUNCH_GMPO(AXON_MASK_I64, 0);
   AXON_CHECK_LAUNCH();
   hipLaunchKernelGGL(reduce_partials_kernel, dim3(1), dim3(1024), 0, st, partials, (int)g.x, 0,
-                     (const int64_t*)nullptr, acc);
+                     (const double*)nullptr, acc);
   AXON_CHECK_LAUNCH();
   hipLaunchKernelGGL(gmpo_rows_kernel, dim3(1), dim3(1024), 0, st, row_vals, n_rows, isw != nullptr,
                      row_coef, acc);

@@ -419,6 +419,7 @@ extern "C" int axon_reverse_scan(int mode, const float* rewards, const float* va
   if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
   if (mode < kScanGae || mode > kScanSuffixSum) return AXON_ERR_ARG;
+  if (uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;  // tokens that belong to no row
   if (n_slots == 0 || n_rows == 0) return AXON_OK;
   if (uniform_len == 0 && !cu_seqlens) return AXON_ERR_ARG;
   if (!rewards || !ret) return AXON_ERR_ARG;

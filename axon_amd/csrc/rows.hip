@@ -235,6 +235,7 @@ static int check_rows(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_
   if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
+  if (uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;  // tokens that belong to no row
   return AXON_OK;
 }
 

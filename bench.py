@@ -161,7 +161,7 @@ def config1_cpu_vs_gpu():
     }
 
 
-def hbm_kernels(n_tokens, dev):
+def hbm_kernels(n_tokens, dev, only=None):
     """Stage-2/3 kernels on a packed batch large enough to show the bandwidth asymptote
     (same lognormal length law as the headline workload).  Each figure is algorithmic bytes
     (one read of every input, one write of every output, fp32) over the median of 20 timed
@@ -188,17 +188,22 @@ def hbm_kernels(n_tokens, dev):
     rows = _ops.rows_of(new, cu)
     seq_scalar = torch.randn(len(lens), device=dev, generator=gd)
 
-    def median_ms(fn, iters=20, warm=5):
+    def median_ms(fn, iters=12, warm=5, inner=8):
+        """Median over `iters` timed regions of `inner` back-to-back calls each, per call: the host enqueues
+        call k + 1 while the GPU runs call k, so the figure is the operator's GPU time (every launch it makes
+        and the gaps between them), not the host's time to issue one eager call to an idle GPU."""
         for _ in range(warm):
             fn()
         ts = []
         for _ in range(iters):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
             a.record()
-            fn()
+            for _ in range(inner):
+                fn()
             b.record()
             b.synchronize()
-            ts.append(a.elapsed_time(b))
+            ts.append(a.elapsed_time(b) / inner)
         return sorted(ts)[len(ts) // 2]
 
     ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
@@ -209,11 +214,11 @@ def hbm_kernels(n_tokens, dev):
         ("device-to-device copy (calibration)", 8, lambda: x.copy_(old)),
         ("policy_loss_kernel: PPO/DAPO loss + gradient, sum/token-mean (one pass)", 20,
          lambda: _ops.policy_loss(0, new, old, adv, mask, None, rows, **ppo)),
-        ("row_stats + policy_loss_kernel: GSPO loss + gradient (two reads of log_probs, old, mask)", 32,
+        ("owned_policy_loss_kernel: GSPO loss + gradient, mean/step-mean (one pass, a workgroup owns whole sequences)", 20,
          lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
         ("sampler_correction_kernel: token IS weights + rejection mask", 20,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=None, **corr)),
-        ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads)", 32,
+        ("owned_correction_kernel: IS + rejection + per-sequence veto (one pass, a workgroup owns whole sequences)", 20,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4), **corr)),
         ("row_stats_kernel: per-sequence count and masked sum", 12, lambda: _ops.row_stats(new, old, mask, rows)),
         ("sampler_diag kernels: all IS / rejection / off-policy / mismatch diagnostics (token pass + row pass)", 12,
@@ -233,6 +238,8 @@ def hbm_kernels(n_tokens, dev):
     ]
     out = []
     for name, bpt, fn in cases:
+        if only is not None and not any(o in name for o in only):
+            continue
         ms = median_ms(fn)
         gbs = n_tokens * bpt / (ms * 1e-3) / 1e9
         out.append({"kernel": name, "bytes_per_token": bpt, "ms": ms, "achieved": gbs, "peak": HBM_PEAK_GBS,
@@ -254,6 +261,8 @@ def hbm_kernels(n_tokens, dev):
             ("logits_stats_kernel: bf16 logits [8192 x 151936] -> log-prob, entropy (one read)", ln * lv * 2,
              lambda: _ops.logits_forward(logits, labels, True)),
             ("logits_grad_kernel: d logits from both gradients (one read, one write)", ln * lv * 4, bwd)):
+        if only is not None and not any(o in name for o in only):
+            continue
         ms = median_ms(fn, iters=10, warm=2)
         gbs = nbytes / (ms * 1e-3) / 1e9
         out.append({"kernel": name, "bytes_per_token": nbytes // ln, "ms": ms, "achieved": gbs, "peak": HBM_PEAK_GBS,

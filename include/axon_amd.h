@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 14
+#define AXON_AMD_ABI_VERSION 16
 
 enum {
   AXON_OK = 0,
@@ -223,13 +223,19 @@ int axon_row_broadcast_mask(const float* row_scalar, const void* mask, int mask_
 
 int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 0 */
 
-/* Bytes of the `partials` workspace of axon_sampler_correction / axon_policy_loss for
- * n_slots tokens (8 floats per workgroup; at most 16384 workgroups walk the tokens).  The scalar sums of those two
- * kernels (the reference's masked_mean metrics and agg_loss totals,
- * axon/utils/torch/ops.py:131-145, axon/trainer/algos/loss/utils.py:224-251) are added
- * from per-workgroup partials in a fixed order by a one-workgroup kernel launched right
- * after, so results are reproducible run to run and no atomics are involved.
- * Contents need no initialisation. */
+/* Bytes of the `partials` workspace of axon_sampler_correction / axon_policy_loss /
+ * axon_side_terms / axon_cov_policy_loss / axon_gmpo_loss (the same for every n_slots: 8 floats for
+ * each of at most 16384 workgroups that walk the tokens, 8 floats for each group of 64 workgroups,
+ * then 2 KB of ticket counters).  The scalar sums of those kernels (the reference's masked_mean
+ * metrics and agg_loss totals, axon/utils/torch/ops.py:131-145,
+ * axon/trainer/algos/loss/utils.py:224-251) are added from per-workgroup partials in a fixed order
+ * inside the same launch (the workgroup that finishes last in a group adds the group, the one that
+ * finishes last of all adds the groups), so results are reproducible run to run and no same-address
+ * float atomics are involved.
+ * The ticket counters (the last 2048 bytes) must be ZERO before the first use; every launch leaves
+ * them zero again, so one zero-filled workspace serves any number of calls that are ordered on a
+ * stream.  Two launches that overlap in time must not share a workspace.  The rows need no
+ * initialisation. */
 int64_t axon_reduce_partials_bytes(int64_t n_slots);
 
 /* Sampler/trainer correction, compute_sampler_correction_and_rejection_mask
@@ -294,14 +300,16 @@ int axon_sampler_diag(const float* old_logp, const float* sampler_logp, const vo
  *   batch_reduce: 0 token-mean, 1 step-mean, 2 program-mean
  *   row_cnt/row_sum from axon_row_stats(logp, old, mask).
  *   per_row_token_count / num_program_tokens / num_program_steps: optional
- *   int64 [n_rows]; valid_count: optional int64 pointer whose element [0] is
+ *   double [n_rows] (counts as floating values, as the reference divides by them,
+ *   utils.py:224-229: a fractional count is not truncated);
+ *   valid_count: optional double pointer whose element [0] is
  *   the mini-batch-wide denominator (utils.py:224-229), else computed locally.
  * Outputs row_scale[n_rows], row_mean[n_rows] (= row_sum / max(row_cnt,1)).
  * Up to 64 workgroups: each repeats the pass over the counts (same order, same totals) and writes its share of the rows. */
 int axon_loss_row_scale(const float* row_cnt, const float* row_sum, int64_t n_rows,
                         int64_t row_len_for_norm, int token_reduce, int batch_reduce,
-                        const int64_t* per_row_token_count, const int64_t* num_program_tokens,
-                        const int64_t* num_program_steps, const int64_t* valid_count,
+                        const double* per_row_token_count, const double* num_program_tokens,
+                        const double* num_program_steps, const double* valid_count,
                         float* row_scale, float* row_mean, void* stream);
 
 /* Clipped policy loss, forward and gradient in one pass.
@@ -334,28 +342,70 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
                      const void* mask, int mask_kind, const float* is_weights,
                      const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
                      int64_t uniform_len, const float* row_scale, const float* row_mean,
-                     float uniform_scale, int post_normalize, const int64_t* valid_count,
+                     float uniform_scale, int post_normalize, const double* valid_count,
                      float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                      float* partials, void* stream);
+
+/* The policy losses that need a per-row quantity, in ONE pass over the tokens: GSPO's sequence mean
+ * log-ratio (axon/trainer/algos/loss/loss.py:141-151) and every aggregation of agg_loss with a per-row
+ * divisor (token_reduce mean / mean-norm / mean-program, batch_reduce step-mean / program-mean,
+ * axon/trainer/algos/loss/utils.py:120-251).  Replaces axon_row_stats + axon_loss_row_scale +
+ * axon_policy_loss for those cases (which read log_probs, old_log_probs and the mask twice): a
+ * workgroup owns whole rows, keeps their tokens in registers between the row sums and the token
+ * pass, and forms the row sums in a fixed order without atomics, so the sequence ratio repeats bit
+ * for bit from run to run.  Rows longer than a workgroup's registers hold (more than 2048 tokens
+ * beyond the workgroup's 2048-token share) are read a second time.
+ *   kind, masks, ratio_lo / ratio_hi / clip_c, grad, acc[0..5]: as in axon_policy_loss (kinds 0-4).
+ *   token_reduce / batch_reduce / per_row_token_count / num_program_tokens / num_program_steps /
+ *   valid_count: as in axon_loss_row_scale.  Without valid_count the batch denominator (sum of the
+ *   mask for token-mean, number of rows with a mask token for step-mean) is known only at the end:
+ *   acc[0] is divided by it, grad[] is left WITHOUT that division and acc[5] returns the factor the
+ *   caller multiplies the gradient by; with valid_count acc[5] = 1.
+ *   Slots that belong to no row (before cu_seqlens[0], after cu_seqlens[n_rows]) receive grad 0.
+ * partials: workspace of axon_reduce_partials_bytes, ticket counters zero (see there). */
+int axon_policy_loss_rows(int kind, const float* logp, const float* old_logp, const float* adv,
+                          const void* mask, int mask_kind, const float* is_weights,
+                          const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
+                          int64_t uniform_len, int token_reduce, int batch_reduce,
+                          const double* per_row_token_count, const double* num_program_tokens,
+                          const double* num_program_steps, const double* valid_count, float ratio_lo,
+                          float ratio_hi, float clip_c, float* grad, float* acc, float* partials,
+                          void* stream);
+
+/* axon_sampler_correction for the modes that need a per-row quantity (the per-sequence veto,
+ * sampler.py:413-428; sequence-level weights :210-214; sequence / geometric rejection :70-79), in ONE
+ * pass over the tokens, same scheme as axon_policy_loss_rows: 20 bytes per token instead of 32, and
+ * row sums formed in a fixed order, so a row whose sum sits next to a rejection bound takes the same
+ * side on every run.  Arguments as axon_sampler_correction without the row inputs; row_cnt /
+ * row_sum / row_flag (each may be NULL) receive the per-row sum of the mask, of (old - sampler) *
+ * mask and the veto decision.  acc as in axon_sampler_correction. */
+int axon_sampler_correction_rows(const float* old_logp, const float* sampler_logp, const void* mask,
+                                 int mask_kind, const int32_t* cu_seqlens, int64_t n_rows,
+                                 int64_t n_slots, int64_t uniform_len, int is_mode, float is_threshold,
+                                 int rs_mode, float rs_lr_lo, float rs_lr_hi, int has_veto,
+                                 float log_veto, float* is_weights, float* new_mask, float* row_cnt,
+                                 float* row_sum, int32_t* row_flag, float* acc, float* partials,
+                                 void* stream);
 
 /* axon_policy_loss for callers that cannot allocate.  No counterpart in the reference: it is
  * for code under HIP graph capture, tight serving loops and harnesses that forbid
  * hipMalloc, which cannot obtain the `partials` workspace.  Arguments, outputs and results
  * are those of axon_policy_loss (same kernels) without `partials`: the per-workgroup partial
- * sums go to a fixed 128 KB array in device memory that the library holds on every GPU it
+ * sums and the ticket counters go to a fixed 522 KB array in device memory that the library holds on every GPU it
  * runs on until the process ends.  Calls no hipMalloc / hipFree and no allocating routine.
- *   n_slots <= 16 777 216 (2^24 tokens: one 4096-token chunk for each of the array's 4096
- *   rows); larger inputs return AXON_ERR_TOO_LARGE and launch nothing.
+ *   n_slots <= 16 777 216 (2^24 tokens, the capacity this entry point states and is tested
+ *   for); larger inputs return AXON_ERR_TOO_LARGE and launch nothing.
  * The first call on a device looks the array's address up (hipGetSymbolAddress, with that
  * device current) and must therefore happen outside stream capture; later calls on that
  * device only launch.  All calls on one GPU share the array: calls that overlap in time on
  * one GPU (different streams) race on it; calls ordered on one stream, or by events, do not.
- * Nothing in the array has to start at zero, so nothing is cleared between calls. */
+ * The array's ticket counter starts at zero (static storage) and every launch leaves it zero, the
+ * partial sums are overwritten before they are read: nothing is cleared between calls. */
 int axon_policy_loss_noalloc(int kind, const float* logp, const float* old_logp, const float* adv,
                              const void* mask, int mask_kind, const float* is_weights,
                              const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
                              int64_t uniform_len, const float* row_scale, const float* row_mean,
-                             float uniform_scale, int post_normalize, const int64_t* valid_count,
+                             float uniform_scale, int post_normalize, const double* valid_count,
                              float ratio_lo, float ratio_hi, float clip_c, float* grad, float* acc,
                              void* stream);
 
@@ -467,7 +517,7 @@ int axon_cov_policy_loss(int kind, const float* logp, const float* old_logp, con
                          const void* mask, int mask_kind, const float* is_weights,
                          const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
                          int64_t uniform_len, const float* row_scale, float uniform_scale,
-                         int post_normalize, const int64_t* valid_count, float ratio_lo,
+                         int post_normalize, const double* valid_count, float ratio_lo,
                          float ratio_hi, float kl_coef, const uint32_t* keys, const void* state,
                          float* grad, float* acc, float* partials, void* stream);
 
@@ -490,7 +540,7 @@ int axon_kl_penalty(const float* logp, const float* ref_logp, int64_t n, int kl_
 int axon_side_terms(const float* entropy, const float* logp, const float* ref_logp, const void* mask,
                     int mask_kind, const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots,
                     int64_t uniform_len, const float* row_scale, float uniform_scale,
-                    int post_normalize, const int64_t* valid_count, int kl_type, int kl_plus,
+                    int post_normalize, const double* valid_count, int kl_type, int kl_plus,
                     float* agg_w, float* grad_kl, float* acc, float* partials, void* stream);
 
 /* GMPO, geo_mean_loss_fn (axon/trainer/algos/loss/loss.py:355-408): the sequence-level loss

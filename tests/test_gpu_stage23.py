@@ -888,3 +888,103 @@ def test_loss_and_correction_in_a_hip_graph():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(g_acc[:6], e_acc[:6]) and torch.equal(g_grad, e_grad) and torch.equal(g_cacc[:6], e_cacc[:6])
+
+
+# ---- kernels in which a workgroup owns whole rows (GSPO, per-row aggregation, veto, sequence level) --------
+def _awkward_packed(lens, seed):
+    """Packed inputs over rows of the given lengths (zeros allowed), padded twins for the oracle."""
+    g = torch.Generator().manual_seed(seed)
+    n = sum(lens)
+    old = -torch.empty(n).exponential_(1.0, generator=g)
+    d = {"lengths": lens, "cu_seqlens": W.cu_from_lengths(lens), "old_log_probs": old,
+         "log_probs": old + 0.3 * torch.randn(n, generator=g), "advantages": torch.randn(n, generator=g),
+         "sampler_log_probs": old + 0.2 * torch.randn(n, generator=g),
+         "response_mask": (torch.rand(n, generator=g) < 0.8).float()}
+    tmax = max(max(lens), 1)
+    pad = {}
+    for k in ("old_log_probs", "log_probs", "advantages", "sampler_log_probs", "response_mask"):
+        pad[k] = torch.zeros(len(lens), tmax)
+        for b, (a, e) in enumerate(zip(d["cu_seqlens"][:-1].tolist(), d["cu_seqlens"][1:].tolist())):
+            pad[k][b, : e - a] = d[k][a:e]
+    return d, pad
+
+
+AWKWARD = {
+    # rows longer than the 4096 tokens a workgroup keeps in registers, next to short ones
+    "long_rows": [5000, 17, 8192, 1, 3, 4097, 2048, 2047, 2049, 6000, 31],
+    # more than 128 rows begin inside one 2048-token range; empty rows in between, first and last
+    "tiny_rows": [0, 0] + [1, 0, 2, 3, 0, 5] * 60 + [700, 0, 0],
+    # a single row, a row that ends exactly on range borders
+    "borders": [2048, 2048, 4096, 1, 2047, 2048],
+}
+
+
+@pytest.mark.parametrize("layout", sorted(AWKWARD))
+def test_row_owned_losses_on_awkward_layouts(layout):
+    lens = AWKWARD[layout]
+    d, pad = _awkward_packed(lens, seed=len(lens))
+    meta = {"cu_seqlens": d["cu_seqlens"]}
+    for name, fn, cfg in (("gspo", OL.gspo_loss, {"clip_ratio_low": 3e-4, "clip_ratio_high": 4e-4,
+                                                   "token_reduce": "mean", "batch_reduce": "step-mean"}),
+                          ("gspo", OL.gspo_loss, {"clip_ratio_low": 0.1, "clip_ratio_high": 0.1,
+                                                   "token_reduce": "sum", "batch_reduce": "token-mean"}),
+                          ("ppo", OL.ppo_loss, {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28,
+                                                "token_reduce": "mean", "batch_reduce": "token-mean"})):
+        first = _check_loss(name, fn, d, cfg, meta=meta, pad=pad)
+        again = _check_loss(name, fn, d, cfg, meta=meta, pad=pad)
+        assert first.item() == again.item()  # fixed summation order: bit-identical from run to run
+
+
+@pytest.mark.parametrize("layout", sorted(AWKWARD))
+@pytest.mark.parametrize("is_l,rs_l", [("token", "token"), ("sequence", "sequence"), ("sequence", "geometric")])
+def test_row_owned_correction_on_awkward_layouts(layout, is_l, rs_l):
+    lens = AWKWARD[layout]
+    d, pad = _awkward_packed(lens, seed=100 + len(lens))
+    kw = dict(sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l, sampler_rs_threshold=2.0,
+              sampler_token_veto_threshold=0.4)
+    outs = []
+    for _ in range(2):
+        proto, new, m = S.compute_sampler_correction_and_rejection_mask(
+            d["old_log_probs"].to(DEV), d["sampler_log_probs"].to(DEV), d["response_mask"].to(DEV),
+            cu_seqlens=d["cu_seqlens"].to(DEV), **kw)
+        outs.append((proto.batch["sampler_is_weights"].clone(), new.clone(), m))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])  # run to run
+    w_ref, new_ref, m_ref = OS.correction(pad["old_log_probs"], pad["sampler_log_probs"], pad["response_mask"], **kw)
+    got_new, got_w = outs[0][1].cpu(), outs[0][0].cpu()
+    assert torch.equal(got_new, pad_to_packed(new_ref, lens))
+    assert torch.allclose(got_w, pad_to_packed(w_ref, lens), rtol=1e-5, atol=1e-7)
+    for k, v in m_ref.items():
+        assert outs[0][2]["sampler_corr/" + k] == pytest.approx(v, rel=1e-4, abs=1e-6), k
+
+
+def test_fractional_valid_count_is_not_truncated():
+    """A count averaged over ranks may be fractional; the reference divides by the value as it is
+    (loss/utils.py:224-229)."""
+    d = _c1_with_adv(5)
+    b = d["old_log_probs"].shape[0]
+    _check_loss("ppo", OL.ppo_loss, d, {"token_reduce": "sum", "batch_reduce": "token-mean"},
+                extra={"valid_token_count": torch.full((b,), 1234.5)})
+    _check_loss("gspo", OL.gspo_loss, d, {"token_reduce": "mean", "batch_reduce": "step-mean"},
+                extra={"valid_batch_size": torch.full((b,), 77.25)})
+
+
+def test_packed_layout_without_rows_is_refused():
+    """cu_seqlens with a single entry (no row) next to a non-empty token array: every kernel that resolves the
+    row of a token returns the shape error instead of reading cu_seqlens[-1]."""
+    from axon_amd import _lib
+    lib = _lib.load()
+    t = torch.zeros(64, device=DEV)
+    cu = torch.zeros(1, dtype=torch.int32, device=DEV)
+    ws = torch.zeros(lib.axon_reduce_partials_bytes(64) // 4, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda x: x.data_ptr()  # noqa: E731
+    assert lib.axon_row_stats(p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 0, 0.0, p(t), p(t), None, st) == -2
+    assert lib.axon_row_broadcast_mask(p(t), p(t), 0, p(cu), 0, 64, 0, 0.0, p(t), st) == -2
+    assert lib.axon_policy_loss(1, p(t), p(t), p(t), p(t), 0, None, p(cu), 0, 64, 0, p(t), p(t), 1.0, 0, None, 0.8,
+                                1.2, 3.0, p(t), p(t), p(ws), st) == -2
+    assert lib.axon_policy_loss_rows(1, p(t), p(t), p(t), p(t), 0, None, p(cu), 0, 64, 0, 1, 1, None, None, None,
+                                     None, 0.8, 1.2, 3.0, p(t), p(t), p(ws), st) == -2
+    assert lib.axon_sampler_correction_rows(p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 1, 2.0, 1, -0.7, 0.7, 1, -9.0,
+                                            p(t), p(t), None, None, None, p(t), p(ws), st) == -2
+    assert lib.axon_reverse_scan(0, p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 1.0, 1.0, None, p(t), p(t), st) == -2
+    torch.cuda.synchronize()

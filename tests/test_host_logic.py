@@ -46,7 +46,7 @@ def test_workspace_queries_and_argument_errors_without_gpu():
     assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None) == -1
     assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0, None, 0.8, 1.2,
                                 3.0, None, None, None, None) == -1
-    assert lib.axon_reduce_partials_bytes(4097) == 2 * 8 * 4 and lib.axon_reduce_partials_bytes(1 << 30) == 16384 * 32 and lib.axon_reduce_partials_bytes(-1) == -1
+    assert lib.axon_reduce_partials_bytes(4097) == lib.axon_reduce_partials_bytes(1 << 30) == 16384 * 32 + 256 * 32 + 2048 and lib.axon_reduce_partials_bytes(-1) == -1
     assert lib.axon_fill_zero(None, 3, None) == -1
 
 

@@ -28,7 +28,7 @@ def _call(fn_name, kind, rl, *, row_scale, row_mean, post_normalize, with_partia
             1.0, post_normalize, None, 0.8, 1.28, 3.0, grad.data_ptr(), acc.data_ptr()]
     keep = None
     if with_partials:
-        keep = torch.empty(max(lib.axon_reduce_partials_bytes(n) // 4, 8), device=dev)
+        keep = torch.zeros(lib.axon_reduce_partials_bytes(n) // 4, device=dev)  # the ticket counter starts at zero
         args.append(keep.data_ptr())
     args.append(torch.cuda.current_stream().cuda_stream)
     rc = getattr(lib, fn_name)(*args)
