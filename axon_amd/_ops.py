@@ -228,13 +228,21 @@ def group_scalar(mode, scores, lens, members, offsets, n_groups, *, eps=1e-6, no
     return out
 
 
+# Operators that need a per-row quantity run as ONE launch in which a workgroup owns whole rows up to this many
+# tokens (any real micro-batch: one launch instead of three or four, and row sums that repeat bit for bit).  That
+# kernel holds 16 tokens per thread across its two phases and runs at about a third of the streaming rate, so
+# beyond this size the token-parallel row pass + token pass is faster (measured crossover: 3-4 M tokens).
+OWNED_ROWS_MAX_SLOTS = 1 << 21
+
 IS_MODES = {None: 0, "token": 1, "sequence": 2}
 RS_MODES = {None: 0, "token": 1, "sequence": 2, "geometric": 3}
 
 
 def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_threshold, rs_mode, rs_lr_lo, rs_lr_hi,
                        log_veto):
-    """One row-stats pass (when a row-level quantity is needed) + one elementwise pass.
+    """Importance weights and rejection / veto mask.  Without a row-level quantity: one elementwise pass.  With
+    one (veto, sequence or geometric level): one launch in which a workgroup owns whole rows, or, beyond
+    ``OWNED_ROWS_MAX_SLOTS`` tokens, a row-stats pass followed by an elementwise pass.
 
     Returns (is_weights | None, new_mask fp32, acc[8] device tensor).
     """
@@ -249,7 +257,8 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
     isw = torch.empty(rows.shape, device=dev, dtype=torch.float32) if is_mode else None
     new_mask = torch.empty(rows.shape, device=dev, dtype=torch.float32)
     acc = _acc8(rows.n_slots, dev)
-    if need_row:  # a workgroup owns whole rows: one pass over the tokens, row sums in a fixed order
+    if need_row and rows.n_slots <= OWNED_ROWS_MAX_SLOTS:
+        # a workgroup owns whole rows: one launch, one pass over the tokens, row sums in a fixed order
         check(
             lib.axon_sampler_correction_rows(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows,
                                              rows.n_slots, rows.uniform_len, is_mode, float(is_threshold), rs_mode,
@@ -259,10 +268,15 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
             "axon_sampler_correction_rows",
         )
         return isw, new_mask, acc
+    cnt = ssum = flag = None
+    if need_row:  # very large batches: a token-parallel row pass, then a token-parallel elementwise pass
+        cnt, ssum, flag = row_stats(old_lp, samp_lp, mk, rows, flag_mode=1 if has_veto else 0,
+                                    threshold=log_veto if has_veto else 0.0)
     check(
         lib.axon_sampler_correction(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows, rows.n_slots,
                                     rows.uniform_len, is_mode, float(is_threshold), rs_mode, float(rs_lr_lo),
-                                    float(rs_lr_hi), 0, 0.0, None, None, None, ptr(isw), ptr(new_mask), ptr(acc),
+                                    float(rs_lr_hi), int(has_veto), float(log_veto if has_veto else 0.0), ptr(cnt),
+                                    ptr(ssum), ptr(flag), ptr(isw), ptr(new_mask), ptr(acc),
                                     ptr(_partials(rows.n_slots, dev)), stream_ptr()),
         "axon_sampler_correction",
     )
@@ -335,12 +349,13 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     # PPO with sum / token-mean needs no per-row quantity: one pass over the tokens, the
     # division by the token count happens when the last workgroup has the total.
     one_pass = kind != 1 and tr == 0 and br == 0
-    if not one_pass:  # a workgroup owns whole rows: still one pass over the tokens
-        if tr == 2 and not rows.uniform_len:
-            raise ValueError("token_reduce='mean-norm' divides by the padded row length: needs a [batch, seq] layout")
-        prtc = _count_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
-        npt = _count_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
-        nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
+    prtc = _count_dev(per_row_token_count, dev, rows.n_rows, "per_row_token_count") if tr == 1 else None
+    npt = _count_dev(num_program_tokens, dev, rows.n_rows, "num_program_tokens") if tr == 3 else None
+    nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
+    if not one_pass and tr == 2 and not rows.uniform_len:
+        raise ValueError("token_reduce='mean-norm' divides by the padded row length: needs a [batch, seq] layout")
+    if not one_pass and rows.n_slots <= OWNED_ROWS_MAX_SLOTS:
+        # a workgroup owns whole rows: one launch, still one pass over the tokens
         check(
             lib.axon_policy_loss_rows(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr,
                                       rows.n_rows, rows.n_slots, rows.uniform_len, tr, br, ptr(prtc), ptr(npt),
@@ -349,11 +364,22 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
             "axon_policy_loss_rows",
         )
         return acc, grad
+    row_scale = row_mean = None
+    if not one_pass:  # very large batches: row pass, row scales, token pass
+        cnt, ssum, _ = row_stats(lp, old, mk, rows, want_sum=(kind == 1))
+        row_scale = torch.empty(rows.n_rows, device=dev, dtype=torch.float32)
+        row_mean = torch.empty(rows.n_rows, device=dev, dtype=torch.float32) if kind == 1 else None
+        check(
+            lib.axon_loss_row_scale(ptr(cnt), ptr(ssum), rows.n_rows, rows.uniform_len if rows.uniform_len else 0, tr,
+                                    br, ptr(prtc), ptr(npt), ptr(nps), ptr(valid), ptr(row_scale), ptr(row_mean),
+                                    stream_ptr()),
+            "axon_loss_row_scale",
+        )
     check(
         lib.axon_policy_loss(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr, rows.n_rows,
-                             rows.n_slots, rows.uniform_len, None, None, 1.0, 1, ptr(valid), float(ratio_lo),
-                             float(ratio_hi), float(clip_c), ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)),
-                             stream_ptr()),
+                             rows.n_slots, rows.uniform_len, ptr(row_scale), ptr(row_mean), 1.0, int(one_pass),
+                             ptr(valid if one_pass else None), float(ratio_lo), float(ratio_hi), float(clip_c),
+                             ptr(grad), ptr(acc), ptr(_partials(rows.n_slots, dev)), stream_ptr()),
         "axon_policy_loss",
     )
     return acc, grad

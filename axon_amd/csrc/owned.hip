@@ -26,6 +26,7 @@ constexpr int kOwnIter = 4;                           // 16-byte vectors per thr
 constexpr int kOwnTokens = kBlock * kVec * kOwnIter;  // tokens a workgroup holds in registers: 4096
 constexpr int kOwnRows = 128;                         // rows whose sums fit the LDS tables at a time
 constexpr int kOwnWaves = kBlock / kWave;
+constexpr int kOwnBatch = 64;                         // ranges whose row boundaries are looked up together
 
 struct RowStarts {
   const int32_t* cu;
@@ -51,15 +52,15 @@ struct RowStarts {
 struct Segment {
   const int32_t* win;  // LDS: win[i] = first slot of row rs + i, i in [0, n]
   int n;
-  __device__ __forceinline__ int row_of(int64_t p) const {  // largest i < n with win[i] <= p
+  __device__ __forceinline__ int row_of(int p) const {  // largest i < n with win[i] <= p
     int a = 0, b = n - 1;
     while (a < b) {
       const int mid = (a + b + 1) >> 1;
-      if ((int64_t)win[mid] <= p) a = mid; else b = mid - 1;
+      if (win[mid] <= p) a = mid; else b = mid - 1;
     }
     return a;
   }
-  __device__ __forceinline__ int64_t end_of(int i) const { return win[i + 1]; }
+  __device__ __forceinline__ int end_of(int i) const { return win[i + 1]; }
 };
 
 // Segmented sum across the wavefront (rows sorted across lanes, -1 = no token); `flush(seg)` is
@@ -90,7 +91,7 @@ __device__ __forceinline__ void row_seg_wave_reduce(RowSeg<NV> s, Flush&& flush)
 }
 
 // What the two kernels share: the walk over ranges, segments and blocks.  `Op` provides
-//   load(p0, lanes_ok[4], it)      one vector of four slots starting at p0 into register set `it`
+//   load(p0, it)                   one vector of four slots starting at p0 into register set `it`
 //   stat(it, j, RowSeg&)           add slot j of register set `it` to the row sums
 //   rows(seg_first_row, i, tot[])  derive the per-row values of local row i from its sums (one thread)
 //   emit(p0, it, ...)              write the outputs of one vector
@@ -100,12 +101,29 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
   constexpr int NV = Op::kNV;
   __shared__ int32_t win[kOwnRows + 1];
   __shared__ float part[kOwnWaves][kOwnRows][NV];
+  __shared__ int32_t bnd[kOwnBatch][2];
   const int wave = threadIdx.x / kWave;
   const int64_t n_ranges = (rs_.n_slots + kOwnStride - 1) / kOwnStride;
+  // this workgroup's ranges: blockIdx.x, blockIdx.x + gridDim.x, ...
+  const int64_t n_mine = (int64_t)blockIdx.x < n_ranges ? (n_ranges - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
 #pragma unroll 1
-  for (int64_t b = blockIdx.x; b < n_ranges; b += gridDim.x) {
-    const int64_t r0 = (b == 0) ? 0 : rs_.first_row_from(b * kOwnStride);
-    const int64_t r1 = (b == n_ranges - 1) ? rs_.n_rows : rs_.first_row_from((b + 1) * kOwnStride);
+  for (int64_t k0 = 0; k0 < n_mine; k0 += kOwnBatch) {
+  // The first and last row of up to kOwnBatch ranges, found by as many threads at once: a bisection
+  // over cu_seqlens is a chain of dependent loads, far too long to sit in front of every range.
+  const int n_batch = (int)min((int64_t)kOwnBatch, n_mine - k0);
+  __syncthreads();
+  if ((int)threadIdx.x < 2 * n_batch) {
+    const int64_t b = blockIdx.x + (k0 + (threadIdx.x >> 1)) * gridDim.x;
+    int64_t r;
+    if ((threadIdx.x & 1) == 0) r = (b == 0) ? 0 : rs_.first_row_from(b * kOwnStride);
+    else r = (b == n_ranges - 1) ? rs_.n_rows : rs_.first_row_from((b + 1) * kOwnStride);
+    bnd[threadIdx.x >> 1][threadIdx.x & 1] = (int32_t)r;
+  }
+  __syncthreads();
+#pragma unroll 1
+  for (int kb = 0; kb < n_batch; ++kb) {
+    const int64_t b = blockIdx.x + (k0 + kb) * gridDim.x;
+    const int64_t r0 = bnd[kb][0], r1 = bnd[kb][1];
 #pragma unroll 1
     for (int64_t rs = r0; rs < r1; rs += kOwnRows) {
       const int n = (int)min((int64_t)kOwnRows, r1 - rs);
@@ -114,21 +132,21 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
       for (int i = threadIdx.x; i < kOwnWaves * kOwnRows * NV; i += kBlock) (&part[0][0][0])[i] = 0.f;
       __syncthreads();
       const Segment seg{win, n};
-      const int64_t t0 = win[0], t1 = win[n];
-      const int64_t base = t0 & ~(int64_t)3;  // vectors stay 16-byte aligned; slots before t0 are not ours
-      const int n_blocks = (int)((t1 - base + kOwnTokens - 1) / kOwnTokens);
+      const int t0 = win[0], t1 = win[n];
+      const int base = t0 & ~3;  // vectors stay 16-byte aligned; slots before t0 are not ours
+      const int n_blocks = (t1 - base + kOwnTokens - 1) / kOwnTokens;
       // ---- pass 1: row sums.  The registers keep the last block that was loaded.
 #pragma unroll 1
       for (int blk = 0; blk < n_blocks; ++blk) {
-        const int64_t b0 = base + (int64_t)blk * kOwnTokens;
+        const int b0 = base + blk * kOwnTokens;
 #pragma unroll
         for (int it = 0; it < kOwnIter; ++it) {
-          const int64_t p0 = b0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
           if (p0 < t1 && p0 + kVec > t0) op.load(p0, it);
         }
 #pragma unroll
         for (int it = 0; it < kOwnIter; ++it) {
-          const int64_t p0 = b0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
           RowSeg<NV> s;
           s.row = -1;
 #pragma unroll
@@ -138,10 +156,10 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
             for (int k = 0; k < NV; ++k) part[wave][f.row][k] += f.v[k];
           };
           if (p0 < t1 && p0 + kVec > t0) {
-            int64_t rend = -1;
+            int rend = -1;
 #pragma unroll
             for (int j = 0; j < kVec; ++j) {
-              const int64_t p = p0 + j;
+              const int p = p0 + j;
               if (p < t0 || p >= t1) continue;
               if (p >= rend) {
                 if (s.row >= 0) flush(s);
@@ -168,22 +186,24 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
       // ---- pass 2: outputs, last block first (its inputs are still in the registers)
 #pragma unroll 1
       for (int blk = n_blocks - 1; blk >= 0; --blk) {
-        const int64_t b0 = base + (int64_t)blk * kOwnTokens;
+        const int b0 = base + blk * kOwnTokens;
         if (blk != n_blocks - 1) {
 #pragma unroll
           for (int it = 0; it < kOwnIter; ++it) {
-            const int64_t p0 = b0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+            const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
             if (p0 < t1 && p0 + kVec > t0) op.load(p0, it);
           }
         }
+#ifdef AXON_EXP_LATE
 #pragma unroll
         for (int it = 0; it < kOwnIter; ++it) {
-          const int64_t p0 = b0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
           if (p0 < t1 && p0 + kVec > t0) op.load_late(p0, it);
         }
+#endif
 #pragma unroll
         for (int it = 0; it < kOwnIter; ++it) {
-          const int64_t p0 = b0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
           if (p0 < t1 && p0 + kVec > t0) op.emit(p0, it, seg, t0, t1);
         }
       }
@@ -192,6 +212,7 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
     // sequence: the first and the last range write zeros there
     if (b == 0) op.fill_gap(0, rs_.at(0));
     if (b == n_ranges - 1) op.fill_gap(rs_.at(rs_.n_rows), rs_.n_slots);
+  }
   }
 }
 
@@ -244,12 +265,16 @@ struct OwnedLossOp {
   __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float (*rowv_)[2], float bd)
       : g(g_), rs(rs_), rowv(rowv_), bden(bd) {}
 
-  __device__ __forceinline__ void load(int64_t p0, int it) {
+  __device__ __forceinline__ void load(int p0, int it) {
     load4_guard(g.logp, p0, rs.n_slots, lv[it]);
     load4_guard(g.oldp, p0, rs.n_slots, ov[it]);
     load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[it]);
+#ifndef AXON_EXP_LATE
+    load_late(p0, it);
+#endif
   }
-  __device__ __forceinline__ void load_late(int64_t p0, int it) {  // read by the output pass only
+  // read by the output pass only
+  __device__ __forceinline__ void load_late(int p0, int it) {
     load4_guard(g.adv, p0, rs.n_slots, av[it]);
     if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[it]);
     else wv[it][0] = wv[it][1] = wv[it][2] = wv[it][3] = 1.f;
@@ -272,13 +297,13 @@ struct OwnedLossOp {
     rowv[i][1] = tot[1] / fmaxf(c, 1.f);
     rows_with_tokens += (c > 0.f) ? 1.f : 0.f;
   }
-  __device__ __forceinline__ void emit(int64_t p0, int it, const Segment& seg, int64_t t0, int64_t t1) {
+  __device__ __forceinline__ void emit(int p0, int it, const Segment& seg, int t0, int t1) {
     float gv[4];
-    int64_t rend = -1;
+    int rend = -1;
     float scale = 0.f, sbar = 0.f;
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
-      const int64_t p = p0 + j;
+      const int p = p0 + j;
       gv[j] = 0.f;
       if (p < t0 || p >= t1) continue;
       if (p >= rend) {
@@ -348,12 +373,12 @@ struct OwnedCorrOp {
   __device__ __forceinline__ OwnedCorrOp(const OwnedCorrArgs& g_, const RowStarts& rs_, CorrRow* rowv_)
       : g(g_), rs(rs_), rowv(rowv_) {}
 
-  __device__ __forceinline__ void load(int64_t p0, int it) {
+  __device__ __forceinline__ void load(int p0, int it) {
     load4_guard(g.oldp, p0, rs.n_slots, ov[it]);
     load4_guard(g.samp, p0, rs.n_slots, sv[it]);
     load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[it]);
   }
-  __device__ __forceinline__ void load_late(int64_t, int) {}
+  __device__ __forceinline__ void load_late(int, int) {}
   __device__ __forceinline__ void stat(int it, int j, RowSeg<3>& s) const {
     const float m = mv[it][j];
     const float d = ov[it][j] - sv[it][j];
@@ -369,13 +394,13 @@ struct OwnedCorrOp {
     if (g.row_sum) g.row_sum[r] = tot[1];
     if (g.row_flag) g.row_flag[r] = vetoed ? 1 : 0;
   }
-  __device__ __forceinline__ void emit(int64_t p0, int it, const Segment& seg, int64_t t0, int64_t t1) {
+  __device__ __forceinline__ void emit(int p0, int it, const Segment& seg, int t0, int t1) {
     float wv[4], nm[4];
-    int64_t rend = -1;
+    int rend = -1;
     CorrRow row{0.f, 1.f, 1.f};
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
-      const int64_t p = p0 + j;
+      const int p = p0 + j;
       wv[j] = 0.f;
       nm[j] = 0.f;
       if (p < t0 || p >= t1) continue;

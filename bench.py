@@ -206,6 +206,13 @@ def hbm_kernels(n_tokens, dev, only=None):
             ts.append(a.elapsed_time(b) / inner)
         return sorted(ts)[len(ts) // 2]
 
+    def forced_owned(fn):
+        keep, _ops.OWNED_ROWS_MAX_SLOTS = _ops.OWNED_ROWS_MAX_SLOTS, 1 << 40
+        try:
+            return fn()
+        finally:
+            _ops.OWNED_ROWS_MAX_SLOTS = keep
+
     ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
     gspo = dict(token_reduce="mean", batch_reduce="step-mean", ratio_lo=1 - 3e-4, ratio_hi=1 + 4e-4, clip_c=3.0)
     corr = dict(is_mode=1, is_threshold=2.0, rs_mode=1, rs_lr_lo=-math.log(2.0), rs_lr_hi=math.log(2.0))
@@ -214,12 +221,20 @@ def hbm_kernels(n_tokens, dev, only=None):
         ("device-to-device copy (calibration)", 8, lambda: x.copy_(old)),
         ("policy_loss_kernel: PPO/DAPO loss + gradient, sum/token-mean (one pass)", 20,
          lambda: _ops.policy_loss(0, new, old, adv, mask, None, rows, **ppo)),
-        ("owned_policy_loss_kernel: GSPO loss + gradient, mean/step-mean (one pass, a workgroup owns whole sequences)", 20,
-         lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
+        ("row_stats + policy_loss_kernel: GSPO loss + gradient (two reads of log_probs, old, mask; the path taken "
+         "beyond 2^21 tokens)", 32, lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
+        ("owned_policy_loss_kernel: GSPO loss + gradient in one launch and one read, a workgroup owns whole "
+         "sequences (the path taken up to 2^21 tokens, forced here)", 20,
+         lambda: forced_owned(lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo))),
         ("sampler_correction_kernel: token IS weights + rejection mask", 20,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=None, **corr)),
-        ("owned_correction_kernel: IS + rejection + per-sequence veto (one pass, a workgroup owns whole sequences)", 20,
+        ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads; the path taken "
+         "beyond 2^21 tokens)", 32,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4), **corr)),
+        ("owned_correction_kernel: IS + rejection + per-sequence veto in one launch and one read (the path taken up "
+         "to 2^21 tokens, forced here)", 20,
+         lambda: forced_owned(lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4),
+                                                              **corr))),
         ("row_stats_kernel: per-sequence count and masked sum", 12, lambda: _ops.row_stats(new, old, mask, rows)),
         ("sampler_diag kernels: all IS / rejection / off-policy / mismatch diagnostics (token pass + row pass)", 12,
          lambda: _ops.sampler_diag(old, samp, mask, rows, is_mode=1, is_lo=0.5, is_hi=2.0, rs_mode=1, rs_lo=0.5,
@@ -305,6 +320,13 @@ def baseline_sizes_cold(dev):
     new, old, mask = (stack(c1[k], sets) for k in ("log_probs", "old_log_probs", "response_mask"))
     adv = stack(torch.randn(c1["log_probs"].shape, generator=torch.Generator().manual_seed(5)), sets) * mask
     rows = _ops.rows_of(new[0])
+    def forced_owned(fn):
+        keep, _ops.OWNED_ROWS_MAX_SLOTS = _ops.OWNED_ROWS_MAX_SLOTS, 1 << 40
+        try:
+            return fn()
+        finally:
+            _ops.OWNED_ROWS_MAX_SLOTS = keep
+
     ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
     f = lambda k: _ops.policy_loss(0, new[k], old[k], adv[k], mask[k], None, rows, **ppo)
     n_slots = rows.n_slots

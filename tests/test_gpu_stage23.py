@@ -243,10 +243,19 @@ def test_ppo_config1_vs_oracle(mask_dtype):
                 {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"})
 
 
+@pytest.fixture(params=["one_launch", "two_pass"])
+def row_path(request):
+    """Operators with a per-row quantity have two implementations, chosen by batch size: run the test on both."""
+    keep = _ops.OWNED_ROWS_MAX_SLOTS
+    _ops.OWNED_ROWS_MAX_SLOTS = keep if request.param == "one_launch" else 0
+    yield request.param
+    _ops.OWNED_ROWS_MAX_SLOTS = keep
+
+
 @pytest.mark.parametrize("tr,br", [("sum", "token-mean"), ("mean", "step-mean"), ("sum", "step-mean"),
                                    ("mean-norm", "step-mean"), ("mean", "token-mean")])
 @pytest.mark.parametrize("name,fn", [("ppo", OL.ppo_loss), ("gspo", OL.gspo_loss)])
-def test_losses_all_reductions_with_is_weights(name, fn, tr, br):
+def test_losses_all_reductions_with_is_weights(name, fn, tr, br, row_path):
     d = _c1_with_adv(2)
     d["log_probs"] = d["old_log_probs"] + 0.3 * torch.randn(d["old_log_probs"].shape)  # exercise every clip region
     d["advantages"] = d["advantages"] + 0.0
@@ -259,7 +268,7 @@ def test_losses_all_reductions_with_is_weights(name, fn, tr, br):
     _check_loss(name, fn, d, cfg, extra={"sampler_is_weights": isw})
 
 
-def test_losses_with_global_counts_and_program_modes():
+def test_losses_with_global_counts_and_program_modes(row_path):
     d = _c1_with_adv(3)
     b = d["old_log_probs"].shape[0]
     agg = {"valid_token_count": torch.full((b,), 70000), "per_row_token_count": d["response_mask"].sum(-1).long() + 3}
@@ -309,7 +318,7 @@ def test_ppo_clip_regions_table_gpu():
 
 
 @pytest.mark.parametrize("n_tokens", [20000, 65536])  # 65536 is the full size of the configuration
-def test_gspo_packed_config4_vs_oracle(n_tokens):
+def test_gspo_packed_config4_vs_oracle(n_tokens, row_path):
     d = W.c4_correction(n_tokens=n_tokens)
     s = len(d["lengths"])
     gidx = T(np.unique(d["uid"], return_inverse=True)[1])
@@ -342,7 +351,7 @@ def _pad_case(seed=4, b=32, t=700):
 @pytest.mark.parametrize("is_l,rs_l", [("token", "token"), ("sequence", "sequence"), ("token", "geometric"),
                                        (None, "token"), ("token", None), (None, None)])
 @pytest.mark.parametrize("mask_dtype", [torch.float32, torch.int64])
-def test_sampler_correction_vs_oracle(is_l, rs_l, mask_dtype):
+def test_sampler_correction_vs_oracle(is_l, rs_l, mask_dtype, row_path):
     old, samp, mask = _pad_case()
     kw = dict(sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l, sampler_rs_threshold=2.0,
               sampler_token_veto_threshold=1e-4)
