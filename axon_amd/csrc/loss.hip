@@ -204,10 +204,14 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
   const int64_t c0 = chunk * kChunk;
   const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
   RowFinder rf;
-  if (need_row) {
-    __syncthreads();  // the previous chunk's row window is no longer read
-    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
-  }
+  // the row search of a chunk is a chain of dependent loads: where a whole chunk is streamed it runs
+  // after the chunk's first loads have been issued, under their latency
+  auto find_rows = [&]() {
+    if (need_row) {
+      __syncthreads();  // the previous chunk's row window is no longer read
+      rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+    }
+  };
   // the per-token arithmetic on one vector of four slots
   auto process = [&](int64_t i, bool full, const float (&lv)[4], const float (&ov)[4], const float (&av)[4],
                      const float (&mv)[4], const float (&wv)[4]) {
@@ -251,12 +255,14 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
         if (isw) load4(isw, i, wv[it]);
         else wv[it][0] = wv[it][1] = wv[it][2] = wv[it][3] = 1.f;
       }
+      if (b0 == 0) find_rows();
 #pragma unroll
       for (int it = 0; it < kB; ++it)
         process(c0 + ((int64_t)(b0 + it) * kBlock + threadIdx.x) * kVec, true, lv[it], ov[it], av[it], mv[it],
                 wv[it]);
     }
   } else {
+    find_rows();
 #pragma unroll 1
     for (int it = 0; it < kIter; ++it) {
       const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;

@@ -63,27 +63,26 @@ __global__ __launch_bounds__(kBlock) void row_stats_kernel(
   const int64_t c0 = (int64_t)blockIdx.x * kChunk;
   const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
   RowFinder rf;
+  const bool whole = (c1 - c0 == kChunk);
+  // whole chunk: every load is issued before the first use (twelve 16-byte requests in flight per
+  // thread), and before the row search, whose chain of dependent loads then runs under them
+  float av_[kIter][4], bv_[kIter][4], mv_[kIter][4];
+  if (whole) {
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      load4(a, i, av_[it]);
+      if (b != nullptr) load4(b, i, bv_[it]);
+      else bv_[it][0] = bv_[it][1] = bv_[it][2] = bv_[it][3] = 0.f;
+      load_mask4<MK>(mask, i, mv_[it]);
+    }
+  }
   rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
 
-#pragma unroll 1
-  for (int it = 0; it < kIter; ++it) {
-    const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+  // the slots of one vector of four -> the wavefront's segmented sums
+  auto fold = [&](int64_t i, const float (&av)[4], const float (&bv)[4], const float (&mv)[4]) {
     Seg s{-1, 0.f, 0.f, 0};
     if (i < c1) {
-      float av[4], bv[4] = {0.f, 0.f, 0.f, 0.f}, mv[4];
-      const bool full = (i + kVec <= n_slots);
-      if (full) {
-        load4(a, i, av);
-        if (b != nullptr) load4(b, i, bv);
-        load_mask4<MK>(mask, i, mv);
-      } else {
-        for (int j = 0; j < 4; ++j) {
-          const bool ok = i + j < n_slots;
-          av[j] = ok ? a[i + j] : 0.f;
-          bv[j] = (ok && b != nullptr) ? b[i + j] : 0.f;
-          mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
-        }
-      }
       int r = rf.row(i);
       int64_t rend = rf.row_end(r);
       s.row = r;
@@ -108,6 +107,33 @@ __global__ __launch_bounds__(kBlock) void row_stats_kernel(
       }
     }
     seg_wave_reduce_flush(s, cnt, sum, flag);
+  };
+  if (whole) {
+#pragma unroll
+    for (int it = 0; it < kIter; ++it)
+      fold(c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec, av_[it], bv_[it], mv_[it]);
+    return;
+  }
+#pragma unroll 1
+  for (int it = 0; it < kIter; ++it) {
+    const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+    float av[4] = {0.f, 0.f, 0.f, 0.f}, bv[4] = {0.f, 0.f, 0.f, 0.f}, mv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (i < c1) {
+      const bool full = (i + kVec <= n_slots);
+      if (full) {
+        load4(a, i, av);
+        if (b != nullptr) load4(b, i, bv);
+        load_mask4<MK>(mask, i, mv);
+      } else {
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = i + j < n_slots;
+          av[j] = ok ? a[i + j] : 0.f;
+          bv[j] = (ok && b != nullptr) ? b[i + j] : 0.f;
+          mv[j] = ok ? load_mask1<MK>(mask, i + j) : 0.f;
+        }
+      }
+    }
+    fold(i, av, bv, mv);
   }
 }
 
@@ -174,6 +200,35 @@ __global__ __launch_bounds__(kBlock) void row_broadcast_kernel(
   const int64_t c0 = (int64_t)blockIdx.x * kChunk;
   const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
   RowFinder rf;
+  if (c1 - c0 == kChunk) {
+    // whole chunk: the mask loads of all four steps are in flight before the row search
+    float mv[kIter][4];
+#pragma unroll
+    for (int it = 0; it < kIter; ++it)
+      load_mask4<MK>(mask, c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec, mv[it]);
+    rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
+#pragma unroll
+    for (int it = 0; it < kIter; ++it) {
+      const int64_t i = c0 + ((int64_t)it * kBlock + threadIdx.x) * kVec;
+      int r = rf.row(i);
+      int64_t rend = rf.row_end(r);
+      float sc = row_scalar[r];
+      float o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (i + j >= rend) {
+          r = rf.row(i + j);
+          rend = rf.row_end(r);
+          sc = row_scalar[r];
+        }
+        float v = sc * mv[it][j];
+        if (clamp_abs > 0.f) v = fminf(fmaxf(v, -clamp_abs), clamp_abs);
+        o[j] = v;
+      }
+      store4(out, i, o);
+    }
+    return;
+  }
   rf.init(cu, n_rows, uniform_len, c0, c1, lds_cu);
 #pragma unroll 1
   for (int it = 0; it < kIter; ++it) {
