@@ -48,6 +48,10 @@ def parse_args():
                          "masked as prompt; 0 disables it")
     ap.add_argument("--hbm-tokens", type=int, default=1 << 26,
                     help="token count for the HBM-bound stage-2/3 kernels' bandwidth figures; 0 disables them")
+    ap.add_argument("--no-calibrate", dest="calibrate", action="store_false",
+                    help="skip the plain-GEMM calibration (torch.matmul and the bare main loop on the dominant shape)")
+    ap.add_argument("--no-other-workloads", dest="other_workloads", action="store_false",
+                    help="skip the short runs of the other head shapes (Qwen2.5-0.5B, GPT-OSS)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run a 1 GiB calibration copy, one head forward and one head backward, then exit: the "
                          "command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken on")
@@ -90,6 +94,7 @@ def cpu_baseline(hid, w, lab, budget_s, check=None):
         "sample": f"{n} of the workload's tokens, full hidden and vocab, fwd+loss+bwd, {t:.1f} s; linear in tokens",
     }
     out["config1"] = config1_cpu_vs_gpu()
+    out["config4"] = config4_cpu_vs_gpu()
     if check is not None:
         idx, got = check
         ref_lp, _ = OM.forward(hid[idx - 1], w, lab[idx])
@@ -159,6 +164,181 @@ def config1_cpu_vs_gpu():
         "loss_rel_err": abs(l_gpu.item() - l_cpu.item()) / abs(l_cpu.item()),
         "grad_rel_l2": ((g_gpu - g_cpu.double()).norm() / g_cpu.double().norm()).item(),
     }
+
+
+def config4_cpu_vs_gpu():
+    """The correction + GSPO configuration at its full size (65536 packed tokens, ragged sequences; token-level
+    importance weights capped at 2, token rejection outside [0.5, 2], per-sequence veto at 1e-4, then the GSPO
+    loss with clip 3e-4 / 4e-4, mean / step-mean, and its gradient): the CPU port on the padded layout the
+    reference uses beside the GPU path on the packed layout, same inputs, with the errors between the two."""
+    import numpy as np
+    import torch
+
+    from axon_amd import workloads as W
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    from axon_amd.utils.rl import sampler as S
+    from oracle import advantage as OA
+    from oracle import loss as OL
+    from oracle import sampler as OS
+
+    d = W.c4_correction()
+    lens, cu = d["lengths"], d["cu_seqlens"]
+    s_, tmax = len(lens), max(lens)
+    pad = {}
+    for k in ("log_probs", "old_log_probs", "sampler_log_probs", "response_mask", "token_level_rewards"):
+        pad[k] = torch.zeros(s_, tmax)
+        for b, (a, e) in enumerate(zip(cu[:-1].tolist(), cu[1:].tolist())):
+            pad[k][b, : e - a] = d[k][a:e]
+    gidx = torch.as_tensor(np.unique(d["uid"], return_inverse=True)[1])
+    adv_pad = OA.grpo_advantage(pad["token_level_rewards"], pad["response_mask"], gidx, 1e-6, True)
+    unpad = lambda x: torch.cat([x[b, :l] for b, l in enumerate(lens)])  # noqa: E731
+    corr = dict(sampler_is="token", sampler_is_threshold=2.0, sampler_rs="token", sampler_rs_threshold=2.0,
+                sampler_token_veto_threshold=1e-4)
+    gspo = {"clip_ratio_low": 3e-4, "clip_ratio_high": 4e-4, "token_reduce": "mean", "batch_reduce": "step-mean"}
+
+    def cpu():
+        w, new_mask, _ = OS.correction(pad["old_log_probs"], pad["sampler_log_probs"], pad["response_mask"], **corr)
+        lp = pad["log_probs"].clone().requires_grad_(True)
+        loss, _ = OL.gspo_loss(lp, pad["old_log_probs"], adv_pad, new_mask, sampler_is_weights=w, **gspo)
+        loss.backward()
+        return loss.detach(), unpad(lp.grad), unpad(new_mask), unpad(w)
+
+    dev = "cuda:0"
+    g_in = {k: d[k].to(dev) for k in ("log_probs", "old_log_probs", "sampler_log_probs", "response_mask")}
+    g_in["advantages"] = unpad(adv_pad).to(dev)
+    cu_d = cu.to(dev)
+
+    def gpu():
+        proto, new_mask, _ = S.compute_sampler_correction_and_rejection_mask(
+            g_in["old_log_probs"], g_in["sampler_log_probs"], g_in["response_mask"], cu_seqlens=cu_d, **corr)
+        lp = g_in["log_probs"].detach().requires_grad_(True)
+        w = proto.batch["sampler_is_weights"]
+        data = DataProto.from_dict(tensors={"log_probs": lp, "old_log_probs": g_in["old_log_probs"],
+                                            "advantages": g_in["advantages"], "response_mask": new_mask,
+                                            "sampler_is_weights": w}, meta_info={"cu_seqlens": cu_d})
+        loss, _ = compute_loss_fn(data, "gspo", gspo)
+        loss.backward()
+        return loss.detach(), lp.grad, new_mask, w
+
+    def timed(fn, reps, sync):
+        fn()
+        if sync:
+            torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            r = fn()
+        if sync:
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps, r
+
+    t_cpu, (l_cpu, g_cpu, m_cpu, w_cpu) = timed(cpu, 10, False)
+    t_gpu, (l_gpu, g_gpu, m_gpu, w_gpu) = timed(gpu, 50, True)
+    g_gpu = g_gpu.cpu().double()
+    return {
+        "workload": "65536 packed tokens: token IS (cap 2) + token rejection [0.5, 2] + veto 1e-4, then GSPO "
+                    "(3e-4 / 4e-4, mean / step-mean) + gradient",
+        "cpu_ms": 1e3 * t_cpu, "cpu_cores": torch.get_num_threads(), "gpu_ms": 1e3 * t_gpu,
+        "sequences": s_, "cpu_layout": f"padded {s_} x {tmax}", "gpu_layout": "packed",
+        "masks_equal": bool(torch.equal(m_gpu.cpu(), m_cpu)),
+        "weights_max_abs_err": (w_gpu.cpu() - w_cpu).abs().max().item(),
+        "loss_rel_err": abs(l_gpu.item() - l_cpu.item()) / abs(l_cpu.item()),
+        "grad_rel_l2": ((g_gpu - g_cpu.double()).norm() / g_cpu.double().norm()).item(),
+    }
+
+
+def gemm_calibration(dev, n, h, chunk=32768):
+    """What a plain bf16 GEMM of the dominant kernel's shape sustains on THIS box, next to the main loop of the
+    fused kernels on the same operands: `torch.matmul` (hipBLASLt) and `axon_gemm_nt_bf16`, dHidden shape
+    [n, chunk] x [chunk, h], random operands, median of 5 regions of 8 calls."""
+    import torch
+
+    from axon_amd import _ops
+
+    g = torch.Generator(device=dev).manual_seed(77)
+    a = torch.randn(h, chunk, device=dev, generator=g).bfloat16()  # [m][k], K-contiguous
+    b = torch.randn(n, chunk, device=dev, generator=g).bfloat16()  # [n][k]
+    out = torch.empty(n, h, device=dev, dtype=torch.bfloat16)
+    flops = 2.0 * n * h * chunk
+
+    def tflops(fn):
+        for _ in range(3):
+            fn()
+        ts = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for _ in range(8):
+                fn()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1) / 8)
+        return flops / (sorted(ts)[2] * 1e-3) / 1e12
+
+    res = {"shape": f"[{n} x {chunk}] x [{chunk} x {h}] bf16, fp32 accumulate",
+           "hipblaslt_matmul_tflops": tflops(lambda: torch.matmul(b, a.t(), out=out)),
+           "axon_gemm_nt_tflops": tflops(lambda: _ops.gemm_nt(a, b))}
+    del a, b, out
+    return res
+
+
+def head_step_summary(workload, dev, steps=3, warmup=1):
+    """One of the other head shapes through the same step as the headline (head forward with roll and shift
+    inside, GRPO advantage, PPO loss, backward to dHidden and dWeight): tokens/s and TFLOP/s per kernel class."""
+    import torch
+
+    from axon_amd import _ops, workloads as W
+    from axon_amd.protocol import DataProto
+    from axon_amd.trainer.algos.advantages import compute_advantage
+    from axon_amd.trainer.algos.loss import compute_loss_fn
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs
+
+    n, h, v, group, seed = WORKLOADS[workload]
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed)
+    rl = W.packed_rl_inputs(n, seed + 100, group=group)
+    hd, wd, ld = hid.to(dev), w.to(dev), lab.to(dev)
+    cu, mask, tlr, uid = rl["cu_seqlens"].to(dev), rl["response_mask"].to(dev), rl["token_level_rewards"].to(dev), rl["uid"]
+    with torch.no_grad():
+        old = packed_logprobs(hd, wd, ld, cu)[0] - 0.05 * torch.randn(n, device=dev)
+    loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
+
+    def step():
+        hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
+        lp_tok, _ = packed_logprobs(hg, wg, ld, cu)
+        a_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
+                                   meta_info={"cu_seqlens": cu})
+        a_in.non_tensor_batch["uid"] = uid
+        adv = compute_advantage(a_in, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}).batch["advantages"]
+        data = DataProto.from_dict(tensors={"log_probs": lp_tok, "old_log_probs": old, "advantages": adv,
+                                            "response_mask": mask}, meta_info={"cu_seqlens": cu})
+        loss, _ = compute_loss_fn(data, "ppo", loss_args)
+        loss.backward()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = _ops.Timer()
+    _ops.set_timing(timer)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    el = time.perf_counter() - t0
+    _ops.set_timing(None)
+    t = timer.collect()
+    timer.close()
+    assert torch.isfinite(loss).item()
+    nhv = float(n) * h * v
+    ms = lambda *keys: sum(t.get(k, {"ms": 0})["ms"] for k in keys) / steps  # noqa: E731
+    tf = lambda fl, m: fl / (m * 1e-3) / 1e12 if m > 0 else None  # noqa: E731
+    return {"workload": workload, "tokens": n, "hidden": h, "vocab": v, "steps": steps,
+            "ms_per_step": 1e3 * el / steps, "tokens_per_s": n * steps / el,
+            "fwd_tflops": tf(2 * nhv, ms("fwd/logits_stats")),
+            "dhidden_dweight_tflops": tf(4 * nhv, ms("bwd/dhidden", "bwd/dweight")),
+            "dlogit_executed_tflops": tf(2 * nhv, ms("bwd/dlogit")),
+            "path_algorithmic_tflops": 6 * nhv / (1e-3 * 1e3 * el / steps) / 1e12}
 
 
 def hbm_kernels(n_tokens, dev, only=None):
@@ -320,13 +500,6 @@ def baseline_sizes_cold(dev):
     new, old, mask = (stack(c1[k], sets) for k in ("log_probs", "old_log_probs", "response_mask"))
     adv = stack(torch.randn(c1["log_probs"].shape, generator=torch.Generator().manual_seed(5)), sets) * mask
     rows = _ops.rows_of(new[0])
-    def forced_owned(fn):
-        keep, _ops.OWNED_ROWS_MAX_SLOTS = _ops.OWNED_ROWS_MAX_SLOTS, 1 << 40
-        try:
-            return fn()
-        finally:
-            _ops.OWNED_ROWS_MAX_SLOTS = keep
-
     ppo = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
     f = lambda k: _ops.policy_loss(0, new[k], old[k], adv[k], mask[k], None, rows, **ppo)
     n_slots = rows.n_slots
@@ -357,10 +530,33 @@ def baseline_sizes_cold(dev):
     return out
 
 
-# HBM-side bytes of ONE launch of the dominant kernel at the default workload, from rocprofv3 --pmc passes
-# over `bench.py --traffic-probe` (FETCH_SIZE scaled by 2.0 and WRITE_SIZE by 1.0, the factors a 1 GiB
-# device copy in the same run calibrates): 12.35e9 read + 0.45e9 written, default vocabulary chunk.
-TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 12.80e9}
+def kernel_source_digest():
+    """Digest of the sources of the LM-head kernels: ties a committed profile to the code it was taken on."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("gemm_nt.h", "lmhead.hip", "common.h"):
+        with open(os.path.join(ROOT, "axon_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def traffic_from_profile(workload):
+    """HBM-side bytes of ONE launch of the dominant kernel, read from the committed summary of the two
+    rocprofv3 --pmc passes over `bench.py --traffic-probe` (profiles/lmhead_<workload>_hbm_traffic.md carries
+    the line `traffic_bytes_per_launch: <bytes> kernel_source_digest: <digest>`).  None when there is no such
+    file or when the kernels have changed since (the digest of their sources differs)."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", f"lmhead_{workload}_hbm_traffic.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)\s+kernel_source_digest:\s*([0-9a-f]+)", text)
+    if not m or m.group(2) != kernel_source_digest():
+        return None
+    return float(m.group(1))
 
 
 def traffic_probe(workload):
@@ -509,10 +705,12 @@ def main():
         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": (dom["algorithmic_tflops"] or dom["executed_tflops"]) / MFMA_BF16_PEAK_TFLOPS,
         "avg_launch_ms": dom["avg_launch_ms"],
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if not args.tokens and not args.vocab_chunk and "gemm_store" in dom["kernel"] else None,
+        "traffic": traffic_from_profile(args.workload) if not args.tokens and not args.vocab_chunk and "gemm_store" in dom["kernel"] else None,
         "kernels": kernels,
         "path_algorithmic_tflops": 6 * nhv / (ms_per_step * 1e-3) / 1e12,
         "path_frac_of_peak": 6 * nhv / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+        # the backward recomputes the logits: 8 N H V are executed for the 6 that count
+        "path_executed_tflops": 8 * nhv / (ms_per_step * 1e-3) / 1e12,
         "other_phases_ms_per_step": {k: t["ms"] / args.steps for k, t in timing.items()
                                      if k in ("fwd/merge", "fwd/label", "bwd/transpose")},
     }
@@ -527,10 +725,24 @@ def main():
                    "vocab_chunk": args.vocab_chunk or "default"},
         "roofline": roofline,
     }
+    if args.calibrate:
+        cal = gemm_calibration(dev, n, h)
+        roofline["calibration_tflops"] = cal
+        best = max(cal["hipblaslt_matmul_tflops"], cal["axon_gemm_nt_tflops"])
+        roofline["ceiling"] = (
+            f"a backward that recomputes the logits executes 8 N H V flop for 6 algorithmic: the path cannot exceed "
+            f"0.75 x what the GEMMs sustain; with the plain GEMM of this run ({best:.0f} TFLOP/s on random operands, "
+            f"{best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak: the part runs at its power limit under matrix "
+            f"load) that is {0.75 * best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak")
     if prompt_variant:
         out["prompt_rows_variant"] = prompt_variant
-    if args.hbm_tokens > 0:
+    if args.other_workloads and not args.tokens:
         del hd, wd, dh, dw
+        hd = wd = dh = dw = None
+        torch.cuda.empty_cache()
+        out["other_workloads"] = [head_step_summary(name, dev) for name in sorted(WORKLOADS) if name != args.workload]
+    if args.hbm_tokens > 0:
+        hd = wd = dh = dw = None
         torch.cuda.empty_cache()
         out["hbm_kernels"] = hbm_kernels(args.hbm_tokens, dev)
         out["hbm_kernels"]["baseline_sizes"] = baseline_sizes_cold(dev)

@@ -203,3 +203,34 @@ def test_logits_oracle_closed_forms():
     assert torch.allclose(M.entropy_from_logits(x.float()).double(), -(p * p.log()).sum(-1), atol=1e-6)
     assert torch.allclose(M.logprobs_from_logits(x.float(), lab).double(), p.log()[torch.arange(4), lab], atol=1e-6)
     assert torch.allclose(M.entropy_from_logits(x.float() + 3.0), M.entropy_from_logits(x.float()), atol=1e-5)
+
+
+# ---- the bf16 torch path timed as the CPU baseline (fused_linear.py run in bf16) -----------------------------
+def test_bf16_torch_path_against_the_fp32_oracle():
+    """`forward_bf16_torch_path` / `backward_bf16_torch_path` are what `bench.py` times on the host cores.  The
+    same formulas evaluated in fp32 are `forward` / `backward`; run in bf16 the results agree to bf16 accuracy:
+    logits rounded to 8 bits (relative 2^-9) move a log-prob by a few hundredths, gradients by a few per cent.
+    In fp32 the two pairs of functions coincide to rounding, which pins the formulas themselves."""
+    g = torch.Generator().manual_seed(4)
+    n, h, v = 700, 64, 900  # more than one 512-token chunk
+    hid = torch.randn(n, h, generator=g)
+    w = torch.randn(v, h, generator=g) * 0.2
+    lab = torch.randint(0, v, (n,), generator=g)
+    dlogp = torch.randn(n, generator=g) / n
+    # fp32 inputs: the bf16-path functions are the same arithmetic as the oracle
+    lp32, ent32 = M.forward_bf16_torch_path(hid, w, lab, 0.7)
+    ref_lp, ref_ent = M.forward(hid, w, lab, 0.7)
+    assert torch.allclose(lp32, ref_lp, atol=1e-5) and torch.allclose(ent32, ref_ent, atol=1e-5)
+    dh32, dw32 = M.backward_bf16_torch_path(dlogp, hid, w, lab, 0.7)
+    ref_dh, ref_dw = M.backward(dlogp, None, hid, w, lab, 0.7, round_dlogits_bf16=False)
+    rel = lambda a, b: ((a.double() - b.double()).norm() / b.double().norm()).item()  # noqa: E731
+    assert rel(dh32, ref_dh) < 1e-5 and rel(dw32, ref_dw) < 1e-5
+    # bf16 inputs: bf16 accuracy
+    hb, wb = hid.bfloat16(), w.bfloat16()
+    lpb, entb = M.forward_bf16_torch_path(hb, wb, lab, 0.7)
+    ref_lp, ref_ent = M.forward(hb, wb, lab, 0.7)
+    assert lpb.dtype == torch.bfloat16 and (lpb.float() - ref_lp).abs().max() < 0.1
+    assert (entb.float() - ref_ent).abs().max() < 0.1
+    dhb, dwb = M.backward_bf16_torch_path(dlogp, hb, wb, lab, 0.7)
+    ref_dh, ref_dw = M.backward(dlogp, None, hb, wb, lab, 0.7)
+    assert dhb.dtype == torch.bfloat16 and rel(dhb, ref_dh) < 5e-2 and rel(dwb, ref_dw) < 5e-2
