@@ -191,10 +191,10 @@ __device__ __forceinline__ void grid_finish(float (&v)[NV], float* lds /* [8 * 4
   if (threadIdx.x == 0) fin(t);
 }
 
-#ifndef AXON_EXP_GRIDCAP
-#define AXON_EXP_GRIDCAP 6144
-#endif
-constexpr int kStreamGridCap = AXON_EXP_GRIDCAP;
+// Workgroups of a streaming launch: beyond this many chunks a workgroup walks several (every
+// workgroup publishes a row of partial sums and takes a ticket when it ends, which costs more than
+// the walk; 6144 measured best between 1024 and 16384 at 2^26 tokens).
+constexpr int kStreamGridCap = 6144;
 inline unsigned stream_grid(int64_t n_slots) {
   const int64_t chunks = (n_slots + kChunk - 1) / kChunk;
   return (unsigned)(chunks < kStreamGridCap ? chunks : kStreamGridCap);

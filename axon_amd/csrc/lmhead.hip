@@ -17,7 +17,6 @@
 
 namespace axon {
 
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -356,14 +355,6 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   int tm, tn;
   tile_coords(tiles_m, tiles_n, tm, tn);
   const TilePos t = Loop::place(g, tm, tn);  // t.m0 is relative to the chunk
-#ifdef AXON_EXP_STAGGER_NS
-  if (blockIdx.x < 256) {
-    const int xcd = blockIdx.x & 7;
-    const uint64_t t0 = wall_clock64();
-    const uint64_t wait = (uint64_t)xcd * (AXON_EXP_STAGGER_NS) / 10;
-    while (wall_clock64() - t0 < wait) __builtin_amdgcn_s_sleep(32);
-  }
-#endif
   AccTile acc;
   Loop::run(g, t, acc, smem);
   __syncthreads();  // every wave is past its last main-loop LDS access
@@ -380,7 +371,6 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   const int n_base = t.n0 + lp.wn * kWaveTile;
   // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
   // destinations by running pointers (no 64-bit multiplies in the loop).
-#ifndef AXON_EXP_SKIP_DL
   {
     const int unit = l32;
     char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
@@ -392,18 +382,12 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
       for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-#ifdef AXON_EXP_NT
-        __builtin_nontemporal_store((u32x2){v[u].x, v[u].y}, reinterpret_cast<u32x2*>(d));
-#else
         *reinterpret_cast<uint2*>(d) = v[u];
-#endif
         d += dstep;
       }
     }
   }
-#endif
   // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
-#ifndef AXON_EXP_SKIP_DLT
   {
     const int nq = l32;  // token quad
     const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
@@ -424,15 +408,10 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
       o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
       o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
 #pragma unroll
-#ifdef AXON_EXP_NT
-      for (int e = 0; e < 4; ++e) __builtin_nontemporal_store((u32x2){o[e].x, o[e].y}, reinterpret_cast<u32x2*>(d + e * rstep));
-#else
       for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
-#endif
       d += 8 * rstep;
     }
   }
-#endif
 }
 
 template <class Loop>
