@@ -14,16 +14,14 @@ Public names and semantics follow axon/utils/rl/sampler.py:
   veto: a row with any masked token whose lr < log(threshold) is zeroed
   new mask = response_mask * rs * veto
 
-Two launches: a ragged row-statistics pass (only when a row-level quantity is
-needed) and one elementwise pass.  The rejection test runs in log space against
-fp32 interval ends computed here on the host, so the 0/1 masks do not depend on
-the last bit of the device's ``exp``.
+One elementwise launch, or, when a row-level quantity is needed (veto, sequence or geometric level),
+one launch in which a workgroup owns whole rows (beyond 2^21 tokens: a row pass, then an elementwise
+pass).  The rejection test runs in log space against fp32 interval ends computed here on the host, so
+the 0/1 masks do not depend on the last bit of the device's ``exp``.
 
-Metrics: the subset that falls out of the same pass (``sampler_is_mean``,
-``sampler_rs_masked_fraction``, ``sampler_is_veto_fraction``,
-``sampler_is_catastrophic_token_fraction``, ``sampler_is_batch_norm_factor``),
-all prefixed ``sampler_corr/``; the reference's remaining diagnostics are not
-produced.
+Metrics: every ``sampler_corr/*`` key of the reference (importance-weight and rejection statistics,
+veto and catastrophic-token fractions, the batch-normalisation factor) from one diagnostics launch
+and ONE readback for everything.
 """
 
 from __future__ import annotations
@@ -217,26 +215,34 @@ def compute_sampler_correction_and_rejection_mask(
 
     An all-zero ``response_mask`` is a no-op: ``(None, response_mask, {})``.
     """
-    _check_shapes(old_log_prob, sampler_log_prob, response_mask)
     use_is = sampler_is is not None and sampler_is_threshold is not None
-    if use_is:
-        _check_is(sampler_is, sampler_is_threshold)
     rs_lo = rs_hi = 0.0
-    if sampler_rs is not None:
-        if sampler_rs_threshold is None:
-            raise ValueError(
-                "sampler_rs_threshold must be explicitly provided when sampler_rs is enabled. "
-                "Set sampler_rs_threshold to the desired threshold value."
-            )
-        _check_rs(sampler_rs, sampler_rs_threshold)
-        upper = sampler_rs_threshold
-        lower = sampler_rs_threshold_lower if sampler_rs_threshold_lower is not None else 1.0 / upper
-        rs_lo, rs_hi = log_interval_for_ratio_bounds(lower, upper)
     log_veto = None
-    if sampler_token_veto_threshold is not None:
-        if sampler_token_veto_threshold <= 0:
-            raise ValueError(f"sampler_token_veto_threshold must be positive, got {sampler_token_veto_threshold}.")
-        log_veto = _log32(sampler_token_veto_threshold)
+    try:
+        _check_shapes(old_log_prob, sampler_log_prob, response_mask)
+        if use_is:
+            _check_is(sampler_is, sampler_is_threshold)
+        if sampler_rs is not None:
+            if sampler_rs_threshold is None:
+                raise ValueError(
+                    "sampler_rs_threshold must be explicitly provided when sampler_rs is enabled. "
+                    "Set sampler_rs_threshold to the desired threshold value."
+                )
+            _check_rs(sampler_rs, sampler_rs_threshold)
+            upper = sampler_rs_threshold
+            lower = sampler_rs_threshold_lower if sampler_rs_threshold_lower is not None else 1.0 / upper
+            rs_lo, rs_hi = log_interval_for_ratio_bounds(lower, upper)
+        if sampler_token_veto_threshold is not None:
+            if sampler_token_veto_threshold <= 0:
+                raise ValueError(f"sampler_token_veto_threshold must be positive, got {sampler_token_veto_threshold}.")
+            log_veto = _log32(sampler_token_veto_threshold)
+    except ValueError:
+        # The reference returns the no-op for an all-padding micro-batch before it validates anything
+        # (sampler.py:368-370): a bad argument only raises when there is a token to correct.  The valid path keeps
+        # its single readback; this one costs an extra one.
+        if not bool(response_mask.any()):
+            return None, response_mask, {}
+        raise
 
     _ops.require_device(old_log_prob, "compute_sampler_correction_and_rejection_mask")
     rows = _ops.rows_of(old_log_prob, cu_seqlens)

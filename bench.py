@@ -52,6 +52,10 @@ def parse_args():
                     help="skip the plain-GEMM calibration (torch.matmul and the bare main loop on the dominant shape)")
     ap.add_argument("--no-other-workloads", dest="other_workloads", action="store_false",
                     help="skip the short runs of the other head shapes (Qwen2.5-0.5B, GPT-OSS)")
+    ap.add_argument("--gemm-probe", choices=("hipblaslt", "axon"),
+                    help="run three plain bf16 GEMMs of the dominant kernel's shape through torch.matmul or through "
+                         "the fused kernels' main loop (axon_gemm_nt_bf16), then exit: the command the rocprofv3 --pmc "
+                         "passes that compare the two are taken on")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run a 1 GiB calibration copy, one head forward and one head backward, then exit: the "
                          "command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken on")
@@ -576,10 +580,29 @@ def traffic_probe(workload):
     torch.cuda.synchronize()
 
 
+def gemm_probe(which, workload):
+    import torch
+
+    from axon_amd import _ops
+
+    n, h, _, _, _ = WORKLOADS[workload]
+    chunk = 32768
+    g = torch.Generator(device="cuda").manual_seed(0)
+    a = torch.randn(h, chunk, device="cuda", generator=g).bfloat16()
+    b = torch.randn(n, chunk, device="cuda", generator=g).bfloat16()
+    for _ in range(3):
+        c = torch.matmul(b, a.t()) if which == "hipblaslt" else _ops.gemm_nt(a, b)
+    torch.cuda.synchronize()
+    del c
+
+
 def main():
     args = parse_args()
     if args.traffic_probe:
         traffic_probe(args.workload)
+        return
+    if args.gemm_probe:
+        gemm_probe(args.gemm_probe, args.workload)
         return
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (--gpus 1); multi-GPU runs are not part of it",

@@ -997,3 +997,17 @@ def test_packed_layout_without_rows_is_refused():
                                             p(t), p(t), None, None, None, p(t), p(ws), st) == -2
     assert lib.axon_reverse_scan(0, p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 1.0, 1.0, None, p(t), p(t), st) == -2
     torch.cuda.synchronize()
+
+
+def test_all_padding_micro_batch_is_a_no_op_before_any_validation():
+    """sampler.py:368-370: an all-zero mask returns (None, mask, {}) even with arguments that would not
+    validate; with a token to correct the same arguments raise."""
+    z = torch.zeros(2, 4, device=DEV)
+    for kw in (dict(sampler_is="token", sampler_is_threshold=0.0), dict(sampler_rs="bogus", sampler_rs_threshold=2.0),
+               dict(sampler_rs="token", sampler_rs_threshold=None), dict(sampler_token_veto_threshold=-1.0)):
+        proto, mask, m = S.compute_sampler_correction_and_rejection_mask(z, z, z, **kw)
+        assert proto is None and mask is z and m == {}
+        with pytest.raises(ValueError):
+            S.compute_sampler_correction_and_rejection_mask(z, z, torch.ones_like(z), **kw)
+    proto, mask, m = S.compute_sampler_correction_and_rejection_mask(z, torch.zeros(2, 5, device=DEV), z)
+    assert proto is None and m == {}

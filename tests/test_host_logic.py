@@ -144,12 +144,15 @@ def test_sampler_validation_messages():
         S.compute_sampler_correction_weights(x, x, "token", 0.0)
     with pytest.raises(ValueError, match="Invalid sampler_is"):
         S.compute_sampler_correction_weights(x, x, "geometric", 2.0)
+    one = torch.ones(2, 3)  # the unified function validates only when there is a token to correct
     with pytest.raises(ValueError, match="must be positive"):
-        S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_token_veto_threshold=-0.1)
+        S.compute_sampler_correction_and_rejection_mask(x, x, one, sampler_token_veto_threshold=-0.1)
     with pytest.raises(ValueError, match="does not match"):
-        S.compute_sampler_correction_and_rejection_mask(x, torch.zeros(2, 4), x)
+        S.compute_sampler_correction_and_rejection_mask(x, torch.zeros(2, 4), one)
     with pytest.raises(ValueError, match="must be explicitly provided"):
-        S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_rs="token", sampler_rs_threshold=None)
+        S.compute_sampler_correction_and_rejection_mask(x, x, one, sampler_rs="token", sampler_rs_threshold=None)
+    # an all-padding micro-batch is a no-op before any validation (sampler.py:368-370)
+    assert S.compute_sampler_correction_and_rejection_mask(x, x, x, sampler_token_veto_threshold=-0.1) == (None, x, {})
 
 
 def test_log_interval_agrees_with_torch_exp_bitwise():
