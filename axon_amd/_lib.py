@@ -21,18 +21,19 @@ SIGNATURES: dict[str, tuple] = {
     "axon_amd_error_string": (ctypes.c_char_p, [_i32]),
     "axon_lmhead_fwd_workspace_bytes": (_i64, [_i64, _i64, _i64]),
     "axon_seq_start_flags": (_i32, [_ptr, _i64, _i64, _ptr, _ptr]),
+    "axon_lmhead_stash_bytes": (_i64, [_i64, _i64, _i64]),
     "axon_lmhead_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr,
-                               _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
+                               _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
     "axon_lmhead_bwd_workspace_bytes": (_i64, [_i64, _i64, _i64, _i64]),
     "axon_lmhead_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                               _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr]),
+                               _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr]),
     "axon_timer_create": (_ptr, [_ptr]),
     "axon_timer_collect": (_i32, [_ptr, _ptr, _ptr]),
     "axon_timer_destroy": (None, [_ptr]),
     "axon_lmhead_fwd_timed": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr,
-                                     _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _ptr]),
+                                     _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                                     _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+                                     _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_active_rows": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_gather_rows": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64,
                                        _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
@@ -83,7 +84,7 @@ SIGNATURES: dict[str, tuple] = {
                                         _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
 }
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -623,9 +623,42 @@ def _head_operands(what, hidden, weight, labels, seq_start):
     return n, int(hidden.shape[1]), int(weight.shape[0])
 
 
+# The forward can leave a stash for its backward (2 bytes per logit: every softmax numerator as fp16 relative to
+# the maximum of its 128-row part of the vocabulary), from which the backward decodes the dlogits instead of
+# recomputing the logits: 6 N H V flop per forward + backward instead of 8.  ``LMHEAD_STASH``: "auto" keeps one
+# when it is at most ``LMHEAD_STASH_MAX_BYTES`` and (outside stream capture) at most half of the free device
+# memory; True always (when the shape allows it); False never (the memory-lean recompute backward).
+LMHEAD_STASH = "auto"
+LMHEAD_STASH_MAX_BYTES = 64 << 30
+
+
+def lmhead_stash_bytes(n: int, h: int, v: int) -> int:
+    """Bytes of the forward's stash for this shape; 0 if the shape cannot be stashed."""
+    return max(0, int(_lib.load().axon_lmhead_stash_bytes(int(n), int(h), int(v))))
+
+
+def _want_stash(n, h, v, dev) -> int:
+    """Bytes of the stash to allocate under the module's policy, or 0."""
+    if LMHEAD_STASH is False or n == 0:
+        return 0
+    need = lmhead_stash_bytes(n, h, v)
+    if need == 0 or LMHEAD_STASH is True:
+        return need
+    if need > LMHEAD_STASH_MAX_BYTES:
+        return 0
+    if not torch.cuda.is_current_stream_capturing():
+        free, _total = torch.cuda.mem_get_info(dev)
+        reusable = torch.cuda.memory_reserved(dev) - torch.cuda.memory_allocated(dev)
+        if need > (free + reusable) // 2:
+            return 0
+    return need
+
+
 def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | None" = None, softcap: float = 0.0,
-                   seq_start=None):
-    """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]).  ``softcap`` > 0 soft-caps the logits
+                   seq_start=None, stash: bool = False):
+    """Returns logprobs, entropy, lse, entropy_b (all fp32 [N]), and with ``stash`` a fifth value: the uint8
+    tensor that ``lmhead_backward(..., stash=)`` decodes the dlogits from (None when the module's policy,
+    ``LMHEAD_STASH``, or the shape says no).  ``softcap`` > 0 soft-caps the logits
     (cap * tanh(logit / cap)) before the temperature.  With ``seq_start`` (``seq_start_flags``) ``labels`` is
     the packed id stream and logprobs / entropy come back aligned to token positions.
 
@@ -640,14 +673,17 @@ def lmhead_forward(hidden, weight, labels, inv_temperature, timing: "Timer | Non
     if ws_bytes < 0:
         raise _lib.AxonAmdError(f"axon_lmhead_fwd: unsupported shape tokens={n} hidden={h} vocab={v} (hidden % 32 != 0?)")
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+    stash_bytes = _want_stash(n, h, v, dev) if stash else 0
+    stash_t = torch.empty(stash_bytes, device=dev, dtype=torch.uint8) if stash_bytes else None
     args = (ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), n, h, v,
             float(inv_temperature), float(softcap), ptr(seq_start), ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), ptr(ws), ws_bytes,
-            stream_ptr())
+            ptr(stash_t), stash_bytes, stream_ptr())
     if timing is None:
         check(lib.axon_lmhead_fwd(*args), "axon_lmhead_fwd")
     else:
         check(lib.axon_lmhead_fwd_timed(*args, timing.handle), "axon_lmhead_fwd_timed")
-    return out[0][:n], out[1][:n], out[2][:n], out[3][:n]
+    res = (out[0][:n], out[1][:n], out[2][:n], out[3][:n])
+    return res + (stash_t,) if stash else res
 
 
 # Opt-in: let the LM-head backward look for rows without an upstream gradient and leave them out.  Finding
@@ -671,9 +707,14 @@ def _active_rows(g_lp, g_en, seq_start, n):
 
 
 def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b, inv_temperature, vocab_chunk=0,
-                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=None):
+                    timing: "Timer | None" = None, softcap: float = 0.0, seq_start=None, skip_zero_rows=None,
+                    stash=None):
     """Returns d_hidden [N,H], d_weight [V,H] in bf16 (``timing`` as in ``lmhead_forward``).  By default the
     call only enqueues launches: no readback, no host synchronisation, and it can be captured into a HIP graph.
+
+    ``stash``: what ``lmhead_forward(..., stash=True)`` returned for the same operands; the dlogits are then
+    decoded from it and the logits are not recomputed.  (It describes all rows: a backward that leaves rows out
+    ignores it and recomputes.)
 
     With ``skip_zero_rows`` (default: the module switch ``SKIP_ZERO_GRAD_ROWS``, off) the rows whose upstream
     gradients are both exactly zero (prompt positions, where the response mask is zero, rejected or clipped
@@ -719,9 +760,15 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
     g_lp = f32(dlogprobs)  # keep the converted copies alive until the launch is enqueued
     g_en = f32(dentropy) if dentropy is not None else None
+    if stash is not None:
+        if stash.dtype != torch.uint8 or stash.device != dev or not stash.is_contiguous():
+            raise ValueError("lmhead_backward: stash must be the uint8 tensor lmhead_forward returned")
+        if int(stash.numel()) != lmhead_stash_bytes(n, h, v) or int(stash.numel()) == 0:
+            raise ValueError(f"lmhead_backward: a stash of {int(stash.numel())} bytes does not belong to a forward of "
+                             f"tokens={n} hidden={h} vocab={v}")
     args = (ptr(g_lp), ptr(g_en), ptr(hidden), ptr(weight), ptr(labels), int(labels.dtype == torch.int64), ptr(lse),
             ptr(entropy_b), n, h, v, float(inv_temperature), float(softcap), ptr(seq_start), ptr(d_hidden), ptr(d_weight), int(vocab_chunk), ptr(ws),
-            ws_bytes, stream_ptr())
+            ws_bytes, ptr(stash), 0 if stash is None else int(stash.numel()), stream_ptr())
     if timing is None:
         check(lib.axon_lmhead_bwd(*args), "axon_lmhead_bwd")
     else:

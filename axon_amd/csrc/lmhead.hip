@@ -41,7 +41,35 @@ struct FwdParams {
   int n_tokens, vocab;
   float c;     // inv_temperature * log2(e)
   float cap, inv_cap;  // logit soft-capping cap * tanh(logit / cap) (SOFTCAP kernels only)
+  uint4* stash;        // STASH kernels only: 128 KB per tile, see StashLayout
 };
+
+// What a stashing forward leaves for the backward: for every logit, w = 2^(y - M) as fp16, where
+// y is the scaled logit in log2 units and M the maximum of y over the 128 vocabulary rows of the
+// same token that one wavefront holds (the `pm` partial of that (token, 128-row part)), so that
+// 0 <= w <= 1 and softmax = w * 2^(M - logsumexp).  fp16 keeps eleven bits of w whatever the size
+// of the logit; entries below 2^-24 of their part's maximum read back as 0 and contribute no
+// gradient.  Each wavefront's 128 x 128 sub-tile is stored in accumulator order, 16 bytes per lane
+// and store (two 16-row blocks), every store one contiguous kilobyte:
+//   uint4 index = ((tile * 4 + wave) * 32 + j * 4 + i / 2) * 64 + lane,   tile = tm * tiles_n + tn.
+// Elements that do not count in their tile (duplicates of the neighbouring tile, rows beyond the
+// matrix) are stored as 0 and never read.
+constexpr int64_t kStashTileBytes = 131072;
+constexpr int kStashWaveVecs = 2048;  // uint4 per wavefront sub-tile
+
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  const f16x2 r = __builtin_convertvector(v, f16x2);  // round to nearest even
+  return *reinterpret_cast<const uint32_t*>(&r);
+}
+__device__ __forceinline__ void unpack_f16(uint32_t w, float& lo, float& hi) {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  const f16x2 r = *reinterpret_cast<const f16x2*>(&w);
+  lo = (float)r[0];
+  hi = (float)r[1];
+}
 
 // tanh(u) = 1 - 2 / (e^(2u) + 1): saturates cleanly at +-1 (2^x -> inf gives rcp 0, 2^x -> 0 gives -1)
 __device__ __forceinline__ float fast_tanh(float u) {
@@ -63,10 +91,11 @@ __device__ __forceinline__ void merge_stats(float M, float& s, float& e, float M
 
 // Fold one 256x256 logits tile into per-token partials.  MASKED: some rows of the tile
 // do not count (beyond the vocabulary, or duplicates of the neighbouring tile); they are
-// excluded by predicate — their accumulators hold finite values.
-template <bool MASKED>
+// excluded by predicate — their accumulators hold finite values.  STASH: also store every
+// 2^(y - M) for the backward (`stash_wave`: this wavefront's 32 KB, already offset by the lane).
+template <bool MASKED, bool STASH>
 __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, const LanePos& lp,
-                                             const TilePos& t, int tm) {
+                                             const TilePos& t, int tm, uint4* stash_wave) {
   const int part = tm * 2 + lp.wm;
 #pragma unroll
   for (int j = 0; j < kBlocks; ++j) {
@@ -79,28 +108,38 @@ __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, c
         const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
         mx = ok ? fmaxf(mx, acc[i][j][r]) : mx;
       }
-    float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
+    // the four lanes that hold the same token (lane ^ 16, lane ^ 32) share one reference
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
     float s = 0.f, e = 0.f;
+    uint32_t hw[kBlocks][2];
 #pragma unroll
-    for (int i = 0; i < kBlocks; ++i)
+    for (int i = 0; i < kBlocks; ++i) {
+      float w[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int mr = lp.m(i, r);
         const bool ok = !MASKED || (mr >= t.m_lo && t.m0 + mr < p.vocab);
         const float y = fmaf(acc[i][j][r], p.c, -M);  // scaled logit relative to the max, <= 0
-        const float w = ok ? fast_exp2(y) : 0.f;
-        s += w;
-        e = fmaf(w, y, e);
+        w[r] = ok ? fast_exp2(y) : 0.f;
+        s += w[r];
+        e = fmaf(w[r], y, e);
       }
-    // merge the four lanes that hold the same token (lane ^ 16, lane ^ 32)
+      if (STASH) {
+        hw[i][0] = pack_f16(w[0], w[1]);
+        hw[i][1] = pack_f16(w[2], w[3]);
+      }
+    }
+    if (STASH) {
+#pragma unroll
+      for (int ip = 0; ip < kBlocks / 2; ++ip)
+        stash_wave[(j * 4 + ip) * 64] = make_uint4(hw[2 * ip][0], hw[2 * ip][1], hw[2 * ip + 1][0], hw[2 * ip + 1][1]);
+    }
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {
-      const float M2 = __shfl_xor(M, off, 64);
-      const float s2 = __shfl_xor(s, off, 64);
-      const float e2 = __shfl_xor(e, off, 64);
-      const float Mn = fmaxf(M, M2);
-      merge_stats(M, s, e, M2, s2, e2, Mn);
-      M = Mn;
+      s += __shfl_xor(s, off, 64);
+      e += __shfl_xor(e, off, 64);
     }
     const int nr = lp.n(j);
     const int n = t.n0 + nr;
@@ -114,7 +153,7 @@ __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, c
 }
 
 // SOFTCAP: the logits go through cap * tanh(. / cap) before the statistics (fused_linear.py:19-23).
-template <class Loop, bool SOFTCAP>
+template <class Loop, bool SOFTCAP, bool STASH>
 __device__ __forceinline__ void fwd_body(const GemmOperands& g, const FwdParams& p, int tiles_m,
                                          int tiles_n) {
   extern __shared__ __align__(16) char smem[];
@@ -132,23 +171,39 @@ __device__ __forceinline__ void fwd_body(const GemmOperands& g, const FwdParams&
         for (int r = 0; r < 4; ++r) acc[i][j][r] = p.cap * fast_tanh(acc[i][j][r] * p.inv_cap);
   }
   const LanePos lp;
+  uint4* const stash_wave =
+      STASH ? p.stash + ((int64_t)(tm * tiles_n + tn) * 4 + lp.wave) * kStashWaveVecs + lp.lane : nullptr;
   if (t.m_lo > 0 || t.m0 + kTile > p.vocab)
-    fwd_epilogue<true>(acc, p, lp, t, tm);
+    fwd_epilogue<true, STASH>(acc, p, lp, t, tm, stash_wave);
   else
-    fwd_epilogue<false>(acc, p, lp, t, tm);
+    fwd_epilogue<false, STASH>(acc, p, lp, t, tm, stash_wave);
 }
 
 template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_kernel(GemmOperands g, FwdParams p,
                                                                   int tiles_m, int tiles_n) {
-  fwd_body<Loop, false>(g, p, tiles_m, tiles_n);
+  fwd_body<Loop, false, false>(g, p, tiles_m, tiles_n);
 }
 
 template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_softcap_kernel(GemmOperands g,
                                                                           FwdParams p, int tiles_m,
                                                                           int tiles_n) {
-  fwd_body<Loop, true>(g, p, tiles_m, tiles_n);
+  fwd_body<Loop, true, false>(g, p, tiles_m, tiles_n);
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_stash_kernel(GemmOperands g, FwdParams p,
+                                                                        int tiles_m, int tiles_n) {
+  fwd_body<Loop, false, true>(g, p, tiles_m, tiles_n);
+}
+
+template <class Loop>
+__global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_softcap_stash_kernel(GemmOperands g,
+                                                                                FwdParams p,
+                                                                                int tiles_m,
+                                                                                int tiles_n) {
+  fwd_body<Loop, true, true>(g, p, tiles_m, tiles_n);
 }
 
 // Token-aligned packed layout.  With `is_start` (one byte per packed position, 1 where a sequence
@@ -295,6 +350,32 @@ __device__ __forceinline__ int stage_off(int nw, int unit) {
 // the derivative 1 - tanh^2 (fused_linear.py:80-83).
 // Accumulators -> bf16 dlogits in the wave's staging area.  MASKED: the tile reaches past the last
 // token or the last vocabulary row; those entries are written as zeros.
+// Per-token factors of dlogit = softmax * (ca + cb * logit) + onehot * gl for tile-relative token
+// row nr; lab_rel is the label's row inside the tile whose first vocabulary row is m0_abs (-1: not
+// in this tile).
+struct TokenCoef {
+  float ca, cb, gl, lse2;
+  int lab_rel, nn;
+  bool n_ok;
+  __device__ __forceinline__ TokenCoef(const DlogitParams& p, int n, int64_t m0_abs) {
+    n_ok = n < p.n_tokens;
+    nn = n_ok ? n : 0;
+    const int src = aligned_pos(nn, p.n_tokens, p.is_start);  // where the label and the gradients live
+    const bool g_ok = n_ok && !(p.is_start && p.is_start[src]);
+    const float g_lp = g_ok ? p.dlogprobs[src] : 0.f;
+    const float g_en = (g_ok && p.dentropy) ? p.dentropy[src] : 0.f;
+    lse2 = p.lse[nn] * kLog2e;
+    const float eb = p.entropy_b[nn];
+    ca = (-g_lp + g_en * eb) * p.inv_temp;
+    cb = -g_en * p.inv_temp * p.inv_temp;
+    gl = g_lp * p.inv_temp;
+    const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[src]
+                                     : (int64_t) static_cast<const int32_t*>(p.labels)[src];
+    const int64_t lab_rel64 = lab - m0_abs;
+    lab_rel = (lab_rel64 >= 0 && lab_rel64 < kTile) ? (int)lab_rel64 : -1;
+  }
+};
+
 template <bool SOFTCAP, bool MASKED>
 __device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p, const LanePos& lp,
                                              const TilePos& t, char* stage) {
@@ -302,24 +383,8 @@ __device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p
 #pragma unroll
   for (int j = 0; j < kBlocks; ++j) {
     const int nw = j * kBlk + lp.l16;  // token row inside the wave's sub-tile
-    const int n = t.n0 + lp.wn * kWaveTile + nw;
-    const bool n_ok = n < p.n_tokens;
-    const int nn = n_ok ? n : 0;
-    const int src = aligned_pos(nn, p.n_tokens, p.is_start);  // where the label and the gradients live
-    const bool g_ok = n_ok && !(p.is_start && p.is_start[src]);
-    const float g_lp = g_ok ? p.dlogprobs[src] : 0.f;
-    const float g_en = (g_ok && p.dentropy) ? p.dentropy[src] : 0.f;
-    const float lse2 = p.lse[nn] * kLog2e;
-    const float eb = p.entropy_b[nn];
-    // dlogit = p * (a + b * logit) + onehot * g / T
-    const float ca = (-g_lp + g_en * eb) * p.inv_temp;
-    const float cb = -g_en * p.inv_temp * p.inv_temp;
-    const float gl = g_lp * p.inv_temp;
-    const int64_t lab = p.labels_i64 ? static_cast<const int64_t*>(p.labels)[src]
-                                     : (int64_t) static_cast<const int32_t*>(p.labels)[src];
-    const int64_t lab_rel64 = lab - (int64_t)(p.v_begin + t.m0);  // label row relative to the tile
-    const int lab_rel = (lab_rel64 >= 0 && lab_rel64 < kTile) ? (int)lab_rel64 : -1;
-    const int m_end = MASKED ? (n_ok ? p.vocab - p.v_begin - t.m0 : 0) : kTile;  // rows that count
+    const TokenCoef k(p, t.n0 + lp.wn * kWaveTile + nw, (int64_t)p.v_begin + t.m0);
+    const int m_end = MASKED ? (k.n_ok ? p.vocab - p.v_begin - t.m0 : 0) : kTile;  // rows that count
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
       float d[4];
@@ -333,9 +398,9 @@ __device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p
           raw = p.cap * th;
           dcap = fmaf(-th, th, 1.f);
         }
-        const float pr = fast_exp2(fmaf(raw, c, -lse2));
-        float v = pr * fmaf(cb, raw, ca);
-        if (mrel == lab_rel) v += gl;
+        const float pr = fast_exp2(fmaf(raw, c, -k.lse2));
+        float v = pr * fmaf(k.cb, raw, k.ca);
+        if (mrel == k.lab_rel) v += k.gl;
         if (SOFTCAP) v *= dcap;
         // rows shared with the neighbouring tile keep their (identical) values
         d[r] = (!MASKED || mrel < m_end) ? v : 0.f;
@@ -344,6 +409,111 @@ __device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p
       w.x = pack_bf16(d[0], d[1]);
       w.y = pack_bf16(d[2], d[3]);
       *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 4 + lp.lq)) = w;
+    }
+  }
+}
+
+// The same from a forward's stash (see StashLayout above FwdParams): softmax = w * 2^(M - lse), scaled
+// logit = log2(w) + M.  SOFTCAP: the stash describes the capped logit, whose derivative factor is
+// 1 - (capped / cap)^2.  EDGE: entries that do not count in this tile are staged as zeros.
+template <bool SOFTCAP, bool EDGE>
+__device__ __forceinline__ void dlogit_stage_stash(const uint4 (&st)[32], const float* __restrict__ pm,
+                                                   int part, const DlogitParams& p, const LanePos& lp,
+                                                   const TilePos& t, char* stage) {
+  const float inv_c = 1.f / (p.inv_temp * kLog2e);
+#pragma unroll
+  for (int j = 0; j < kBlocks; ++j) {
+    const int nw = j * kBlk + lp.l16;
+    const int nr = lp.wn * kWaveTile + nw;
+    const TokenCoef k(p, t.n0 + nr, (int64_t)p.v_begin + t.m0);
+    const float Mp = pm[(int64_t)part * p.n_tokens + k.nn];
+    const float scale = fast_exp2(Mp - k.lse2);
+    const bool n_counts = !EDGE || (k.n_ok && nr >= t.n_lo);
+#pragma unroll
+    for (int i = 0; i < kBlocks; ++i) {
+      const uint4 q = st[j * 4 + (i >> 1)];
+      float wv[4];
+      unpack_f16((i & 1) ? q.z : q.x, wv[0], wv[1]);
+      unpack_f16((i & 1) ? q.w : q.y, wv[2], wv[3]);
+      float d[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int mrel = lp.m(i, r);
+        const float pr = wv[r] * scale;
+        const float raw = (__builtin_amdgcn_logf(fmaxf(wv[r], 1e-30f)) + Mp) * inv_c;
+        float v = pr * fmaf(k.cb, raw, k.ca);
+        if (mrel == k.lab_rel) v += k.gl;
+        if (SOFTCAP) {
+          const float th = raw * p.inv_cap;
+          v *= fmaf(-th, th, 1.f);
+        }
+        const bool ok = !EDGE || (n_counts && mrel >= t.m_lo && p.v_begin + t.m0 + mrel < p.vocab);
+        d[r] = ok ? v : 0.f;
+      }
+      uint2 w;
+      w.x = pack_bf16(d[0], d[1]);
+      w.y = pack_bf16(d[2], d[3]);
+      *reinterpret_cast<uint2*>(stage + stage_off(nw, i * 4 + lp.lq)) = w;
+    }
+  }
+}
+
+// The wave's staged 128 x 128 bf16 sub-tile -> dl (token-major) and dlT (vocab-major).  The wave
+// reads back only what it wrote itself; LDS operations of one wave complete in order.  EDGE: entries
+// that duplicate the neighbouring tile (tile-relative token < n_lo, vocabulary row < m_lo; both
+// multiples of 4) are left to that tile.
+template <bool EDGE>
+__device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitParams& p,
+                                                const LanePos& lp, const TilePos& t) {
+  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
+  const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
+  const int n_base = t.n0 + lp.wn * kWaveTile;
+  const int m_skip = t.m_lo - lp.wm * kWaveTile, n_skip = t.n_lo - lp.wn * kWaveTile;  // sub-tile relative
+  // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
+  // destinations by running pointers (no 64-bit multiplies in the loop).
+  {
+    const int unit = l32;
+    char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
+    const int64_t dstep = p.ld_dl * 4;  // two rows of bf16
+    const bool col_ok = !EDGE || unit * 4 >= m_skip;
+#pragma unroll 1
+    for (int nw0 = lhi; nw0 < kWaveTile; nw0 += 16) {
+      uint2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (col_ok && (!EDGE || nw0 + 2 * u >= n_skip)) *reinterpret_cast<uint2*>(d) = v[u];
+        d += dstep;
+      }
+    }
+  }
+  // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
+  {
+    const int nq = l32;  // token quad
+    const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
+    char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + lhi * 4) * p.ld_dlT + n_base + nq * 4);
+    const bool tok_ok = !EDGE || nq * 4 >= n_skip;
+#pragma unroll 2
+    for (int unit = lhi; unit < 32; unit += 2) {
+      uint2 rws[4];
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+        rws[f] = *reinterpret_cast<const uint2*>(stage + stage_off(nq * 4 + f, unit));
+      uint2 o[4];
+      o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
+      o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
+      o[1].x = (rws[0].x >> 16) | (rws[1].x & 0xffff0000u);
+      o[1].y = (rws[2].x >> 16) | (rws[3].x & 0xffff0000u);
+      o[2].x = (rws[0].y & 0xffffu) | (rws[1].y << 16);
+      o[2].y = (rws[2].y & 0xffffu) | (rws[3].y << 16);
+      o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
+      o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
+      if (tok_ok && (!EDGE || unit * 4 >= m_skip)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
+      }
+      d += 8 * rstep;
     }
   }
 }
@@ -360,58 +530,12 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
   __syncthreads();  // every wave is past its last main-loop LDS access
 
   const LanePos lp;
-  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
   char* const stage = smem + lp.wave * 32768;
   if (t.n0 + kTile > p.n_tokens || p.v_begin + t.m0 + kTile > p.vocab)
     dlogit_stage<SOFTCAP, true>(acc, p, lp, t, stage);
   else
     dlogit_stage<SOFTCAP, false>(acc, p, lp, t, stage);
-  // the wave reads back only what it wrote itself; LDS operations of one wave complete in order
-  const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
-  const int n_base = t.n0 + lp.wn * kWaveTile;
-  // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
-  // destinations by running pointers (no 64-bit multiplies in the loop).
-  {
-    const int unit = l32;
-    char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
-    const int64_t dstep = p.ld_dl * 4;  // two rows of bf16
-#pragma unroll 1
-    for (int nw0 = lhi; nw0 < kWaveTile; nw0 += 16) {
-      uint2 v[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        *reinterpret_cast<uint2*>(d) = v[u];
-        d += dstep;
-      }
-    }
-  }
-  // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
-  {
-    const int nq = l32;  // token quad
-    const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
-    char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + lhi * 4) * p.ld_dlT + n_base + nq * 4);
-#pragma unroll 2
-    for (int unit = lhi; unit < 32; unit += 2) {
-      uint2 rws[4];
-#pragma unroll
-      for (int f = 0; f < 4; ++f)
-        rws[f] = *reinterpret_cast<const uint2*>(stage + stage_off(nq * 4 + f, unit));
-      uint2 o[4];
-      o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
-      o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
-      o[1].x = (rws[0].x >> 16) | (rws[1].x & 0xffff0000u);
-      o[1].y = (rws[2].x >> 16) | (rws[3].x & 0xffff0000u);
-      o[2].x = (rws[0].y & 0xffffu) | (rws[1].y << 16);
-      o[2].y = (rws[2].y & 0xffffu) | (rws[3].y << 16);
-      o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
-      o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
-      d += 8 * rstep;
-    }
-  }
+  dlogit_copy_out<false>(stage, p, lp, t);
 }
 
 template <class Loop>
@@ -426,6 +550,53 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_softcap_kernel(Gem
                                                                              int tiles_m,
                                                                              int tiles_n) {
   dlogit_body<Loop, true>(g, p, tiles_m, tiles_n);
+}
+
+// Backward B1 without the recompute: one wavefront per workgroup turns the 128 x 128 sub-tile a
+// stashing forward stored into bf16 dlogits in both orientations.  A streaming kernel: 2 bytes
+// read and 4 written per logit.  Tiles are the forward's (same shifted or clamped placement), so
+// `tm0` is the forward tile row of the chunk's first vocabulary row and t.m0 is made chunk-relative
+// only after the edge tests; it is negative only for rows that the tile does not own.
+struct StashSource {
+  const uint4* stash;
+  const float* pm;
+  int tiles_n, tm0, shifted;
+};
+
+template <bool SOFTCAP>
+__global__ __launch_bounds__(64) void lmhead_dlogit_stash_kernel(DlogitParams p, StashSource src) {
+  __shared__ __align__(16) char stage[32768];
+  const int wave = blockIdx.x & 3, tile = blockIdx.x >> 2;
+  const int tm = src.tm0 + tile / src.tiles_n, tn = tile % src.tiles_n;
+  TilePos t{tm * kTile, tn * kTile, 0, 0};
+  if (src.shifted) {
+    t.m0 = min(t.m0, p.vocab - kTile);
+    t.n0 = min(t.n0, p.n_tokens - kTile);
+    t.m_lo = tm * kTile - t.m0;
+    t.n_lo = tn * kTile - t.n0;
+  }
+  LanePos lp;
+  lp.wave = wave;
+  lp.wm = wave >> 1;
+  lp.wn = wave & 1;
+  const uint4* sv = src.stash + ((int64_t)(tm * src.tiles_n + tn) * 4 + wave) * kStashWaveVecs + lp.lane;
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  uint4 st[32];
+#pragma unroll
+  for (int q = 0; q < 32; ++q) {  // read once: keep it out of the way of the GEMMs' operands in L2
+    const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sv + q * 64));
+    st[q] = make_uint4(x[0], x[1], x[2], x[3]);
+  }
+  const bool edge = t.m_lo > 0 || t.n_lo > 0 || t.m0 + kTile > p.vocab || t.n0 + kTile > p.n_tokens;
+  t.m0 -= p.v_begin;
+  const int part = tm * 2 + lp.wm;
+  if (edge) {
+    dlogit_stage_stash<SOFTCAP, true>(st, src.pm, part, p, lp, t, stage);
+    dlogit_copy_out<true>(stage, p, lp, t);
+  } else {
+    dlogit_stage_stash<SOFTCAP, false>(st, src.pm, part, p, lp, t, stage);
+    dlogit_copy_out<false>(stage, p, lp, t);
+  }
 }
 
 // ----------------------------------------------------------------------------
@@ -692,6 +863,31 @@ FwdWs fwd_ws(int64_t n, int64_t vocab, void* base) {
   return w;
 }
 
+// The stash of a forward for its backward: the tiles' fp16 sub-tiles, then the per-part maxima
+// (which the forward then writes there instead of into its workspace).
+struct StashWs {
+  uint4* tiles;
+  float* pm;
+  int tiles_m, tiles_n, shifted;
+  int64_t bytes;  // 0: this shape cannot be stashed
+};
+StashWs stash_ws(int64_t n, int64_t h, int64_t v, void* base) {
+  StashWs w{};
+  if (n <= 0) return w;
+  GemmOperands g{};
+  g.lda = g.ldb = h;  g.m_rows = (int)v;  g.n_rows = (int)n;  g.k = (int)h;
+  w.shifted = dma_ok(g);
+  // shifted edge tiles hand their duplicated rows to the neighbouring tile in groups of four
+  if (w.shifted && ((v % 4) != 0 || (n % 4) != 0)) return w;
+  w.tiles_m = (int)(round_up(v, kTile) / kTile);
+  w.tiles_n = (int)(round_up(n, kTile) / kTile);
+  const int64_t tile_bytes = (int64_t)w.tiles_m * w.tiles_n * kStashTileBytes;
+  w.tiles = static_cast<uint4*>(base);
+  w.pm = reinterpret_cast<float*>(static_cast<char*>(base) + tile_bytes);
+  w.bytes = tile_bytes + round_up((int64_t)w.tiles_m * 2 * n * 4, kAlign);
+  return w;
+}
+
 struct BwdWs {
   __bf16 *wT, *hT, *dl, *dlT;
   float* dh_acc;
@@ -810,7 +1006,7 @@ int launch_zero_cols(void* p, int64_t ld, int rows, int col0, int ncols, hipStre
 int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64, int64_t n,
              int64_t h, int64_t v, float inv_temp, float softcap, const uint8_t* is_start,
              float* logprobs, float* entropy, float* lse, float* entropy_b, void* workspace,
-             int64_t ws_bytes, void* stream, PhaseTimer* timer) {
+             int64_t ws_bytes, void* stash, int64_t stash_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
@@ -820,22 +1016,36 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
   if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight)) & 15)
     return AXON_ERR_ARG;
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
-  const FwdWs w = fwd_ws(n, v, base);
+  FwdWs w = fwd_ws(n, v, base);
   if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
   const hipStream_t st = (hipStream_t)stream;
+  StashWs sw{};
+  if (stash) {
+    if (reinterpret_cast<uintptr_t>(stash) & 15) return AXON_ERR_ARG;
+    sw = stash_ws(n, h, v, stash);
+    if (sw.bytes == 0) return AXON_ERR_SHAPE;
+    if (sw.bytes > stash_bytes) return AXON_ERR_WORKSPACE;
+    w.pm = sw.pm;  // the backward needs the per-part maxima: they live in the stash
+  }
 
   GemmOperands g;
   g.a = static_cast<const __bf16*>(weight);  g.lda = h;  g.m_rows = (int)v;
   g.b = static_cast<const __bf16*>(hidden);  g.ldb = h;  g.n_rows = (int)n;
   g.k = (int)h;
   FwdParams p{w.pm, w.ps, w.pe, (int)n, (int)v, inv_temp * kLog2e, softcap,
-              softcap > 0.f ? 1.f / softcap : 0.f};
+              softcap > 0.f ? 1.f / softcap : 0.f, sw.tiles};
   {
     Span span(timer, 0);
-    if (softcap > 0.f)
+    if (stash) {
+      if (softcap > 0.f)
+        AXON_LAUNCH_GEMM(lmhead_fwd_softcap_stash_kernel, g, p, st);
+      else
+        AXON_LAUNCH_GEMM(lmhead_fwd_stash_kernel, g, p, st);
+    } else if (softcap > 0.f) {
       AXON_LAUNCH_GEMM(lmhead_fwd_softcap_kernel, g, p, st);
-    else
+    } else {
       AXON_LAUNCH_GEMM(lmhead_fwd_kernel, g, p, st);
+    }
   }
   {
     Span span(timer, 1);
@@ -865,7 +1075,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
              const void* labels, int labels_i64, const float* lse, const float* entropy_b,
              int64_t n, int64_t h, int64_t v, float inv_temp, float softcap,
              const uint8_t* is_start, void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
-             int64_t ws_bytes, void* stream, PhaseTimer* timer) {
+             int64_t ws_bytes, const void* stash, int64_t stash_bytes, void* stream, PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
@@ -881,6 +1091,13 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
   const BwdWs w = bwd_ws(n, h, v, chunk, base);
   if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
+  StashWs sw{};
+  if (stash) {
+    if (reinterpret_cast<uintptr_t>(stash) & 15) return AXON_ERR_ARG;
+    sw = stash_ws(n, h, v, const_cast<void*>(stash));
+    if (sw.bytes == 0) return AXON_ERR_SHAPE;
+    if (sw.bytes > stash_bytes) return AXON_ERR_WORKSPACE;
+  }
 
   // K-contiguous copies for the two output GEMMs
   {
@@ -910,10 +1127,19 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
       p.cap = softcap; p.inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
       p.is_start = is_start;
-      if (softcap > 0.f)
+      if (stash) {
+        const StashSource src{sw.tiles, sw.pm, sw.tiles_n, (int)(v0 / kTile), sw.shifted};
+        const unsigned blocks = (unsigned)(round_up(vc, kTile) / kTile) * (unsigned)sw.tiles_n * 4u;
+        if (softcap > 0.f)
+          hipLaunchKernelGGL(lmhead_dlogit_stash_kernel<true>, dim3(blocks), dim3(64), 0, st, p, src);
+        else
+          hipLaunchKernelGGL(lmhead_dlogit_stash_kernel<false>, dim3(blocks), dim3(64), 0, st, p, src);
+        AXON_CHECK_LAUNCH();
+      } else if (softcap > 0.f) {
         AXON_LAUNCH_GEMM(lmhead_dlogit_softcap_kernel, g, p, st);
-      else
+      } else {
         AXON_LAUNCH_GEMM(lmhead_dlogit_kernel, g, p, st);
+      }
       // reduction padding the tiles did not cover (the shifted-tile path writes no padding; the
       // clamped path writes zeros there already, the extra fill is then redundant but harmless)
       rc = launch_zero_cols(w.dl, w.ld_c, (int)n, (int)vc, (int)(vc_red - vc), st);
@@ -1037,13 +1263,19 @@ extern "C" int64_t axon_lmhead_fwd_workspace_bytes(int64_t n, int64_t h, int64_t
   return fwd_ws(n, v, nullptr).bytes + kAlign;
 }
 
+extern "C" int64_t axon_lmhead_stash_bytes(int64_t n, int64_t h, int64_t v) {
+  if (check_head_shape(n, h, v) != AXON_OK) return -1;
+  return stash_ws(n, h, v, nullptr).bytes;
+}
+
 extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const void* labels,
                                int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
                                float softcap, const uint8_t* seq_start, float* logprobs,
                                float* entropy, float* lse, float* entropy_b, void* workspace,
-                               int64_t ws_bytes, void* stream) {
+                               int64_t ws_bytes, void* stash, int64_t stash_bytes, void* stream) {
   return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start,
-                  logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stream, nullptr);
+                  logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stash, stash_bytes, stream,
+                  nullptr);
 }
 
 extern "C" void* axon_timer_create(void* stream) { return new (std::nothrow) PhaseTimer((hipStream_t)stream); }
@@ -1067,13 +1299,13 @@ extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, con
                                      float inv_temp, float softcap, const uint8_t* seq_start,
                                      float* logprobs, float* entropy, float* lse,
                                      float* entropy_b, void* workspace, int64_t ws_bytes,
-                                     void* stream, void* timer) {
+                                     void* stash, int64_t stash_bytes, void* stream, void* timer) {
   if (!timer) return AXON_ERR_ARG;
   PhaseTimer* t = static_cast<PhaseTimer*>(timer);
   if (t->st != (hipStream_t)stream) return AXON_ERR_ARG;
   t->base = 0;
   return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, logprobs,
-                  entropy, lse, entropy_b, workspace, ws_bytes, stream, t);
+                  entropy, lse, entropy_b, workspace, ws_bytes, stash, stash_bytes, stream, t);
 }
 
 extern "C" int64_t axon_lmhead_bwd_workspace_bytes(int64_t n, int64_t h, int64_t v,
@@ -1088,10 +1320,10 @@ extern "C" int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, co
                                const float* lse, const float* entropy_b, int64_t n, int64_t h,
                                int64_t v, float inv_temp, float softcap, const uint8_t* seq_start,
                                void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
-                               int64_t ws_bytes, void* stream) {
+                               int64_t ws_bytes, const void* stash, int64_t stash_bytes, void* stream) {
   return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
                   inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes,
-                  stream, nullptr);
+                  stash, stash_bytes, stream, nullptr);
 }
 
 extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy,
@@ -1100,14 +1332,15 @@ extern "C" int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentro
                                      int64_t n, int64_t h, int64_t v, float inv_temp,
                                      float softcap, const uint8_t* seq_start, void* d_hidden,
                                      void* d_weight, int64_t chunk, void* workspace,
-                                     int64_t ws_bytes, void* stream, void* timer) {
+                                     int64_t ws_bytes, const void* stash, int64_t stash_bytes,
+                                     void* stream, void* timer) {
   if (!timer) return AXON_ERR_ARG;
   PhaseTimer* t = static_cast<PhaseTimer*>(timer);
   if (t->st != (hipStream_t)stream) return AXON_ERR_ARG;
   t->base = 4;
   return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
-                  inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes, stream,
-                  t);
+                  inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes, stash,
+                  stash_bytes, stream, t);
 }
 
 extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int64_t ldb, float* out,

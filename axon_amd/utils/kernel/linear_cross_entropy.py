@@ -21,7 +21,10 @@ Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntro
   every sequence).  That is ``torch.roll(ids, -1)`` before the head and the shift-right after it
   (axon/utils/fsdp/forward_utils.py:131,164-182) done inside the kernels, forward and backward.
 
-The [tokens x vocab] logits are never written to memory, forward or backward.
+The [tokens x vocab] logits are never written to memory.  When a gradient is wanted and memory allows
+(``axon_amd._ops.LMHEAD_STASH``), the forward keeps 2 bytes per logit for its backward (each softmax
+numerator as fp16), which then decodes the dlogits instead of recomputing the logits; otherwise the
+backward recomputes them chunk by chunk as the reference's kernels do (kernels.py:1377-1585).
 """
 
 from __future__ import annotations
@@ -61,9 +64,12 @@ class LinearCrossEntropy(torch.autograd.Function):
         if not cap >= 0.0:
             raise ValueError(f"logit_softcapping must be positive, got {logit_softcapping}")
         seq_start = None if cu_seqlens is None else _ops.seq_start_flags(cu_seqlens, hidden2.shape[0])
-        logprobs, entropy, lse, entropy_b = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING,
-                                                                softcap=cap, seq_start=seq_start)
-        ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b, seq_start)
+        want_grad = bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        res = _ops.lmhead_forward(hidden2, weight, labels1, inv_t, timing=_ops.TIMING, softcap=cap,
+                                  seq_start=seq_start, stash=want_grad)
+        logprobs, entropy, lse, entropy_b = res[:4]
+        stash = res[4] if want_grad else None
+        ctx.save_for_backward(hidden2, weight, labels1, lse, entropy_b, seq_start, stash)
         ctx.shape, ctx.inv_t, ctx.reduction, ctx.cap = shape, inv_t, reduction, cap
         if reduction == "sum":
             logprobs = logprobs.sum()
@@ -73,7 +79,7 @@ class LinearCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dlogprobs, dentropy):
-        hidden2, weight, labels1, lse, entropy_b, seq_start = ctx.saved_tensors
+        hidden2, weight, labels1, lse, entropy_b, seq_start, stash = ctx.saved_tensors
         n = hidden2.shape[0]
         if dlogprobs is None:
             dlogprobs = torch.zeros(n, device=hidden2.device, dtype=torch.float32)
@@ -83,7 +89,7 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs = (dlogprobs / n).expand(n)
         d_hidden, d_weight = _ops.lmhead_backward(
             dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
-            entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap, seq_start=seq_start,
+            entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap, seq_start=seq_start, stash=stash,
         )
         return d_hidden.view(ctx.shape), d_weight, None, None, None, None, None, None
 

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 16
+#define AXON_AMD_ABI_VERSION 17
 
 enum {
   AXON_OK = 0,
@@ -80,8 +80,22 @@ const char* axon_amd_error_string(int code);
  *        lse / entropy_b stay indexed by hidden position.  The backward takes the
  *        same flags and reads dlogprobs / dentropy in the aligned layout, ignoring
  *        them at sequence starts.
+ *   stash (may be NULL): device memory of axon_lmhead_stash_bytes bytes, 16-byte aligned, that
+ *        the forward fills for its backward: every softmax numerator as fp16, relative to the
+ *        maximum of its 128-row part of the vocabulary (2 bytes per logit, in tile order), and
+ *        those maxima.  A backward given the same buffer reads the dlogits off it instead of
+ *        recomputing the logits: 6 N H V flop per forward + backward instead of 8, for
+ *        2 * n_tokens * vocab bytes that must live from the forward to the backward (10 GB at
+ *        32768 x 151936; the part has 288 GB).  The reference keeps no such buffer (its kernels
+ *        recompute, kernels.py:1377-1585; its torch path keeps the fp32 logits of one chunk,
+ *        fused_linear.py:26-46).  fp16 holds eleven bits of each numerator whatever the size of
+ *        the logit; numerators below 2^-24 of their part's maximum read back as 0.
  * Constraints: hidden % 32 == 0, hidden >= 32, vocab >= 1, n_tokens >= 0. */
 int64_t axon_lmhead_fwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab);
+/* Bytes of the forward's stash for this shape; 0 if the shape cannot be stashed (tiles that are
+ * shifted back inside the matrix need n_tokens % 4 == 0 and vocab % 4 == 0), -1 for an invalid
+ * shape.  The layout is private to the library and depends on the shape only. */
+int64_t axon_lmhead_stash_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab);
 /* flags[p] = 1 where a non-empty sequence of cu_seqlens[n_seqs + 1] begins, else 0.
  * `flags` holds n_tokens bytes rounded up to a multiple of 4. */
 int axon_seq_start_flags(const int32_t* cu_seqlens, int64_t n_seqs, int64_t n_tokens,
@@ -90,7 +104,8 @@ int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void
                     int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
                     float inv_temperature, float softcap, const uint8_t* seq_start,
                     float* logprobs, float* entropy, float* lse,
-                    float* entropy_b, void* workspace, int64_t workspace_bytes, void* stream);
+                    float* entropy_b, void* workspace, int64_t workspace_bytes, void* stash,
+                    int64_t stash_bytes, void* stream);
 
 /* Backward.  Replaces efficient_entropy_backward
  * (axon/utils/kernel/kernels.py:1377-1585, default _Split_Dlogits_N) and
@@ -100,7 +115,9 @@ int axon_lmhead_fwd(const void* hidden_bf16, const void* weight_bf16, const void
  * With softcap > 0 dlogit is additionally multiplied by 1 - tanh^2(raw logit / softcap)
  * (fused_linear.py:80-83).  dentropy may be NULL (treated as zeros).  vocab_chunk (multiple of 256, or 0
  * for the library default, 32768) bounds the bf16 dlogit scratch to
- * 2 * n_tokens_padded * vocab_chunk * 2 bytes. */
+ * 2 * n_tokens_padded * vocab_chunk * 2 bytes.  stash (may be NULL): what axon_lmhead_fwd left
+ * for the same operands, shape, temperature and softcap; the dlogits are then decoded from it by
+ * a streaming kernel (2 bytes read, 4 written per logit) and the logits are not recomputed. */
 int64_t axon_lmhead_bwd_workspace_bytes(int64_t n_tokens, int64_t hidden, int64_t vocab,
                                         int64_t vocab_chunk);
 int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
@@ -108,7 +125,8 @@ int axon_lmhead_bwd(const float* dlogprobs, const float* dentropy, const void* h
                     const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
                     int64_t vocab, float inv_temperature, float softcap,
                     const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
-                    int64_t vocab_chunk, void* workspace, int64_t workspace_bytes, void* stream);
+                    int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
+                    const void* stash, int64_t stash_bytes, void* stream);
 
 /* Rows of the backward without an upstream gradient.  The reference's trainer runs the head over every
  * packed token, prompt included (fsdp_model_forward, axon/utils/fsdp/forward_utils.py:236-265), and the
@@ -147,7 +165,7 @@ int axon_lmhead_scatter_rows(const void* d_hidden_c_bf16, const int32_t* row_ran
  * and launch counts of everything recorded since the last collect to the two HOST
  * arrays of 8 entries (zero them first) and forgets the spans:
  *   [0] forward logits+statistics kernel, [1] merge, [2] label logit, [3] unused,
- *   [4] backward transposes, [5] dlogit recompute, [6] dHidden GEMM, [7] dWeight GEMM.
+ *   [4] backward transposes, [5] dlogit (recompute, or decode of the stash), [6] dHidden GEMM, [7] dWeight GEMM.
  * The timer creates and destroys events and owns host memory (the exception to
  * "never allocates"); `stream` of a timed call must be the timer's.
  * No reference counterpart (measurement only). */
@@ -158,14 +176,15 @@ int axon_lmhead_fwd_timed(const void* hidden_bf16, const void* weight_bf16, cons
                           int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
                           float inv_temperature, float softcap, const uint8_t* seq_start,
                           float* logprobs, float* entropy, float* lse, float* entropy_b,
-                          void* workspace, int64_t workspace_bytes, void* stream, void* timer);
+                          void* workspace, int64_t workspace_bytes, void* stash,
+                          int64_t stash_bytes, void* stream, void* timer);
 int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
                           const void* weight_bf16, const void* labels, int labels_are_i64,
                           const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
                           int64_t vocab, float inv_temperature, float softcap,
                           const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
                           int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
-                          void* stream, void* timer);
+                          const void* stash, int64_t stash_bytes, void* stream, void* timer);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
  * (fp32 accumulate, fp32 output).  No reference counterpart: it exists so tests

@@ -154,6 +154,19 @@ def _spread_rows(v, chunk=32768):
     return torch.tensor(sorted(r for r in rows if 0 <= r < v))
 
 
+def _stash_backward(hd, wd, ld, g_lp, g_en, plain_forward):
+    """Forward with a stash (its outputs must be those of the plain forward, bit for bit) and the backward
+    that decodes it."""
+    from axon_amd import _ops
+    saved, _ops.LMHEAD_STASH = _ops.LMHEAD_STASH, True
+    try:
+        *out, stash = _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)
+    finally:
+        _ops.LMHEAD_STASH = saved
+    assert stash is not None and all(torch.equal(a, b) for a, b in zip(out, plain_forward))
+    return _ops.lmhead_backward(g_lp, g_en, hd, wd, ld, out[2], out[3], 1.0, stash=stash)
+
+
 def test_qwen3_8b_dweight_rows_vs_fp32_torch():
     """Config 3 at full size: d_weight on ~120 vocabulary rows spread over all five vocabulary chunks of the
     backward (rows >= 131072 and the last tile included), log-prob and entropy of every token, against an
@@ -176,6 +189,13 @@ def test_qwen3_8b_dweight_rows_vs_fp32_torch():
     assert rel_l2(got, ref_dw) < 2e-2
     per_row = (got - ref_dw).norm(dim=1) / ref_dw.norm(dim=1).clamp_min(1e-30)
     assert per_row.max().item() < 5e-2, (per_row.argmax().item(), per_row.max().item())  # no single row is off
+    # the same from the forward's stash (10 GB at this shape) instead of the recomputed logits
+    dh_s, dw_s = _stash_backward(hd, wd, ld, g_lp, g_en, (lp, ent, lse, eb))
+    got_s = dw_s[rows.to(DEV)].double()
+    assert rel_l2(got_s, ref_dw) < 2e-2
+    per_row = (got_s - ref_dw).norm(dim=1) / ref_dw.norm(dim=1).clamp_min(1e-30)
+    assert per_row.max().item() < 5e-2, (per_row.argmax().item(), per_row.max().item())
+    assert rel_l2(dh_s, dh.float()) < 5e-3 and rel_l2(dw_s, dw.float()) < 5e-3
 
 
 def test_gpt_oss_head_full_shape():
@@ -205,6 +225,10 @@ def test_gpt_oss_head_full_shape():
     assert rel_l2(dh[idx.to(DEV)], o_dh) < 2e-2
     dh2, dw2 = _ops.lmhead_backward(2 * g_lp, None, hd, wd, ld, lse, eb, 1.0)
     assert rel_l2(dh2, 2 * dh.float()) < 1e-2 and rel_l2(dw2, 2 * dw.float()) < 1e-2
+    del dh2, dw2
+    dh_s, dw_s = _stash_backward(hd, wd, ld, g_lp, None, (lp, ent, lse, eb))
+    assert rel_l2(dw_s[rows.to(DEV)].double(), ref_dw) < 2e-2 and rel_l2(dh_s[idx.to(DEV)], o_dh) < 2e-2
+    assert rel_l2(dh_s, dh.float()) < 5e-3 and rel_l2(dw_s, dw.float()) < 5e-3
 
 
 def test_micro_batched_dapo_chain_vs_whole_batch_oracle():
