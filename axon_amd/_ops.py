@@ -623,12 +623,14 @@ def _head_operands(what, hidden, weight, labels, seq_start):
     return n, int(hidden.shape[1]), int(weight.shape[0])
 
 
-# The forward can leave a stash for its backward (2 bytes per logit: every softmax numerator as fp16 relative to
-# the maximum of its 128-row part of the vocabulary), from which the backward decodes the dlogits instead of
-# recomputing the logits: 6 N H V flop per forward + backward instead of 8.  ``LMHEAD_STASH``: "auto" keeps one
-# when it is at most ``LMHEAD_STASH_MAX_BYTES`` and (outside stream capture) at most half of the free device
-# memory; True always (when the shape allows it); False never (the memory-lean recompute backward).
-LMHEAD_STASH = "auto"
+# Opt-in: the forward can leave a stash for its backward (2 bytes per logit: every softmax numerator as fp16
+# relative to the maximum of its 128-row part of the vocabulary), from which the backward decodes the dlogits
+# instead of recomputing the logits: 6 N H V flop per forward + backward instead of 8, for tokens x vocab x 2
+# bytes held from forward to backward (10 GB at 32768 x 151936).  Off by default: like the reference's kernels,
+# the default path never holds anything of size tokens x vocab.  ``LMHEAD_STASH``: False never; True whenever
+# the shape allows it; "auto" when it is at most ``LMHEAD_STASH_MAX_BYTES`` and (outside stream capture) at
+# most half of the free device memory.
+LMHEAD_STASH = False
 LMHEAD_STASH_MAX_BYTES = 64 << 30
 
 

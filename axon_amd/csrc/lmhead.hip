@@ -335,6 +335,18 @@ struct DlogitParams {
   const uint8_t* is_start;  // token-aligned packed layout (see aligned_pos), or null
 };
 
+// Four rows of four bf16 (rws[f] = row f) -> their transpose (o[e] = column e).
+__device__ __forceinline__ void transpose_4x4_bf16(const uint2 (&rws)[4], uint2 (&o)[4]) {
+  o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
+  o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
+  o[1].x = (rws[0].x >> 16) | (rws[1].x & 0xffff0000u);
+  o[1].y = (rws[2].x >> 16) | (rws[3].x & 0xffff0000u);
+  o[2].x = (rws[0].y & 0xffffu) | (rws[1].y << 16);
+  o[2].y = (rws[2].y & 0xffffu) | (rws[3].y << 16);
+  o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
+  o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
+}
+
 // Per-wave staging of the wave's 128(n) x 128(m) bf16 sub-tile in its own 32 KB of LDS:
 // row nw (256 bytes = 32 units of 4 bf16), unit u stored at slot perm(u) ^ swz(nw),
 // swz(nw) = (nw & 31) ^ (nw >> 5), perm(u) = u rotated right by two bits (unit = 4 * block + lane
@@ -414,24 +426,28 @@ __device__ __forceinline__ void dlogit_stage(AccTile& acc, const DlogitParams& p
 }
 
 // The same from a forward's stash (see StashLayout above FwdParams): softmax = w * 2^(M - lse), scaled
-// logit = log2(w) + M.  SOFTCAP: the stash describes the capped logit, whose derivative factor is
-// 1 - (capped / cap)^2.  EDGE: entries that do not count in this tile are staged as zeros.
+// logit = log2(w) + M.  One call covers 64 tokens (four 16-token blocks, j0 .. j0 + 3) x 128 vocabulary
+// rows of a wavefront's sub-tile; staged row = token - 16 * j0.  SOFTCAP: the stash describes the capped
+// logit, whose derivative factor is 1 - (capped / cap)^2.  EDGE: entries that do not count in this tile
+// are staged as zeros.
+constexpr int kStashHalfBlocks = kBlocks / 2;
 template <bool SOFTCAP, bool EDGE>
-__device__ __forceinline__ void dlogit_stage_stash(const uint4 (&st)[32], const float* __restrict__ pm,
-                                                   int part, const DlogitParams& p, const LanePos& lp,
+__device__ __forceinline__ void dlogit_stage_stash(const uint4 (&st)[4 * kStashHalfBlocks], int j0,
+                                                   const float* __restrict__ pm, int part,
+                                                   const DlogitParams& p, const LanePos& lp,
                                                    const TilePos& t, char* stage) {
   const float inv_c = 1.f / (p.inv_temp * kLog2e);
 #pragma unroll
-  for (int j = 0; j < kBlocks; ++j) {
-    const int nw = j * kBlk + lp.l16;
-    const int nr = lp.wn * kWaveTile + nw;
+  for (int jl = 0; jl < kStashHalfBlocks; ++jl) {
+    const int nw = jl * kBlk + lp.l16;
+    const int nr = lp.wn * kWaveTile + j0 * kBlk + nw;
     const TokenCoef k(p, t.n0 + nr, (int64_t)p.v_begin + t.m0);
     const float Mp = pm[(int64_t)part * p.n_tokens + k.nn];
     const float scale = fast_exp2(Mp - k.lse2);
     const bool n_counts = !EDGE || (k.n_ok && nr >= t.n_lo);
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
-      const uint4 q = st[j * 4 + (i >> 1)];
+      const uint4 q = st[jl * 4 + (i >> 1)];
       float wv[4];
       unpack_f16((i & 1) ? q.z : q.x, wv[0], wv[1]);
       unpack_f16((i & 1) ? q.w : q.y, wv[2], wv[3]);
@@ -458,26 +474,25 @@ __device__ __forceinline__ void dlogit_stage_stash(const uint4 (&st)[32], const 
   }
 }
 
-// The wave's staged 128 x 128 bf16 sub-tile -> dl (token-major) and dlT (vocab-major).  The wave
-// reads back only what it wrote itself; LDS operations of one wave complete in order.  EDGE: entries
-// that duplicate the neighbouring tile (tile-relative token < n_lo, vocabulary row < m_lo; both
-// multiples of 4) are left to that tile.
+// A staged 64 x 128 half sub-tile (tokens 16 * j0 .. of the wavefront's sub-tile) -> dl and dlT.  Token-major
+// as in dlogit_copy_out (below); vocab-major: sixteen lanes cover the 64 tokens of one vocabulary row (one
+// 128-byte line), the four lane groups take units u, u + 8, u + 16, u + 24, whose permuted slots differ in
+// a bit that the rows' swizzles (a set with that bit fixed) cannot cancel.  EDGE: entries that duplicate the
+// neighbouring tile (tile-relative token < n_lo, vocabulary row < m_lo; both multiples of 4) are left to it.
 template <bool EDGE>
-__device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitParams& p,
-                                                const LanePos& lp, const TilePos& t) {
+__device__ __forceinline__ void dlogit_copy_out_half(const char* stage, int j0, const DlogitParams& p,
+                                                     const LanePos& lp, const TilePos& t) {
   const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
-  const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
-  const int n_base = t.n0 + lp.wn * kWaveTile;
-  const int m_skip = t.m_lo - lp.wm * kWaveTile, n_skip = t.n_lo - lp.wn * kWaveTile;  // sub-tile relative
-  // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
-  // destinations by running pointers (no 64-bit multiplies in the loop).
+  const int m_base = t.m0 + lp.wm * kWaveTile;
+  const int n_base = t.n0 + lp.wn * kWaveTile + j0 * kBlk;
+  const int m_skip = t.m_lo - lp.wm * kWaveTile, n_skip = t.n_lo - lp.wn * kWaveTile - j0 * kBlk;
   {
     const int unit = l32;
     char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
     const int64_t dstep = p.ld_dl * 4;  // two rows of bf16
     const bool col_ok = !EDGE || unit * 4 >= m_skip;
 #pragma unroll 1
-    for (int nw0 = lhi; nw0 < kWaveTile; nw0 += 16) {
+    for (int nw0 = lhi; nw0 < kStashHalfBlocks * kBlk; nw0 += 16) {
       uint2 v[8];
 #pragma unroll
       for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
@@ -488,12 +503,59 @@ __device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitP
       }
     }
   }
+  {
+    const int nq = lp.lane & 15, grp = lp.lane >> 4;
+    const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
+    char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + grp * 32) * p.ld_dlT + n_base + nq * 4);
+    const bool tok_ok = !EDGE || nq * 4 >= n_skip;
+#pragma unroll 2
+    for (int u8 = 0; u8 < 8; ++u8) {
+      const int unit = grp * 8 + u8;
+      uint2 rws[4];
+#pragma unroll
+      for (int f = 0; f < 4; ++f)
+        rws[f] = *reinterpret_cast<const uint2*>(stage + stage_off(nq * 4 + f, unit));
+      uint2 o[4];
+      transpose_4x4_bf16(rws, o);
+      if (tok_ok && (!EDGE || unit * 4 >= m_skip)) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
+      }
+      d += 4 * rstep;
+    }
+  }
+}
+
+// The wave's staged 128 x 128 bf16 sub-tile -> dl (token-major) and dlT (vocab-major).  The wave
+// reads back only what it wrote itself; LDS operations of one wave complete in order.
+__device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitParams& p,
+                                                const LanePos& lp, const TilePos& t) {
+  const int l32 = lp.lane & 31, lhi = lp.lane >> 5;
+  const int m_base = t.m0 + lp.wm * kWaveTile;  // chunk-relative column of the sub-tile
+  const int n_base = t.n0 + lp.wn * kWaveTile;
+  // token-major copy: 32 lanes cover one 256-byte row.  Eight rows per trip, reads before writes;
+  // destinations by running pointers (no 64-bit multiplies in the loop).
+  {
+    const int unit = l32;
+    char* d = reinterpret_cast<char*>(p.dl + (int64_t)(n_base + lhi) * p.ld_dl + m_base + unit * 4);
+    const int64_t dstep = p.ld_dl * 4;  // two rows of bf16
+#pragma unroll 1
+    for (int nw0 = lhi; nw0 < kWaveTile; nw0 += 16) {
+      uint2 v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const uint2*>(stage + stage_off(nw0 + 2 * u, unit));
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        *reinterpret_cast<uint2*>(d) = v[u];
+        d += dstep;
+      }
+    }
+  }
   // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
   {
     const int nq = l32;  // token quad
     const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
     char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + lhi * 4) * p.ld_dlT + n_base + nq * 4);
-    const bool tok_ok = !EDGE || nq * 4 >= n_skip;
 #pragma unroll 2
     for (int unit = lhi; unit < 32; unit += 2) {
       uint2 rws[4];
@@ -501,18 +563,9 @@ __device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitP
       for (int f = 0; f < 4; ++f)
         rws[f] = *reinterpret_cast<const uint2*>(stage + stage_off(nq * 4 + f, unit));
       uint2 o[4];
-      o[0].x = (rws[0].x & 0xffffu) | (rws[1].x << 16);
-      o[0].y = (rws[2].x & 0xffffu) | (rws[3].x << 16);
-      o[1].x = (rws[0].x >> 16) | (rws[1].x & 0xffff0000u);
-      o[1].y = (rws[2].x >> 16) | (rws[3].x & 0xffff0000u);
-      o[2].x = (rws[0].y & 0xffffu) | (rws[1].y << 16);
-      o[2].y = (rws[2].y & 0xffffu) | (rws[3].y << 16);
-      o[3].x = (rws[0].y >> 16) | (rws[1].y & 0xffff0000u);
-      o[3].y = (rws[2].y >> 16) | (rws[3].y & 0xffff0000u);
-      if (tok_ok && (!EDGE || unit * 4 >= m_skip)) {
+      transpose_4x4_bf16(rws, o);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
-      }
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint2*>(d + e * rstep) = o[e];
       d += 8 * rstep;
     }
   }
@@ -535,7 +588,7 @@ __device__ __forceinline__ void dlogit_body(const GemmOperands& g, const DlogitP
     dlogit_stage<SOFTCAP, true>(acc, p, lp, t, stage);
   else
     dlogit_stage<SOFTCAP, false>(acc, p, lp, t, stage);
-  dlogit_copy_out<false>(stage, p, lp, t);
+  dlogit_copy_out(stage, p, lp, t);
 }
 
 template <class Loop>
@@ -552,8 +605,9 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_dlogit_softcap_kernel(Gem
   dlogit_body<Loop, true>(g, p, tiles_m, tiles_n);
 }
 
-// Backward B1 without the recompute: one wavefront per workgroup turns the 128 x 128 sub-tile a
-// stashing forward stored into bf16 dlogits in both orientations.  A streaming kernel: 2 bytes
+// Backward B1 without the recompute: one wavefront per workgroup turns half (64 tokens x 128 rows) of a
+// sub-tile that a stashing forward stored into bf16 dlogits in both orientations (16 KB of LDS and few
+// registers: ten wavefronts per CU hide the latency of the loads and of the per-token operands).  A streaming kernel: 2 bytes
 // read and 4 written per logit.  Tiles are the forward's (same shifted or clamped placement), so
 // `tm0` is the forward tile row of the chunk's first vocabulary row and t.m0 is made chunk-relative
 // only after the edge tests; it is negative only for rows that the tile does not own.
@@ -565,8 +619,8 @@ struct StashSource {
 
 template <bool SOFTCAP>
 __global__ __launch_bounds__(64) void lmhead_dlogit_stash_kernel(DlogitParams p, StashSource src) {
-  __shared__ __align__(16) char stage[32768];
-  const int wave = blockIdx.x & 3, tile = blockIdx.x >> 2;
+  __shared__ __align__(16) char stage[kStashHalfBlocks * kBlk * 256];  // 64 tokens x 128 bf16
+  const int half = blockIdx.x & 1, wave = (blockIdx.x >> 1) & 3, tile = blockIdx.x >> 3;
   const int tm = src.tm0 + tile / src.tiles_n, tn = tile % src.tiles_n;
   TilePos t{tm * kTile, tn * kTile, 0, 0};
   if (src.shifted) {
@@ -579,11 +633,13 @@ __global__ __launch_bounds__(64) void lmhead_dlogit_stash_kernel(DlogitParams p,
   lp.wave = wave;
   lp.wm = wave >> 1;
   lp.wn = wave & 1;
-  const uint4* sv = src.stash + ((int64_t)(tm * src.tiles_n + tn) * 4 + wave) * kStashWaveVecs + lp.lane;
+  const int j0 = half * kStashHalfBlocks;
+  const uint4* sv = src.stash + ((int64_t)(tm * src.tiles_n + tn) * 4 + wave) * kStashWaveVecs +
+                    j0 * 4 * 64 + lp.lane;
   typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-  uint4 st[32];
+  uint4 st[4 * kStashHalfBlocks];
 #pragma unroll
-  for (int q = 0; q < 32; ++q) {  // read once: keep it out of the way of the GEMMs' operands in L2
+  for (int q = 0; q < 4 * kStashHalfBlocks; ++q) {  // read once: keep it out of the way of the GEMMs' operands in L2
     const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sv + q * 64));
     st[q] = make_uint4(x[0], x[1], x[2], x[3]);
   }
@@ -591,11 +647,11 @@ __global__ __launch_bounds__(64) void lmhead_dlogit_stash_kernel(DlogitParams p,
   t.m0 -= p.v_begin;
   const int part = tm * 2 + lp.wm;
   if (edge) {
-    dlogit_stage_stash<SOFTCAP, true>(st, src.pm, part, p, lp, t, stage);
-    dlogit_copy_out<true>(stage, p, lp, t);
+    dlogit_stage_stash<SOFTCAP, true>(st, j0, src.pm, part, p, lp, t, stage);
+    dlogit_copy_out_half<true>(stage, j0, p, lp, t);
   } else {
-    dlogit_stage_stash<SOFTCAP, false>(st, src.pm, part, p, lp, t, stage);
-    dlogit_copy_out<false>(stage, p, lp, t);
+    dlogit_stage_stash<SOFTCAP, false>(st, j0, src.pm, part, p, lp, t, stage);
+    dlogit_copy_out_half<false>(stage, j0, p, lp, t);
   }
 }
 
@@ -1129,7 +1185,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       p.is_start = is_start;
       if (stash) {
         const StashSource src{sw.tiles, sw.pm, sw.tiles_n, (int)(v0 / kTile), sw.shifted};
-        const unsigned blocks = (unsigned)(round_up(vc, kTile) / kTile) * (unsigned)sw.tiles_n * 4u;
+        const unsigned blocks = (unsigned)(round_up(vc, kTile) / kTile) * (unsigned)sw.tiles_n * 8u;
         if (softcap > 0.f)
           hipLaunchKernelGGL(lmhead_dlogit_stash_kernel<true>, dim3(blocks), dim3(64), 0, st, p, src);
         else

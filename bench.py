@@ -42,10 +42,12 @@ def parse_args():
     ap.add_argument("--workload", default="qwen3-8b", choices=sorted(WORKLOADS))
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (debugging)")
     ap.add_argument("--vocab-chunk", type=int, default=0)
-    ap.add_argument("--head-backward", choices=("auto", "stash", "recompute"), default="auto",
-                    help="where the head's backward takes its dlogits from: the forward's stash (2 bytes per "
-                         "logit kept from forward to backward), a recompute of the logits, or the library's own "
-                         "choice (the stash when it fits)")
+    ap.add_argument("--head-backward", choices=("recompute", "stash"), default="recompute",
+                    help="where the headline's backward takes its dlogits from: a recompute of the logits (nothing "
+                         "of size tokens x vocab is ever in memory, as the reference's kernels and the library's "
+                         "default), or the forward's stash (2 bytes per logit kept from forward to backward, opt-in)")
+    ap.add_argument("--no-stash-variant", dest="stash_variant", action="store_false",
+                    help="skip the short second measurement of the same step with the opt-in stash")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
     ap.add_argument("--prompt-fraction", type=float, default=1 / 3,
                     help="after the headline, time the step again with this leading share of every sequence "
@@ -61,7 +63,8 @@ def parse_args():
                          "the fused kernels' main loop (axon_gemm_nt_bf16), then exit: the command the rocprofv3 --pmc "
                          "passes that compare the two are taken on")
     ap.add_argument("--traffic-probe", action="store_true",
-                    help="run a 1 GiB calibration copy, one head forward and one head backward, then exit: the "
+                    help="run a 1 GiB calibration copy, then one head forward and backward on each of the two "
+                         "backward paths (recompute, stash), then exit: the "
                          "command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken on")
     return ap.parse_args()
 
@@ -539,6 +542,40 @@ def baseline_sizes_cold(dev):
     return out
 
 
+def kernel_table(timing, steps, n, h, v, stash_bytes):
+    """Per kernel class of the head: launches and milliseconds per step (HIP events on the launch stream),
+    algorithmic and executed TFLOP/s.  With the forward's stash the backward's first kernel is a streaming one:
+    per logit it reads 2 bytes of stash and writes the bf16 dlogit twice (token-major and vocab-major), and no
+    flop of the path is executed twice; without it that kernel recomputes the logits (2 N H V executed flop that
+    do not count as algorithmic)."""
+    nhv = float(n) * h * v
+    classes = [
+        ("gemm_store_kernel (dHidden + dWeight GEMMs)", ("bwd/dhidden", "bwd/dweight"), 4 * nhv, 4 * nhv, 0.0),
+        ("lmhead_fwd_stash_kernel (logits + online softmax statistics + stash)" if stash_bytes else
+         "lmhead_fwd_kernel (logits + online softmax statistics)", ("fwd/logits_stats",), 2 * nhv, 2 * nhv, 0.0),
+        ("lmhead_dlogit_stash_kernel (stash -> dlogit in both orientations; HBM-bound)", ("bwd/dlogit",), 0.0, 0.0,
+         6.0 * n * v) if stash_bytes else
+        ("lmhead_dlogit_kernel (logit recompute + dlogit)", ("bwd/dlogit",), 0.0, 2 * nhv, 0.0),
+    ]
+    kernels = []
+    for label, keys, algo, execd, hbm_bytes in classes:
+        ms = sum(timing.get(k, {"ms": 0})["ms"] for k in keys)
+        launches = sum(timing.get(k, {"launches": 0})["launches"] for k in keys)
+        if launches == 0:
+            continue
+        kernels.append({
+            "kernel": label, "launches_per_step": launches / steps, "ms_per_step": ms / steps,
+            "avg_launch_ms": ms / launches,
+            "algorithmic_tflops": algo * steps / (ms * 1e-3) / 1e12,
+            "executed_tflops": execd * steps / (ms * 1e-3) / 1e12,
+        })
+        if hbm_bytes:
+            gbps = hbm_bytes * steps / (ms * 1e-3) / 1e9
+            kernels[-1].update({"algorithmic_bytes_per_step": hbm_bytes, "achieved_GBps": gbps,
+                                "frac_of_hbm_peak": gbps / HBM_PEAK_GBS})
+    return kernels
+
+
 def kernel_source_digest():
     """Digest of the sources of the LM-head kernels: ties a committed profile to the code it was taken on."""
     import hashlib
@@ -579,8 +616,11 @@ def traffic_probe(workload):
     src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()  # 1 GiB
     dst = torch.empty_like(src)
     dst.copy_(src)  # calibration kernel: reads 1 GiB, writes 1 GiB
-    _, _, lse, eb, stash = _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)
     g = torch.randn(n, device="cuda")
+    _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)  # the default path: the backward recomputes the logits
+    _ops.lmhead_backward(g, torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0)
+    _ops.LMHEAD_STASH = True  # the opt-in path: the forward's stash, decoded by the backward
+    _, _, lse, eb, stash = _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)
     _ops.lmhead_backward(g, torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0, stash=stash)
     torch.cuda.synchronize()
 
@@ -662,7 +702,7 @@ def main():
         return loss, hg.grad, wg.grad
 
     _ops.DEFAULT_VOCAB_CHUNK = args.vocab_chunk
-    _ops.LMHEAD_STASH = {"auto": "auto", "stash": True, "recompute": False}[args.head_backward]
+    _ops.LMHEAD_STASH = args.head_backward == "stash"
     stash_bytes = _ops._want_stash(n, h, v, torch.device(dev))  # what every timed forward will allocate
     for _ in range(args.warmup):
         step()
@@ -682,6 +722,39 @@ def main():
 
     ms_per_step = 1e3 * elapsed / args.steps
     tokens_per_s = n * args.steps / elapsed
+
+    # Not the headline: the same step with the opt-in stash (the forward keeps 2 bytes per logit, the backward
+    # decodes the dlogits from them instead of recomputing the logits)
+    stash_variant = None
+    if args.stash_variant and not stash_bytes and _ops.lmhead_stash_bytes(n, h, v):
+        _ops.LMHEAD_STASH = True
+        step()
+        torch.cuda.synchronize()
+        timer = _ops.Timer()
+        _ops.set_timing(timer)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            loss_s, dh_s, dw_s = step()
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        _ops.set_timing(None)
+        timing_s = timer.collect()
+        timer.close()
+        _ops.LMHEAD_STASH = False
+        rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()  # noqa: E731
+        stash_variant = {
+            "what": "same step, forward keeps 2 bytes per logit (fp16 softmax numerators) for the backward: "
+                    "6 N H V flop executed instead of 8, tokens x vocab x 2 bytes held from forward to backward",
+            "stash_bytes": _ops.lmhead_stash_bytes(n, h, v), "steps": 3,
+            "ms_per_step": 1e3 * el / 3, "tokens_per_s": 3 * n / el,
+            "path_algorithmic_tflops": 6 * float(n) * h * v / (el / 3) / 1e12,
+            "path_frac_of_peak": 6 * float(n) * h * v / (el / 3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+            "loss": loss_s.item(), "headline_loss": loss.item(),
+            "dhidden_rel_l2_vs_headline": rel(dh_s, dh), "dweight_rel_l2_vs_headline": rel(dw_s, dw),
+            "kernels": kernel_table(timing_s, 3, n, h, v, _ops.lmhead_stash_bytes(n, h, v)),
+        }
+        del loss_s, dh_s, dw_s
+        torch.cuda.empty_cache()
 
     # Not the headline: the same step when the first third of every sequence is prompt (response_mask 0), as in
     # the trainer's batches.  Those positions send exact zeros back into the head, whose backward leaves their
@@ -712,33 +785,8 @@ def main():
     nhv = float(n) * h * v
 
     # kernel classes: (label, timing keys, algorithmic flops per step, executed flops per step)
-    # with the forward's stash the backward's first kernel is a streaming one: per logit it reads 2 bytes of
-    # stash and writes the bf16 dlogit twice (token-major and vocab-major), and no flop of the path is executed twice
     executed = 6 if stash_bytes else 8
-    classes = [
-        ("gemm_store_kernel (dHidden + dWeight GEMMs)", ("bwd/dhidden", "bwd/dweight"), 4 * nhv, 4 * nhv, 0.0),
-        ("lmhead_fwd_stash_kernel (logits + online softmax statistics + stash)" if stash_bytes else
-         "lmhead_fwd_kernel (logits + online softmax statistics)", ("fwd/logits_stats",), 2 * nhv, 2 * nhv, 0.0),
-        ("lmhead_dlogit_stash_kernel (stash -> dlogit in both orientations; HBM-bound)", ("bwd/dlogit",), 0.0, 0.0,
-         6.0 * n * v) if stash_bytes else
-        ("lmhead_dlogit_kernel (logit recompute + dlogit)", ("bwd/dlogit",), 0.0, 2 * nhv, 0.0),
-    ]
-    kernels = []
-    for label, keys, algo, execd, hbm_bytes in classes:
-        ms = sum(timing.get(k, {"ms": 0})["ms"] for k in keys)
-        launches = sum(timing.get(k, {"launches": 0})["launches"] for k in keys)
-        if launches == 0:
-            continue
-        kernels.append({
-            "kernel": label, "launches_per_step": launches / args.steps, "ms_per_step": ms / args.steps,
-            "avg_launch_ms": ms / launches,
-            "algorithmic_tflops": algo * args.steps / (ms * 1e-3) / 1e12,
-            "executed_tflops": execd * args.steps / (ms * 1e-3) / 1e12,
-        })
-        if hbm_bytes:
-            gbps = hbm_bytes * args.steps / (ms * 1e-3) / 1e9
-            kernels[-1].update({"algorithmic_bytes_per_step": hbm_bytes, "achieved_GBps": gbps,
-                                "frac_of_hbm_peak": gbps / HBM_PEAK_GBS})
+    kernels = kernel_table(timing, args.steps, n, h, v, stash_bytes)
     dom = max(kernels, key=lambda k: k["ms_per_step"])
     roofline = {
         "bound": "mfma", "kernel": dom["kernel"], "achieved": dom["algorithmic_tflops"] or dom["executed_tflops"],
@@ -781,6 +829,8 @@ def main():
             f"with the plain GEMM of this run ({best:.0f} TFLOP/s on random operands, "
             f"{best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak: the part runs at its power limit under matrix "
             f"load) the path's ceiling is {share * best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak")
+    if stash_variant:
+        out["stash_variant"] = stash_variant
     if prompt_variant:
         out["prompt_rows_variant"] = prompt_variant
     if args.other_workloads and not args.tokens:

@@ -377,7 +377,9 @@ def test_stash_policy_and_refusals():
     hid, w, lab = W.lmhead_inputs(513, 256, 1500, seed=4)
     hd, wd, ld = hid.to(DEV), w.to(DEV), lab.to(DEV)
     saved = _ops.LMHEAD_STASH
+    assert saved is False  # opt-in: by default nothing of size tokens x vocab is kept
     try:
+        assert _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)[4] is None
         _ops.LMHEAD_STASH = True
         assert _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)[4] is None
         hg, wg = hd.clone().requires_grad_(True), wd.clone().requires_grad_(True)
