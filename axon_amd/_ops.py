@@ -228,11 +228,19 @@ def group_scalar(mode, scores, lens, members, offsets, n_groups, *, eps=1e-6, no
     return out
 
 
-# Operators that need a per-row quantity run as ONE launch in which a workgroup owns whole rows up to this many
-# tokens (any real micro-batch: one launch instead of three or four, and row sums that repeat bit for bit).  That
-# kernel holds 16 tokens per thread across its two phases and runs at about a third of the streaming rate, so
-# beyond this size the token-parallel row pass + token pass is faster (measured crossover: 3-4 M tokens).
-OWNED_ROWS_MAX_SLOTS = 1 << 21
+# Operators that need a per-row quantity run as ONE launch in which a workgroup owns whole rows (one read of every
+# input, row sums that repeat bit for bit) when the rows are long enough to fill a workgroup: it works on one row
+# at a time, so a batch of rows of a few tokens each would leave most of its threads idle.  Otherwise, and beyond
+# ``OWNED_ROWS_MAX_SLOTS`` tokens, a token-parallel row pass followed by a token pass (two reads, float atomics
+# per row).  At 2^26 tokens the two take the same time (0.39 ms); at the sizes of real micro-batches the single
+# launch is 2-3 times faster.
+OWNED_ROWS_MAX_SLOTS = 1 << 40
+OWNED_ROWS_MIN_MEAN_LEN = 64
+
+
+def _own_rows(rows: "Rows") -> bool:
+    return rows.n_slots <= OWNED_ROWS_MAX_SLOTS and rows.n_slots >= OWNED_ROWS_MIN_MEAN_LEN * max(rows.n_rows, 1)
+
 
 IS_MODES = {None: 0, "token": 1, "sequence": 2}
 RS_MODES = {None: 0, "token": 1, "sequence": 2, "geometric": 3}
@@ -241,8 +249,8 @@ RS_MODES = {None: 0, "token": 1, "sequence": 2, "geometric": 3}
 def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_threshold, rs_mode, rs_lr_lo, rs_lr_hi,
                        log_veto):
     """Importance weights and rejection / veto mask.  Without a row-level quantity: one elementwise pass.  With
-    one (veto, sequence or geometric level): one launch in which a workgroup owns whole rows, or, beyond
-    ``OWNED_ROWS_MAX_SLOTS`` tokens, a row-stats pass followed by an elementwise pass.
+    one (veto, sequence or geometric level): one launch in which a workgroup owns whole rows, or (short rows, see
+    ``OWNED_ROWS_MIN_MEAN_LEN``) a row-stats pass followed by an elementwise pass.
 
     Returns (is_weights | None, new_mask fp32, acc[8] device tensor).
     """
@@ -257,7 +265,7 @@ def sampler_correction(old_lp, samp_lp, mask, rows: Rows, *, is_mode, is_thresho
     isw = torch.empty(rows.shape, device=dev, dtype=torch.float32) if is_mode else None
     new_mask = torch.empty(rows.shape, device=dev, dtype=torch.float32)
     acc = _acc8(rows.n_slots, dev)
-    if need_row and rows.n_slots <= OWNED_ROWS_MAX_SLOTS:
+    if need_row and _own_rows(rows):
         # a workgroup owns whole rows: one launch, one pass over the tokens, row sums in a fixed order
         check(
             lib.axon_sampler_correction_rows(ptr(old_lp), ptr(samp_lp), ptr(mk), kind, rows.cu_ptr, rows.n_rows,
@@ -354,7 +362,7 @@ def policy_loss(kind, log_probs, old_log_probs, advantages, mask, is_weights, ro
     nps = _count_dev(num_program_steps, dev, rows.n_rows, "num_program_steps") if br == 2 else None
     if not one_pass and tr == 2 and not rows.uniform_len:
         raise ValueError("token_reduce='mean-norm' divides by the padded row length: needs a [batch, seq] layout")
-    if not one_pass and rows.n_slots <= OWNED_ROWS_MAX_SLOTS:
+    if not one_pass and _own_rows(rows):
         # a workgroup owns whole rows: one launch, still one pass over the tokens
         check(
             lib.axon_policy_loss_rows(kind, ptr(lp), ptr(old), ptr(adv), ptr(mk), mkind, ptr(isw), rows.cu_ptr,

@@ -3,30 +3,28 @@
 // batch_reduce step-mean / program-mean), the per-sequence veto, and sequence-level / geometric
 // importance weights and rejection.
 //
-// A workgroup owns WHOLE rows: range b covers the rows that begin in [b * kOwnStride,
-// (b + 1) * kOwnStride), whatever their length.  It loads the tokens of its rows once (16 per thread,
-// kept in registers), forms the per-row sums in LDS, and then writes the per-token outputs from the
-// registers.  A range longer than the registers hold (a row of more than 2048 tokens in it) is
-// walked in blocks of kOwnTokens and read a second time for the output pass (the re-read follows
-// the first read within microseconds and is mostly served by the L2); the common case reads every
-// input exactly once: 20 bytes per token for GSPO or the veto against 32 for a row pass followed by
-// a token pass.
+// A WORKGROUP owns whole rows.  The slots are cut into as many ranges of `stride` tokens as the
+// launch has workgroups (all resident at once); workgroup b takes the rows that BEGIN in range b,
+// whatever their length, so every workgroup has the same number of tokens up to one row.  A row is
+// walked in chunks of 1024 slots (16 bytes per thread), kRowHold chunks (2048 slots) per wait: the
+// row sums are formed across the workgroup, the per-row values derived from them, and the
+// per-token outputs written from the registers.  A row of more than 2048 slots is read a second
+// time for the output pass, all but its last group (it was read microseconds earlier).  The common
+// case reads every input exactly once: 20 bytes per token for GSPO or the veto against 32 for a
+// row pass followed by a token pass.  Few registers per thread (two chunks) keep six wavefronts per
+// SIMD resident, which is what hides the two waits per row.
 //
-// The per-row sums are formed without atomics and in a fixed order: every wavefront adds the tokens
-// it sees into its own slots in LDS (in program order), and the four wavefronts' slots are added
-// 0 + 1 + 2 + 3.  The sequence ratio, the sequence-level masks and weights are therefore the same
-// on every run.
+// The per-row sums are formed without atomics and in a fixed order (a thread adds its slots chunk
+// by chunk, then the fixed tree of the wavefront sum, then the four wavefronts 0 + 1 + 2 + 3), so
+// the sequence ratio, the sequence-level masks and weights are the same on every run.
 #include "common.h"
 #include "token_math.h"
 
 namespace axon {
 
-constexpr int kOwnStride = 2048;                      // tokens between the starts of two ranges
-constexpr int kOwnIter = 4;                           // 16-byte vectors per thread per block
-constexpr int kOwnTokens = kBlock * kVec * kOwnIter;  // tokens a workgroup holds in registers: 4096
-constexpr int kOwnRows = 128;                         // rows whose sums fit the LDS tables at a time
+constexpr int kRowChunk = kBlock * kVec;  // slots one workgroup instruction covers: 1024
+constexpr int kRowHold = 2;               // chunks of a row kept in registers
 constexpr int kOwnWaves = kBlock / kWave;
-constexpr int kOwnBatch = 64;                         // ranges whose row boundaries are looked up together
 
 struct RowStarts {
   const int32_t* cu;
@@ -48,171 +46,132 @@ struct RowStarts {
   }
 };
 
-// The rows [rs, re) of one segment: their starts in LDS, and the row of a slot by bisection.
-struct Segment {
-  const int32_t* win;  // LDS: win[i] = first slot of row rs + i, i in [0, n]
-  int n;
-  __device__ __forceinline__ int row_of(int p) const {  // largest i < n with win[i] <= p
-    int a = 0, b = n - 1;
-    while (a < b) {
-      const int mid = (a + b + 1) >> 1;
-      if (win[mid] <= p) a = mid; else b = mid - 1;
-    }
-    return a;
-  }
-  __device__ __forceinline__ int end_of(int i) const { return win[i + 1]; }
-};
-
-// Segmented sum across the wavefront (rows sorted across lanes, -1 = no token); `flush(seg)` is
-// called once per run by its first lane.
-template <int NV, class Flush>
-__device__ __forceinline__ void row_seg_wave_reduce(RowSeg<NV> s, Flush&& flush) {
-  const int lane = threadIdx.x & (kWave - 1);
-  const int first = __builtin_amdgcn_readfirstlane(s.row);
-  if (first >= 0 && __builtin_amdgcn_readlane(s.row, kWave - 1) == first) {
-#pragma unroll
-    for (int k = 0; k < NV; ++k) s.v[k] = wave_sum_to_last(s.v[k]);
-    if (lane == kWave - 1) flush(s);
-    return;
-  }
-#pragma unroll
-  for (int off = 1; off < kWave; off <<= 1) {
-    const int r2 = __shfl_down(s.row, off, kWave);
-    float t[NV];
-#pragma unroll
-    for (int k = 0; k < NV; ++k) t[k] = __shfl_down(s.v[k], off, kWave);
-    if (lane + off < kWave && r2 == s.row) {
-#pragma unroll
-      for (int k = 0; k < NV; ++k) s.v[k] += t[k];
+// first_row_from by the whole wavefront: every step probes 64 evenly spaced rows (three dependent loads
+// for 10^5 rows instead of seventeen).  The same value in every lane.
+__device__ __forceinline__ int first_row_from_wave(const RowStarts& rs, int64_t pos, int lane) {
+  if (rs.uniform > 0) return (int)rs.first_row_from(pos);
+  int lo = 0, hi = (int)rs.n_rows;  // the answer lies in [lo, hi]
+  while (hi > lo) {
+    const int step = (hi - lo + kWave - 1) / kWave;
+    const int idx = lo + lane * step;
+    const bool ge = idx >= hi || (int64_t)rs.cu[idx] >= pos;
+    const unsigned long long m = __ballot(ge);
+    if (m == 0ull) {  // every probed row begins before pos
+      lo = lo + (kWave - 1) * step + 1;
+    } else {
+      const int f = __builtin_ctzll(m);
+      hi = min(hi, lo + f * step);
+      if (f > 0) lo = lo + (f - 1) * step + 1;
     }
   }
-  const int prev = __shfl_up(s.row, 1, kWave);
-  if ((lane == 0 || prev != s.row) && s.row >= 0) flush(s);
+  return lo;
 }
 
-// What the two kernels share: the walk over ranges, segments and blocks.  `Op` provides
-//   load(p0, it)                   one vector of four slots starting at p0 into register set `it`
-//   stat(it, j, RowSeg&)           add slot j of register set `it` to the row sums
-//   rows(seg_first_row, i, tot[])  derive the per-row values of local row i from its sums (one thread)
-//   emit(p0, it, ...)              write the outputs of one vector
-// and kNV row sums.  Written as a macro-free template: the kernels below instantiate it.
+__device__ __forceinline__ float wave_total(float v) {  // the same value in every lane
+  v = wave_sum_to_last(v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), kWave - 1));
+}
+
+// What the two kernels share: the walk over ranges, rows and chunks.  `Op` provides
+//   kNV                               number of row sums
+//   load(p0, c)                       the vector of four slots starting at p0 into register set c (every input)
+//   stat(c, j, s[])                   add slot j of register set c to the thread's row sums
+//   rows(r, tot[], first) -> RowVals  the per-row values from the row's sums (every thread the same)
+//   emit(p0, c, rv, t0, t1)           write the outputs of the vector in register set c
+//   fill_gap(a, b)                    zeros for slots that belong to no row
+// Every thread of the workgroup walks the same rows (the loop bounds are uniform), so the barriers
+// inside the loop are reached by all.
 template <class Op>
-__device__ __forceinline__ void walk_owned_rows(const RowStarts& rs_, Op& op) {
+__device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride, Op& op) {
   constexpr int NV = Op::kNV;
-  __shared__ int32_t win[kOwnRows + 1];
-  __shared__ float part[kOwnWaves][kOwnRows][NV];
-  __shared__ int32_t bnd[kOwnBatch][2];
-  const int wave = threadIdx.x / kWave;
-  const int64_t n_ranges = (rs_.n_slots + kOwnStride - 1) / kOwnStride;
-  // this workgroup's ranges: blockIdx.x, blockIdx.x + gridDim.x, ...
-  const int64_t n_mine = (int64_t)blockIdx.x < n_ranges ? (n_ranges - blockIdx.x + gridDim.x - 1) / gridDim.x : 0;
+  __shared__ float red[2][kOwnWaves][NV];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t n_ranges = (rs.n_slots + stride - 1) / stride;  // <= workgroups of the launch
+  // this workgroup's rows: those that begin in [blockIdx.x * stride, range_end).  Only the first is
+  // looked up (by every wavefront, to the same result); the walk ends at the first row that begins
+  // beyond the range.
+  const int64_t range_end = ((int64_t)blockIdx.x >= n_ranges - 1) ? INT64_MAX : ((int64_t)blockIdx.x + 1) * stride;
+  int r = (int)rs.n_rows;
+  if ((int64_t)blockIdx.x < n_ranges)
+    r = (blockIdx.x == 0) ? 0 : first_row_from_wave(rs, (int64_t)blockIdx.x * stride, lane);
+  // row starts, 64 at a time: lane l holds the start of row win0 + l (of row n_rows: the end of the last)
+  int win0 = r;
+  int win = (int)rs.at(min((int64_t)win0 + lane, rs.n_rows));
+  int parity = 0;
 #pragma unroll 1
-  for (int64_t k0 = 0; k0 < n_mine; k0 += kOwnBatch) {
-  // The first and last row of up to kOwnBatch ranges, found by as many threads at once: a bisection
-  // over cu_seqlens is a chain of dependent loads, far too long to sit in front of every range.
-  const int n_batch = (int)min((int64_t)kOwnBatch, n_mine - k0);
-  __syncthreads();
-  if ((int)threadIdx.x < 2 * n_batch) {
-    const int64_t b = blockIdx.x + (k0 + (threadIdx.x >> 1)) * gridDim.x;
-    int64_t r;
-    if ((threadIdx.x & 1) == 0) r = (b == 0) ? 0 : rs_.first_row_from(b * kOwnStride);
-    else r = (b == n_ranges - 1) ? rs_.n_rows : rs_.first_row_from((b + 1) * kOwnStride);
-    bnd[threadIdx.x >> 1][threadIdx.x & 1] = (int32_t)r;
-  }
-  __syncthreads();
+  for (; r < (int)rs.n_rows; ++r) {
+    if (r - win0 >= kWave - 1) {
+      win0 = r;
+      win = (int)rs.at(min((int64_t)win0 + lane, rs.n_rows));
+    }
+    const int k = __builtin_amdgcn_readfirstlane(r - win0);
+    const int t0 = __builtin_amdgcn_readlane(win, k), t1 = __builtin_amdgcn_readlane(win, k + 1);
+    if ((int64_t)t0 >= range_end) break;
+    const int base = t0 & ~3;  // vectors stay 16-byte aligned; slots before t0 are not this row's
+    const int n_chunks = (t1 > t0) ? (t1 - base + kRowChunk - 1) / kRowChunk : 0;
+    const int n_groups = (n_chunks + kRowHold - 1) / kRowHold;
+    const int thread_p = base + (int)threadIdx.x * kVec;
+    float s[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) s[i] = 0.f;
+    // ---- pass 1: the row's sums, kRowHold chunks (one wait) at a time; the registers keep the last group
 #pragma unroll 1
-  for (int kb = 0; kb < n_batch; ++kb) {
-    const int64_t b = blockIdx.x + (k0 + kb) * gridDim.x;
-    const int64_t r0 = bnd[kb][0], r1 = bnd[kb][1];
-#pragma unroll 1
-    for (int64_t rs = r0; rs < r1; rs += kOwnRows) {
-      const int n = (int)min((int64_t)kOwnRows, r1 - rs);
-      __syncthreads();  // the tables of the previous segment are no longer read
-      for (int i = threadIdx.x; i <= n; i += kBlock) win[i] = (int32_t)rs_.at(rs + i);
-      for (int i = threadIdx.x; i < kOwnWaves * kOwnRows * NV; i += kBlock) (&part[0][0][0])[i] = 0.f;
-      __syncthreads();
-      const Segment seg{win, n};
-      const int t0 = win[0], t1 = win[n];
-      const int base = t0 & ~3;  // vectors stay 16-byte aligned; slots before t0 are not ours
-      const int n_blocks = (t1 - base + kOwnTokens - 1) / kOwnTokens;
-      // ---- pass 1: row sums.  The registers keep the last block that was loaded.
-#pragma unroll 1
-      for (int blk = 0; blk < n_blocks; ++blk) {
-        const int b0 = base + blk * kOwnTokens;
+    for (int grp = 0; grp < n_groups; ++grp) {
+      const int c0 = grp * kRowHold;
 #pragma unroll
-        for (int it = 0; it < kOwnIter; ++it) {
-          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
-          if (p0 < t1 && p0 + kVec > t0) op.load(p0, it);
-        }
-#pragma unroll
-        for (int it = 0; it < kOwnIter; ++it) {
-          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
-          RowSeg<NV> s;
-          s.row = -1;
-#pragma unroll
-          for (int k = 0; k < NV; ++k) s.v[k] = 0.f;
-          auto flush = [&](const RowSeg<NV>& f) {
-#pragma unroll
-            for (int k = 0; k < NV; ++k) part[wave][f.row][k] += f.v[k];
-          };
-          if (p0 < t1 && p0 + kVec > t0) {
-            int rend = -1;
-#pragma unroll
-            for (int j = 0; j < kVec; ++j) {
-              const int p = p0 + j;
-              if (p < t0 || p >= t1) continue;
-              if (p >= rend) {
-                if (s.row >= 0) flush(s);
-                s.row = seg.row_of(p);
-                rend = seg.end_of(s.row);
-#pragma unroll
-                for (int k = 0; k < NV; ++k) s.v[k] = 0.f;
-              }
-              op.stat(it, j, s);
-            }
-          }
-          row_seg_wave_reduce<NV>(s, flush);
-        }
+      for (int c = 0; c < kRowHold; ++c) {
+        const int p0 = thread_p + (c0 + c) * kRowChunk;
+        if (p0 < t1 && p0 + kVec > t0) op.load(p0, c);
       }
-      __syncthreads();
-      // ---- the rows of the segment: sums of the four wavefronts in a fixed order -> derived values
-      for (int i = threadIdx.x; i < n; i += kBlock) {
-        float tot[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k) tot[k] = ((part[0][i][k] + part[1][i][k]) + part[2][i][k]) + part[3][i][k];
-        op.rows(rs + i, i, tot);
-      }
-      __syncthreads();
-      // ---- pass 2: outputs, last block first (its inputs are still in the registers)
-#pragma unroll 1
-      for (int blk = n_blocks - 1; blk >= 0; --blk) {
-        const int b0 = base + blk * kOwnTokens;
-        if (blk != n_blocks - 1) {
+      for (int c = 0; c < kRowHold; ++c) {
+        const int p0 = thread_p + (c0 + c) * kRowChunk;
+        if (p0 >= t0 && p0 + kVec <= t1) {  // the whole vector belongs to the row
 #pragma unroll
-          for (int it = 0; it < kOwnIter; ++it) {
-            const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
-            if (p0 < t1 && p0 + kVec > t0) op.load(p0, it);
-          }
-        }
-#ifdef AXON_EXP_LATE
+          for (int j = 0; j < kVec; ++j) op.stat(c, j, s);
+        } else if (p0 < t1 && p0 + kVec > t0) {
 #pragma unroll
-        for (int it = 0; it < kOwnIter; ++it) {
-          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
-          if (p0 < t1 && p0 + kVec > t0) op.load_late(p0, it);
-        }
-#endif
-#pragma unroll
-        for (int it = 0; it < kOwnIter; ++it) {
-          const int p0 = b0 + (it * kBlock + (int)threadIdx.x) * kVec;
-          if (p0 < t1 && p0 + kVec > t0) op.emit(p0, it, seg, t0, t1);
+          for (int j = 0; j < kVec; ++j)
+            if (p0 + j >= t0 && p0 + j < t1) op.stat(c, j, s);
         }
       }
     }
-    // slots outside every row (before the first row's start, after the last row's end) belong to no
-    // sequence: the first and the last range write zeros there
-    if (b == 0) op.fill_gap(0, rs_.at(0));
-    if (b == n_ranges - 1) op.fill_gap(rs_.at(rs_.n_rows), rs_.n_slots);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) s[i] = wave_total(s[i]);
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) red[parity][wave][i] = s[i];
+    }
+    __syncthreads();  // one barrier per row: the next row writes the other half of `red`
+    float tot[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+      tot[i] = ((red[parity][0][i] + red[parity][1][i]) + red[parity][2][i]) + red[parity][3][i];
+    parity ^= 1;
+    const auto rv = op.rows(r, tot, threadIdx.x == 0);
+    // ---- pass 2: outputs, last group first (its inputs are still in the registers)
+#pragma unroll 1
+    for (int grp = n_groups - 1; grp >= 0; --grp) {
+      const int c0 = grp * kRowHold;
+      if (grp != n_groups - 1) {
+#pragma unroll
+        for (int c = 0; c < kRowHold; ++c) {
+          const int p0 = thread_p + (c0 + c) * kRowChunk;
+          if (p0 < t1 && p0 + kVec > t0) op.load(p0, c);
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) {
+        const int p0 = thread_p + (c0 + c) * kRowChunk;
+        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, c, rv, t0, t1);
+      }
+    }
   }
+  // slots outside every row (before the first row's start, after the last row's end) belong to no
+  // sequence: one workgroup writes zeros there
+  if (blockIdx.x == 0) {
+    op.fill_gap(0, rs.at(0));
+    op.fill_gap(rs.at(rs.n_rows), rs.n_slots);
   }
 }
 
@@ -254,67 +213,54 @@ struct OwnedLossArgs {
 template <int MK, int KIND>
 struct OwnedLossOp {
   static constexpr int kNV = 2;  // sum mask, sum (logp - old) * mask
+  struct RowVals { float scale, sbar; };
   const OwnedLossArgs& g;
   const RowStarts& rs;
-  float (*rowv)[2];  // LDS [kOwnRows]: scale, mean log-ratio
-  float bden;        // the batch denominator when the caller supplied it
-  float lv[kOwnIter][4], ov[kOwnIter][4], mv[kOwnIter][4], av[kOwnIter][4], wv[kOwnIter][4];
+  float bden;  // the batch denominator when the caller supplied it
+  float lv[kRowHold][4], ov[kRowHold][4], mv[kRowHold][4], av[kRowHold][4], wv[kRowHold][4];
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float rows_with_tokens = 0.f;
 
-  __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float (*rowv_)[2], float bd)
-      : g(g_), rs(rs_), rowv(rowv_), bden(bd) {}
+  __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float bd)
+      : g(g_), rs(rs_), bden(bd) {}
 
-  __device__ __forceinline__ void load(int p0, int it) {
-    load4_guard(g.logp, p0, rs.n_slots, lv[it]);
-    load4_guard(g.oldp, p0, rs.n_slots, ov[it]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[it]);
-#ifndef AXON_EXP_LATE
-    load_late(p0, it);
-#endif
+  __device__ __forceinline__ void load(int p0, int c) {
+    load4_guard(g.logp, p0, rs.n_slots, lv[c]);
+    load4_guard(g.oldp, p0, rs.n_slots, ov[c]);
+    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[c]);
+    // read by the output pass only, requested with the rest so that one wait covers all
+    load4_guard(g.adv, p0, rs.n_slots, av[c]);
+    if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[c]);
+    else wv[c][0] = wv[c][1] = wv[c][2] = wv[c][3] = 1.f;
   }
-  // read by the output pass only
-  __device__ __forceinline__ void load_late(int p0, int it) {
-    load4_guard(g.adv, p0, rs.n_slots, av[it]);
-    if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[it]);
-    else wv[it][0] = wv[it][1] = wv[it][2] = wv[it][3] = 1.f;
-  }
-  __device__ __forceinline__ void stat(int it, int j, RowSeg<2>& s) const {
-    const float m = mv[it][j];
-    s.v[0] += m;
+  __device__ __forceinline__ void stat(int c, int j, float (&s)[2]) const {
+    const float m = mv[c][j];
+    s[0] += m;
     // masked sum: values outside the mask never reach it (NaN / Inf in padding)
-    s.v[1] += (m != 0.f) ? (lv[it][j] - ov[it][j]) * m : 0.f;
+    s[1] += (m != 0.f) ? (lv[c][j] - ov[c][j]) * m : 0.f;
   }
-  __device__ __forceinline__ void rows(int64_t r, int i, const float (&tot)[2]) {
+  __device__ __forceinline__ RowVals rows(int64_t r, const float (&tot)[2], bool first) {
     const float c = tot[0];
     float td = 1.f;
     if (g.token_reduce == 1) td = fmaxf(g.prtc ? (float)g.prtc[r] : c, 1.f);
     if (g.token_reduce == 2) td = (float)rs.uniform;
     if (g.token_reduce == 3) td = fmaxf((float)g.npt[r], 1.f);
     if (g.batch_reduce == 2) td *= fmaxf((float)g.nps[r], 1.f);
+    rows_with_tokens += (first && c > 0.f) ? 1.f : 0.f;
     // with the batch denominator known this is the scale of the two-pass path, 1 / (td * bden)
-    rowv[i][0] = (g.valid != nullptr) ? 1.f / (td * bden) : 1.f / td;
-    rowv[i][1] = tot[1] / fmaxf(c, 1.f);
-    rows_with_tokens += (c > 0.f) ? 1.f : 0.f;
+    return RowVals{(g.valid != nullptr) ? 1.f / (td * bden) : 1.f / td, tot[1] / fmaxf(c, 1.f)};
   }
-  __device__ __forceinline__ void emit(int p0, int it, const Segment& seg, int t0, int t1) {
+  __device__ __forceinline__ void emit(int p0, int c, const RowVals& rv, int t0, int t1) {
+    const bool whole = p0 >= t0 && p0 + kVec <= t1;
     float gv[4];
-    int rend = -1;
-    float scale = 0.f, sbar = 0.f;
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
       const int p = p0 + j;
       gv[j] = 0.f;
-      if (p < t0 || p >= t1) continue;
-      if (p >= rend) {
-        const int i = seg.row_of(p);
-        rend = seg.end_of(i);
-        scale = rowv[i][0];
-        sbar = rowv[i][1];
-      }
+      if (!whole && (p < t0 || p >= t1)) continue;
       const TokenTerm t =
-          policy_token<KIND>(lv[it][j], ov[it][j], av[it][j], wv[it][j], sbar, g.lo, g.hi, g.clip_c, false);
-      gv[j] = accumulate_token(t, mv[it][j], scale, a);
+          policy_token<KIND>(lv[c][j], ov[c][j], av[c][j], wv[c][j], rv.sbar, g.lo, g.hi, g.clip_c, false);
+      gv[j] = accumulate_token(t, mv[c][j], rv.scale, a);
     }
     store4_range(g.grad, p0, t0, t1, gv);
   }
@@ -322,14 +268,13 @@ struct OwnedLossOp {
 };
 
 template <int MK, int KIND>
-__global__ __launch_bounds__(kBlock) void owned_policy_loss_kernel(OwnedLossArgs g, RowStarts rs, float* ws,
-                                                                   float* __restrict__ acc) {
-  __shared__ float rowv[kOwnRows][2];
+__global__ __launch_bounds__(kBlock) void owned_policy_loss_kernel(OwnedLossArgs g, RowStarts rs, int stride,
+                                                                   float* ws, float* __restrict__ acc) {
   __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   // a caller-supplied batch denominator (utils.py:224-229) is known before the first token
   const float bden = (g.valid != nullptr) ? fmaxf((float)g.valid[0], 1.f) : 1.f;
-  OwnedLossOp<MK, KIND> op(g, rs, rowv, bden);
-  walk_owned_rows(rs, op);
+  OwnedLossOp<MK, KIND> op(g, rs, bden);
+  walk_owned_rows(rs, stride, op);
   float part[7] = {op.a[0], op.a[1], op.a[2], op.a[3], op.a[4], 0.f, op.rows_with_tokens};
   const int batch_reduce = g.batch_reduce;
   const bool known = (g.valid != nullptr);
@@ -363,53 +308,47 @@ struct OwnedCorrArgs {
 template <int MK>
 struct OwnedCorrOp {
   static constexpr int kNV = 3;  // sum mask, sum (old - sampler) * mask, tokens under the veto threshold
+  typedef CorrRow RowVals;
   const OwnedCorrArgs& g;
   const RowStarts& rs;
-  CorrRow* rowv;  // LDS [kOwnRows]
-  float ov[kOwnIter][4], sv[kOwnIter][4], mv[kOwnIter][4];
+  float ov[kRowHold][4], sv[kRowHold][4], mv[kRowHold][4];
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float vetoed_rows = 0.f;
 
-  __device__ __forceinline__ OwnedCorrOp(const OwnedCorrArgs& g_, const RowStarts& rs_, CorrRow* rowv_)
-      : g(g_), rs(rs_), rowv(rowv_) {}
+  __device__ __forceinline__ OwnedCorrOp(const OwnedCorrArgs& g_, const RowStarts& rs_) : g(g_), rs(rs_) {}
 
-  __device__ __forceinline__ void load(int p0, int it) {
-    load4_guard(g.oldp, p0, rs.n_slots, ov[it]);
-    load4_guard(g.samp, p0, rs.n_slots, sv[it]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[it]);
+  __device__ __forceinline__ void load(int p0, int c) {
+    load4_guard(g.oldp, p0, rs.n_slots, ov[c]);
+    load4_guard(g.samp, p0, rs.n_slots, sv[c]);
+    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[c]);
   }
-  __device__ __forceinline__ void load_late(int, int) {}
-  __device__ __forceinline__ void stat(int it, int j, RowSeg<3>& s) const {
-    const float m = mv[it][j];
-    const float d = ov[it][j] - sv[it][j];
-    s.v[0] += m;
-    s.v[1] += (m != 0.f) ? d * m : 0.f;
-    s.v[2] += (g.cfg.has_veto && m != 0.f && d < g.cfg.log_veto) ? 1.f : 0.f;
+  __device__ __forceinline__ void stat(int c, int j, float (&s)[3]) const {
+    const float m = mv[c][j];
+    const float d = ov[c][j] - sv[c][j];
+    s[0] += m;
+    s[1] += (m != 0.f) ? d * m : 0.f;
+    s[2] += (g.cfg.has_veto && m != 0.f && d < g.cfg.log_veto) ? 1.f : 0.f;
   }
-  __device__ __forceinline__ void rows(int64_t r, int i, const float (&tot)[3]) {
+  __device__ __forceinline__ RowVals rows(int64_t r, const float (&tot)[3], bool first) {
     const bool vetoed = tot[2] > 0.f;
-    rowv[i] = corr_row(g.cfg, tot[1], tot[0], vetoed);
-    vetoed_rows += (g.cfg.has_veto && vetoed) ? 1.f : 0.f;
-    if (g.row_cnt) g.row_cnt[r] = tot[0];
-    if (g.row_sum) g.row_sum[r] = tot[1];
-    if (g.row_flag) g.row_flag[r] = vetoed ? 1 : 0;
+    vetoed_rows += (first && g.cfg.has_veto && vetoed) ? 1.f : 0.f;
+    if (first) {
+      if (g.row_cnt) g.row_cnt[r] = tot[0];
+      if (g.row_sum) g.row_sum[r] = tot[1];
+      if (g.row_flag) g.row_flag[r] = vetoed ? 1 : 0;
+    }
+    return corr_row(g.cfg, tot[1], tot[0], vetoed);
   }
-  __device__ __forceinline__ void emit(int p0, int it, const Segment& seg, int t0, int t1) {
+  __device__ __forceinline__ void emit(int p0, int c, const RowVals& row, int t0, int t1) {
+    const bool whole = p0 >= t0 && p0 + kVec <= t1;
     float wv[4], nm[4];
-    int rend = -1;
-    CorrRow row{0.f, 1.f, 1.f};
 #pragma unroll
     for (int j = 0; j < kVec; ++j) {
       const int p = p0 + j;
       wv[j] = 0.f;
       nm[j] = 0.f;
-      if (p < t0 || p >= t1) continue;
-      if (p >= rend) {
-        const int i = seg.row_of(p);
-        rend = seg.end_of(i);
-        row = rowv[i];
-      }
-      corr_token(g.cfg, row, ov[it][j], sv[it][j], mv[it][j], wv[j], nm[j], a);
+      if (!whole && (p < t0 || p >= t1)) continue;
+      corr_token(g.cfg, row, ov[c][j], sv[c][j], mv[c][j], wv[j], nm[j], a);
     }
     if (g.isw) store4_range(g.isw, p0, t0, t1, wv);
     store4_range(g.new_mask, p0, t0, t1, nm);
@@ -421,12 +360,11 @@ struct OwnedCorrOp {
 };
 
 template <int MK>
-__global__ __launch_bounds__(kBlock) void owned_correction_kernel(OwnedCorrArgs g, RowStarts rs, float* ws,
-                                                                  float* __restrict__ acc) {
-  __shared__ CorrRow rowv[kOwnRows];
+__global__ __launch_bounds__(kBlock) void owned_correction_kernel(OwnedCorrArgs g, RowStarts rs, int stride,
+                                                                  float* ws, float* __restrict__ acc) {
   __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
-  OwnedCorrOp<MK> op(g, rs, rowv);
-  walk_owned_rows(rs, op);
+  OwnedCorrOp<MK> op(g, rs);
+  walk_owned_rows(rs, stride, op);
   float part[6] = {op.a[0], op.a[1], op.a[2], op.a[3], op.vetoed_rows, op.a[5]};
   grid_finish<6>(part, lds_red, ws, [&](float (&tot)[kPartialStride]) {
     for (int k = 0; k < kPartialStride; ++k) acc[k] = tot[k];
@@ -439,16 +377,34 @@ using namespace axon;
 
 namespace {
 
-// one resident wave of workgroups per launch keeps the number of partial rows small; the ranges are
-// short (2048 tokens), so the walk balances itself
-unsigned owned_grid(int64_t n_slots) {
-  const int64_t ranges = (n_slots + kOwnStride - 1) / kOwnStride;
-  return (unsigned)(ranges < kStreamGridCap ? ranges : kStreamGridCap);
+// Ranges and workgroups of a launch: one range per workgroup, as many workgroups as are resident at
+// once (a workgroup that had to wait for a free slot would start its range late), ranges of at
+// least one chunk.
+struct OwnedLaunch {
+  int stride;
+  unsigned grid;
+};
+template <typename K>
+int resident_blocks(K kernel) {  // 0 when the runtime cannot say
+  int dev = 0, cus = 0, per_cu = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kernel), kBlock, 0) !=
+      hipSuccess)
+    return 0;
+  return cus * per_cu;
+}
+OwnedLaunch owned_launch(int64_t n_slots, int resident) {
+  const int64_t max_blocks = resident > 0 ? resident : 1024;
+  int64_t stride = (n_slots + max_blocks - 1) / max_blocks;
+  stride = (stride + kVec - 1) / kVec * kVec;
+  if (stride < kRowChunk) stride = kRowChunk;
+  return OwnedLaunch{(int)stride, (unsigned)((n_slots + stride - 1) / stride)};
 }
 
 int check_owned_rows(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len) {
   if (n_rows < 0 || n_slots < 0 || uniform_len < 0) return AXON_ERR_ARG;
-  if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX - kOwnTokens) return AXON_ERR_SHAPE;
+  if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX - 4 * kRowChunk) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;  // slots without rows
@@ -476,10 +432,14 @@ extern "C" int axon_policy_loss_rows(int kind, const float* logp, const float* o
   const OwnedLossArgs g{logp, oldp, adv, isw, mask, token_reduce, batch_reduce, prtc, npt, nps, valid,
                         ratio_lo, ratio_hi, clip_c, grad};
   const RowStarts rs{cu, uniform_len, n_rows, n_slots};
-  const dim3 grid(owned_grid(n_slots)), blk(kBlock);
   const hipStream_t st = (hipStream_t)stream;
-#define AXON_LAUNCH_OWNED(MK, KD) \
-  hipLaunchKernelGGL((owned_policy_loss_kernel<MK, KD>), grid, blk, 0, st, g, rs, partials, acc)
+#define AXON_LAUNCH_OWNED(MK, KD)                                                                       \
+  do {                                                                                                  \
+    static const int resident = resident_blocks(owned_policy_loss_kernel<MK, KD>);                      \
+    const OwnedLaunch ol = owned_launch(n_slots, resident);                                             \
+    hipLaunchKernelGGL((owned_policy_loss_kernel<MK, KD>), dim3(ol.grid), dim3(kBlock), 0, st, g, rs,   \
+                       ol.stride, partials, acc);                                                       \
+  } while (0)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_OWNED(AXON_MASK_F32, 0);
     else if (kind == 1) AXON_LAUNCH_OWNED(AXON_MASK_F32, 1);
@@ -514,13 +474,17 @@ extern "C" int axon_sampler_correction_rows(const float* oldp, const float* samp
   const OwnedCorrArgs g{oldp, samp, mask, CorrCfg{is_mode, is_thr, rs_mode, rs_lo, rs_hi, has_veto, log_veto},
                         isw, new_mask, row_cnt, row_sum, row_flag};
   const RowStarts rs{cu, uniform_len, n_rows, n_slots};
-  const dim3 grid(owned_grid(n_slots)), blk(kBlock);
-  if (mask_kind == AXON_MASK_F32)
-    hipLaunchKernelGGL(owned_correction_kernel<AXON_MASK_F32>, grid, blk, 0, (hipStream_t)stream, g, rs,
-                       partials, acc);
-  else
-    hipLaunchKernelGGL(owned_correction_kernel<AXON_MASK_I64>, grid, blk, 0, (hipStream_t)stream, g, rs,
-                       partials, acc);
+  if (mask_kind == AXON_MASK_F32) {
+    static const int resident = resident_blocks(owned_correction_kernel<AXON_MASK_F32>);
+    const OwnedLaunch ol = owned_launch(n_slots, resident);
+    hipLaunchKernelGGL(owned_correction_kernel<AXON_MASK_F32>, dim3(ol.grid), dim3(kBlock), 0,
+                       (hipStream_t)stream, g, rs, ol.stride, partials, acc);
+  } else {
+    static const int resident = resident_blocks(owned_correction_kernel<AXON_MASK_I64>);
+    const OwnedLaunch ol = owned_launch(n_slots, resident);
+    hipLaunchKernelGGL(owned_correction_kernel<AXON_MASK_I64>, dim3(ol.grid), dim3(kBlock), 0,
+                       (hipStream_t)stream, g, rs, ol.stride, partials, acc);
+  }
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }

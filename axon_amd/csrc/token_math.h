@@ -9,10 +9,12 @@ namespace axon {
 // max/min with PyTorch's gradient convention: ties split the gradient evenly.
 struct ValGrad { float v, g; };
 __device__ __forceinline__ ValGrad vg_max(ValGrad a, ValGrad b) {
-  if (a.v > b.v) return a;
-  if (a.v < b.v) return b;
-  if (a.v == b.v) return ValGrad{a.v, 0.5f * (a.g + b.g)};
-  return ValGrad{a.v + b.v, 0.f};  // NaN operand: propagate
+  // selects, not branches: the four outcomes cost a handful of instructions each, a divergent
+  // branch per token costs more than all of them
+  const bool gt = a.v > b.v, lt = a.v < b.v, eq = a.v == b.v;
+  const float v_tie = eq ? a.v : a.v + b.v;          // NaN operand: propagate
+  const float g_tie = eq ? 0.5f * (a.g + b.g) : 0.f;
+  return ValGrad{gt ? a.v : (lt ? b.v : v_tie), gt ? a.g : (lt ? b.g : g_tie)};
 }
 
 // One token of a policy loss.  vw / gw: loss term and its derivative w.r.t. log_prob, already times
@@ -97,10 +99,11 @@ __device__ __forceinline__ TokenTerm policy_token(float lp, float old, float A, 
   if (KIND == 0) {
     const float pg3 = -A * clip_c;
     t.c3 = (c.v > pg3 && A < 0.f) ? 1.f : 0.f;
-    if (A < 0.f) {  // torch.min(pg3, c1), pg3 carries no gradient
-      if (pg3 < c.v) c = ValGrad{pg3, 0.f};
-      else if (pg3 == c.v) c = ValGrad{c.v, 0.5f * c.g};
-      else if (!(pg3 > c.v)) c = ValGrad{pg3 + c.v, 0.f};
+    {  // A < 0: torch.min(pg3, c1), pg3 carries no gradient (selects: see vg_max)
+      const bool neg = A < 0.f, lt = pg3 < c.v, eq = pg3 == c.v, gt = pg3 > c.v;
+      const float v_min = lt ? pg3 : (eq ? c.v : (gt ? c.v : pg3 + c.v));
+      const float g_min = lt ? 0.f : (eq ? 0.5f * c.g : (gt ? c.g : 0.f));
+      c = ValGrad{neg ? v_min : c.v, neg ? g_min : c.g};
     }
   }
   t.vw = c.v * w;

@@ -398,8 +398,8 @@ def hbm_kernels(n_tokens, dev, only=None):
             ts.append(a.elapsed_time(b) / inner)
         return sorted(ts)[len(ts) // 2]
 
-    def forced_owned(fn):
-        keep, _ops.OWNED_ROWS_MAX_SLOTS = _ops.OWNED_ROWS_MAX_SLOTS, 1 << 40
+    def forced_two_pass(fn):
+        keep, _ops.OWNED_ROWS_MAX_SLOTS = _ops.OWNED_ROWS_MAX_SLOTS, 0
         try:
             return fn()
         finally:
@@ -413,20 +413,21 @@ def hbm_kernels(n_tokens, dev, only=None):
         ("device-to-device copy (calibration)", 8, lambda: x.copy_(old)),
         ("policy_loss_kernel: PPO/DAPO loss + gradient, sum/token-mean (one pass)", 20,
          lambda: _ops.policy_loss(0, new, old, adv, mask, None, rows, **ppo)),
-        ("row_stats + policy_loss_kernel: GSPO loss + gradient (two reads of log_probs, old, mask; the path taken "
-         "beyond 2^21 tokens)", 32, lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
         ("owned_policy_loss_kernel: GSPO loss + gradient in one launch and one read, a workgroup owns whole "
-         "sequences (the path taken up to 2^21 tokens, forced here)", 20,
-         lambda: forced_owned(lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo))),
+         "sequences (the path taken unless the rows are short)", 20,
+         lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo)),
+        ("row_stats + policy_loss_kernel: GSPO loss + gradient (two reads of log_probs, old, mask; the path for "
+         "batches of short rows, forced here)", 32,
+         lambda: forced_two_pass(lambda: _ops.policy_loss(1, new, old, adv, mask, None, rows, **gspo))),
         ("sampler_correction_kernel: token IS weights + rejection mask", 20,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=None, **corr)),
-        ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads; the path taken "
-         "beyond 2^21 tokens)", 32,
+        ("owned_correction_kernel: IS + rejection + per-sequence veto in one launch and one read (the path taken "
+         "unless the rows are short)", 20,
          lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4), **corr)),
-        ("owned_correction_kernel: IS + rejection + per-sequence veto in one launch and one read (the path taken up "
-         "to 2^21 tokens, forced here)", 20,
-         lambda: forced_owned(lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4),
-                                                              **corr))),
+        ("row_stats + sampler_correction_kernel: IS + rejection + per-sequence veto (two reads; the path for batches "
+         "of short rows, forced here)", 32,
+         lambda: forced_two_pass(lambda: _ops.sampler_correction(old, samp, mask, rows, log_veto=math.log(1e-4),
+                                                                 **corr))),
         ("row_stats_kernel: per-sequence count and masked sum", 12, lambda: _ops.row_stats(new, old, mask, rows)),
         ("sampler_diag kernels: all IS / rejection / off-policy / mismatch diagnostics (token pass + row pass)", 12,
          lambda: _ops.sampler_diag(old, samp, mask, rows, is_mode=1, is_lo=0.5, is_hi=2.0, rs_mode=1, rs_lo=0.5,

@@ -246,10 +246,11 @@ def test_ppo_config1_vs_oracle(mask_dtype):
 @pytest.fixture(params=["one_launch", "two_pass"])
 def row_path(request):
     """Operators with a per-row quantity have two implementations, chosen by batch size: run the test on both."""
-    keep = _ops.OWNED_ROWS_MAX_SLOTS
-    _ops.OWNED_ROWS_MAX_SLOTS = keep if request.param == "one_launch" else 0
+    keep = _ops.OWNED_ROWS_MAX_SLOTS, _ops.OWNED_ROWS_MIN_MEAN_LEN
+    _ops.OWNED_ROWS_MAX_SLOTS = keep[0] if request.param == "one_launch" else 0
+    _ops.OWNED_ROWS_MIN_MEAN_LEN = 0  # rows of any length, also the short ones the dispatch would send elsewhere
     yield request.param
-    _ops.OWNED_ROWS_MAX_SLOTS = keep
+    _ops.OWNED_ROWS_MAX_SLOTS, _ops.OWNED_ROWS_MIN_MEAN_LEN = keep
 
 
 @pytest.mark.parametrize("tr,br", [("sum", "token-mean"), ("mean", "step-mean"), ("sum", "step-mean"),
