@@ -26,6 +26,18 @@ __device__ __forceinline__ float clampf(float x, float lo, float hi) {
   return (x != x) ? x : fminf(fmaxf(x, lo), hi);
 }
 
+// expf for an argument already clamped into [-20, 20] (or NaN, which propagates): the same steps and
+// the same bits as expf's (product with log2 e in two parts, round to nearest integer, 2^fraction,
+// scale by 2^integer) without its tests for overflow and underflow, five instructions fewer per token.
+__device__ __forceinline__ float exp_bounded(float x) {
+  constexpr float kLog2eHi = 0x1.715476p+0f, kLog2eLo = 0x1.4ae0bep-26f;
+  const float t = x * kLog2eHi;
+  float e = fmaf(x, kLog2eHi, -t);
+  const float n = rintf(t);
+  e = fmaf(x, kLog2eLo, e);
+  return ldexpf(__builtin_amdgcn_exp2f((t - n) + e), (int)n);
+}
+
 // State of a top-k selection over 32-bit keys (largest keys win; key 0 never wins).  A token i is
 // selected when key > threshold, or key == threshold and i < index_limit (ties go to the lowest indices).
 struct SelectState {

@@ -1,6 +1,8 @@
 // (c) Elementwise stage-2/3 kernels: sampler correction and the clipped policy
 // loss with its gradient.  One read of every input, one write of every output;
 // scalar sums leave through per-workgroup partials that the last workgroup adds up.
+#include <type_traits>
+
 #include "common.h"
 #include "token_math.h"
 #include <mutex>
@@ -213,15 +215,18 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
     }
   };
   // the per-token arithmetic on one vector of four slots
-  auto process = [&](int64_t i, bool full, const float (&lv)[4], const float (&ov)[4], const float (&av)[4],
+  // (full_c: a compile-time true where every slot of the vector exists, so that the common path carries
+  // no test per token)
+  auto process = [&](int64_t i, auto full_c, const float (&lv)[4], const float (&ov)[4], const float (&av)[4],
                      const float (&mv)[4], const float (&wv)[4]) {
+    constexpr bool full = decltype(full_c)::value;
     float gv[4];
     int64_t rend = -1;
     float scale = uniform_scale, sbar = 0.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int64_t p = i + j;
-      if (p >= n_slots) { gv[j] = 0.f; continue; }
+      if (!full && p >= n_slots) { gv[j] = 0.f; continue; }
       if (need_row && p >= rend) {
         const int r = rf.row(p);
         rend = rf.row_end(r);
@@ -258,8 +263,8 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
       if (b0 == 0) find_rows();
 #pragma unroll
       for (int it = 0; it < kB; ++it)
-        process(c0 + ((int64_t)(b0 + it) * kBlock + threadIdx.x) * kVec, true, lv[it], ov[it], av[it], mv[it],
-                wv[it]);
+        process(c0 + ((int64_t)(b0 + it) * kBlock + threadIdx.x) * kVec, std::true_type{}, lv[it], ov[it], av[it],
+                mv[it], wv[it]);
     }
   } else {
     find_rows();
@@ -285,7 +290,7 @@ __global__ __launch_bounds__(kBlock) void policy_loss_kernel(
           wv[j] = (ok && isw) ? isw[i + j] : 1.f;
         }
       }
-      process(i, full, lv, ov, av, mv, wv);
+      process(i, std::false_type{}, lv, ov, av, mv, wv);
     }
   }
   }  // chunk

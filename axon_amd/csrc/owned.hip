@@ -11,12 +11,14 @@
 // per-token outputs written from the registers.  A row of more than 2048 slots is read a second
 // time for the output pass, all but its last group (it was read microseconds earlier).  The common
 // case reads every input exactly once: 20 bytes per token for GSPO or the veto against 32 for a
-// row pass followed by a token pass.  Few registers per thread (two chunks) keep six wavefronts per
-// SIMD resident, which is what hides the two waits per row.
+// row pass followed by a token pass.  The first group of the next row is requested before the
+// current row is worked on (two banks of two chunks in registers).
 //
 // The per-row sums are formed without atomics and in a fixed order (a thread adds its slots chunk
 // by chunk, then the fixed tree of the wavefront sum, then the four wavefronts 0 + 1 + 2 + 3), so
 // the sequence ratio, the sequence-level masks and weights are the same on every run.
+#include <type_traits>
+
 #include "common.h"
 #include "token_math.h"
 
@@ -74,40 +76,60 @@ __device__ __forceinline__ float wave_total(float v) {  // the same value in eve
 
 // What the two kernels share: the walk over ranges, rows and chunks.  `Op` provides
 //   kNV                               number of row sums
-//   load(p0, c)                       the vector of four slots starting at p0 into register set c (every input)
-//   stat(c, j, s[])                   add slot j of register set c to the thread's row sums
+//   load(p0, b, c)                    the vector of four slots starting at p0 into register set (b, c) (every input)
+//   stat(b, c, j, s[])                add slot j of register set (b, c) to the thread's row sums
 //   rows(r, tot[], first) -> RowVals  the per-row values from the row's sums (every thread the same)
-//   emit(p0, c, rv, t0, t1)           write the outputs of the vector in register set c
+//   emit(p0, b, c, rv, t0, t1)        write the outputs of the vector in register set (b, c)
 //   fill_gap(a, b)                    zeros for slots that belong to no row
-// Every thread of the workgroup walks the same rows (the loop bounds are uniform), so the barriers
-// inside the loop are reached by all.
+// Two banks of register sets: while a row is worked on in one bank, the first group of the next row
+// is already on its way into the other, so a row's loads have a whole row's time to arrive.  Every
+// thread of the workgroup walks the same rows (the loop bounds are uniform), so the barrier inside
+// the loop is reached by all; it waits for LDS only, not for the loads in flight.
 template <class Op>
 __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride, Op& op) {
   constexpr int NV = Op::kNV;
   __shared__ float red[2][kOwnWaves][NV];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int n_rows = (int)rs.n_rows;
   const int64_t n_ranges = (rs.n_slots + stride - 1) / stride;  // <= workgroups of the launch
   // this workgroup's rows: those that begin in [blockIdx.x * stride, range_end).  Only the first is
   // looked up (by every wavefront, to the same result); the walk ends at the first row that begins
   // beyond the range.
   const int64_t range_end = ((int64_t)blockIdx.x >= n_ranges - 1) ? INT64_MAX : ((int64_t)blockIdx.x + 1) * stride;
-  int r = (int)rs.n_rows;
+  int r = n_rows;
   if ((int64_t)blockIdx.x < n_ranges)
     r = (blockIdx.x == 0) ? 0 : first_row_from_wave(rs, (int64_t)blockIdx.x * stride, lane);
   // row starts, 64 at a time: lane l holds the start of row win0 + l (of row n_rows: the end of the last)
   int win0 = r;
   int win = (int)rs.at(min((int64_t)win0 + lane, rs.n_rows));
-  int parity = 0;
-#pragma unroll 1
-  for (; r < (int)rs.n_rows; ++r) {
-    if (r - win0 >= kWave - 1) {
-      win0 = r;
+  // [t0, t1) of row rr; false when the walk ends before it
+  auto fetch = [&](int rr, int& t0, int& t1) -> bool {
+    if (rr >= n_rows) return false;
+    if (rr - win0 >= kWave - 1) {
+      win0 = rr;
       win = (int)rs.at(min((int64_t)win0 + lane, rs.n_rows));
     }
-    const int k = __builtin_amdgcn_readfirstlane(r - win0);
-    const int t0 = __builtin_amdgcn_readlane(win, k), t1 = __builtin_amdgcn_readlane(win, k + 1);
-    if ((int64_t)t0 >= range_end) break;
-    const int base = t0 & ~3;  // vectors stay 16-byte aligned; slots before t0 are not this row's
+    const int k = __builtin_amdgcn_readfirstlane(rr - win0);
+    t0 = __builtin_amdgcn_readlane(win, k);
+    t1 = __builtin_amdgcn_readlane(win, k + 1);
+    return (int64_t)t0 < range_end;
+  };
+  // the loads of group `grp` of the row [t0, t1) into bank B
+  auto load_group = [&](auto bank, int grp, int t0, int t1) {
+    constexpr int B = decltype(bank)::value;
+    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;  // vectors stay 16-byte aligned
+#pragma unroll
+    for (int c = 0; c < kRowHold; ++c) {
+      const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
+      if (p0 < t1 && p0 + kVec > t0) op.load(p0, B, c);
+    }
+  };
+  int parity = 0;
+  // one row in bank B; its first group has been requested; (n0, n1) is the next row, if there is one
+  auto row = [&](auto bank, int rr, int t0, int t1, bool has_next, int n0, int n1) {
+    constexpr int B = decltype(bank)::value;
+    if (has_next) load_group(std::integral_constant<int, B ^ 1>{}, 0, n0, n1);
+    const int base = t0 & ~3;  // slots before t0 are not this row's
     const int n_chunks = (t1 > t0) ? (t1 - base + kRowChunk - 1) / kRowChunk : 0;
     const int n_groups = (n_chunks + kRowHold - 1) / kRowHold;
     const int thread_p = base + (int)threadIdx.x * kVec;
@@ -117,22 +139,17 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
     // ---- pass 1: the row's sums, kRowHold chunks (one wait) at a time; the registers keep the last group
 #pragma unroll 1
     for (int grp = 0; grp < n_groups; ++grp) {
-      const int c0 = grp * kRowHold;
+      if (grp > 0) load_group(bank, grp, t0, t1);
 #pragma unroll
       for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (c0 + c) * kRowChunk;
-        if (p0 < t1 && p0 + kVec > t0) op.load(p0, c);
-      }
-#pragma unroll
-      for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (c0 + c) * kRowChunk;
+        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
         if (p0 >= t0 && p0 + kVec <= t1) {  // the whole vector belongs to the row
 #pragma unroll
-          for (int j = 0; j < kVec; ++j) op.stat(c, j, s);
+          for (int j = 0; j < kVec; ++j) op.stat(B, c, j, s);
         } else if (p0 < t1 && p0 + kVec > t0) {
 #pragma unroll
           for (int j = 0; j < kVec; ++j)
-            if (p0 + j >= t0 && p0 + j < t1) op.stat(c, j, s);
+            if (p0 + j >= t0 && p0 + j < t1) op.stat(B, c, j, s);
         }
       }
     }
@@ -148,24 +165,32 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
     for (int i = 0; i < NV; ++i)
       tot[i] = ((red[parity][0][i] + red[parity][1][i]) + red[parity][2][i]) + red[parity][3][i];
     parity ^= 1;
-    const auto rv = op.rows(r, tot, threadIdx.x == 0);
+    const auto rv = op.rows(rr, tot, threadIdx.x == 0);
     // ---- pass 2: outputs, last group first (its inputs are still in the registers)
 #pragma unroll 1
     for (int grp = n_groups - 1; grp >= 0; --grp) {
-      const int c0 = grp * kRowHold;
-      if (grp != n_groups - 1) {
-#pragma unroll
-        for (int c = 0; c < kRowHold; ++c) {
-          const int p0 = thread_p + (c0 + c) * kRowChunk;
-          if (p0 < t1 && p0 + kVec > t0) op.load(p0, c);
-        }
-      }
+      if (grp != n_groups - 1) load_group(bank, grp, t0, t1);
 #pragma unroll
       for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (c0 + c) * kRowChunk;
-        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, c, rv, t0, t1);
+        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
+        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, B, c, rv, t0, t1);
       }
     }
+  };
+  using Bank0 = std::integral_constant<int, 0>;
+  using Bank1 = std::integral_constant<int, 1>;
+  int t0 = 0, t1 = 0, n0 = 0, n1 = 0;
+  bool more = fetch(r, t0, t1);
+  if (more) load_group(Bank0{}, 0, t0, t1);
+#pragma unroll 1
+  while (more) {
+    bool next = fetch(r + 1, n0, n1);
+    row(Bank0{}, r, t0, t1, next, n0, n1);
+    ++r;
+    if (!next) break;
+    more = fetch(r + 1, t0, t1);
+    row(Bank1{}, r, n0, n1, more, t0, t1);
+    ++r;
   }
   // slots outside every row (before the first row's start, after the last row's end) belong to no
   // sequence: one workgroup writes zeros there
@@ -217,27 +242,27 @@ struct OwnedLossOp {
   const OwnedLossArgs& g;
   const RowStarts& rs;
   float bden;  // the batch denominator when the caller supplied it
-  float lv[kRowHold][4], ov[kRowHold][4], mv[kRowHold][4], av[kRowHold][4], wv[kRowHold][4];
+  float lv[2][kRowHold][4], ov[2][kRowHold][4], mv[2][kRowHold][4], av[2][kRowHold][4], wv[2][kRowHold][4];
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float rows_with_tokens = 0.f;
 
   __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float bd)
       : g(g_), rs(rs_), bden(bd) {}
 
-  __device__ __forceinline__ void load(int p0, int c) {
-    load4_guard(g.logp, p0, rs.n_slots, lv[c]);
-    load4_guard(g.oldp, p0, rs.n_slots, ov[c]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[c]);
+  __device__ __forceinline__ void load(int p0, int b, int c) {
+    load4_guard(g.logp, p0, rs.n_slots, lv[b][c]);
+    load4_guard(g.oldp, p0, rs.n_slots, ov[b][c]);
+    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[b][c]);
     // read by the output pass only, requested with the rest so that one wait covers all
-    load4_guard(g.adv, p0, rs.n_slots, av[c]);
-    if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[c]);
-    else wv[c][0] = wv[c][1] = wv[c][2] = wv[c][3] = 1.f;
+    load4_guard(g.adv, p0, rs.n_slots, av[b][c]);
+    if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[b][c]);
+    else wv[b][c][0] = wv[b][c][1] = wv[b][c][2] = wv[b][c][3] = 1.f;
   }
-  __device__ __forceinline__ void stat(int c, int j, float (&s)[2]) const {
-    const float m = mv[c][j];
+  __device__ __forceinline__ void stat(int b, int c, int j, float (&s)[2]) const {
+    const float m = mv[b][c][j];
     s[0] += m;
     // masked sum: values outside the mask never reach it (NaN / Inf in padding)
-    s[1] += (m != 0.f) ? (lv[c][j] - ov[c][j]) * m : 0.f;
+    s[1] += (m != 0.f) ? (lv[b][c][j] - ov[b][c][j]) * m : 0.f;
   }
   __device__ __forceinline__ RowVals rows(int64_t r, const float (&tot)[2], bool first) {
     const float c = tot[0];
@@ -250,7 +275,7 @@ struct OwnedLossOp {
     // with the batch denominator known this is the scale of the two-pass path, 1 / (td * bden)
     return RowVals{(g.valid != nullptr) ? 1.f / (td * bden) : 1.f / td, tot[1] / fmaxf(c, 1.f)};
   }
-  __device__ __forceinline__ void emit(int p0, int c, const RowVals& rv, int t0, int t1) {
+  __device__ __forceinline__ void emit(int p0, int b, int c, const RowVals& rv, int t0, int t1) {
     const bool whole = p0 >= t0 && p0 + kVec <= t1;
     float gv[4];
 #pragma unroll
@@ -259,8 +284,8 @@ struct OwnedLossOp {
       gv[j] = 0.f;
       if (!whole && (p < t0 || p >= t1)) continue;
       const TokenTerm t =
-          policy_token<KIND>(lv[c][j], ov[c][j], av[c][j], wv[c][j], rv.sbar, g.lo, g.hi, g.clip_c, false);
-      gv[j] = accumulate_token(t, mv[c][j], rv.scale, a);
+          policy_token<KIND>(lv[b][c][j], ov[b][c][j], av[b][c][j], wv[b][c][j], rv.sbar, g.lo, g.hi, g.clip_c, false);
+      gv[j] = accumulate_token(t, mv[b][c][j], rv.scale, a);
     }
     store4_range(g.grad, p0, t0, t1, gv);
   }
@@ -311,20 +336,20 @@ struct OwnedCorrOp {
   typedef CorrRow RowVals;
   const OwnedCorrArgs& g;
   const RowStarts& rs;
-  float ov[kRowHold][4], sv[kRowHold][4], mv[kRowHold][4];
+  float ov[2][kRowHold][4], sv[2][kRowHold][4], mv[2][kRowHold][4];
   float a[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float vetoed_rows = 0.f;
 
   __device__ __forceinline__ OwnedCorrOp(const OwnedCorrArgs& g_, const RowStarts& rs_) : g(g_), rs(rs_) {}
 
-  __device__ __forceinline__ void load(int p0, int c) {
-    load4_guard(g.oldp, p0, rs.n_slots, ov[c]);
-    load4_guard(g.samp, p0, rs.n_slots, sv[c]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[c]);
+  __device__ __forceinline__ void load(int p0, int b, int c) {
+    load4_guard(g.oldp, p0, rs.n_slots, ov[b][c]);
+    load4_guard(g.samp, p0, rs.n_slots, sv[b][c]);
+    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[b][c]);
   }
-  __device__ __forceinline__ void stat(int c, int j, float (&s)[3]) const {
-    const float m = mv[c][j];
-    const float d = ov[c][j] - sv[c][j];
+  __device__ __forceinline__ void stat(int b, int c, int j, float (&s)[3]) const {
+    const float m = mv[b][c][j];
+    const float d = ov[b][c][j] - sv[b][c][j];
     s[0] += m;
     s[1] += (m != 0.f) ? d * m : 0.f;
     s[2] += (g.cfg.has_veto && m != 0.f && d < g.cfg.log_veto) ? 1.f : 0.f;
@@ -339,7 +364,7 @@ struct OwnedCorrOp {
     }
     return corr_row(g.cfg, tot[1], tot[0], vetoed);
   }
-  __device__ __forceinline__ void emit(int p0, int c, const RowVals& row, int t0, int t1) {
+  __device__ __forceinline__ void emit(int p0, int b, int c, const RowVals& row, int t0, int t1) {
     const bool whole = p0 >= t0 && p0 + kVec <= t1;
     float wv[4], nm[4];
 #pragma unroll
@@ -348,7 +373,7 @@ struct OwnedCorrOp {
       wv[j] = 0.f;
       nm[j] = 0.f;
       if (!whole && (p < t0 || p >= t1)) continue;
-      corr_token(g.cfg, row, ov[c][j], sv[c][j], mv[c][j], wv[j], nm[j], a);
+      corr_token(g.cfg, row, ov[b][c][j], sv[b][c][j], mv[b][c][j], wv[j], nm[j], a);
     }
     if (g.isw) store4_range(g.isw, p0, t0, t1, wv);
     store4_range(g.new_mask, p0, t0, t1, nm);

@@ -37,7 +37,7 @@ __device__ __forceinline__ TokenTerm policy_token(float lp, float old, float A, 
   }
   if (KIND == 3) {  // CISPO (loss.py:411-468): -sg(clip(r)) * A * log_prob, IS weights not used
     const float xc = clampf(d, -kSafetyBound, kSafetyBound);
-    const float r_ = expf(xc);
+    const float r_ = exp_bounded(xc);
     const float rc = clampf(r_, lo, hi);
     float tm = 1.f;  // optional token-level mask of the unified formulation (clip_c != 0)
     if (clip_c != 0.f && ((A > 0.f && r_ > hi) || (A < 0.f && r_ < lo))) tm = 0.f;
@@ -66,7 +66,7 @@ __device__ __forceinline__ TokenTerm policy_token(float lp, float old, float A, 
   if (KIND == 5) {  // KL-Cov (loss.py:283-352): -A*ratio, plus clip_c * |log ratio| on the selected tokens
     const bool pass = (d >= -kSafetyBound && d <= kSafetyBound);
     const float xc = clampf(d, -kSafetyBound, kSafetyBound);
-    const float r_ = expf(xc);
+    const float r_ = exp_bounded(xc);
     float v = -A * r_, g = -A * r_;
     if (hit) {
       v += clip_c * fabsf(xc);
@@ -83,7 +83,7 @@ __device__ __forceinline__ TokenTerm policy_token(float lp, float old, float A, 
   else x = (lp - lp) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
   const bool pass = (x >= -kSafetyBound && x <= kSafetyBound);  // clamp passes grad inclusively
   const float xc = clampf(x, -kSafetyBound, kSafetyBound);
-  const float r_ = expf(xc);
+  const float r_ = exp_bounded(xc);
   const ValGrad p1{-A * r_, -A * r_};
   const float rc = clampf(r_, lo, hi);
   const bool rin = (r_ >= lo && r_ <= hi);
@@ -153,7 +153,7 @@ __device__ __forceinline__ void corr_token(const CorrCfg& c, const CorrRow& row,
   const float lr = oldv - sampv;
   const bool on = (m != 0.f);
   float w = 0.f;
-  if (c.is_mode == 1) w = expf(clampf(lr, -kSafetyBound, kSafetyBound)) * m;
+  if (c.is_mode == 1) w = exp_bounded(clampf(lr, -kSafetyBound, kSafetyBound)) * m;
   if (c.is_mode == 2) w = row.w * m;
   a[1] += on ? w * m : 0.f;
   w = (w != w) ? w : fminf(w, c.is_thr);  // clamp(max=thr), NaN propagates
