@@ -15,7 +15,7 @@ Public names and semantics follow axon/utils/rl/sampler.py:
   new mask = response_mask * rs * veto
 
 One elementwise launch, or, when a row-level quantity is needed (veto, sequence or geometric level),
-one launch in which a workgroup owns whole rows (beyond 2^21 tokens: a row pass, then an elementwise
+one launch in which a workgroup owns whole rows (batches of short rows: a row pass, then an elementwise
 pass).  The rejection test runs in log space against fp32 interval ends computed here on the host, so
 the 0/1 masks do not depend on the last bit of the device's ``exp``.
 
