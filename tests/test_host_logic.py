@@ -254,3 +254,22 @@ def test_kl_controllers_known_answers():
         get_kl_controller(SimpleNamespace(type="adaptive", kl_coef=0.2, target_kl=6.0, horizon=0))
     with pytest.raises(NotImplementedError):
         get_kl_controller(SimpleNamespace(type="bogus", kl_coef=0.2))
+
+
+def test_row_owning_dispatch_rule():
+    """Operators with a per-row quantity take the one-launch kernel (a workgroup works on one row at a time)
+    when the rows average at least OWNED_ROWS_MIN_MEAN_LEN tokens, the row pass + token pass otherwise."""
+    import torch
+
+    from axon_amd import _ops
+
+    assert _ops._own_rows(_ops.rows_of(torch.zeros(128, 1024)))           # padded 128 x 1024
+    assert _ops._own_rows(_ops.rows_of(torch.zeros(65536), torch.tensor([0, 30000, 65536], dtype=torch.int32)))
+    assert not _ops._own_rows(_ops.rows_of(torch.zeros(4096, 8)))         # rows of 8 tokens
+    assert not _ops._own_rows(_ops.rows_of(torch.zeros(12), torch.arange(0, 13, 3, dtype=torch.int32)))
+    keep = _ops.OWNED_ROWS_MAX_SLOTS
+    try:
+        _ops.OWNED_ROWS_MAX_SLOTS = 0
+        assert not _ops._own_rows(_ops.rows_of(torch.zeros(128, 1024)))
+    finally:
+        _ops.OWNED_ROWS_MAX_SLOTS = keep
