@@ -429,7 +429,8 @@ OwnedLaunch owned_launch(int64_t n_slots, int resident) {
 
 int check_owned_rows(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len) {
   if (n_rows < 0 || n_slots < 0 || uniform_len < 0) return AXON_ERR_ARG;
-  if (n_rows >= (int64_t)INT32_MAX || n_slots >= (int64_t)INT32_MAX - 4 * kRowChunk) return AXON_ERR_SHAPE;
+  // 32-bit positions: a chunk past the last slot and a search step past the last row must still fit
+  if (n_rows >= (int64_t)INT32_MAX - kWave || n_slots >= (int64_t)INT32_MAX - 4 * kRowChunk) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;  // slots without rows
