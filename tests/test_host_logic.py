@@ -42,6 +42,12 @@ def test_workspace_queries_and_argument_errors_without_gpu():
     assert lib.axon_lmhead_fwd_workspace_bytes(16, 100, 50) == -1  # hidden % 32 != 0
     assert lib.axon_lmhead_bwd_workspace_bytes(64, 128, 1000, 100) == -1  # chunk % 256 != 0
     assert lib.axon_lmhead_bwd_workspace_bytes(64, 128, 1000, 256) > 0
+    # the forward's optional stash: 128 KB per 256 x 256 tile + the per-part maxima; 0 where shifted edge tiles
+    # could not hand rows over in fours; -1 for an invalid shape
+    assert lib.axon_lmhead_stash_bytes(32768, 4096, 151936) == 594 * 128 * 131072 + 594 * 2 * 32768 * 4
+    assert lib.axon_lmhead_stash_bytes(513, 256, 1500) == 0 and lib.axon_lmhead_stash_bytes(516, 256, 1502) == 0
+    assert lib.axon_lmhead_stash_bytes(513, 96, 1501) == 3 * 6 * 131072 + 256 * ((6 * 2 * 513 * 4 + 255) // 256)
+    assert lib.axon_lmhead_stash_bytes(16, 100, 50) == -1 and lib.axon_lmhead_stash_bytes(0, 128, 1000) == 0
     # null pointers are rejected before any launch
     assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None) == -1
     assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0, None, 0.8, 1.2,
