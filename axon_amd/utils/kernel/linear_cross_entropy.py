@@ -6,7 +6,10 @@ Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntro
 
     logprobs, entropy = linear_cross_entropy(hidden, weight, labels, temperature, "none")
 
-* ``hidden`` ``[N, H]`` or ``[1, N, H]`` bf16, ``weight`` ``[V, H]`` bf16, ``labels`` int32/int64;
+* ``hidden`` ``[N, H]`` or ``[1, N, H]``, ``weight`` ``[V, H]``, ``labels`` int32/int64.  The kernels compute in
+  bf16 with fp32 accumulation (the trainer runs under bf16 autocast, forward_utils.py:216); fp16 or fp32
+  operands are accepted like the reference accepts any float dtype (kernels.py:517-522 asserts layout only),
+  are rounded to bf16 first, and receive their gradients in their own dtype;
 * outputs are flat fp32 ``[N]`` (never reshaped back, like the reference);
 * differentiable w.r.t. ``hidden`` and ``weight``; gradients come back in the input dtype;
 * ``reduction`` "sum"/"mean" reduce the log-probs as the reference's epilogue does
@@ -50,7 +53,8 @@ class LinearCrossEntropy(torch.autograd.Function):
             raise NotImplementedError("vocab-parallel LM head (dist_process_group) is not part of the one-GPU path")
         _lib.require_device(hidden, "linear_cross_entropy")
         assert weight.device == hidden.device and labels.device == hidden.device
-        assert hidden.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, "hidden and weight must be bf16"
+        floats = (torch.bfloat16, torch.float16, torch.float32)
+        assert hidden.dtype in floats and weight.dtype in floats, "hidden and weight must be bf16, fp16 or fp32"
         assert labels.dtype in (torch.int32, torch.int64), "labels must be int32 or int64"
 
         shape = hidden.shape
@@ -59,6 +63,8 @@ class LinearCrossEntropy(torch.autograd.Function):
         assert weight.dim() == 2 and hidden2.shape[1] == weight.shape[1]
         assert hidden2.shape[0] == labels1.shape[0]
         assert hidden2.is_contiguous() and weight.is_contiguous() and labels1.is_contiguous()
+        ctx.in_dtypes = (hidden.dtype, weight.dtype)
+        hidden2, weight = hidden2.to(torch.bfloat16), weight.to(torch.bfloat16)  # no copy when already bf16
 
         inv_t = 1.0 / temperature
         cap = 0.0 if logit_softcapping is None else float(logit_softcapping)
@@ -92,7 +98,8 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs.reshape(-1), None if dentropy is None else dentropy.reshape(-1), hidden2, weight, labels1, lse,
             entropy_b, ctx.inv_t, timing=_ops.TIMING, softcap=ctx.cap, seq_start=seq_start, stash=stash,
         )
-        return d_hidden.view(ctx.shape), d_weight, None, None, None, None, None, None
+        return (d_hidden.view(ctx.shape).to(ctx.in_dtypes[0]), d_weight.to(ctx.in_dtypes[1]), None, None, None, None,
+                None, None)
 
 
 linear_cross_entropy = LinearCrossEntropy.apply

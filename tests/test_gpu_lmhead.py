@@ -69,6 +69,26 @@ def test_forward_vs_oracle(n, h, v, temp, ldt):
     assert (ent.cpu() - ref_ent).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("dt", [torch.float16, torch.float32])
+def test_other_float_dtypes_are_rounded_to_bf16(dt):
+    """fp16 / fp32 operands (the reference's op takes any float dtype, kernels.py:517-522): the result is that of
+    the bf16-rounded operands, and the gradients come back in the operands' own dtype."""
+    n, h, v = 300, 128, 1000
+    hid, w, lab = W.lmhead_inputs(n, h, v, seed=31)
+    w = (w.float() * 8).bfloat16()
+    hd, wd = hid.to(DEV).to(dt).requires_grad_(True), w.to(DEV).to(dt).requires_grad_(True)  # exact in fp32; fp16 rounds
+    lp, ent = linear_cross_entropy(hd, wd, lab.to(DEV), 1.0, "none")
+    hb, wb = hd.detach().bfloat16().cpu(), wd.detach().bfloat16().cpu()
+    ref_lp, ref_ent = OM.forward(hb, wb, lab)
+    assert lp.dtype == torch.float32 and (lp.cpu() - ref_lp).abs().max() < 1e-3 and (ent.cpu() - ref_ent).abs().max() < 1e-3
+    g = torch.Generator().manual_seed(2)
+    g_lp = torch.randn(n, generator=g) / n
+    (lp * g_lp.to(DEV)).sum().backward()
+    assert hd.grad.dtype == dt and wd.grad.dtype == dt
+    ref_dh, ref_dw = OM.backward(g_lp, None, hb, wb, lab, 1.0)
+    assert rel_l2(hd.grad, ref_dh) < 2e-2 and rel_l2(wd.grad, ref_dw) < 2e-2
+
+
 def test_forward_closed_forms_gpu():
     n, h, v = 130, 64, 3000
     hid = torch.randn(n, h).bfloat16()
