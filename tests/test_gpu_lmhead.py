@@ -122,6 +122,10 @@ def test_3d_hidden_reductions_and_errors():
     mod = FusedLinearForPPO()
     lp2, ent2 = mod(hid.view(2, 48, 64).to(DEV), w.to(DEV), lab.view(2, 48).to(DEV).int(), temperature=1.0)
     assert lp2.shape == (2, 48) and torch.allclose(lp2.flatten().cpu(), ref, atol=1e-3)
+    lp3, ent3 = FusedLinearForPPO(round_outputs_to_input_dtype=True)(hid.view(2, 48, 64).to(DEV), w.to(DEV),
+                                                                      lab.view(2, 48).to(DEV), temperature=1.0)
+    assert lp3.dtype == torch.bfloat16 and ent3.dtype == torch.bfloat16  # as fused_linear.py:46
+    assert torch.equal(lp3, lp2.bfloat16()) and torch.equal(ent3, ent2.bfloat16())
 
 
 @pytest.mark.parametrize("n,h,v,temp,ldt", CASES)
