@@ -134,7 +134,11 @@ __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, c
     if (STASH) {
 #pragma unroll
       for (int ip = 0; ip < kBlocks / 2; ++ip)
-        stash_wave[(j * 4 + ip) * 64] = make_uint4(hw[2 * ip][0], hw[2 * ip][1], hw[2 * ip + 1][0], hw[2 * ip + 1][1]);
+      {  // written once, read once by the backward: kept out of the way of the operand slices in L2
+        typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 x = {hw[2 * ip][0], hw[2 * ip][1], hw[2 * ip + 1][0], hw[2 * ip + 1][1]};
+        __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(stash_wave + (j * 4 + ip) * 64));
+      }
     }
 #pragma unroll
     for (int off = 16; off <= 32; off <<= 1) {
