@@ -239,7 +239,7 @@ OWNED_ROWS_MIN_MEAN_LEN = 64
 
 
 def _own_rows(rows: "Rows") -> bool:
-    return rows.n_slots <= OWNED_ROWS_MAX_SLOTS and rows.n_slots >= OWNED_ROWS_MIN_MEAN_LEN * max(rows.n_rows, 1)
+    return 4 <= rows.n_slots <= OWNED_ROWS_MAX_SLOTS and rows.n_slots >= OWNED_ROWS_MIN_MEAN_LEN * max(rows.n_rows, 1)
 
 
 IS_MODES = {None: 0, "token": 1, "sequence": 2}

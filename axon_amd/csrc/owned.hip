@@ -9,10 +9,12 @@
 // walked in chunks of 1024 slots (16 bytes per thread), kRowHold chunks (2048 slots) per wait: the
 // row sums are formed across the workgroup, the per-row values derived from them, and the
 // per-token outputs written from the registers.  A row of more than 2048 slots is read a second
-// time for the output pass, all but its last group (it was read microseconds earlier).  The common
-// case reads every input exactly once: 20 bytes per token for GSPO or the veto against 32 for a
-// row pass followed by a token pass.  The first group of the next row is requested before the
-// current row is worked on (two banks of two chunks in registers).
+// time for the output pass, all but its last group: its first read goes without the streaming hint,
+// so that the second finds the lines in the L2.  The common case reads every input exactly once:
+// 20 bytes per token for GSPO or the veto against 32 for a row pass followed by a token pass.  The
+// first group of the next row is requested before the current row is worked on (two banks of two
+// chunks in registers), as a fixed number of loads in straight-line code: the compiler then waits
+// for the current row's loads by count and leaves the next row's in flight.
 //
 // The per-row sums are formed without atomics and in a fixed order (a thread adds its slots chunk
 // by chunk, then the fixed tree of the wavefront sum, then the four wavefronts 0 + 1 + 2 + 3), so
@@ -76,7 +78,9 @@ __device__ __forceinline__ float wave_total(float v) {  // the same value in eve
 
 // What the two kernels share: the walk over ranges, rows and chunks.  `Op` provides
 //   kNV                               number of row sums
-//   load(p0, b, c)                    the vector of four slots starting at p0 into register set (b, c) (every input)
+//   load(p0, b, c)                    the vector of four slots starting at p0 into register set (b, c) (every input):
+//                                     a fixed number of 16-byte loads, p0 + 4 <= n_slots
+//   load_edge(p0, b, c)               the same for a vector that may reach beyond the last slot
 //   stat(b, c, j, s[])                add slot j of register set (b, c) to the thread's row sums
 //   rows(r, tot[], first) -> RowVals  the per-row values from the row's sums (every thread the same)
 //   emit(p0, b, c, rv, t0, t1)        write the outputs of the vector in register set (b, c)
@@ -114,32 +118,69 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
     t1 = __builtin_amdgcn_readlane(win, k + 1);
     return (int64_t)t0 < range_end;
   };
-  // the loads of group `grp` of the row [t0, t1) into bank B
-  auto load_group = [&](auto bank, int grp, int t0, int t1) {
+  // With a slot count that is no multiple of four the last vector is incomplete: `tail_p0` is its
+  // first slot (none: -1) and `last_full` the last vector that can be read with one 16-byte load.
+  const int n4 = (int)(rs.n_slots & ~(int64_t)3);
+  const int tail_p0 = (n4 < rs.n_slots) ? n4 : -1;
+  const int last_full = max(n4 - kVec, 0);  // n_slots >= 4 (the host's check)
+  // The first group of the row [t0, t1) into bank B, as a FIXED number of loads in straight-line code: a
+  // vector beyond the row's end is requested at the row's last vector instead (one cache line for the
+  // whole wavefront, never used).  A load under a condition would leave the compiler unable to count
+  // the loads in flight behind the ones it waits for, and every wait would drain the prefetch as well.
+  auto prefetch = [&](auto bank, int t0, int t1) {
     constexpr int B = decltype(bank)::value;
     const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;  // vectors stay 16-byte aligned
+    const int hi = min(max(t1 - 1, t0) & ~3, last_full);
+    // a row of several groups comes back to this one for its outputs: both arms issue the same loads
+    if (t1 - (t0 & ~3) > kRowHold * kRowChunk) {
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) op.template load<true>(min(thread_p + c * kRowChunk, hi), B, c);
+    } else {
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) op.template load<false>(min(thread_p + c * kRowChunk, hi), B, c);
+    }
+  };
+  // The incomplete last vector of the arrays, when the first group of [t0, t1) holds it: one thread of
+  // the launch reads it slot by slot, and waits at once so that the compiler's count of the loads in
+  // flight stays what it is on the path without this block.
+  auto fetch_tail = [&](auto bank, int t0, int t1) {
+    constexpr int B = decltype(bank)::value;
+    if (tail_p0 < 0 || tail_p0 >= t1) return;
+    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;
+#pragma unroll
+    for (int c = 0; c < kRowHold; ++c) {
+      if (thread_p + c * kRowChunk == tail_p0) {
+        op.template load_edge<false>(tail_p0, B, c);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+      }
+    }
+  };
+  // a later group of a long row (or an earlier one again, for the output pass)
+  auto load_group = [&](auto bank, int grp, int t0, int t1, bool keep) {
+    constexpr int B = decltype(bank)::value;
+    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;
 #pragma unroll
     for (int c = 0; c < kRowHold; ++c) {
       const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
-      if (p0 < t1 && p0 + kVec > t0) op.load(p0, B, c);
+      if (p0 < t1 && p0 + kVec > t0) {
+        if (keep) op.template load_edge<true>(p0, B, c);
+        else op.template load_edge<false>(p0, B, c);
+      }
     }
   };
   int parity = 0;
   // one row in bank B; its first group has been requested; (n0, n1) is the next row, if there is one
   auto row = [&](auto bank, int rr, int t0, int t1, bool has_next, int n0, int n1) {
     constexpr int B = decltype(bank)::value;
-    if (has_next) load_group(std::integral_constant<int, B ^ 1>{}, 0, n0, n1);
+    prefetch(std::integral_constant<int, B ^ 1>{}, has_next ? n0 : 0, has_next ? n1 : 0);
     const int base = t0 & ~3;  // slots before t0 are not this row's
     const int n_chunks = (t1 > t0) ? (t1 - base + kRowChunk - 1) / kRowChunk : 0;
-    const int n_groups = (n_chunks + kRowHold - 1) / kRowHold;
+    const int n_groups = max((n_chunks + kRowHold - 1) / kRowHold, 1);
     const int thread_p = base + (int)threadIdx.x * kVec;
     float s[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) s[i] = 0.f;
-    // ---- pass 1: the row's sums, kRowHold chunks (one wait) at a time; the registers keep the last group
-#pragma unroll 1
-    for (int grp = 0; grp < n_groups; ++grp) {
-      if (grp > 0) load_group(bank, grp, t0, t1);
+    auto stat_group = [&](int grp) {
 #pragma unroll
       for (int c = 0; c < kRowHold; ++c) {
         const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
@@ -152,6 +193,23 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
             if (p0 + j >= t0 && p0 + j < t1) op.stat(B, c, j, s);
         }
       }
+    };
+    auto emit_group = [&](int grp, const typename Op::RowVals& rv) {
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) {
+        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
+        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, B, c, rv, t0, t1);
+      }
+    };
+    // ---- pass 1: the row's sums.  The first group is in flight since the previous row (straight-line
+    // code up to its first use, so the wait leaves the prefetch alone); a long row fetches the others
+    // one wait at a time and the registers keep the last.
+    fetch_tail(bank, t0, t1);
+    stat_group(0);
+#pragma unroll 1
+    for (int grp = 1; grp < n_groups; ++grp) {
+      load_group(bank, grp, t0, t1, grp < n_groups - 1);
+      stat_group(grp);
     }
 #pragma unroll
     for (int i = 0; i < NV; ++i) s[i] = wave_total(s[i]);
@@ -167,21 +225,18 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
     parity ^= 1;
     const auto rv = op.rows(rr, tot, threadIdx.x == 0);
     // ---- pass 2: outputs, last group first (its inputs are still in the registers)
+    emit_group(n_groups - 1, rv);
 #pragma unroll 1
-    for (int grp = n_groups - 1; grp >= 0; --grp) {
-      if (grp != n_groups - 1) load_group(bank, grp, t0, t1);
-#pragma unroll
-      for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
-        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, B, c, rv, t0, t1);
-      }
+    for (int grp = n_groups - 2; grp >= 0; --grp) {
+      load_group(bank, grp, t0, t1, false);
+      emit_group(grp, rv);
     }
   };
   using Bank0 = std::integral_constant<int, 0>;
   using Bank1 = std::integral_constant<int, 1>;
   int t0 = 0, t1 = 0, n0 = 0, n1 = 0;
   bool more = fetch(r, t0, t1);
-  if (more) load_group(Bank0{}, 0, t0, t1);
+  if (more) prefetch(Bank0{}, t0, t1);
 #pragma unroll 1
   while (more) {
     bool next = fetch(r + 1, n0, n1);
@@ -200,15 +255,35 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
   }
 }
 
+// Loads of the row walk.  KEEP: the vector will be read a second time soon (a group of a long row that
+// the output pass comes back to), so it is requested without the streaming hint and stays in the L2.
+template <bool KEEP>
+__device__ __forceinline__ void row_load4(const float* p, int64_t i, float (&v)[4]) {
+  const f32x4* q = reinterpret_cast<const f32x4*>(p + i);
+  const f32x4 x = KEEP ? *q : __builtin_nontemporal_load(q);
+  v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+}
+// the mask is known to be there: no branch around the loads
+template <int MK, bool KEEP>
+__device__ __forceinline__ void row_load_mask4(const void* mask, int64_t i, float (&m)[4]) {
+  if (MK == AXON_MASK_F32) {
+    row_load4<KEEP>(static_cast<const float*>(mask), i, m);
+  } else {
+    const i64x2* p = reinterpret_cast<const i64x2*>(static_cast<const int64_t*>(mask) + i);
+    const i64x2 a = KEEP ? p[0] : __builtin_nontemporal_load(p), b = KEEP ? p[1] : __builtin_nontemporal_load(p + 1);
+    m[0] = (float)a.x; m[1] = (float)a.y; m[2] = (float)b.x; m[3] = (float)b.y;
+  }
+}
 // four slots starting at p0 (p0 % 4 == 0): one 16-byte load when all four exist
-__device__ __forceinline__ void load4_guard(const float* p, int64_t p0, int64_t n_slots, float (&v)[4]) {
-  if (p0 + kVec <= n_slots) { load4(p, p0, v); return; }
+template <bool KEEP>
+__device__ __forceinline__ void row_load4_guard(const float* p, int64_t p0, int64_t n_slots, float (&v)[4]) {
+  if (p0 + kVec <= n_slots) { row_load4<KEEP>(p, p0, v); return; }
 #pragma unroll
   for (int j = 0; j < kVec; ++j) v[j] = (p0 + j < n_slots) ? p[p0 + j] : 0.f;
 }
-template <int MK>
-__device__ __forceinline__ void load_mask4_guard(const void* mask, int64_t p0, int64_t n_slots, float (&m)[4]) {
-  if (p0 + kVec <= n_slots) { load_mask4<MK>(mask, p0, m); return; }
+template <int MK, bool KEEP>
+__device__ __forceinline__ void row_load_mask4_guard(const void* mask, int64_t p0, int64_t n_slots, float (&m)[4]) {
+  if (p0 + kVec <= n_slots) { row_load_mask4<MK, KEEP>(mask, p0, m); return; }
 #pragma unroll
   for (int j = 0; j < kVec; ++j) m[j] = (p0 + j < n_slots) ? load_mask1<MK>(mask, p0 + j) : 0.f;
 }
@@ -238,7 +313,7 @@ struct OwnedLossArgs {
 template <int MK, int KIND>
 struct OwnedLossOp {
   static constexpr int kNV = 2;  // sum mask, sum (logp - old) * mask
-  struct RowVals { float scale, sbar; };
+  struct RowVals { float scale, sbar; Ratio seq; };  // seq: GSPO's ratio of the sequence (KIND 1)
   const OwnedLossArgs& g;
   const RowStarts& rs;
   float bden;  // the batch denominator when the caller supplied it
@@ -249,14 +324,24 @@ struct OwnedLossOp {
   __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float bd)
       : g(g_), rs(rs_), bden(bd) {}
 
+  // Always the same number of loads (the walk counts on it): without importance weights the slot of
+  // `wv` is filled from the advantages' lines, which are on their way anyway, and not used.
+  template <bool KEEP>
   __device__ __forceinline__ void load(int p0, int b, int c) {
-    load4_guard(g.logp, p0, rs.n_slots, lv[b][c]);
-    load4_guard(g.oldp, p0, rs.n_slots, ov[b][c]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[b][c]);
+    row_load4<KEEP>(g.logp, p0, lv[b][c]);
+    row_load4<KEEP>(g.oldp, p0, ov[b][c]);
+    row_load_mask4<MK, KEEP>(g.mask, p0, mv[b][c]);
     // read by the output pass only, requested with the rest so that one wait covers all
-    load4_guard(g.adv, p0, rs.n_slots, av[b][c]);
-    if (g.isw) load4_guard(g.isw, p0, rs.n_slots, wv[b][c]);
-    else wv[b][c][0] = wv[b][c][1] = wv[b][c][2] = wv[b][c][3] = 1.f;
+    row_load4<KEEP>(g.adv, p0, av[b][c]);
+    row_load4<KEEP>(g.isw ? g.isw : g.adv, p0, wv[b][c]);
+  }
+  template <bool KEEP>
+  __device__ __forceinline__ void load_edge(int p0, int b, int c) {
+    row_load4_guard<KEEP>(g.logp, p0, rs.n_slots, lv[b][c]);
+    row_load4_guard<KEEP>(g.oldp, p0, rs.n_slots, ov[b][c]);
+    row_load_mask4_guard<MK, KEEP>(g.mask, p0, rs.n_slots, mv[b][c]);
+    row_load4_guard<KEEP>(g.adv, p0, rs.n_slots, av[b][c]);
+    row_load4_guard<KEEP>(g.isw ? g.isw : g.adv, p0, rs.n_slots, wv[b][c]);
   }
   __device__ __forceinline__ void stat(int b, int c, int j, float (&s)[2]) const {
     const float m = mv[b][c][j];
@@ -273,7 +358,10 @@ struct OwnedLossOp {
     if (g.batch_reduce == 2) td *= fmaxf((float)g.nps[r], 1.f);
     rows_with_tokens += (first && c > 0.f) ? 1.f : 0.f;
     // with the batch denominator known this is the scale of the two-pass path, 1 / (td * bden)
-    return RowVals{(g.valid != nullptr) ? 1.f / (td * bden) : 1.f / td, tot[1] / fmaxf(c, 1.f)};
+    RowVals rv{(g.valid != nullptr) ? 1.f / (td * bden) : 1.f / td, tot[1] / fmaxf(c, 1.f), Ratio{}};
+    // GSPO's ratio is the same for every token of the sequence: the exponential once per row
+    if (KIND == 1) rv.seq = ratio_of(0.f + rv.sbar, g.lo, g.hi);
+    return rv;
   }
   __device__ __forceinline__ void emit(int p0, int b, int c, const RowVals& rv, int t0, int t1) {
     const bool whole = p0 >= t0 && p0 + kVec <= t1;
@@ -283,8 +371,10 @@ struct OwnedLossOp {
       const int p = p0 + j;
       gv[j] = 0.f;
       if (!whole && (p < t0 || p >= t1)) continue;
-      const TokenTerm t =
-          policy_token<KIND>(lv[b][c][j], ov[b][c][j], av[b][c][j], wv[b][c][j], rv.sbar, g.lo, g.hi, g.clip_c, false);
+      const float w = g.isw ? wv[b][c][j] : 1.f;
+      const TokenTerm t = (KIND == 1) ? gspo_token(rv.seq, lv[b][c][j], ov[b][c][j], av[b][c][j], w, g.clip_c)
+                                      : policy_token<KIND>(lv[b][c][j], ov[b][c][j], av[b][c][j], w, rv.sbar, g.lo,
+                                                           g.hi, g.clip_c, false);
       gv[j] = accumulate_token(t, mv[b][c][j], rv.scale, a);
     }
     store4_range(g.grad, p0, t0, t1, gv);
@@ -342,10 +432,17 @@ struct OwnedCorrOp {
 
   __device__ __forceinline__ OwnedCorrOp(const OwnedCorrArgs& g_, const RowStarts& rs_) : g(g_), rs(rs_) {}
 
+  template <bool KEEP>
   __device__ __forceinline__ void load(int p0, int b, int c) {
-    load4_guard(g.oldp, p0, rs.n_slots, ov[b][c]);
-    load4_guard(g.samp, p0, rs.n_slots, sv[b][c]);
-    load_mask4_guard<MK>(g.mask, p0, rs.n_slots, mv[b][c]);
+    row_load4<KEEP>(g.oldp, p0, ov[b][c]);
+    row_load4<KEEP>(g.samp, p0, sv[b][c]);
+    row_load_mask4<MK, KEEP>(g.mask, p0, mv[b][c]);
+  }
+  template <bool KEEP>
+  __device__ __forceinline__ void load_edge(int p0, int b, int c) {
+    row_load4_guard<KEEP>(g.oldp, p0, rs.n_slots, ov[b][c]);
+    row_load4_guard<KEEP>(g.samp, p0, rs.n_slots, sv[b][c]);
+    row_load_mask4_guard<MK, KEEP>(g.mask, p0, rs.n_slots, mv[b][c]);
   }
   __device__ __forceinline__ void stat(int b, int c, int j, float (&s)[3]) const {
     const float m = mv[b][c][j];
@@ -431,6 +528,8 @@ int check_owned_rows(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_t
   if (n_rows < 0 || n_slots < 0 || uniform_len < 0) return AXON_ERR_ARG;
   // 32-bit positions: a chunk past the last slot and a search step past the last row must still fit
   if (n_rows >= (int64_t)INT32_MAX - kWave || n_slots >= (int64_t)INT32_MAX - 4 * kRowChunk) return AXON_ERR_SHAPE;
+  // the kernels read whole 16-byte vectors wherever one fits: fewer than four slots is the other path's case
+  if (n_slots > 0 && n_slots < kVec) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && cu == nullptr && n_slots > 0) return AXON_ERR_ARG;
   if (uniform_len > 0 && n_rows * uniform_len != n_slots) return AXON_ERR_SHAPE;
   if (uniform_len == 0 && n_rows == 0 && n_slots > 0) return AXON_ERR_SHAPE;  // slots without rows

@@ -22,6 +22,51 @@ __device__ __forceinline__ ValGrad vg_max(ValGrad a, ValGrad b) {
 // whose masked sum is the third metric.  The caller multiplies by mask and aggregation scale.
 struct TokenTerm { float vw, gw, c1, k2, c3; };
 
+// The ratio of a clipped surrogate loss and what depends on it alone: the exponent clamped to +-20
+// (the clamp passes the gradient inclusively), the ratio, the ratio clipped to [lo, hi] and whether it
+// lies inside.
+struct Ratio { float xc, r, rc; bool pass, rin; };
+__device__ __forceinline__ Ratio ratio_of(float x, float lo, float hi) {
+  Ratio q;
+  q.pass = (x >= -kSafetyBound && x <= kSafetyBound);
+  q.xc = clampf(x, -kSafetyBound, kSafetyBound);
+  q.r = exp_bounded(q.xc);
+  q.rc = clampf(q.r, lo, hi);
+  q.rin = (q.r >= lo && q.r <= hi);
+  return q;
+}
+
+// PPO (0), GSPO (1) and Clip-Cov (6) from the ratio on: max(-A r, -A clip(r)), the dual clip of PPO,
+// the metrics.  d = log_prob - old.
+template <int KIND>
+__device__ __forceinline__ TokenTerm clipped_token(const Ratio& q, float d, float A, float w, float clip_c,
+                                                   bool hit) {
+  TokenTerm t{0.f, 0.f, 0.f, 0.f, 0.f};
+  const ValGrad p1{-A * q.r, -A * q.r};
+  const ValGrad p2{-A * q.rc, q.rin ? -A * q.r : 0.f};
+  ValGrad c = vg_max(p1, p2);
+  if (KIND == 6) {  // Clip-Cov (loss.py:198-280): the selected tokens drop out of the loss
+    if (hit) c = ValGrad{c.v * 0.f, 0.f};
+    t.c1 = hit ? 1.f : 0.f;
+  } else {
+    t.c1 = (p2.v > p1.v) ? 1.f : 0.f;
+  }
+  t.k2 = (KIND == 1) ? -d : -q.xc;  // ppo_kl: raw for GSPO (loss.py:173), clamped otherwise (loss.py:77-79)
+  if (KIND == 0) {
+    const float pg3 = -A * clip_c;
+    t.c3 = (c.v > pg3 && A < 0.f) ? 1.f : 0.f;
+    {  // A < 0: torch.min(pg3, c1), pg3 carries no gradient (selects: see vg_max)
+      const bool neg = A < 0.f, lt = pg3 < c.v, eq = pg3 == c.v, gt = pg3 > c.v;
+      const float v_min = lt ? pg3 : (eq ? c.v : (gt ? c.v : pg3 + c.v));
+      const float g_min = lt ? 0.f : (eq ? 0.5f * c.g : (gt ? c.g : 0.f));
+      c = ValGrad{neg ? v_min : c.v, neg ? g_min : c.g};
+    }
+  }
+  t.vw = c.v * w;
+  t.gw = (q.pass ? c.g : 0.f) * w;
+  return t;
+}
+
 // KIND 0 PPO, 1 GSPO (sbar = the sequence's mean log-ratio), 2 REINFORCE / GPG, 3 CISPO, 4 clipped
 // value loss, 5 KL-Cov, 6 Clip-Cov (hit: the token is among the selected ones).
 template <int KIND>
@@ -81,34 +126,19 @@ __device__ __forceinline__ TokenTerm policy_token(float lp, float old, float A, 
   float x;  // exponent before the +-20 clamp
   if (KIND == 0 || KIND == 6) x = d;
   else x = (lp - lp) + sbar;  // log_prob - sg(log_prob) + sg(seq mean)
-  const bool pass = (x >= -kSafetyBound && x <= kSafetyBound);  // clamp passes grad inclusively
-  const float xc = clampf(x, -kSafetyBound, kSafetyBound);
-  const float r_ = exp_bounded(xc);
-  const ValGrad p1{-A * r_, -A * r_};
-  const float rc = clampf(r_, lo, hi);
-  const bool rin = (r_ >= lo && r_ <= hi);
-  const ValGrad p2{-A * rc, rin ? -A * r_ : 0.f};
-  ValGrad c = vg_max(p1, p2);
-  if (KIND == 6) {  // Clip-Cov (loss.py:198-280): the selected tokens drop out of the loss
-    if (hit) c = ValGrad{c.v * 0.f, 0.f};
-    t.c1 = hit ? 1.f : 0.f;
-  } else {
-    t.c1 = (p2.v > p1.v) ? 1.f : 0.f;
-  }
-  t.k2 = (KIND == 1) ? -d : -xc;  // ppo_kl: raw for GSPO (loss.py:173), clamped otherwise (loss.py:77-79)
-  if (KIND == 0) {
-    const float pg3 = -A * clip_c;
-    t.c3 = (c.v > pg3 && A < 0.f) ? 1.f : 0.f;
-    {  // A < 0: torch.min(pg3, c1), pg3 carries no gradient (selects: see vg_max)
-      const bool neg = A < 0.f, lt = pg3 < c.v, eq = pg3 == c.v, gt = pg3 > c.v;
-      const float v_min = lt ? pg3 : (eq ? c.v : (gt ? c.v : pg3 + c.v));
-      const float g_min = lt ? 0.f : (eq ? 0.5f * c.g : (gt ? c.g : 0.f));
-      c = ValGrad{neg ? v_min : c.v, neg ? g_min : c.g};
-    }
-  }
-  t.vw = c.v * w;
-  t.gw = (pass ? c.g : 0.f) * w;
-  return t;
+  return clipped_token<KIND>(ratio_of(x, lo, hi), d, A, w, clip_c, hit);
+}
+
+// GSPO where the sequence's ratio is at hand (ratio_of((0 + sbar), lo, hi), once per sequence): the
+// same token as policy_token<1>, bit for bit.  log_prob - sg(log_prob) is zero for a finite log_prob and
+// NaN otherwise; added to the ratio and its clipped value it leaves them as they are or makes them
+// NaN, which is what the exponential of a NaN exponent gives.
+__device__ __forceinline__ TokenTerm gspo_token(const Ratio& seq, float lp, float old, float A, float w,
+                                                float clip_c) {
+  const float z = lp - lp;
+  const bool fin = (z == 0.f);
+  return clipped_token<1>(Ratio{seq.xc + z, seq.r + z, seq.rc + z, seq.pass && fin, seq.rin && fin}, lp - old, A, w,
+                          clip_c, false);
 }
 
 // Adds one token to the running sums a[0..4] (loss, three metrics, mask) and returns its gradient.

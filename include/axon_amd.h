@@ -382,6 +382,8 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
  *   acc[0] is divided by it, grad[] is left WITHOUT that division and acc[5] returns the factor the
  *   caller multiplies the gradient by; with valid_count acc[5] = 1.
  *   Slots that belong to no row (before cu_seqlens[0], after cu_seqlens[n_rows]) receive grad 0.
+ *   n_slots of 1, 2 or 3 is refused (AXON_ERR_SHAPE): the kernel reads 16-byte vectors; such inputs are
+ *   for the calls it replaces.  The same holds for axon_sampler_correction_rows.
  * partials: workspace of axon_reduce_partials_bytes, ticket counters zero (see there). */
 int axon_policy_loss_rows(int kind, const float* logp, const float* old_logp, const float* adv,
                           const void* mask, int mask_kind, const float* is_weights,

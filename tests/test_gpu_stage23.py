@@ -926,11 +926,28 @@ AWKWARD = {
     "tiny_rows": [0, 0] + [1, 0, 2, 3, 0, 5] * 60 + [700, 0, 0],
     # a single row, a row that ends exactly on range borders
     "borders": [2048, 2048, 4096, 1, 2047, 2048],
+    # slot counts that are no multiple of four: the incomplete last 16-byte vector shared by two rows, in a
+    # later group of a long row, in the first group of the only row; the smallest input the kernels take
+    "tail_two_rows": [3000, 2, 1],
+    "tail_in_long_row": [6145],
+    "tail_in_first_group": [5],
+    "four_slots": [1, 3],
 }
 
 
+@pytest.fixture
+def owned_rows_forced():
+    """Rows of any length through the kernels in which a workgroup owns whole rows (the dispatch would send
+    batches of short rows to the row pass + token pass)."""
+    from axon_amd import _ops
+    keep = _ops.OWNED_ROWS_MIN_MEAN_LEN
+    _ops.OWNED_ROWS_MIN_MEAN_LEN = 0
+    yield
+    _ops.OWNED_ROWS_MIN_MEAN_LEN = keep
+
+
 @pytest.mark.parametrize("layout", sorted(AWKWARD))
-def test_row_owned_losses_on_awkward_layouts(layout):
+def test_row_owned_losses_on_awkward_layouts(layout, owned_rows_forced):
     lens = AWKWARD[layout]
     d, pad = _awkward_packed(lens, seed=len(lens))
     meta = {"cu_seqlens": d["cu_seqlens"]}
@@ -947,7 +964,7 @@ def test_row_owned_losses_on_awkward_layouts(layout):
 
 @pytest.mark.parametrize("layout", sorted(AWKWARD))
 @pytest.mark.parametrize("is_l,rs_l", [("token", "token"), ("sequence", "sequence"), ("sequence", "geometric")])
-def test_row_owned_correction_on_awkward_layouts(layout, is_l, rs_l):
+def test_row_owned_correction_on_awkward_layouts(layout, is_l, rs_l, owned_rows_forced):
     lens = AWKWARD[layout]
     d, pad = _awkward_packed(lens, seed=100 + len(lens))
     kw = dict(sampler_is=is_l, sampler_is_threshold=2.0, sampler_rs=rs_l, sampler_rs_threshold=2.0,

@@ -279,3 +279,10 @@ def test_row_owning_dispatch_rule():
         assert not _ops._own_rows(_ops.rows_of(torch.zeros(128, 1024)))
     finally:
         _ops.OWNED_ROWS_MAX_SLOTS = keep
+    keep = _ops.OWNED_ROWS_MIN_MEAN_LEN
+    try:  # whatever the threshold: never fewer slots than one 16-byte vector
+        _ops.OWNED_ROWS_MIN_MEAN_LEN = 0
+        assert _ops._own_rows(_ops.rows_of(torch.zeros(1, 4)))
+        assert not _ops._own_rows(_ops.rows_of(torch.zeros(1, 3)))
+    finally:
+        _ops.OWNED_ROWS_MIN_MEAN_LEN = keep
