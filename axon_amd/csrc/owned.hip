@@ -92,7 +92,7 @@ __device__ __forceinline__ float wave_total(float v) {  // the same value in eve
 template <class Op>
 __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride, Op& op) {
   constexpr int NV = Op::kNV;
-  __shared__ float red[2][kOwnWaves][NV];
+  __shared__ float red[2][kOwnWaves][kRowHold * NV];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int n_rows = (int)rs.n_rows;
   const int64_t n_ranges = (rs.n_slots + stride - 1) / stride;  // <= workgroups of the launch
@@ -123,45 +123,78 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
   const int n4 = (int)(rs.n_slots & ~(int64_t)3);
   const int tail_p0 = (n4 < rs.n_slots) ? n4 : -1;
   const int last_full = max(n4 - kVec, 0);  // n_slots >= 4 (the host's check)
-  // The first group of the row [t0, t1) into bank B, as a FIXED number of loads in straight-line code: a
-  // vector beyond the row's end is requested at the row's last vector instead (one cache line for the
-  // whole wavefront, never used).  A load under a condition would leave the compiler unable to count
-  // the loads in flight behind the ones it waits for, and every wait would drain the prefetch as well.
-  auto prefetch = [&](auto bank, int t0, int t1) {
-    constexpr int B = decltype(bank)::value;
-    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;  // vectors stay 16-byte aligned
-    const int hi = min(max(t1 - 1, t0) & ~3, last_full);
-    // a row of several groups comes back to this one for its outputs: both arms issue the same loads
-    if (t1 - (t0 & ~3) > kRowHold * kRowChunk) {
-#pragma unroll
-      for (int c = 0; c < kRowHold; ++c) op.template load<true>(min(thread_p + c * kRowChunk, hi), B, c);
-    } else {
-#pragma unroll
-      for (int c = 0; c < kRowHold; ++c) op.template load<false>(min(thread_p + c * kRowChunk, hi), B, c);
+  // What one step of the walk works on: row r = [a0, a1) and, when that row and the next one fit a
+  // chunk each, the next row [b0, b1) beside it (`pair`): the second chunk of the registers would
+  // otherwise idle through every short row.  Uniform across the workgroup.
+  static_assert(kRowHold == 2, "a step pairs two one-chunk rows in the two chunks of a bank");
+  struct Span { int r, a0, a1, b0, b1; bool valid, pair; };
+  auto chunks_of = [](int t0, int t1) { return (t1 > t0) ? (t1 - (t0 & ~3) + kRowChunk - 1) / kRowChunk : 0; };
+  auto span_at = [&](int rr) -> Span {
+    Span sp{rr, 0, 0, 0, 0, false, false};
+    int t0 = 0, t1 = 0;
+    sp.valid = fetch(rr, t0, t1);
+    if (!sp.valid) return sp;
+    sp.a0 = t0;
+    sp.a1 = t1;
+    if (chunks_of(t0, t1) <= 1 && fetch(rr + 1, t0, t1) && chunks_of(t0, t1) <= 1) {
+      sp.pair = true;
+      sp.b0 = t0;
+      sp.b1 = t1;
     }
+    return sp;
   };
-  // The incomplete last vector of the arrays, when the first group of [t0, t1) holds it: one thread of
-  // the launch reads it slot by slot, and waits at once so that the compiler's count of the loads in
-  // flight stays what it is on the path without this block.
-  auto fetch_tail = [&](auto bank, int t0, int t1) {
+  // Chunk c of group grp of a span: this thread's vector p0 and the row [t0, t1) it is part of.
+  auto unit = [&](const Span& sp, int c, int grp, int& p0, int& t0, int& t1) {
+    const bool other = (c == 1) && sp.pair;
+    t0 = other ? sp.b0 : sp.a0;
+    t1 = other ? sp.b1 : sp.a1;
+    p0 = (t0 & ~3) + (int)threadIdx.x * kVec + (other ? 0 : (grp * kRowHold + c) * kRowChunk);  // 16-byte aligned
+  };
+  // The first group of a span into bank B, as a FIXED number of loads in straight-line code: a vector
+  // beyond the row's end is requested at the row's last vector instead (one cache line for the whole
+  // wavefront, never used).  A load under a condition would leave the compiler unable to count the
+  // loads in flight behind the ones it waits for, and every wait would drain the prefetch as well.
+  auto prefetch = [&](auto bank, const Span& sp) {
     constexpr int B = decltype(bank)::value;
-    if (tail_p0 < 0 || tail_p0 >= t1) return;
-    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;
+    int p0[kRowHold];
 #pragma unroll
     for (int c = 0; c < kRowHold; ++c) {
-      if (thread_p + c * kRowChunk == tail_p0) {
+      int t0, t1;
+      unit(sp, c, 0, p0[c], t0, t1);
+      p0[c] = min(p0[c], min(max(t1 - 1, t0) & ~3, last_full));
+    }
+    // a row of several groups comes back to this one for its outputs: both arms issue the same loads
+    if (sp.a1 - (sp.a0 & ~3) > kRowHold * kRowChunk) {
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) op.template load<true>(p0[c], B, c);
+    } else {
+#pragma unroll
+      for (int c = 0; c < kRowHold; ++c) op.template load<false>(p0[c], B, c);
+    }
+  };
+  // The incomplete last vector of the arrays, when the first group of the span holds it: one thread of
+  // the launch reads it slot by slot, and waits at once so that the compiler's count of the loads in
+  // flight stays what it is on the path without this block.
+  auto fetch_tail = [&](auto bank, const Span& sp) {
+    constexpr int B = decltype(bank)::value;
+    if (tail_p0 < 0) return;
+#pragma unroll
+    for (int c = 0; c < kRowHold; ++c) {
+      int p0, t0, t1;
+      unit(sp, c, 0, p0, t0, t1);
+      if (p0 == tail_p0 && tail_p0 < t1) {
         op.template load_edge<false>(tail_p0, B, c);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
       }
     }
   };
   // a later group of a long row (or an earlier one again, for the output pass)
-  auto load_group = [&](auto bank, int grp, int t0, int t1, bool keep) {
+  auto load_group = [&](auto bank, const Span& sp, int grp, bool keep) {
     constexpr int B = decltype(bank)::value;
-    const int thread_p = (t0 & ~3) + (int)threadIdx.x * kVec;
 #pragma unroll
     for (int c = 0; c < kRowHold; ++c) {
-      const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
+      int p0, t0, t1;
+      unit(sp, c, grp, p0, t0, t1);
       if (p0 < t1 && p0 + kVec > t0) {
         if (keep) op.template load_edge<true>(p0, B, c);
         else op.template load_edge<false>(p0, B, c);
@@ -169,83 +202,93 @@ __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride,
     }
   };
   int parity = 0;
-  // one row in bank B; its first group has been requested; (n0, n1) is the next row, if there is one
-  auto row = [&](auto bank, int rr, int t0, int t1, bool has_next, int n0, int n1) {
+  // one span in bank B; its first group has been requested; `nxt` is the next span (not valid: none)
+  auto step = [&](auto bank, const Span& sp, const Span& nxt) {
     constexpr int B = decltype(bank)::value;
-    prefetch(std::integral_constant<int, B ^ 1>{}, has_next ? n0 : 0, has_next ? n1 : 0);
-    const int base = t0 & ~3;  // slots before t0 are not this row's
-    const int n_chunks = (t1 > t0) ? (t1 - base + kRowChunk - 1) / kRowChunk : 0;
-    const int n_groups = max((n_chunks + kRowHold - 1) / kRowHold, 1);
-    const int thread_p = base + (int)threadIdx.x * kVec;
-    float s[NV];
+    prefetch(std::integral_constant<int, B ^ 1>{}, nxt);
+    const int n_groups = max((chunks_of(sp.a0, sp.a1) + kRowHold - 1) / kRowHold, 1);
+    float s[kRowHold][NV];  // the sums of the chunks apart: two rows, or the two halves of one
 #pragma unroll
-    for (int i = 0; i < NV; ++i) s[i] = 0.f;
+    for (int c = 0; c < kRowHold; ++c)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) s[c][i] = 0.f;
     auto stat_group = [&](int grp) {
 #pragma unroll
       for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
+        int p0, t0, t1;
+        unit(sp, c, grp, p0, t0, t1);
         if (p0 >= t0 && p0 + kVec <= t1) {  // the whole vector belongs to the row
 #pragma unroll
-          for (int j = 0; j < kVec; ++j) op.stat(B, c, j, s);
+          for (int j = 0; j < kVec; ++j) op.stat(B, c, j, s[c]);
         } else if (p0 < t1 && p0 + kVec > t0) {
 #pragma unroll
           for (int j = 0; j < kVec; ++j)
-            if (p0 + j >= t0 && p0 + j < t1) op.stat(B, c, j, s);
+            if (p0 + j >= t0 && p0 + j < t1) op.stat(B, c, j, s[c]);
         }
       }
     };
-    auto emit_group = [&](int grp, const typename Op::RowVals& rv) {
-#pragma unroll
-      for (int c = 0; c < kRowHold; ++c) {
-        const int p0 = thread_p + (grp * kRowHold + c) * kRowChunk;
-        if (p0 < t1 && p0 + kVec > t0) op.emit(p0, B, c, rv, t0, t1);
-      }
+    auto emit_unit = [&](int c, int grp, const typename Op::RowVals& rv) {
+      int p0, t0, t1;
+      unit(sp, c, grp, p0, t0, t1);
+      if (p0 < t1 && p0 + kVec > t0) op.emit(p0, B, c, rv, t0, t1);
     };
-    // ---- pass 1: the row's sums.  The first group is in flight since the previous row (straight-line
+    // ---- pass 1: the rows' sums.  The first group is in flight since the previous step (straight-line
     // code up to its first use, so the wait leaves the prefetch alone); a long row fetches the others
     // one wait at a time and the registers keep the last.
-    fetch_tail(bank, t0, t1);
+    fetch_tail(bank, sp);
     stat_group(0);
 #pragma unroll 1
     for (int grp = 1; grp < n_groups; ++grp) {
-      load_group(bank, grp, t0, t1, grp < n_groups - 1);
+      load_group(bank, sp, grp, grp < n_groups - 1);
       stat_group(grp);
     }
 #pragma unroll
-    for (int i = 0; i < NV; ++i) s[i] = wave_total(s[i]);
+    for (int c = 0; c < kRowHold; ++c)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) s[c][i] = wave_total(s[c][i]);
     if (lane == 0) {
 #pragma unroll
-      for (int i = 0; i < NV; ++i) red[parity][wave][i] = s[i];
-    }
-    __syncthreads();  // one barrier per row: the next row writes the other half of `red`
-    float tot[NV];
+      for (int c = 0; c < kRowHold; ++c)
 #pragma unroll
-    for (int i = 0; i < NV; ++i)
-      tot[i] = ((red[parity][0][i] + red[parity][1][i]) + red[parity][2][i]) + red[parity][3][i];
+        for (int i = 0; i < NV; ++i) red[parity][wave][c * NV + i] = s[c][i];
+    }
+    __syncthreads();  // one barrier per step: the next step writes the other half of `red`
+    float tot[kRowHold][NV];
+#pragma unroll
+    for (int c = 0; c < kRowHold; ++c)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int k = c * NV + i;
+        tot[c][i] = ((red[parity][0][k] + red[parity][1][k]) + red[parity][2][k]) + red[parity][3][k];
+      }
     parity ^= 1;
-    const auto rv = op.rows(rr, tot, threadIdx.x == 0);
+    if (!sp.pair) {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) tot[0][i] += tot[1][i];
+    }
+    auto rv = op.rows(sp.r, tot[0], threadIdx.x == 0);
     // ---- pass 2: outputs, last group first (its inputs are still in the registers)
-    emit_group(n_groups - 1, rv);
+    emit_unit(0, n_groups - 1, rv);
+    if (sp.pair) rv = op.rows(sp.r + 1, tot[1], threadIdx.x == 0);
+    emit_unit(1, n_groups - 1, rv);
 #pragma unroll 1
     for (int grp = n_groups - 2; grp >= 0; --grp) {
-      load_group(bank, grp, t0, t1, false);
-      emit_group(grp, rv);
+      load_group(bank, sp, grp, false);
+      emit_unit(0, grp, rv);
+      emit_unit(1, grp, rv);
     }
   };
   using Bank0 = std::integral_constant<int, 0>;
   using Bank1 = std::integral_constant<int, 1>;
-  int t0 = 0, t1 = 0, n0 = 0, n1 = 0;
-  bool more = fetch(r, t0, t1);
-  if (more) prefetch(Bank0{}, t0, t1);
+  Span cur = span_at(r);
+  if (cur.valid) prefetch(Bank0{}, cur);
 #pragma unroll 1
-  while (more) {
-    bool next = fetch(r + 1, n0, n1);
-    row(Bank0{}, r, t0, t1, next, n0, n1);
-    ++r;
-    if (!next) break;
-    more = fetch(r + 1, t0, t1);
-    row(Bank1{}, r, n0, n1, more, t0, t1);
-    ++r;
+  while (cur.valid) {
+    const Span nxt = span_at(cur.r + (cur.pair ? 2 : 1));
+    step(Bank0{}, cur, nxt);
+    if (!nxt.valid) break;
+    cur = span_at(nxt.r + (nxt.pair ? 2 : 1));
+    step(Bank1{}, nxt, cur);
   }
   // slots outside every row (before the first row's start, after the last row's end) belong to no
   // sequence: one workgroup writes zeros there
@@ -383,7 +426,8 @@ struct OwnedLossOp {
 };
 
 template <int MK, int KIND>
-__global__ __launch_bounds__(kBlock) void owned_policy_loss_kernel(OwnedLossArgs g, RowStarts rs, int stride,
+// four workgroups per CU: the kernel is bound by the latencies of a step, which only other steps hide
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void owned_policy_loss_kernel(OwnedLossArgs g, RowStarts rs, int stride,
                                                                    float* ws, float* __restrict__ acc) {
   __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   // a caller-supplied batch denominator (utils.py:224-229) is known before the first token
@@ -482,7 +526,7 @@ struct OwnedCorrOp {
 };
 
 template <int MK>
-__global__ __launch_bounds__(kBlock) void owned_correction_kernel(OwnedCorrArgs g, RowStarts rs, int stride,
+__global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void owned_correction_kernel(OwnedCorrArgs g, RowStarts rs, int stride,
                                                                   float* ws, float* __restrict__ acc) {
   __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   OwnedCorrOp<MK> op(g, rs);
