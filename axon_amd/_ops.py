@@ -49,17 +49,24 @@ def _on_16_bytes(t: torch.Tensor) -> torch.Tensor:
 
 
 def f32(t: torch.Tensor) -> torch.Tensor:
-    return _on_16_bytes(t.detach().to(torch.float32).contiguous())
+    if t.requires_grad:
+        t = t.detach()
+    if t.dtype != torch.float32 or not t.is_contiguous():  # the usual operand passes through untouched
+        t = t.to(torch.float32).contiguous()
+    return _on_16_bytes(t)
 
 
 def mask_arg(mask: torch.Tensor):
     """Normalise a response mask once: fp32 and int64 are read natively by the kernels."""
-    mask = mask.detach()
+    if mask.requires_grad:
+        mask = mask.detach()
+    if not mask.is_contiguous():
+        mask = mask.contiguous()
     if mask.dtype == torch.int64:
-        return _on_16_bytes(mask.contiguous()), MASK_I64
+        return _on_16_bytes(mask), MASK_I64
     if mask.dtype != torch.float32:
         mask = mask.to(torch.float32)
-    return _on_16_bytes(mask.contiguous()), MASK_F32
+    return _on_16_bytes(mask), MASK_F32
 
 
 def _same_len(what: str, n: int, **tensors) -> None:
