@@ -186,14 +186,17 @@ __device__ __forceinline__ double wave_sum_d(double v) {
   return v;
 }
 
+// Four wavefronts per workgroup: what a wavefront spends here is mostly the 50 + 20 reductions at the end,
+// which cost the same for one row per lane as for four, and sixteen wavefronts would queue four deep on a SIMD.
+constexpr int kDiagRowThreads = 256;
 // Workgroup b of the grid takes token partials b, b + gridDim.x, ... and rows likewise, and leaves its
 // 70 sums / maxima / minima in out[b][kDiagOut]; sampler_diag_final_kernel folds the workgroups.
-__global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
+__global__ __launch_bounds__(kDiagRowThreads) void sampler_diag_rows_kernel(
     const float* __restrict__ partials, int n_blocks, const float* __restrict__ row_vals,
     int64_t n_rows, DiagCfg cfg, double* __restrict__ out_all) {
   double* out = out_all + (size_t)blockIdx.x * kDiagOut;
-  __shared__ double red[16][kOutSums];
-  __shared__ float red_mx[16][kOutMM], red_mn[16][kOutMM];
+  __shared__ double red[kDiagRowThreads / kWave][kOutSums];
+  __shared__ float red_mx[kDiagRowThreads / kWave][kOutMM], red_mn[kDiagRowThreads / kWave][kOutMM];
   const float kInf = __builtin_huge_valf();
   double acc[kOutSums];
 #pragma unroll
@@ -315,18 +318,27 @@ __global__ __launch_bounds__(1024) void sampler_diag_rows_kernel(
   }
 }
 
-__global__ __launch_bounds__(128) void sampler_diag_final_kernel(const double* __restrict__ parts, int n_parts,
-                                                                 double* __restrict__ out) {
-  const int k = threadIdx.x;
-  if (k >= kOutSums + 2 * kOutMM) return;
-  double v = parts[k];
-  for (int b = 1; b < n_parts; ++b) {
-    const double x = parts[(size_t)b * kDiagOut + k];
-    if (k < kOutSums) v += x;
-    else if (k < kOutSums + kOutMM) v = fmax(v, x);
-    else v = fmin(v, x);
+// One workgroup folds the row pass's per-workgroup results: wavefront w takes outputs w, w + 16, ...,
+// its lanes read the parts side by side (a serial walk over 128 parts would be 128 dependent loads).
+// Fixed order: lane l adds parts l, l + 64, ..., then the wavefront's fixed tree.
+__global__ __launch_bounds__(1024) void sampler_diag_final_kernel(const double* __restrict__ parts, int n_parts,
+                                                                  double* __restrict__ out) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n_waves = (int)(blockDim.x >> 6);
+  const double kInf = (double)__builtin_huge_valf();
+  for (int k = wave; k < kOutSums + 2 * kOutMM; k += n_waves) {
+    const bool is_sum = k < kOutSums, is_max = !is_sum && k < kOutSums + kOutMM;
+    double v = is_sum ? 0.0 : (is_max ? -kInf : kInf);
+    for (int b = lane; b < n_parts; b += kWave) {
+      const double x = parts[(size_t)b * kDiagOut + k];
+      v = is_sum ? v + x : (is_max ? fmax(v, x) : fmin(v, x));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const double x = __shfl_down(v, off, kWave);
+      v = is_sum ? v + x : (is_max ? fmax(v, x) : fmin(v, x));
+    }
+    if (lane == 0) out[k] = v;
   }
-  out[k] = v;
 }
 
 }  // namespace axon
@@ -384,10 +396,10 @@ extern "C" int axon_sampler_diag(const float* oldp, const float* samp, const voi
   const int64_t floats = kDiagRowVals * n_rows + (int64_t)g.x * kDiagStride;
   double* parts = reinterpret_cast<double*>(workspace + (floats + 1) / 2 * 2);
   const int rb = diag_row_blocks(n_rows, g.x);
-  hipLaunchKernelGGL(sampler_diag_rows_kernel, dim3(rb), dim3(1024), 0, st, partials, (int)g.x, row_vals,
+  hipLaunchKernelGGL(sampler_diag_rows_kernel, dim3(rb), dim3(kDiagRowThreads), 0, st, partials, (int)g.x, row_vals,
                      n_rows, cfg, parts);
   AXON_CHECK_LAUNCH();
-  hipLaunchKernelGGL(sampler_diag_final_kernel, dim3(1), dim3(128), 0, st, parts, rb, out);
+  hipLaunchKernelGGL(sampler_diag_final_kernel, dim3(1), dim3(1024), 0, st, parts, rb, out);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
