@@ -236,11 +236,11 @@ def group_scalar(mode, scores, lens, members, offsets, n_groups, *, eps=1e-6, no
 
 
 # Operators that need a per-row quantity run as ONE launch in which a workgroup owns whole rows (one read of every
-# input, row sums that repeat bit for bit) when the rows are long enough to fill a workgroup: it works on one row
-# at a time, so a batch of rows of a few tokens each would leave most of its threads idle.  Otherwise, and beyond
-# ``OWNED_ROWS_MAX_SLOTS`` tokens, a token-parallel row pass followed by a token pass (two reads, float atomics
-# per row).  At 2^26 tokens the two take the same time (0.39 ms); at the sizes of real micro-batches the single
-# launch is 2-3 times faster.
+# input, row sums that repeat bit for bit) when the rows are long enough to fill a workgroup: it works on one or
+# two rows at a time, so a batch of rows of a few tokens each would leave most of its threads idle.  Otherwise, and
+# beyond ``OWNED_ROWS_MAX_SLOTS`` tokens, a token-parallel row pass followed by a token pass (two reads, float
+# atomics per row).  At 2^26 tokens 0.31-0.34 ms against 0.40-0.43; at the sizes of real micro-batches one launch
+# instead of four or five.
 OWNED_ROWS_MAX_SLOTS = 1 << 40
 OWNED_ROWS_MIN_MEAN_LEN = 64
 

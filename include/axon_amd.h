@@ -373,8 +373,9 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
  * workgroup owns whole rows, keeps their tokens in registers between the row sums and the token
  * pass, and forms the row sums in a fixed order without atomics, so the sequence ratio repeats bit
  * for bit from run to run.  A row of more than 2048 tokens is read a second time, all but its last
- * 2048.  A workgroup works on one row at a time, so the kernel suits batches whose rows are at least
- * some tens of tokens long on average (for shorter rows use the calls it replaces).
+ * 2048.  A workgroup works on one row (or two short ones) at a time, so the kernel suits batches
+ * whose rows are at least some tens of tokens long on average (for shorter rows use the calls it
+ * replaces).
  *   kind, masks, ratio_lo / ratio_hi / clip_c, grad, acc[0..5]: as in axon_policy_loss (kinds 0-4).
  *   token_reduce / batch_reduce / per_row_token_count / num_program_tokens / num_program_steps /
  *   valid_count: as in axon_loss_row_scale.  Without valid_count the batch denominator (sum of the
