@@ -353,7 +353,9 @@ struct OwnedLossArgs {
   float* grad;
 };
 
-template <int MK, int KIND>
+// HAS_W: importance weights are given (their loads are part of the fixed count of a step's loads, so the
+// two cases are two kernels and not a branch)
+template <int MK, int KIND, bool HAS_W>
 struct OwnedLossOp {
   static constexpr int kNV = 2;  // sum mask, sum (logp - old) * mask
   struct RowVals { float scale, sbar; Ratio seq; };  // seq: GSPO's ratio of the sequence (KIND 1)
@@ -367,8 +369,6 @@ struct OwnedLossOp {
   __device__ __forceinline__ OwnedLossOp(const OwnedLossArgs& g_, const RowStarts& rs_, float bd)
       : g(g_), rs(rs_), bden(bd) {}
 
-  // Always the same number of loads (the walk counts on it): without importance weights the slot of
-  // `wv` is filled from the advantages' lines, which are on their way anyway, and not used.
   template <bool KEEP>
   __device__ __forceinline__ void load(int p0, int b, int c) {
     row_load4<KEEP>(g.logp, p0, lv[b][c]);
@@ -376,7 +376,7 @@ struct OwnedLossOp {
     row_load_mask4<MK, KEEP>(g.mask, p0, mv[b][c]);
     // read by the output pass only, requested with the rest so that one wait covers all
     row_load4<KEEP>(g.adv, p0, av[b][c]);
-    row_load4<KEEP>(g.isw ? g.isw : g.adv, p0, wv[b][c]);
+    if (HAS_W) row_load4<KEEP>(g.isw, p0, wv[b][c]);
   }
   template <bool KEEP>
   __device__ __forceinline__ void load_edge(int p0, int b, int c) {
@@ -384,7 +384,7 @@ struct OwnedLossOp {
     row_load4_guard<KEEP>(g.oldp, p0, rs.n_slots, ov[b][c]);
     row_load_mask4_guard<MK, KEEP>(g.mask, p0, rs.n_slots, mv[b][c]);
     row_load4_guard<KEEP>(g.adv, p0, rs.n_slots, av[b][c]);
-    row_load4_guard<KEEP>(g.isw ? g.isw : g.adv, p0, rs.n_slots, wv[b][c]);
+    if (HAS_W) row_load4_guard<KEEP>(g.isw, p0, rs.n_slots, wv[b][c]);
   }
   __device__ __forceinline__ void stat(int b, int c, int j, float (&s)[2]) const {
     const float m = mv[b][c][j];
@@ -414,7 +414,7 @@ struct OwnedLossOp {
       const int p = p0 + j;
       gv[j] = 0.f;
       if (!whole && (p < t0 || p >= t1)) continue;
-      const float w = g.isw ? wv[b][c][j] : 1.f;
+      const float w = HAS_W ? wv[b][c][j] : 1.f;
       const TokenTerm t = (KIND == 1) ? gspo_token(rv.seq, lv[b][c][j], ov[b][c][j], av[b][c][j], w, g.clip_c)
                                       : policy_token<KIND>(lv[b][c][j], ov[b][c][j], av[b][c][j], w, rv.sbar, g.lo,
                                                            g.hi, g.clip_c, false);
@@ -425,14 +425,14 @@ struct OwnedLossOp {
   __device__ __forceinline__ void fill_gap(int64_t a0, int64_t b0) { zero_range(g.grad, a0, b0); }
 };
 
-template <int MK, int KIND>
+template <int MK, int KIND, bool HAS_W>
 // four workgroups per CU: the kernel is bound by the latencies of a step, which only other steps hide
 __global__ __launch_bounds__(kBlock) __attribute__((amdgpu_waves_per_eu(4))) void owned_policy_loss_kernel(OwnedLossArgs g, RowStarts rs, int stride,
                                                                    float* ws, float* __restrict__ acc) {
   __shared__ float lds_red[kPartialStride * (kBlock / kWave)];
   // a caller-supplied batch denominator (utils.py:224-229) is known before the first token
   const float bden = (g.valid != nullptr) ? fmaxf((float)g.valid[0], 1.f) : 1.f;
-  OwnedLossOp<MK, KIND> op(g, rs, bden);
+  OwnedLossOp<MK, KIND, HAS_W> op(g, rs, bden);
   walk_owned_rows(rs, stride, op);
   float part[7] = {op.a[0], op.a[1], op.a[2], op.a[3], op.a[4], 0.f, op.rows_with_tokens};
   const int batch_reduce = g.batch_reduce;
@@ -602,12 +602,17 @@ extern "C" int axon_policy_loss_rows(int kind, const float* logp, const float* o
                         ratio_lo, ratio_hi, clip_c, grad};
   const RowStarts rs{cu, uniform_len, n_rows, n_slots};
   const hipStream_t st = (hipStream_t)stream;
-#define AXON_LAUNCH_OWNED(MK, KD)                                                                       \
+#define AXON_LAUNCH_OWNED_W(MK, KD, HW)                                                                   \
   do {                                                                                                  \
-    static const int resident = resident_blocks(owned_policy_loss_kernel<MK, KD>);                      \
+    static const int resident = resident_blocks(owned_policy_loss_kernel<MK, KD, HW>);                  \
     const OwnedLaunch ol = owned_launch(n_slots, resident);                                             \
-    hipLaunchKernelGGL((owned_policy_loss_kernel<MK, KD>), dim3(ol.grid), dim3(kBlock), 0, st, g, rs,   \
-                       ol.stride, partials, acc);                                                       \
+    hipLaunchKernelGGL((owned_policy_loss_kernel<MK, KD, HW>), dim3(ol.grid), dim3(kBlock), 0, st, g,   \
+                       rs, ol.stride, partials, acc);                                                   \
+  } while (0)
+#define AXON_LAUNCH_OWNED(MK, KD)                 \
+  do {                                            \
+    if (isw) AXON_LAUNCH_OWNED_W(MK, KD, true);   \
+    else AXON_LAUNCH_OWNED_W(MK, KD, false);      \
   } while (0)
   if (mask_kind == AXON_MASK_F32) {
     if (kind == 0) AXON_LAUNCH_OWNED(AXON_MASK_F32, 0);
@@ -623,6 +628,7 @@ extern "C" int axon_policy_loss_rows(int kind, const float* logp, const float* o
     else AXON_LAUNCH_OWNED(AXON_MASK_I64, 4);
   }
 #undef AXON_LAUNCH_OWNED
+#undef AXON_LAUNCH_OWNED_W
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
