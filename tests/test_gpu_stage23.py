@@ -1017,6 +1017,23 @@ def test_packed_layout_without_rows_is_refused():
     torch.cuda.synchronize()
 
 
+def test_row_owned_entry_points_refuse_fewer_than_four_slots():
+    """The kernels in which a workgroup owns whole rows read 16-byte vectors: one to three slots are refused
+    with the shape error (the host sends such inputs through the row pass + token pass), four are taken."""
+    from axon_amd import _lib
+    lib = _lib.load()
+    t = torch.zeros(8, device=DEV)
+    ws = torch.zeros(lib.axon_reduce_partials_bytes(8) // 4, device=DEV)
+    st = torch.cuda.current_stream().cuda_stream
+    p = lambda x: x.data_ptr()  # noqa: E731
+    for n, want in ((1, -2), (3, -2), (4, 0)):
+        assert lib.axon_policy_loss_rows(1, p(t), p(t), p(t), p(t), 0, None, None, 1, n, n, 1, 1, None, None, None,
+                                         None, 0.8, 1.2, 3.0, p(t), p(t), p(ws), st) == want
+        assert lib.axon_sampler_correction_rows(p(t), p(t), p(t), 0, None, 1, n, n, 1, 2.0, 1, -0.7, 0.7, 1, -9.0,
+                                                p(t), p(t), None, None, None, p(t), p(ws), st) == want
+    torch.cuda.synchronize()
+
+
 def test_all_padding_micro_batch_is_a_no_op_before_any_validation():
     """sampler.py:368-370: an all-zero mask returns (None, mask, {}) even with arguments that would not
     validate; with a token to correct the same arguments raise."""
