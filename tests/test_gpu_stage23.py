@@ -1017,6 +1017,36 @@ def test_packed_layout_without_rows_is_refused():
     torch.cuda.synchronize()
 
 
+def _random_layout(seed):
+    """Row lengths drawn from a mixture: empty and tiny rows, rows under a chunk of 1024 slots (which share a step
+    in pairs), rows of one to two chunks, rows of several groups of 2048; any slot count modulo four."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    kinds = torch.randint(0, 5, (40,), generator=g).tolist()
+    lens = []
+    for k in kinds:
+        lo, hi = ((0, 4), (4, 200), (200, 1025), (1025, 2100), (2100, 7000))[k]
+        lens.append(int(torch.randint(lo, hi, (1,), generator=g)))
+    return lens
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_row_owned_kernels_on_random_layouts(seed, owned_rows_forced):
+    """GSPO (sequence ratio and per-row mean), the veto and sequence-level weights on random mixtures of row
+    lengths against the oracle: every kind of step of the row walk next to every other."""
+    lens = _random_layout(seed)
+    d, pad = _awkward_packed(lens, seed=500 + seed)
+    _check_loss("gspo", OL.gspo_loss, d, {"clip_ratio_low": 0.1, "clip_ratio_high": 0.1, "token_reduce": "mean",
+                                          "batch_reduce": "step-mean"}, meta={"cu_seqlens": d["cu_seqlens"]}, pad=pad)
+    kw = dict(sampler_is="sequence", sampler_is_threshold=2.0, sampler_rs="geometric", sampler_rs_threshold=2.0,
+              sampler_token_veto_threshold=0.4)
+    proto, new, _ = S.compute_sampler_correction_and_rejection_mask(
+        d["old_log_probs"].to(DEV), d["sampler_log_probs"].to(DEV), d["response_mask"].to(DEV),
+        cu_seqlens=d["cu_seqlens"].to(DEV), **kw)
+    w_ref, new_ref, _ = OS.correction(pad["old_log_probs"], pad["sampler_log_probs"], pad["response_mask"], **kw)
+    assert torch.equal(new.cpu(), pad_to_packed(new_ref, lens))
+    assert torch.allclose(proto.batch["sampler_is_weights"].cpu(), pad_to_packed(w_ref, lens), rtol=1e-5, atol=1e-7)
+
+
 def test_row_owned_entry_points_refuse_fewer_than_four_slots():
     """The kernels in which a workgroup owns whole rows read 16-byte vectors: one to three slots are refused
     with the shape error (the host sends such inputs through the row pass + token pass), four are taken."""
