@@ -85,10 +85,11 @@ __device__ __forceinline__ float wave_total(float v) {  // the same value in eve
 //   rows(r, tot[], first) -> RowVals  the per-row values from the row's sums (every thread the same)
 //   emit(p0, b, c, rv, t0, t1)        write the outputs of the vector in register set (b, c)
 //   fill_gap(a, b)                    zeros for slots that belong to no row
-// Two banks of register sets: while a row is worked on in one bank, the first group of the next row
-// is already on its way into the other, so a row's loads have a whole row's time to arrive.  Every
-// thread of the workgroup walks the same rows (the loop bounds are uniform), so the barrier inside
-// the loop is reached by all; it waits for LDS only, not for the loads in flight.
+// Two banks of register sets: while a step (a row, or two short ones) is worked on in one bank, the
+// first group of the next step is already on its way into the other, so its loads have a whole
+// step's time to arrive.  Every thread of the workgroup walks the same rows (the loop bounds are
+// uniform), so the barrier inside the loop is reached by all; it waits for LDS only, not for the
+// loads in flight.
 template <class Op>
 __device__ __forceinline__ void walk_owned_rows(const RowStarts& rs, int stride, Op& op) {
   constexpr int NV = Op::kNV;
