@@ -68,9 +68,6 @@ def build(verbose: bool = False) -> str:
 
 
 def ensure_built() -> str:
-    override = os.environ.get("AXON_AMD_LIB")  # an explicitly named build of the same sources
-    if override:
-        return override
     if not os.path.exists(LIB_PATH):
         build()
     return LIB_PATH

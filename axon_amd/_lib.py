@@ -34,6 +34,13 @@ SIGNATURES: dict[str, tuple] = {
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                      _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_block_begin": (_i32, [_ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_block_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr, _i64,
+                                     _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_block_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
+                                     _f32, _f32, _ptr, _i64, _ptr, _ptr, _ptr, _i32, _i32, _i64, _ptr, _i64,
+                                     _ptr, _i64, _ptr, _ptr]),
+    "axon_scale_bf16_unless_one": (_i32, [_ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_active_rows": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_gather_rows": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64,
                                        _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
@@ -84,7 +91,7 @@ SIGNATURES: dict[str, tuple] = {
                                         _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
 }
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

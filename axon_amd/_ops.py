@@ -793,6 +793,131 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
     return d_hidden, d_weight
 
 
+DW_STORE, DW_FIRST, DW_ADD, DW_LAST = 0, 1, 2, 3
+
+
+class HeadBlocks:
+    """One step of the head as blocks of consecutive tokens (``axon_lmhead_block_*``): forward of a block over
+    the whole vocabulary with a stash, then (by the caller) the loss on the block's positions, then the block's
+    backward from the stash, then the next block.  Holds the step's operands and everything the blocks share:
+    the stash and the workspaces (sized for the largest block, allocated once), the transposed weight, the
+    fp32 accumulator of the weight gradient, and the whole-stream outputs.
+
+    ``hidden`` ``[N, H]`` and ``weight`` ``[V, H]`` bf16; ``labels`` ``[N]`` (with ``seq_start``: the packed id
+    stream, outputs and gradients aligned to token positions, see ``lmhead_forward``).  ``ranges``: the hidden
+    rows ``(first, end)`` of every block, in ascending order and covering all rows.  A block may begin before
+    the previous one ends: the shared rows must reach the earlier block with a zero gradient (it then adds
+    nothing for them), the later block writes their outputs and their ``d_hidden`` again.  ``vocab_chunk``: 0 =
+    the backward of a block takes the whole vocabulary in one piece (no fp32 read-modify-write of the block's
+    d_hidden; bf16 dlogits of 2 x block x vocab x 2 bytes), else a multiple of 256."""
+
+    def __init__(self, hidden, weight, labels, inv_temperature, ranges, *, softcap=0.0, seq_start=None,
+                 vocab_chunk=0, stash=True, timing: "Timer | None" = None):
+        self.lib = _lib.load()
+        require_device(hidden, "HeadBlocks")
+        self.n, self.h, self.v = _head_operands("HeadBlocks", hidden, weight, labels, seq_start)
+        self.ranges = [(int(a), int(b)) for a, b in ranges]
+        ok = bool(self.ranges) and self.ranges[0][0] == 0 and self.ranges[-1][1] == self.n
+        ok = ok and all(a < b for a, b in self.ranges)
+        ok = ok and all(a1 < a2 <= b1 <= b2 for (a1, b1), (a2, b2) in zip(self.ranges, self.ranges[1:]))
+        if not ok:
+            raise ValueError(f"HeadBlocks: row ranges {self.ranges} do not cover {self.n} rows in ascending order")
+        self.hidden, self.weight, self.labels, self.seq_start = hidden, weight, labels, seq_start
+        self.inv_t, self.softcap, self.timing = float(inv_temperature), float(softcap), timing
+        dev = hidden.device
+        n_max = max(b - a for a, b in self.ranges)
+        self.chunk = int(vocab_chunk) if vocab_chunk else (self.v + 255) // 256 * 256
+        self.fwd_ws_bytes = self.lib.axon_lmhead_fwd_workspace_bytes(n_max, self.h, self.v)
+        self.bwd_ws_bytes = self.lib.axon_lmhead_bwd_workspace_bytes(n_max, self.h, self.v, self.chunk)
+        if self.fwd_ws_bytes < 0 or self.bwd_ws_bytes < 0:
+            raise _lib.AxonAmdError(f"HeadBlocks: unsupported shape tokens={n_max} hidden={self.h} vocab={self.v}")
+        self.fwd_ws = torch.empty(self.fwd_ws_bytes, device=dev, dtype=torch.uint8)
+        self.bwd_ws = torch.empty(self.bwd_ws_bytes, device=dev, dtype=torch.uint8)
+        self.stash_bytes = max(lmhead_stash_bytes(b - a, self.h, self.v) for a, b in self.ranges) if stash else 0
+        self.stash = torch.empty(self.stash_bytes, device=dev, dtype=torch.uint8) if self.stash_bytes else None
+        self.stats = torch.empty(2, n_max, device=dev, dtype=torch.float32)  # lse, entropy_b of the current block
+        # whole-stream outputs; position 0 is a sequence start (the aligned layout writes it from the last row)
+        self.out = torch.zeros(2, max(self.n, 1), device=dev, dtype=torch.float32)
+        self.d_hidden = torch.empty_like(hidden)
+        self.d_weight = torch.empty_like(weight)
+        self.one_block = len(self.ranges) == 1
+        self.dw_acc = None if self.one_block else torch.empty(self.v, self.h, device=dev, dtype=torch.float32)
+        self.wt_ready = False
+        self.block_stash_bytes = 0
+        self.workspace_bytes = (self.fwd_ws_bytes + self.bwd_ws_bytes + self.stash_bytes +
+                                (0 if self.one_block else self.v * self.h * 4))
+
+    @property
+    def logprobs(self):
+        return self.out[0][: self.n]
+
+    @property
+    def entropy(self):
+        return self.out[1][: self.n]
+
+    def _block(self, k):
+        n0, n1 = self.ranges[k]
+        last_dst = 0 if self.seq_start is None else (n1 - n0 if n1 < self.n else -n0)
+        return n0, n1, last_dst
+
+    def _at(self, t, n0):
+        """Pointer to element ``n0`` of a whole-stream array (None stays None)."""
+        return None if t is None else t.data_ptr() + n0 * t.element_size()
+
+    def forward(self, k):
+        """Forward of block ``k``: its positions of ``logprobs`` / ``entropy`` (with ``seq_start``: positions
+        ``first + 1 .. end`` of its rows, the stream's last row goes to position 0) are valid once the
+        stream reaches the point after the call."""
+        n0, n1, last_dst = self._block(k)
+        nb = n1 - n0
+        self.block_stash_bytes = lmhead_stash_bytes(nb, self.h, self.v) if self.stash is not None else 0
+        check(self.lib.axon_lmhead_block_fwd(
+            self.hidden.data_ptr() + n0 * self.h * 2, ptr(self.weight), self._at(self.labels, n0),
+            int(self.labels.dtype == torch.int64), nb, self.h, self.v, self.inv_t, self.softcap,
+            self._at(self.seq_start, n0), last_dst, self._at(self.out[0], n0), self._at(self.out[1], n0),
+            ptr(self.stats[0]), ptr(self.stats[1]), ptr(self.fwd_ws), self.fwd_ws_bytes,
+            ptr(self.stash) if self.block_stash_bytes else None, self.block_stash_bytes, stream_ptr(),
+            self.timing.handle if self.timing else None), "axon_lmhead_block_fwd")
+
+    def backward(self, k, dlogprobs, dentropy):
+        """Backward of block ``k`` (after its ``forward``; no other block's forward in between).  ``dlogprobs`` /
+        ``dentropy`` (fp32, ``dentropy`` may be None): whole-stream arrays, read at the block's positions."""
+        n0, n1, last_dst = self._block(k)
+        nb = n1 - n0
+        if dlogprobs.dtype != torch.float32 or int(dlogprobs.numel()) < self.n or not dlogprobs.is_contiguous():
+            raise ValueError("HeadBlocks.backward: dlogprobs must be a contiguous fp32 array over the whole stream")
+        if dentropy is not None and (dentropy.dtype != torch.float32 or int(dentropy.numel()) < self.n
+                                     or not dentropy.is_contiguous()):
+            raise ValueError("HeadBlocks.backward: dentropy must be a contiguous fp32 array over the whole stream")
+        st = stream_ptr()
+        th = self.timing.handle if self.timing else None
+        if not self.wt_ready:
+            check(self.lib.axon_lmhead_block_begin(ptr(self.weight), self.h, self.v, self.chunk, ptr(self.bwd_ws),
+                                                   self.bwd_ws_bytes, st, th), "axon_lmhead_block_begin")
+            self.wt_ready = True
+        last = k == len(self.ranges) - 1
+        mode = DW_STORE if self.one_block else DW_FIRST if k == 0 else DW_LAST if last else DW_ADD
+        check(self.lib.axon_lmhead_block_bwd(
+            self._at(dlogprobs, n0), self._at(dentropy, n0), self.hidden.data_ptr() + n0 * self.h * 2,
+            ptr(self.weight), self._at(self.labels, n0), int(self.labels.dtype == torch.int64),
+            ptr(self.stats[0]), ptr(self.stats[1]), nb, self.h, self.v, self.inv_t, self.softcap,
+            self._at(self.seq_start, n0), last_dst, self.d_hidden.data_ptr() + n0 * self.h * 2,
+            ptr(self.d_weight), ptr(self.dw_acc), mode, 1, self.chunk, ptr(self.bwd_ws), self.bwd_ws_bytes,
+            ptr(self.stash) if self.block_stash_bytes else None, self.block_stash_bytes, st, th),
+            "axon_lmhead_block_bwd")
+
+
+def scale_bf16_unless_one(x, scale):
+    """``x *= scale`` in place (bf16 ``x``, ``scale`` a device scalar); no memory traffic when it is exactly 1."""
+    lib = _lib.load()
+    require_device(x, "scale_bf16_unless_one")
+    if x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("scale_bf16_unless_one: x must be contiguous bf16")
+    s = scale.detach().to(device=x.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
+    check(lib.axon_scale_bf16_unless_one(ptr(x), int(x.numel()), ptr(s), stream_ptr()), "axon_scale_bf16_unless_one")
+    return x
+
+
 _LOGITS_DTYPES = {torch.float32: 0, torch.bfloat16: 1}
 
 

@@ -216,10 +216,14 @@ __global__ __launch_bounds__(kGemmThreads) void lmhead_fwd_softcap_stash_kernel(
 // sequence's first position receives 0 (there is no prediction for it) and its upstream gradient
 // is ignored.  This is roll(ids, -1) before and the shift-right after the head
 // (axon/utils/fsdp/forward_utils.py:131,180-182) without the extra passes.  The position after the
-// last one wraps to 0, which is always a sequence start.
-__device__ __forceinline__ int aligned_pos(int n, int n_tokens, const uint8_t* is_start) {
+// last one is `last_dst`: 0 for a whole packed stream (it wraps to the first position, which is always
+// a sequence start).  A call that covers a block of consecutive positions of a longer stream hands
+// over its arrays offset to the block's first position and names where its last row's output goes:
+// n_tokens (the stream goes on: the first position of the next block) or minus the block's first
+// position (the block ends the stream: position 0 of the stream).
+__device__ __forceinline__ int aligned_pos(int n, int n_tokens, const uint8_t* is_start, int last_dst) {
   if (is_start == nullptr) return n;
-  return (n + 1 == n_tokens) ? 0 : n + 1;
+  return (n + 1 == n_tokens) ? last_dst : n + 1;
 }
 
 __global__ __launch_bounds__(256) void seq_start_kernel(const int32_t* __restrict__ cu, int n_seqs,
@@ -240,7 +244,7 @@ __global__ __launch_bounds__(kMergeTokens * kMergeGroups) void lmhead_merge_kern
     const float* __restrict__ pm, const float* __restrict__ ps, const float* __restrict__ pe,
     int parts, int n_tokens, float* __restrict__ lse, float* __restrict__ entropy_b,
     float* __restrict__ entropy, float* __restrict__ fin_max, float* __restrict__ fin_log2s,
-    const uint8_t* __restrict__ is_start) {
+    const uint8_t* __restrict__ is_start, int last_dst) {
   __shared__ float red[3][kMergeGroups][kMergeTokens];
   const int tok = threadIdx.x % kMergeTokens, grp = threadIdx.x / kMergeTokens;
   const int n = blockIdx.x * kMergeTokens + tok;
@@ -279,7 +283,7 @@ __global__ __launch_bounds__(kMergeTokens * kMergeGroups) void lmhead_merge_kern
   const float d = e / s;
   lse[n] = (M + L) * kLn2;
   entropy_b[n] = (M + d) * kLn2;
-  const int dst = aligned_pos(n, n_tokens, is_start);
+  const int dst = aligned_pos(n, n_tokens, is_start, last_dst);
   entropy[dst] = (is_start && is_start[dst]) ? 0.f : (L - d) * kLn2;
   fin_max[n] = M;
   fin_log2s[n] = L;
@@ -291,11 +295,11 @@ __global__ __launch_bounds__(256) void lmhead_label_kernel(
     const __bf16* __restrict__ hidden, const __bf16* __restrict__ weight,
     const LabelT* __restrict__ labels, int n_tokens, int hidden_sz, int vocab, float inv_temp,
     float cap, const float* __restrict__ fin_max, const float* __restrict__ fin_log2s,
-    float* __restrict__ logprobs, const uint8_t* __restrict__ is_start) {
+    float* __restrict__ logprobs, const uint8_t* __restrict__ is_start, int last_dst) {
   const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= n_tokens) return;
   const int lane = threadIdx.x & 63;
-  const int dst = aligned_pos(n, n_tokens, is_start);
+  const int dst = aligned_pos(n, n_tokens, is_start, last_dst);
   const int64_t lab = (int64_t)labels[dst];
   float dot = 0.f;
   if (lab >= 0 && lab < vocab) {
@@ -337,6 +341,7 @@ struct DlogitParams {
   float inv_temp;
   float cap, inv_cap;  // soft-capping (SOFTCAP kernels only)
   const uint8_t* is_start;  // token-aligned packed layout (see aligned_pos), or null
+  int last_dst;             // where the last row's label and gradients live (see aligned_pos)
 };
 
 // Four rows of four bf16 (rws[f] = row f) -> their transpose (o[e] = column e).
@@ -376,7 +381,7 @@ struct TokenCoef {
   __device__ __forceinline__ TokenCoef(const DlogitParams& p, int n, int64_t m0_abs) {
     n_ok = n < p.n_tokens;
     nn = n_ok ? n : 0;
-    const int src = aligned_pos(nn, p.n_tokens, p.is_start);  // where the label and the gradients live
+    const int src = aligned_pos(nn, p.n_tokens, p.is_start, p.last_dst);  // where the label and the gradients live
     const bool g_ok = n_ok && !(p.is_start && p.is_start[src]);
     const float g_lp = g_ok ? p.dlogprobs[src] : 0.f;
     const float g_en = (g_ok && p.dentropy) ? p.dentropy[src] : 0.f;
@@ -668,6 +673,7 @@ struct StoreParams {
   int64_t ld_f32, ld_bf16;
   int m_valid, n_valid;
   int accumulate;     // add the previous contents of out_f32 first
+  int keep_f32;       // write the sum back to out_f32 (0: out_f32 is only read, the sum leaves as bf16)
 };
 
 template <class Loop>
@@ -698,7 +704,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g
           const float4 old = *dst;
           v.x += old.x; v.y += old.y; v.z += old.z; v.w += old.w;
         }
-        *dst = v;
+        if (p.keep_f32) *dst = v;
       }
       if (p.out_bf16) {
         uint2 w;
@@ -787,7 +793,7 @@ __global__ __launch_bounds__(1024) void active_rows_kernel(
       const int n = first + j;
       act[j] = false;
       if (n < n_tokens) {
-        const int src = aligned_pos(n, n_tokens, is_start);
+        const int src = aligned_pos(n, n_tokens, is_start, 0);
         if (!(is_start && is_start[src]))
           act[j] = dlogprobs[src] != 0.f || (dentropy && dentropy[src] != 0.f);  // NaN counts as active
       }
@@ -835,7 +841,7 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(
   uint4* dst_row = hidden_c + (int64_t)r * row_vec;
   for (int c = threadIdx.x; c < row_vec; c += 256) dst_row[c] = src_row[c];
   if (threadIdx.x == 0) {
-    const int src = aligned_pos(n, n_tokens, is_start);
+    const int src = aligned_pos(n, n_tokens, is_start, 0);
     labels_c[r] = labels[src];
     lse_c[r] = lse[n];
     entropy_b_c[r] = entropy_b[n];
@@ -857,6 +863,22 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(const uint4* __restri
   }
   const uint4* src_row = d_hidden_c + (int64_t)r * row_vec;
   for (int c = threadIdx.x; c < row_vec; c += 256) dst_row[c] = src_row[c];
+}
+
+// x *= scale[0] in place on bf16 values, eight per thread and access; nothing is read or written when the
+// factor is exactly one (the factor lives on the device: the host does not know it without waiting).
+__global__ __launch_bounds__(256) void scale_bf16_kernel(uint4* __restrict__ x, int64_t n_vec,
+                                                         const float* __restrict__ scale) {
+  const float s = scale[0];
+  if (s == 1.f) return;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n_vec; i += (int64_t)gridDim.x * 256) {
+    uint4 v = x[i];
+    uint32_t* w = reinterpret_cast<uint32_t*>(&v);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      w[k] = pack_bf16(__uint_as_float(w[k] << 16) * s, __uint_as_float(w[k] & 0xffff0000u) * s);
+    x[i] = v;
+  }
 }
 
 }  // namespace axon
@@ -1065,8 +1087,9 @@ int launch_zero_cols(void* p, int64_t ld, int rows, int col0, int ncols, hipStre
 
 int fwd_impl(const void* hidden, const void* weight, const void* labels, int labels_i64, int64_t n,
              int64_t h, int64_t v, float inv_temp, float softcap, const uint8_t* is_start,
-             float* logprobs, float* entropy, float* lse, float* entropy_b, void* workspace,
-             int64_t ws_bytes, void* stash, int64_t stash_bytes, void* stream, PhaseTimer* timer) {
+             int64_t last_dst, float* logprobs, float* entropy, float* lse, float* entropy_b,
+             void* workspace, int64_t ws_bytes, void* stash, int64_t stash_bytes, void* stream,
+             PhaseTimer* timer) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (n == 0) return AXON_OK;
@@ -1112,7 +1135,7 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
     hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned)((n + kMergeTokens - 1) / kMergeTokens)),
                        dim3(kMergeTokens * kMergeGroups), 0, st,
                        w.pm, w.ps, w.pe, w.parts, (int)n, lse, entropy_b, entropy, w.fin_max,
-                       w.fin_log2s, is_start);
+                       w.fin_log2s, is_start, (int)last_dst);
   }
   AXON_CHECK_LAUNCH();
   const dim3 lg((unsigned)((n + 3) / 4));
@@ -1121,32 +1144,50 @@ int fwd_impl(const void* hidden, const void* weight, const void* labels, int lab
     hipLaunchKernelGGL(lmhead_label_kernel<int64_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int64_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start);
+                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start, (int)last_dst);
   else
     hipLaunchKernelGGL(lmhead_label_kernel<int32_t>, lg, dim3(256), 0, st,
                        static_cast<const __bf16*>(hidden), static_cast<const __bf16*>(weight),
                        static_cast<const int32_t*>(labels), (int)n, (int)h, (int)v, inv_temp,
-                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start);
+                       softcap, w.fin_max, w.fin_log2s, logprobs, is_start, (int)last_dst);
   AXON_CHECK_LAUNCH();
   return AXON_OK;
 }
+
+// A backward over a block of consecutive tokens of a longer stream (one call per block, one stream):
+// where the last row's label and gradients live (aligned_pos), whether the workspace already holds the
+// transposed weight (written by the step's first call), and how this block's share of the weight
+// gradient leaves: the blocks of a step add up in one fp32 array, the last one rounds the sum to bf16.
+enum { kDwStore = 0, kDwFirst = 1, kDwAdd = 2, kDwLast = 3 };
+struct BlockArgs {
+  int64_t last_dst = 0;
+  int wt_ready = 0;
+  int dw_mode = kDwStore;
+  float* dw_acc = nullptr;  // [vocab][hidden] fp32 (modes other than kDwStore)
+};
 
 int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
              const void* labels, int labels_i64, const float* lse, const float* entropy_b,
              int64_t n, int64_t h, int64_t v, float inv_temp, float softcap,
              const uint8_t* is_start, void* d_hidden, void* d_weight, int64_t chunk, void* workspace,
-             int64_t ws_bytes, const void* stash, int64_t stash_bytes, void* stream, PhaseTimer* timer) {
+             int64_t ws_bytes, const void* stash, int64_t stash_bytes, void* stream, PhaseTimer* timer,
+             const BlockArgs& blk = BlockArgs()) {
   int rc = check_head_shape(n, h, v);
   if (rc != AXON_OK) return rc;
   if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
-  if (!d_weight || !weight) return AXON_ERR_ARG;
+  if (!weight) return AXON_ERR_ARG;
+  if (blk.dw_mode < kDwStore || blk.dw_mode > kDwLast) return AXON_ERR_ARG;
+  if (blk.dw_mode != kDwStore && (!blk.dw_acc || (reinterpret_cast<uintptr_t>(blk.dw_acc) & 15) || n == 0))
+    return AXON_ERR_ARG;
+  const bool dw_bf16 = blk.dw_mode == kDwStore || blk.dw_mode == kDwLast;
+  if (dw_bf16 && !d_weight) return AXON_ERR_ARG;
   const hipStream_t st = (hipStream_t)stream;
   if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
   if (!dlogprobs || !hidden || !labels || !lse || !entropy_b || !d_hidden || !workspace)
     return AXON_ERR_ARG;
   if (!(inv_temp > 0.f) || !(softcap >= 0.f)) return AXON_ERR_ARG;
   if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
-       reinterpret_cast<uintptr_t>(d_hidden) | reinterpret_cast<uintptr_t>(d_weight)) & 15)
+       reinterpret_cast<uintptr_t>(d_hidden) | (dw_bf16 ? reinterpret_cast<uintptr_t>(d_weight) : 0)) & 15)
     return AXON_ERR_ARG;
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
   const BwdWs w = bwd_ws(n, h, v, chunk, base);
@@ -1162,8 +1203,10 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   // K-contiguous copies for the two output GEMMs
   {
     Span span(timer, 0);
-    rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.ld_v, (int)w.v_pad, st);
-    if (rc != AXON_OK) return rc;
+    if (!blk.wt_ready) {
+      rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.ld_v, (int)w.v_pad, st);
+      if (rc != AXON_OK) return rc;
+    }
     rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.ld_n, (int)w.n_pad, st);
     if (rc != AXON_OK) return rc;
   }
@@ -1187,6 +1230,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
       p.cap = softcap; p.inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
       p.is_start = is_start;
+      p.last_dst = (int)blk.last_dst;
       if (stash) {
         const StashSource src{sw.tiles, sw.pm, sw.tiles_n, (int)(v0 / kTile), sw.shifted};
         const unsigned blocks = (unsigned)(round_up(vc, kTile) / kTile) * (unsigned)sw.tiles_n * 8u;
@@ -1218,7 +1262,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       const bool last = (ci == w.chunks - 1);
       sp.out_f32 = (w.chunks > 1) ? w.dh_acc : nullptr;  sp.ld_f32 = h;
       sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
-      sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0);
+      sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0); sp.keep_f32 = 1;
       rc = launch_store(g, sp, st);
       if (rc != AXON_OK) return rc;
     }
@@ -1230,9 +1274,11 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       g.b = w.dlT;  g.ldb = w.ld_n;  g.n_rows = (int)vc;
       g.k = (int)n_red;
       StoreParams sp;
-      sp.out_f32 = nullptr; sp.ld_f32 = 0;
-      sp.out_bf16 = static_cast<__bf16*>(d_weight) + v0 * h;  sp.ld_bf16 = h;
-      sp.m_valid = (int)h; sp.n_valid = (int)vc; sp.accumulate = 0;
+      sp.out_f32 = blk.dw_mode == kDwStore ? nullptr : blk.dw_acc + v0 * h;  sp.ld_f32 = h;
+      sp.out_bf16 = dw_bf16 ? static_cast<__bf16*>(d_weight) + v0 * h : nullptr;  sp.ld_bf16 = h;
+      sp.m_valid = (int)h; sp.n_valid = (int)vc;
+      sp.accumulate = blk.dw_mode == kDwAdd || blk.dw_mode == kDwLast;
+      sp.keep_f32 = blk.dw_mode != kDwLast;
       rc = launch_store(g, sp, st);
       if (rc != AXON_OK) return rc;
     }
@@ -1333,7 +1379,7 @@ extern "C" int axon_lmhead_fwd(const void* hidden, const void* weight, const voi
                                float softcap, const uint8_t* seq_start, float* logprobs,
                                float* entropy, float* lse, float* entropy_b, void* workspace,
                                int64_t ws_bytes, void* stash, int64_t stash_bytes, void* stream) {
-  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start,
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, 0,
                   logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stash, stash_bytes, stream,
                   nullptr);
 }
@@ -1364,7 +1410,7 @@ extern "C" int axon_lmhead_fwd_timed(const void* hidden, const void* weight, con
   PhaseTimer* t = static_cast<PhaseTimer*>(timer);
   if (t->st != (hipStream_t)stream) return AXON_ERR_ARG;
   t->base = 0;
-  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, logprobs,
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, 0, logprobs,
                   entropy, lse, entropy_b, workspace, ws_bytes, stash, stash_bytes, stream, t);
 }
 
@@ -1416,6 +1462,87 @@ extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int6
   g.k = (int)k;
   StoreParams sp;
   sp.out_f32 = out; sp.ld_f32 = ldo; sp.out_bf16 = nullptr; sp.ld_bf16 = 0;
-  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0;
+  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0; sp.keep_f32 = 1;
   return launch_store(g, sp, (hipStream_t)stream);
+}
+
+// ----------------------------------------------------------------------------
+// One step as token blocks: forward (with stash), loss and backward of one block of consecutive
+// tokens before the next block's forward, so that what is kept from a forward to its backward is
+// one block's stash whatever the number of tokens.  One call per block and phase, all on one stream.
+// ----------------------------------------------------------------------------
+namespace {
+PhaseTimer* block_timer(void* timer, void* stream, int base, int* rc) {
+  *rc = AXON_OK;
+  if (!timer) return nullptr;
+  PhaseTimer* t = static_cast<PhaseTimer*>(timer);
+  if (t->st != (hipStream_t)stream) { *rc = AXON_ERR_ARG; return nullptr; }
+  t->base = base;
+  return t;
+}
+bool last_dst_ok(int64_t last_dst, int64_t n) { return last_dst <= n && last_dst > -(int64_t(1) << 30); }
+}  // namespace
+
+extern "C" int axon_lmhead_block_begin(const void* weight, int64_t h, int64_t v, int64_t chunk,
+                                       void* workspace, int64_t ws_bytes, void* stream, void* timer) {
+  int rc = check_head_shape(0, h, v);
+  if (rc != AXON_OK) return rc;
+  if (chunk < 0 || chunk % kTile != 0) return AXON_ERR_ARG;
+  if (!weight || !workspace || (reinterpret_cast<uintptr_t>(weight) & 15)) return AXON_ERR_ARG;
+  PhaseTimer* t = block_timer(timer, stream, 4, &rc);
+  if (rc != AXON_OK) return rc;
+  char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
+  const BwdWs w = bwd_ws(0, h, v, chunk, base);
+  if ((base - static_cast<char*>(workspace)) + round_up(h * w.ld_v * 2, kAlign) > ws_bytes)
+    return AXON_ERR_WORKSPACE;
+  Span span(t, 0);
+  return launch_transpose(weight, h, (int)v, (int)h, w.wT, w.ld_v, (int)w.v_pad, (hipStream_t)stream);
+}
+
+extern "C" int axon_lmhead_block_fwd(const void* hidden, const void* weight, const void* labels,
+                                     int labels_i64, int64_t n, int64_t h, int64_t v, float inv_temp,
+                                     float softcap, const uint8_t* seq_start, int64_t last_dst,
+                                     float* logprobs, float* entropy, float* lse, float* entropy_b,
+                                     void* workspace, int64_t ws_bytes, void* stash,
+                                     int64_t stash_bytes, void* stream, void* timer) {
+  if (!last_dst_ok(last_dst, n)) return AXON_ERR_ARG;
+  int rc;
+  PhaseTimer* t = block_timer(timer, stream, 0, &rc);
+  if (rc != AXON_OK) return rc;
+  return fwd_impl(hidden, weight, labels, labels_i64, n, h, v, inv_temp, softcap, seq_start, last_dst,
+                  logprobs, entropy, lse, entropy_b, workspace, ws_bytes, stash, stash_bytes, stream, t);
+}
+
+extern "C" int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentropy, const void* hidden,
+                                     const void* weight, const void* labels, int labels_i64,
+                                     const float* lse, const float* entropy_b, int64_t n, int64_t h,
+                                     int64_t v, float inv_temp, float softcap,
+                                     const uint8_t* seq_start, int64_t last_dst, void* d_hidden,
+                                     void* d_weight, float* dw_acc, int dw_mode, int wt_ready,
+                                     int64_t chunk, void* workspace, int64_t ws_bytes,
+                                     const void* stash, int64_t stash_bytes, void* stream,
+                                     void* timer) {
+  if (!last_dst_ok(last_dst, n) || n <= 0) return AXON_ERR_ARG;
+  int rc;
+  PhaseTimer* t = block_timer(timer, stream, 4, &rc);
+  if (rc != AXON_OK) return rc;
+  BlockArgs blk;
+  blk.last_dst = last_dst;
+  blk.wt_ready = wt_ready != 0;
+  blk.dw_mode = dw_mode;
+  blk.dw_acc = dw_acc;
+  return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
+                  inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes, stash,
+                  stash_bytes, stream, t, blk);
+}
+
+extern "C" int axon_scale_bf16_unless_one(void* x, int64_t n, const float* scale, void* stream) {
+  if (n < 0 || n % 8 != 0) return AXON_ERR_SHAPE;
+  if (n == 0) return AXON_OK;
+  if (!x || !scale || (reinterpret_cast<uintptr_t>(x) & 15)) return AXON_ERR_ARG;
+  const int64_t n_vec = n / 8, blocks = (n_vec + 255) / 256;
+  hipLaunchKernelGGL(scale_bf16_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(256), 0,
+                     (hipStream_t)stream, static_cast<uint4*>(x), n_vec, scale);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
 }

@@ -68,9 +68,12 @@ def _aggregation(b, config, default_token_reduce: str) -> dict:
                 num_program_steps=nps, valid_count=valid)
 
 
-def _run(kind: int, data, config, default_token_reduce: str):
+def policy_loss_spec(kind: int, data, config, default_token_reduce: str, with_log_probs: bool = True):
+    """The operands and hyper-parameters of one clipped-policy-loss call, validated as the reference does:
+    ``(log_probs, rows, tensors, hp)`` for ``_ops.policy_loss(kind, log_probs, **tensors, rows, **hp)``.
+    Without ``with_log_probs`` (a caller that produces them block by block) the first two are None."""
     b = data.batch
-    log_probs = b["log_probs"]
+    log_probs = b["log_probs"] if with_log_probs else None
     clip = config.get("clip_ratio", 0.2)
     lo = config.get("clip_ratio_low", None)
     hi = config.get("clip_ratio_high", None)
@@ -84,8 +87,10 @@ def _run(kind: int, data, config, default_token_reduce: str):
         clip_c = 1.0 if config.get("token_level_mask", False) else 0.0
     agg = _aggregation(b, config, default_token_reduce)
 
-    _lib.require_device(log_probs, "policy loss")
-    rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
+    rows = None
+    if with_log_probs:
+        _lib.require_device(log_probs, "policy loss")
+        rows = _ops.rows_of(log_probs, data.meta_info.get("cu_seqlens", None) if data.meta_info else None)
     tensors = {
         "old_log_probs": b["old_log_probs"],
         "advantages": b["advantages"],
@@ -95,15 +100,30 @@ def _run(kind: int, data, config, default_token_reduce: str):
     }
     # bounds evaluated in double and rounded once, as torch.clamp does with Python scalars
     hp = dict(ratio_lo=1 - lo, ratio_hi=1 + hi, clip_c=clip_c, **agg)
-    loss, acc = _ClippedPolicyLoss.apply(log_probs, kind, tensors, rows, hp)
-    sums = acc.tolist()  # the only host sync of the loss
+    return log_probs, rows, tensors, hp
+
+
+def policy_loss_metrics(kind: int, sums) -> dict[str, Any]:
+    """The metrics of a clipped policy loss from the kernel's sums (``acc[1:5]`` as a list)."""
     denom = max(sums[4], 1.0)
     metrics: dict[str, Any] = {"ppo_kl": sums[2] / denom}
     if kind != _KIND_REINFORCE:
         metrics["pg_clipfrac"] = sums[1] / denom
     if kind in (_KIND_PPO, _KIND_GSPO):
         metrics["pg_clipfrac_lower"] = (sums[3] / denom) if kind == _KIND_PPO else 0.0
-    return loss, metrics
+    return metrics
+
+
+# registry name -> (kernel kind, default token_reduce) of the losses that run on ``_ops.policy_loss``
+POLICY_LOSS_KINDS = {"ppo": (_KIND_PPO, "sum"), "gspo": (_KIND_GSPO, "mean"), "reinforce": (_KIND_REINFORCE, "sum"),
+                     "gpg": (_KIND_REINFORCE, "sum"), "cispo": (_KIND_CISPO, "sum")}
+
+
+def _run(kind: int, data, config, default_token_reduce: str):
+    log_probs, rows, tensors, hp = policy_loss_spec(kind, data, config, default_token_reduce)
+    loss, acc = _ClippedPolicyLoss.apply(log_probs, kind, tensors, rows, hp)
+    sums = acc.tolist()  # the only host sync of the loss
+    return loss, policy_loss_metrics(kind, sums)
 
 
 @register_loss(LossFn.PPO)

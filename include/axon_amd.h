@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 17
+#define AXON_AMD_ABI_VERSION 18
 
 enum {
   AXON_OK = 0,
@@ -185,6 +185,54 @@ int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const v
                           const uint8_t* seq_start, void* d_hidden_bf16, void* d_weight_bf16,
                           int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
                           const void* stash, int64_t stash_bytes, void* stream, void* timer);
+
+/* One step as token blocks.  The reference's per-micro-batch step (CausalLM.forward_backward_fn,
+ * axon/models/fsdp_models.py:183-279) runs the head forward over all tokens, then the loss, then the
+ * head backward; its kernels hold [tokens, 9504]-column slices of logits on the way
+ * (efficient_entropy_forward / _backward, axon/utils/kernel/kernels.py:1523-1580).  These entry
+ * points run the same three stages block of consecutive tokens by block: forward of the block over the whole
+ * vocabulary with a stash (axon_lmhead_fwd above), the caller's loss kernels on the block's positions,
+ * backward of the block from the stash, then the next block.  What lives from a forward to its
+ * backward is ONE block's stash (2 bytes x block tokens x vocab), whatever the number of tokens, and
+ * the path executes 6 N H V flop for the 6 that count.  All calls of a step go to one stream.
+ *   Arrays: `hidden`, `labels`, `seq_start`, `logprobs`, `entropy`, `dlogprobs`, `dentropy`, `d_hidden`
+ *        point at the BLOCK's first position inside the step's whole arrays (hidden rows and d_hidden
+ *        rows of the block; the per-position arrays offset by the block's first position); `lse`,
+ *        `entropy_b` are per block (n_tokens entries).  `weight`, `d_weight`, `dw_acc` are whole.
+ *   last_dst (token-aligned layout only, seq_start != NULL): a block's last row predicts the position
+ *        after the block: pass n_tokens when the stream goes on (its label, outputs and gradients are
+ *        then read and written at index n_tokens of the block-offset arrays, i.e. the next block's
+ *        first position), and minus the block's first position when the block ends the stream (index 0
+ *        of the whole arrays, a sequence start).  0 is the whole-stream call, as axon_lmhead_fwd.
+ *   axon_lmhead_block_begin: once per step, before the first backward: the transposed weight into
+ *        `workspace` (the same workspace, of axon_lmhead_bwd_workspace_bytes(largest block, ...) bytes,
+ *        must then be handed to every axon_lmhead_block_bwd of the step, with wt_ready = 1).
+ *   axon_lmhead_block_bwd: d_hidden rows of the block (bf16, complete: a row sums over the vocabulary
+ *        only).  The weight gradient sums over all blocks: dw_mode 0 = this block is the whole step,
+ *        d_weight (bf16) is written; 1 = first block, dw_acc[vocab][hidden] (fp32) is written;
+ *        2 = a middle block, added to dw_acc; 3 = last block, dw_acc + this block's share is rounded
+ *        to bf16 into d_weight and dw_acc is left as it was.  stash may be NULL (the block's logits are then recomputed).
+ *   timer: NULL, or an axon_timer_create object on `stream` (phases as below).
+ * axon_scale_bf16_unless_one multiplies n bf16 values in place by the DEVICE scalar scale[0] and touches
+ * nothing when it is exactly 1 (the step's gradients are finished before autograd hands over the
+ * factor of the loss, which is 1 unless the caller scaled the loss); n % 8 == 0, x on a 16-byte boundary. */
+int axon_lmhead_block_begin(const void* weight_bf16, int64_t hidden, int64_t vocab, int64_t vocab_chunk,
+                            void* workspace, int64_t workspace_bytes, void* stream, void* timer);
+int axon_lmhead_block_fwd(const void* hidden_bf16, const void* weight_bf16, const void* labels,
+                          int labels_are_i64, int64_t n_tokens, int64_t hidden, int64_t vocab,
+                          float inv_temperature, float softcap, const uint8_t* seq_start,
+                          int64_t last_dst, float* logprobs, float* entropy, float* lse,
+                          float* entropy_b, void* workspace, int64_t workspace_bytes, void* stash,
+                          int64_t stash_bytes, void* stream, void* timer);
+int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentropy, const void* hidden_bf16,
+                          const void* weight_bf16, const void* labels, int labels_are_i64,
+                          const float* lse, const float* entropy_b, int64_t n_tokens, int64_t hidden,
+                          int64_t vocab, float inv_temperature, float softcap,
+                          const uint8_t* seq_start, int64_t last_dst, void* d_hidden_bf16,
+                          void* d_weight_bf16, float* dw_acc, int dw_mode, int wt_ready,
+                          int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
+                          const void* stash, int64_t stash_bytes, void* stream, void* timer);
+int axon_scale_bf16_unless_one(void* x_bf16, int64_t n, const float* scale, void* stream);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
  * (fp32 accumulate, fp32 output).  No reference counterpart: it exists so tests

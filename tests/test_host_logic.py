@@ -286,3 +286,15 @@ def test_row_owning_dispatch_rule():
         assert not _ops._own_rows(_ops.rows_of(torch.zeros(1, 3)))
     finally:
         _ops.OWNED_ROWS_MIN_MEAN_LEN = keep
+
+
+def test_fused_step_block_plans():
+    from axon_amd.models.fused_head_loss import sequence_blocks, token_blocks
+    assert token_blocks(32768, 8192) == [(0, 8192), (8192, 16384), (16384, 24576), (24576, 32768)]
+    assert token_blocks(1500, 512) == [(0, 512), (512, 1024), (1024, 1500)]
+    assert token_blocks(1500, 4096) == [(0, 1500)]
+    assert token_blocks(33000, 8192) == [(0, 6656), (6656, 13312), (13312, 19968), (19968, 26624), (26624, 33000)]
+    cu = [0, 400, 433, 933, 997, 1297, 1500]
+    assert sequence_blocks(cu, 512) == [(0, 2), (2, 3), (3, 5), (5, 6)]
+    assert sequence_blocks(cu, 499) is None
+    assert sequence_blocks([0, 0, 5, 5, 5], 8) == [(0, 4)]
