@@ -34,6 +34,7 @@ SIGNATURES: dict[str, tuple] = {
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_bwd_timed": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
                                      _f32, _f32, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_block_dw_acc_bytes": (_i64, [_i64, _i64]),
     "axon_lmhead_block_begin": (_i32, [_ptr, _i64, _i64, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_block_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr, _i64,
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),

@@ -841,11 +841,11 @@ class HeadBlocks:
         self.d_hidden = torch.empty_like(hidden)
         self.d_weight = torch.empty_like(weight)
         self.one_block = len(self.ranges) == 1
-        self.dw_acc = None if self.one_block else torch.empty(self.v, self.h, device=dev, dtype=torch.float32)
+        self.dw_acc_bytes = 0 if self.one_block else int(self.lib.axon_lmhead_block_dw_acc_bytes(self.h, self.v))
+        self.dw_acc = torch.empty(self.dw_acc_bytes // 4, device=dev, dtype=torch.float32) if self.dw_acc_bytes else None
         self.wt_ready = False
         self.block_stash_bytes = 0
-        self.workspace_bytes = (self.fwd_ws_bytes + self.bwd_ws_bytes + self.stash_bytes +
-                                (0 if self.one_block else self.v * self.h * 4))
+        self.workspace_bytes = self.fwd_ws_bytes + self.bwd_ws_bytes + self.stash_bytes + self.dw_acc_bytes
 
     @property
     def logprobs(self):

@@ -672,9 +672,15 @@ struct StoreParams {
   __bf16* out_bf16;   // [n][ld_bf16] (may be null)
   int64_t ld_f32, ld_bf16;
   int m_valid, n_valid;
-  int accumulate;     // add the previous contents of out_f32 first
-  int keep_f32;       // write the sum back to out_f32 (0: out_f32 is only read, the sum leaves as bf16)
+  int accumulate;     // add the previous contents of out_f32 (or tile_acc) first
+  int keep_f32;       // write the sum back to out_f32 / tile_acc (0: it is only read, the sum leaves as bf16)
+  // fp32 partial sums that only this kernel ever reads back (the weight gradient carried from one token
+  // block to the next): kept per tile in the order the accumulators lie in the registers, so that every
+  // wavefront load and store is one contiguous kilobyte.  float4 index =
+  // ((tile * 4 + wave) * 64 + i * 8 + j) * 64 + lane, tile = tm * tiles_n + tn.  Null: not used.
+  float4* tile_acc;
 };
+constexpr int64_t kTileAccVecs = 4 * kBlocks * kBlocks * 64;  // float4 per tile (256 KB)
 
 template <class Loop>
 __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g, StoreParams p,
@@ -686,6 +692,31 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_store_kernel(GemmOperands g
   AccTile acc;
   Loop::run(g, t, acc, smem);
   const LanePos lp;
+  if (p.tile_acc) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    f32x4* ta = reinterpret_cast<f32x4*>(p.tile_acc) +
+                ((int64_t)(tm * tiles_n + tn) * 4 + lp.wave) * (kBlocks * kBlocks * 64) + lp.lane;
+#pragma unroll
+    for (int i = 0; i < kBlocks; ++i) {
+      f32x4 old[kBlocks];
+      if (p.accumulate) {
+#pragma unroll
+        for (int j = 0; j < kBlocks; ++j) old[j] = __builtin_nontemporal_load(ta + (i * kBlocks + j) * 64);
+      }
+#pragma unroll
+      for (int j = 0; j < kBlocks; ++j) {
+        if (p.accumulate) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[i][j][r] += old[j][r];
+        }
+        if (p.keep_f32) {
+          const f32x4 v = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+          __builtin_nontemporal_store(v, ta + (i * kBlocks + j) * 64);
+        }
+      }
+    }
+    if (!p.out_bf16) return;
+  }
 #pragma unroll
   for (int j = 0; j < kBlocks; ++j) {
     const int nr = lp.n(j);
@@ -1163,7 +1194,7 @@ struct BlockArgs {
   int64_t last_dst = 0;
   int wt_ready = 0;
   int dw_mode = kDwStore;
-  float* dw_acc = nullptr;  // [vocab][hidden] fp32 (modes other than kDwStore)
+  float* dw_acc = nullptr;  // axon_lmhead_block_dw_acc_bytes of fp32 partial sums, tile order (modes other than kDwStore)
 };
 
 int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
@@ -1211,6 +1242,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
     if (rc != AXON_OK) return rc;
   }
   const int64_t n_red = round_up(n, 64);  // reduction length of B3
+  const int64_t tiles_h = round_up(h, kTile) / kTile;
 
   for (int ci = 0; ci < w.chunks; ++ci) {
     const int64_t v0 = (int64_t)ci * w.chunk;
@@ -1263,6 +1295,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       sp.out_f32 = (w.chunks > 1) ? w.dh_acc : nullptr;  sp.ld_f32 = h;
       sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
       sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0); sp.keep_f32 = 1;
+      sp.tile_acc = nullptr;
       rc = launch_store(g, sp, st);
       if (rc != AXON_OK) return rc;
     }
@@ -1274,7 +1307,10 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       g.b = w.dlT;  g.ldb = w.ld_n;  g.n_rows = (int)vc;
       g.k = (int)n_red;
       StoreParams sp;
-      sp.out_f32 = blk.dw_mode == kDwStore ? nullptr : blk.dw_acc + v0 * h;  sp.ld_f32 = h;
+      sp.out_f32 = nullptr;  sp.ld_f32 = 0;
+      sp.tile_acc = blk.dw_mode == kDwStore
+                        ? nullptr
+                        : reinterpret_cast<float4*>(blk.dw_acc) + (v0 / kTile) * tiles_h * kTileAccVecs;
       sp.out_bf16 = dw_bf16 ? static_cast<__bf16*>(d_weight) + v0 * h : nullptr;  sp.ld_bf16 = h;
       sp.m_valid = (int)h; sp.n_valid = (int)vc;
       sp.accumulate = blk.dw_mode == kDwAdd || blk.dw_mode == kDwLast;
@@ -1462,7 +1498,7 @@ extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int6
   g.k = (int)k;
   StoreParams sp;
   sp.out_f32 = out; sp.ld_f32 = ldo; sp.out_bf16 = nullptr; sp.ld_bf16 = 0;
-  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0; sp.keep_f32 = 1;
+  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0; sp.keep_f32 = 1; sp.tile_acc = nullptr;
   return launch_store(g, sp, (hipStream_t)stream);
 }
 
@@ -1482,6 +1518,11 @@ PhaseTimer* block_timer(void* timer, void* stream, int base, int* rc) {
 }
 bool last_dst_ok(int64_t last_dst, int64_t n) { return last_dst <= n && last_dst > -(int64_t(1) << 30); }
 }  // namespace
+
+extern "C" int64_t axon_lmhead_block_dw_acc_bytes(int64_t h, int64_t v) {
+  if (check_head_shape(0, h, v) != AXON_OK) return -1;
+  return (round_up(h, kTile) / kTile) * (round_up(v, kTile) / kTile) * kTileAccVecs * 16;
+}
 
 extern "C" int axon_lmhead_block_begin(const void* weight, int64_t h, int64_t v, int64_t chunk,
                                        void* workspace, int64_t ws_bytes, void* stream, void* timer) {

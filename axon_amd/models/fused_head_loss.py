@@ -35,9 +35,12 @@ _TILE = 256
 
 
 def token_blocks(n: int, block_tokens: int):
-    """Hidden-row ranges of equal size (a multiple of the GEMM tile) that cover ``n`` rows."""
-    n_blocks = max(1, -(-n // max(int(block_tokens), _TILE)))
-    nb = -(-(-(-n // n_blocks)) // _TILE) * _TILE
+    """Hidden-row ranges that cover ``n`` rows: blocks of ``block_tokens`` rows (rounded up to the GEMM tile), the
+    last one shorter; when that would leave a last block of under a quarter of a block, equal blocks instead."""
+    nb = max(-(-int(block_tokens) // _TILE), 1) * _TILE
+    n_blocks = max(1, -(-n // nb))
+    if n_blocks > 1 and n - (n_blocks - 1) * nb < nb // 4:
+        nb = -(-(-(-n // n_blocks)) // _TILE) * _TILE
     return [(a, min(a + nb, n)) for a in range(0, n, nb)]
 
 
@@ -68,6 +71,27 @@ def _global_count(mask, rows, batch_reduce, given):
                                    want_sum=False)
         return (cnt > 0).sum(dtype=torch.float64).reshape(1)
     raise AssertionError("valid_program_count required for batch_reduce='program-mean'")
+
+
+_PINNED: dict = {}
+
+
+def _start_readback(values):
+    """Start the device-to-host copy of a small float64 tensor into pinned memory on the current stream and
+    return ``(host tensor, event)``: the host waits for the event only, so launches enqueued after this call
+    keep the GPU busy while the host reads the values and goes on.  One pinned buffer per device, reused: read
+    the values before the next call."""
+    dev = values.device
+    n = int(values.numel())
+    buf = _PINNED.get(dev.index)
+    if buf is None or buf.numel() < n:
+        buf = torch.empty(max(n, 128), dtype=torch.float64, pin_memory=True)
+        _PINNED[dev.index] = buf
+    host = buf[:n]
+    host.copy_(values, non_blocking=True)
+    event = torch.cuda.Event()
+    event.record()
+    return host, event
 
 
 def _rows_slice(x, r0, r1):
@@ -106,11 +130,28 @@ class _BlockedHeadLoss(torch.autograd.Function):
         g_en = torch.zeros(n + 4, device=dev, dtype=torch.float32) if want_ent_grad else None
         accs, side_accs = [], []
 
+        out = {}
+
+        def finish():
+            """After the last block's loss, before its backward: the step's scalars are complete.  Their readback
+            starts here, so that the host can pick them up (and prepare whatever comes next) while the GPU still
+            works through the last block's backward."""
+            sums = torch.stack(accs).sum(0) if accs else torch.zeros(8, device=dev)
+            side_sums = torch.stack(side_accs).sum(0) if side_accs else torch.zeros(8, device=dev)
+            loss = sums[0].clone()
+            if side is not None:
+                if side["entropy_coef"] != 0:
+                    loss = loss - side_sums[0] * side["entropy_coef"]
+                if side["kl_type"] and side["kl_coef"] != 0:
+                    loss = loss + side_sums[1] * side["kl_coef"]
+            scalars = [sums[:5].double(), side_sums[:5].double()]
+            if spec.get("after_forward") is not None:  # more scalars from the whole-stream outputs (device tensors)
+                scalars += [t.double().reshape(-1) for t in spec["after_forward"](hb.logprobs, hb.entropy)]
+            spec["readback"] = _start_readback(torch.cat(scalars))
+            out.update(loss=loss, sums=sums, side_sums=side_sums)
+
         for k, (lo, hi) in enumerate(slots):
             hb.forward(k)
-            if hi <= lo:
-                hb.backward(k, g_lp, g_en)
-                continue
             cut = lambda t: None if t is None else t.reshape(-1)[lo:hi]  # noqa: E731
             if seq_mode:
                 r0, r1 = spec["row_blocks"][k]
@@ -138,16 +179,11 @@ class _BlockedHeadLoss(torch.autograd.Function):
                     torch.mul(agg_w.reshape(-1), s_acc[5] * (-side["entropy_coef"]), out=g_en[lo:hi])
                 if side["kl_type"] and side["kl_coef"] != 0:
                     g_lp[lo:hi].addcmul_(grad_kl.reshape(-1), s_acc[5], value=side["kl_coef"])
+            if k == len(slots) - 1:
+                finish()
             hb.backward(k, g_lp, g_en)
 
-        sums = torch.stack(accs).sum(0) if accs else torch.zeros(8, device=dev)
-        loss = sums[0].clone()
-        side_sums = torch.stack(side_accs).sum(0) if side_accs else torch.zeros(8, device=dev)
-        if side is not None:
-            if side["entropy_coef"] != 0:
-                loss = loss - side_sums[0] * side["entropy_coef"]
-            if side["kl_type"] and side["kl_coef"] != 0:
-                loss = loss + side_sums[1] * side["kl_coef"]
+        loss, sums, side_sums = out["loss"], out["sums"], out["side_sums"]
         ctx.grads = (hb.d_hidden, hb.d_weight)
         ctx.head_workspace_bytes = hb.workspace_bytes
         spec["stash_bytes"], spec["workspace_bytes"], spec["n_blocks"] = hb.stash_bytes, hb.workspace_bytes, len(ranges)
@@ -245,8 +281,8 @@ def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
     from axon_amd.models.fsdp_models import loss_from_outputs
     from axon_amd.trainer.algos.loss.registry import _SAMPLER_SWITCHES
     from axon_amd.utils.fsdp.forward_utils import packed_logprobs
-    from axon_amd.utils.rl.sampler import (compute_sampler_corr_metrics_from_logprobs,
-                                           compute_sampler_correction_and_add_to_batch)
+    from axon_amd.utils.rl.sampler import (compute_sampler_correction_and_add_to_batch, sampler_gap_metrics,
+                                           sampler_gap_sums)
 
     loss_fn = meta_info["loss_fn"]
     loss_fn_args = meta_info["loss_fn_args"] or {}
@@ -279,17 +315,19 @@ def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
         data.meta_info["head_backward"] = "recompute"
         return loss_from_outputs(data, log_prob, entropy, meta_info)
 
-    loss, log_prob, entropy, sums, side_sums = blocked_head_loss(hidden2, weight, spec)
+    sampler_log_prob = b.get("sampler_log_probs", None)
+    if sampler_log_prob is not None:  # the gap between the current policy and the sampler (fsdp_models.py:232-241)
+        spec["after_forward"] = lambda lp, _ent: [sampler_gap_sums(lp, sampler_log_prob, side_mask, cu_seqlens)]
+    loss, log_prob, entropy, _sums, _side_sums = blocked_head_loss(hidden2, weight, spec)
     b["log_probs"], b["entropys"] = log_prob, entropy
     data.meta_info.update(head_backward="blocked-stash", stash_bytes=spec["stash_bytes"],
                           head_workspace_bytes=spec["workspace_bytes"], n_blocks=spec["n_blocks"])
-    metrics = {}
-    sampler_log_prob = b.get("sampler_log_probs", None)
+    host, event = spec["readback"]  # the one readback of the step's scalars, started before the last block's backward
+    event.synchronize()
+    vals = host.tolist()
+    metrics = {**policy_loss_metrics(spec["kind"], vals[:5]), **corr_metrics}
     if sampler_log_prob is not None:
-        metrics.update(compute_sampler_corr_metrics_from_logprobs(log_prob=log_prob, sampler_log_prob=sampler_log_prob,
-                                                                  response_mask=side_mask, cu_seqlens=cu_seqlens))
-    vals = torch.cat([sums[:5], side_sums[:5]]).tolist()  # the one readback of the step's scalars
-    metrics = {**policy_loss_metrics(spec["kind"], vals[:5]), **corr_metrics, **metrics}
+        metrics.update(sampler_gap_metrics(vals[10:], int(cu_seqlens.numel()) - 1))
     metrics["pg_loss"] = vals[0] * n_micro_batches
     metrics["entropy"] = vals[5] * n_micro_batches
     metrics["entropy_token_mean"] = vals[7] / max(vals[9], 1.0)

@@ -344,11 +344,8 @@ def compute_sampler_rejection_mask(
 
 
 def _diag_plain(old_log_prob, sampler_log_prob, response_mask, cu_seqlens):
-    rows = _ops.rows_of(old_log_prob, cu_seqlens)
-    d = _ops.sampler_diag(old_log_prob, sampler_log_prob, response_mask, rows, is_mode=0, is_lo=1.0, is_hi=1.0,
-                          rs_mode=0, rs_lo=1.0, rs_hi=1.0, rs_lr_lo=-math.inf, rs_lr_hi=math.inf, log_is_lo=0.0,
-                          log_is_hi=0.0, log_rs_lo=0.0, log_rs_hi=0.0)
-    return d.tolist(), rows.n_rows
+    d = sampler_gap_sums(old_log_prob, sampler_log_prob, response_mask, cu_seqlens)
+    return d.tolist(), _ops.rows_of(old_log_prob, cu_seqlens).n_rows
 
 
 def compute_offpolicy_metrics(old_log_prob, sampler_log_prob, response_mask,
@@ -368,6 +365,22 @@ def compute_offpolicy_metrics(old_log_prob, sampler_log_prob, response_mask,
     if d[0] == 0:
         return {}
     return _offpolicy_from_diag(d, n_rows)
+
+
+def sampler_gap_sums(log_prob, sampler_log_prob, response_mask, cu_seqlens=None):
+    """The device half of ``compute_sampler_corr_metrics_from_logprobs``: the raw sums as a float64 device tensor
+    (no readback), for a caller that collects them with other scalars; ``sampler_gap_metrics`` is the host half."""
+    rows = _ops.rows_of(log_prob, cu_seqlens)
+    return _ops.sampler_diag(log_prob.detach(), sampler_log_prob, response_mask, rows, is_mode=0, is_lo=1.0, is_hi=1.0,
+                             rs_mode=0, rs_lo=1.0, rs_hi=1.0, rs_lr_lo=-math.inf, rs_lr_hi=math.inf, log_is_lo=0.0,
+                             log_is_hi=0.0, log_rs_lo=0.0, log_rs_hi=0.0)
+
+
+def sampler_gap_metrics(sums: list, n_rows: int) -> dict[str, float]:
+    """``sampler_corr/``-prefixed off-policy metrics from ``sampler_gap_sums`` read back as a list."""
+    if sums[0] == 0:
+        return {}
+    return {f"sampler_corr/{k}": v for k, v in _offpolicy_from_diag(sums, n_rows).items()}
 
 
 def compute_sampler_corr_metrics_from_logprobs(log_prob, sampler_log_prob, response_mask,

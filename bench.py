@@ -1,10 +1,13 @@
 #!/usr/bin/env python3
 """Benchmark of the trainer-side per-token hot path on one MI355X.
 
-One step = fused LM-head log-prob/entropy forward -> packed shift -> GRPO advantage ->
+One step = GRPO advantage -> fused LM-head log-prob/entropy forward (label roll and shift inside) ->
 PPO (DAPO clip) loss forward+backward -> LM-head backward (dHidden, dWeight), on
 synthetic inputs already resident in HBM.  Default workload: Qwen3-8B head shape,
-32768 packed tokens, hidden 4096, vocab 151936, bf16.
+32768 packed tokens, hidden 4096, vocab 151936, bf16.  The headline runs head forward, loss and
+head backward block of tokens by block in one autograd node (a stash of fixed size, no logit
+computed twice); the same step with the head as a plain autograd function whose backward
+recomputes the logits is timed beside it.
 
 Prints ONE JSON line: trained tokens/s, the MFMA roofline of the dominant kernel
 (HIP-event times over the timed region) and the CPU port of the reference torch path
@@ -42,12 +45,15 @@ def parse_args():
     ap.add_argument("--workload", default="qwen3-8b", choices=sorted(WORKLOADS))
     ap.add_argument("--tokens", type=int, default=0, help="override the token count (debugging)")
     ap.add_argument("--vocab-chunk", type=int, default=0)
-    ap.add_argument("--head-backward", choices=("recompute", "stash"), default="recompute",
-                    help="where the headline's backward takes its dlogits from: a recompute of the logits (nothing "
-                         "of size tokens x vocab is ever in memory, as the reference's kernels and the library's "
-                         "default), or the forward's stash (2 bytes per logit kept from forward to backward, opt-in)")
-    ap.add_argument("--no-stash-variant", dest="stash_variant", action="store_false",
-                    help="skip the short second measurement of the same step with the opt-in stash")
+    ap.add_argument("--head-backward", choices=("blocked-stash", "recompute", "stash"), default="blocked-stash",
+                    help="where the headline's backward takes its dlogits from: the stash of one block of tokens "
+                         "(forward, loss and backward block by block in one autograd node; 2 bytes x block x vocab "
+                         "held whatever the token count), a recompute of the logits (head, loss and backward as "
+                         "separate autograd functions, nothing of size tokens x vocab in memory), or a stash of "
+                         "ALL tokens kept from the forward to the backward (opt-in)")
+    ap.add_argument("--block-tokens", type=int, default=8192, help="tokens per block of the blocked-stash step")
+    ap.add_argument("--no-variants", dest="variants", action="store_false",
+                    help="skip the short measurements of the same step on the other head-backward paths")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
     ap.add_argument("--prompt-fraction", type=float, default=1 / 3,
                     help="after the headline, time the step again with this leading share of every sequence "
@@ -62,10 +68,10 @@ def parse_args():
                     help="run three plain bf16 GEMMs of the dominant kernel's shape through torch.matmul or through "
                          "the fused kernels' main loop (axon_gemm_nt_bf16), then exit: the command the rocprofv3 --pmc "
                          "passes that compare the two are taken on")
-    ap.add_argument("--traffic-probe", action="store_true",
-                    help="run a 1 GiB calibration copy, then one head forward and backward on each of the two "
-                         "backward paths (recompute, stash), then exit: the "
-                         "command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes are taken on")
+    ap.add_argument("--traffic-probe", choices=("blocked-stash", "recompute", "stash"),
+                    help="run a 1 GiB calibration copy, then one head forward and backward on the named "
+                         "head-backward path, then exit: the command the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "passes are taken on")
     return ap.parse_args()
 
 
@@ -294,15 +300,16 @@ def gemm_calibration(dev, n, h, chunk=32768):
     return res
 
 
-def head_step_summary(workload, dev, steps=3, warmup=1):
-    """One of the other head shapes through the same step as the headline (head forward with roll and shift
-    inside, GRPO advantage, PPO loss, backward to dHidden and dWeight): tokens/s and TFLOP/s per kernel class."""
+def head_step_summary(workload, dev, steps=3, warmup=1, block_tokens=8192):
+    """One of the other head shapes through the same step as the headline (GRPO advantage, then head forward with
+    roll and shift inside, PPO loss and backward to dHidden and dWeight block of tokens by block): tokens/s and
+    TFLOP/s per kernel class."""
     import torch
 
     from axon_amd import _ops, workloads as W
+    from axon_amd.models.fused_head_loss import fused_head_loss
     from axon_amd.protocol import DataProto
     from axon_amd.trainer.algos.advantages import compute_advantage
-    from axon_amd.trainer.algos.loss import compute_loss_fn
     from axon_amd.utils.fsdp.forward_utils import packed_logprobs
 
     n, h, v, group, seed = WORKLOADS[workload]
@@ -314,17 +321,19 @@ def head_step_summary(workload, dev, steps=3, warmup=1):
         old = packed_logprobs(hd, wd, ld, cu)[0] - 0.05 * torch.randn(n, device=dev)
     loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
 
+    meta = {"loss_fn": "ppo", "loss_fn_args": loss_args, "temperature": 1.0, "dp_replicas": 1}
+    info = {}
+
     def step():
         hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
-        lp_tok, _ = packed_logprobs(hg, wg, ld, cu)
         a_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
                                    meta_info={"cu_seqlens": cu})
         a_in.non_tensor_batch["uid"] = uid
         adv = compute_advantage(a_in, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}).batch["advantages"]
-        data = DataProto.from_dict(tensors={"log_probs": lp_tok, "old_log_probs": old, "advantages": adv,
-                                            "response_mask": mask}, meta_info={"cu_seqlens": cu})
-        loss, _ = compute_loss_fn(data, "ppo", loss_args)
+        data = DataProto.from_dict(tensors={"old_log_probs": old, "advantages": adv, "response_mask": mask})
+        loss, _ = fused_head_loss(hg, wg, ld, cu, data, meta, block_tokens=block_tokens)
         loss.backward()
+        info.update(data.meta_info)
         return loss
 
     for _ in range(warmup):
@@ -348,8 +357,8 @@ def head_step_summary(workload, dev, steps=3, warmup=1):
             "ms_per_step": 1e3 * el / steps, "tokens_per_s": n * steps / el,
             "fwd_tflops": tf(2 * nhv, ms("fwd/logits_stats")),
             "dhidden_dweight_tflops": tf(4 * nhv, ms("bwd/dhidden", "bwd/dweight")),
-            "head_backward": "stash" if _ops._want_stash(n, h, v, torch.device(dev)) else "recompute",
-            "dlogit_ms_per_step": ms("bwd/dlogit"),
+            "head_backward": info.get("head_backward"), "n_blocks": info.get("n_blocks"),
+            "stash_bytes": info.get("stash_bytes"), "dlogit_ms_per_step": ms("bwd/dlogit"),
             "path_algorithmic_tflops": 6 * nhv / (1e-3 * 1e3 * el / steps) / 1e12}
 
 
@@ -588,11 +597,12 @@ def kernel_source_digest():
     return h.hexdigest()[:16]
 
 
-def traffic_from_profile(workload):
-    """HBM-side bytes of ONE launch of the dominant kernel, read from the committed summary of the two
-    rocprofv3 --pmc passes over `bench.py --traffic-probe` (profiles/lmhead_<workload>_hbm_traffic.md carries
-    the line `traffic_bytes_per_launch: <bytes> kernel_source_digest: <digest>`).  None when there is no such
-    file or when the kernels have changed since (the digest of their sources differs)."""
+def traffic_from_profile(workload, head_path):
+    """HBM-side bytes of ONE launch of the dominant kernel on the named head-backward path, read from the
+    committed summary of the two rocprofv3 --pmc passes over `bench.py --traffic-probe <path>`
+    (profiles/lmhead_<workload>_hbm_traffic.md carries one line
+    `traffic_bytes_per_launch[<path>]: <bytes> kernel_source_digest: <digest>` per path).  None when there is no
+    such line or when the kernels have changed since (the digest of their sources differs)."""
     import re
 
     path = os.path.join(ROOT, "profiles", f"lmhead_{workload}_hbm_traffic.md")
@@ -600,13 +610,14 @@ def traffic_from_profile(workload):
         text = open(path).read()
     except OSError:
         return None
-    m = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)\s+kernel_source_digest:\s*([0-9a-f]+)", text)
+    m = re.search(r"traffic_bytes_per_launch\[" + re.escape(head_path) +
+                  r"\]:\s*([0-9.eE+]+)\s+kernel_source_digest:\s*([0-9a-f]+)", text)
     if not m or m.group(2) != kernel_source_digest():
         return None
     return float(m.group(1))
 
 
-def traffic_probe(workload):
+def traffic_probe(workload, head_path):
     import torch
 
     from axon_amd import _ops, workloads as W
@@ -617,12 +628,19 @@ def traffic_probe(workload):
     src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()  # 1 GiB
     dst = torch.empty_like(src)
     dst.copy_(src)  # calibration kernel: reads 1 GiB, writes 1 GiB
-    g = torch.randn(n, device="cuda")
-    _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)  # the default path: the backward recomputes the logits
-    _ops.lmhead_backward(g, torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0)
-    _ops.LMHEAD_STASH = True  # the opt-in path: the forward's stash, decoded by the backward
-    _, _, lse, eb, stash = _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)
-    _ops.lmhead_backward(g, torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0, stash=stash)
+    g = torch.randn(n + 4, device="cuda")
+    if head_path == "blocked-stash":  # four blocks of 8192 tokens: forward with stash, backward from it
+        hb = _ops.HeadBlocks(hd, wd, ld, 1.0, [(a, min(a + 8192, n)) for a in range(0, n, 8192)])
+        for k in range(len(hb.ranges)):
+            hb.forward(k)
+            hb.backward(k, g, None)
+    elif head_path == "recompute":  # the library's default: the backward recomputes the logits
+        _, _, lse, eb = _ops.lmhead_forward(hd, wd, ld, 1.0)
+        _ops.lmhead_backward(g[:n], torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0)
+    else:  # the opt-in stash of all tokens
+        _ops.LMHEAD_STASH = True
+        _, _, lse, eb, stash = _ops.lmhead_forward(hd, wd, ld, 1.0, stash=True)
+        _ops.lmhead_backward(g[:n], torch.zeros(n, device="cuda"), hd, wd, ld, lse, eb, 1.0, stash=stash)
     torch.cuda.synchronize()
 
 
@@ -645,7 +663,7 @@ def gemm_probe(which, workload):
 def main():
     args = parse_args()
     if args.traffic_probe:
-        traffic_probe(args.workload)
+        traffic_probe(args.workload, args.traffic_probe)
         return
     if args.gemm_probe:
         gemm_probe(args.gemm_probe, args.workload)
@@ -688,74 +706,105 @@ def main():
     lp_subset = lp0.cpu()[idx]
 
     loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
+    adv_cfg = {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}
+    meta = {"loss_fn": "ppo", "loss_fn_args": loss_args, "temperature": 1.0, "dp_replicas": 1}
+    from axon_amd.models.fused_head_loss import fused_head_loss
 
-    def step(mask=mask, head_mask=None):
-        hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
-        lp_tok, _ent = packed_logprobs(hg, wg, ld, cu, response_mask=head_mask)
+    def advantages(mask):
         adv_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
                                      meta_info={"cu_seqlens": cu})
         adv_in.non_tensor_batch["uid"] = uid
-        adv = compute_advantage(adv_in, {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}).batch["advantages"]
-        data = DataProto.from_dict(tensors={"log_probs": lp_tok, "old_log_probs": old, "advantages": adv,
+        return compute_advantage(adv_in, adv_cfg).batch["advantages"]
+
+    def step_unfused(mask=mask, head_mask=None):
+        """Head, loss and head backward as separate autograd functions (the reference's structure)."""
+        hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
+        lp_tok, _ent = packed_logprobs(hg, wg, ld, cu, response_mask=head_mask)
+        data = DataProto.from_dict(tensors={"log_probs": lp_tok, "old_log_probs": old, "advantages": advantages(mask),
                                             "response_mask": mask}, meta_info={"cu_seqlens": cu})
         loss, _ = compute_loss_fn(data, "ppo", loss_args)
         loss.backward()
         return loss, hg.grad, wg.grad
 
-    _ops.DEFAULT_VOCAB_CHUNK = args.vocab_chunk
-    _ops.LMHEAD_STASH = args.head_backward == "stash"
-    stash_bytes = _ops._want_stash(n, h, v, torch.device(dev))  # what every timed forward will allocate
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    block_info = {}
 
-    timer = _ops.Timer()
-    _ops.set_timing(timer)  # HIP events around every LM-head launch, on the launch stream, no synchronisation
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        loss, dh, dw = step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    _ops.set_timing(None)
-    timing = timer.collect()  # events of the timed region, read after it has ended
-    timer.close()
-    assert torch.isfinite(loss).item() and torch.isfinite(dh.float()).all().item()
+    def step_blocked(mask=mask):
+        """Head forward, loss and head backward block of tokens by block, one autograd node."""
+        hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
+        data = DataProto.from_dict(tensors={"old_log_probs": old, "advantages": advantages(mask), "response_mask": mask})
+        loss, _ = fused_head_loss(hg, wg, ld, cu, data, meta, block_tokens=args.block_tokens,
+                                  vocab_chunk=args.vocab_chunk)
+        loss.backward()
+        block_info.update(data.meta_info)
+        return loss, hg.grad, wg.grad
 
-    ms_per_step = 1e3 * elapsed / args.steps
-    tokens_per_s = n * args.steps / elapsed
-
-    # Not the headline: the same step with the opt-in stash (the forward keeps 2 bytes per logit, the backward
-    # decodes the dlogits from them instead of recomputing the logits)
-    stash_variant = None
-    if args.stash_variant and not stash_bytes and _ops.lmhead_stash_bytes(n, h, v):
-        _ops.LMHEAD_STASH = True
-        step()
+    def timed_steps(step_fn, steps, warmup):
+        """`warmup` untimed steps, then exactly `steps` steps between two synchronisations, with HIP events
+        around every LM-head launch (recorded on the launch stream without synchronising)."""
+        for _ in range(warmup):
+            step_fn()
         torch.cuda.synchronize()
         timer = _ops.Timer()
         _ops.set_timing(timer)
         t0 = time.perf_counter()
-        for _ in range(3):
-            loss_s, dh_s, dw_s = step()
+        for _ in range(steps):
+            res = step_fn()
         torch.cuda.synchronize()
         el = time.perf_counter() - t0
         _ops.set_timing(None)
-        timing_s = timer.collect()
+        timing = timer.collect()  # events of the timed region, read after it has ended
         timer.close()
-        _ops.LMHEAD_STASH = False
-        rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()  # noqa: E731
-        stash_variant = {
-            "what": "same step, forward keeps 2 bytes per logit (fp16 softmax numerators) for the backward: "
-                    "6 N H V flop executed instead of 8, tokens x vocab x 2 bytes held from forward to backward",
-            "stash_bytes": _ops.lmhead_stash_bytes(n, h, v), "steps": 3,
-            "ms_per_step": 1e3 * el / 3, "tokens_per_s": 3 * n / el,
-            "path_algorithmic_tflops": 6 * float(n) * h * v / (el / 3) / 1e12,
-            "path_frac_of_peak": 6 * float(n) * h * v / (el / 3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-            "loss": loss_s.item(), "headline_loss": loss.item(),
-            "dhidden_rel_l2_vs_headline": rel(dh_s, dh), "dweight_rel_l2_vs_headline": rel(dw_s, dw),
-            "kernels": kernel_table(timing_s, 3, n, h, v, _ops.lmhead_stash_bytes(n, h, v)),
-        }
-        del loss_s, dh_s, dw_s
-        torch.cuda.empty_cache()
+        return el, timing, res
+
+    def run_path(path, steps, warmup):
+        _ops.LMHEAD_STASH = path == "stash"
+        try:
+            return timed_steps(step_blocked if path == "blocked-stash" else step_unfused, steps, warmup)
+        finally:
+            _ops.LMHEAD_STASH = False
+
+    _ops.DEFAULT_VOCAB_CHUNK = args.vocab_chunk
+    head_path = args.head_backward
+    elapsed, timing, (loss, dh, dw) = run_path(head_path, args.steps, args.warmup)
+    assert torch.isfinite(loss).item() and torch.isfinite(dh.float()).all().item()
+    if head_path == "blocked-stash":
+        assert block_info.get("head_backward") == "blocked-stash", block_info
+        stash_bytes = int(block_info["stash_bytes"])
+    else:
+        stash_bytes = _ops.lmhead_stash_bytes(n, h, v) if head_path == "stash" else 0
+
+    ms_per_step = 1e3 * elapsed / args.steps
+    tokens_per_s = n * args.steps / elapsed
+    nhv = float(n) * h * v
+
+    # Not the headline: the same step on the other head-backward paths (three steps each)
+    variants = {}
+    rel = lambda a, b: ((a.float() - b.float()).norm() / b.float().norm()).item()  # noqa: E731
+    what = {
+        "blocked-stash": "head forward, loss and head backward block of tokens by block in one autograd node: one "
+                         "block's stash (2 bytes per logit) held, 6 N H V flop executed",
+        "recompute": "head as an autograd function whose backward recomputes the logits (the library's default and the "
+                     "reference's structure): nothing of size tokens x vocab held, 8 N H V flop executed for 6",
+        "stash": "head as an autograd function whose forward keeps 2 bytes per logit for ALL tokens (opt-in): "
+                 "tokens x vocab x 2 bytes held from forward to backward, 6 N H V flop executed",
+    }
+    if args.variants and not args.tokens:
+        for path in ("blocked-stash", "recompute", "stash"):
+            if path == head_path or (path == "stash" and not _ops.lmhead_stash_bytes(n, h, v)):
+                continue
+            el, timing_v, (loss_v, dh_v, dw_v) = run_path(path, 3, 1)
+            sb = (int(block_info["stash_bytes"]) if path == "blocked-stash" else
+                  _ops.lmhead_stash_bytes(n, h, v) if path == "stash" else 0)
+            variants[path] = {
+                "what": what[path], "stash_bytes": sb, "steps": 3, "ms_per_step": 1e3 * el / 3,
+                "tokens_per_s": 3 * n / el, "path_algorithmic_tflops": 6 * nhv / (el / 3) / 1e12,
+                "path_frac_of_peak": 6 * nhv / (el / 3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                "loss": loss_v.item(), "headline_loss": loss.item(),
+                "dhidden_rel_l2_vs_headline": rel(dh_v, dh), "dweight_rel_l2_vs_headline": rel(dw_v, dw),
+                "kernels": kernel_table(timing_v, 3, n, h, v, sb),
+            }
+            del loss_v, dh_v, dw_v
+            torch.cuda.empty_cache()
 
     # Not the headline: the same step when the first third of every sequence is prompt (response_mask 0), as in
     # the trainer's batches.  Those positions send exact zeros back into the head, whose backward leaves their
@@ -767,15 +816,16 @@ def main():
         row = torch.searchsorted(cu.long(), pos, right=True) - 1
         start, length = cu.long()[row], (cu.long()[1:] - cu.long()[:-1])[row]
         mask_p = mask * (pos - start >= (length.float() * args.prompt_fraction).long()).to(mask.dtype)
-        prompt_variant = {"prompt_fraction_of_tokens": 1.0 - mask_p.sum().item() / n, "steps": 3}
+        prompt_variant = {"prompt_fraction_of_tokens": 1.0 - mask_p.sum().item() / n, "steps": 3,
+                          "head_backward": "recompute"}
         for name, head_mask in (("backward", None), ("forward_and_backward", mask_p)):
             # "backward": the opt-in search for rows without a gradient (one readback per backward)
             _ops.SKIP_ZERO_GRAD_ROWS = head_mask is None
-            step(mask_p, head_mask)
+            step_unfused(mask_p, head_mask)
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for _ in range(3):
-                loss_p, dh_p, _ = step(mask_p, head_mask)
+                loss_p, dh_p, _ = step_unfused(mask_p, head_mask)
             torch.cuda.synchronize()
             el = time.perf_counter() - t0
             assert torch.isfinite(loss_p).item() and torch.isfinite(dh_p.float()).all().item()
@@ -783,28 +833,36 @@ def main():
         _ops.SKIP_ZERO_GRAD_ROWS = False
         del loss_p, dh_p
 
-    nhv = float(n) * h * v
-
     # kernel classes: (label, timing keys, algorithmic flops per step, executed flops per step)
-    executed = 6 if stash_bytes else 8
+    executed = 8 if head_path == "recompute" else 6
     kernels = kernel_table(timing, args.steps, n, h, v, stash_bytes)
     dom = max(kernels, key=lambda k: k["ms_per_step"])
     roofline = {
         "bound": "mfma", "kernel": dom["kernel"], "achieved": dom["algorithmic_tflops"] or dom["executed_tflops"],
         "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
         "frac": (dom["algorithmic_tflops"] or dom["executed_tflops"]) / MFMA_BF16_PEAK_TFLOPS,
-        "avg_launch_ms": dom["avg_launch_ms"],
-        "traffic": traffic_from_profile(args.workload) if not args.tokens and not args.vocab_chunk and "gemm_store" in dom["kernel"] else None,
+        "avg_launch_ms": dom["avg_launch_ms"], "launches_per_step": dom["launches_per_step"],
+        "traffic": traffic_from_profile(args.workload, head_path) if not args.tokens and not args.vocab_chunk
+        and args.block_tokens == 8192 and "gemm_store" in dom["kernel"] else None,
         "kernels": kernels,
         "path_algorithmic_tflops": 6 * nhv / (ms_per_step * 1e-3) / 1e12,
         "path_frac_of_peak": 6 * nhv / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
-        # a backward that recomputes the logits executes 8 N H V for the 6 that count; one that decodes the
-        # forward's stash executes the 6
+        # a backward that recomputes the logits executes 8 N H V for the 6 that count; one that decodes a
+        # stash executes the 6
         "path_executed_flop_per_algorithmic": executed / 6,
         "path_executed_tflops": executed * nhv / (ms_per_step * 1e-3) / 1e12,
         "other_phases_ms_per_step": {k: t["ms"] / args.steps for k, t in timing.items()
                                      if k in ("fwd/merge", "fwd/label", "bwd/transpose")},
+        "gemm_dhidden_ms_per_step": timing.get("bwd/dhidden", {"ms": 0.0})["ms"] / args.steps,
+        "gemm_dweight_ms_per_step": timing.get("bwd/dweight", {"ms": 0.0})["ms"] / args.steps,
     }
+    head_ms = sum(t["ms"] for t in timing.values()) / args.steps
+    roofline["head_kernels_ms_per_step"] = head_ms  # the rest of the step: advantage, loss kernels, fills, gaps
+    roofline["outside_head_kernels_ms_per_step"] = ms_per_step - head_ms
+    for path, var in variants.items():  # scalars, so that a reader of the first level sees them
+        key = path.replace("-", "_")
+        roofline[f"{key}_variant_ms_per_step"] = var["ms_per_step"]
+        roofline[f"{key}_variant_path_frac"] = var["path_frac_of_peak"]
 
     out = {
         "metric": "trained tokens/sec for fused logprob+GRPO loss fwd+bwd, Qwen3-8B shape; % MFMA peak",
@@ -814,24 +872,24 @@ def main():
         "config": {"workload": f"{args.workload}: fused LM-head logprob + GRPO/PPO loss fwd+bwd", "tokens": n,
                    "hidden": h, "vocab": v, "sequences": len(rl["lengths"]), "group": group,
                    "vocab_chunk": args.vocab_chunk or "default",
-                   "head_backward": "stash" if stash_bytes else "recompute", "stash_bytes": stash_bytes},
+                   "head_backward": head_path, "stash_bytes": stash_bytes},
         "roofline": roofline,
     }
+    if head_path == "blocked-stash":
+        out["config"].update(block_tokens=args.block_tokens, n_blocks=int(block_info["n_blocks"]),
+                             head_workspace_bytes=int(block_info["head_workspace_bytes"]))
     if args.calibrate:
         cal = gemm_calibration(dev, n, h)
         roofline["calibration_tflops"] = cal
         best = max(cal["hipblaslt_matmul_tflops"], cal["axon_gemm_nt_tflops"])
         share = 6 / executed
-        roofline["ceiling"] = (
-            (f"the backward decodes the forward's stash: 6 N H V flop are executed for 6 algorithmic, plus a "
-             f"streaming pass of 6 bytes per logit; " if stash_bytes else
-             f"a backward that recomputes the logits executes 8 N H V flop for 6 algorithmic: the path cannot exceed "
-             f"0.75 x what the GEMMs sustain; ") +
-            f"with the plain GEMM of this run ({best:.0f} TFLOP/s on random operands, "
-            f"{best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak: the part runs at its power limit under matrix "
-            f"load) the path's ceiling is {share * best / MFMA_BF16_PEAK_TFLOPS:.2f} of the published peak")
-    if stash_variant:
-        out["stash_variant"] = stash_variant
+        roofline["calibration_hipblaslt_tflops"] = cal["hipblaslt_matmul_tflops"]
+        roofline["calibration_axon_gemm_tflops"] = cal["axon_gemm_nt_tflops"]
+        roofline["path_ceiling_frac"] = share * best / MFMA_BF16_PEAK_TFLOPS
+        roofline["ceiling"] = (f"{share * best / MFMA_BF16_PEAK_TFLOPS:.2f} of peak = {6}/{executed} executed x best "
+                               f"plain GEMM of this run ({best:.0f} TFLOP/s, power-limited)")
+    if variants:
+        out["variants"] = variants
     if prompt_variant:
         out["prompt_rows_variant"] = prompt_variant
     if args.other_workloads and not args.tokens:

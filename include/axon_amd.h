@@ -209,13 +209,17 @@ int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const v
  *        must then be handed to every axon_lmhead_block_bwd of the step, with wt_ready = 1).
  *   axon_lmhead_block_bwd: d_hidden rows of the block (bf16, complete: a row sums over the vocabulary
  *        only).  The weight gradient sums over all blocks: dw_mode 0 = this block is the whole step,
- *        d_weight (bf16) is written; 1 = first block, dw_acc[vocab][hidden] (fp32) is written;
+ *        d_weight (bf16) is written; 1 = first block, dw_acc (fp32 partial sums,
+ *        axon_lmhead_block_dw_acc_bytes(hidden, vocab) bytes, 16-byte aligned; its layout is private:
+ *        tile by tile in register order, so that it streams at full width) is written;
  *        2 = a middle block, added to dw_acc; 3 = last block, dw_acc + this block's share is rounded
- *        to bf16 into d_weight and dw_acc is left as it was.  stash may be NULL (the block's logits are then recomputed).
+ *        to bf16 into d_weight and dw_acc is left as it was.  The same vocab_chunk in every call of a
+ *        step.  stash may be NULL (the block's logits are then recomputed).
  *   timer: NULL, or an axon_timer_create object on `stream` (phases as below).
  * axon_scale_bf16_unless_one multiplies n bf16 values in place by the DEVICE scalar scale[0] and touches
  * nothing when it is exactly 1 (the step's gradients are finished before autograd hands over the
  * factor of the loss, which is 1 unless the caller scaled the loss); n % 8 == 0, x on a 16-byte boundary. */
+int64_t axon_lmhead_block_dw_acc_bytes(int64_t hidden, int64_t vocab);
 int axon_lmhead_block_begin(const void* weight_bf16, int64_t hidden, int64_t vocab, int64_t vocab_chunk,
                             void* workspace, int64_t workspace_bytes, void* stream, void* timer);
 int axon_lmhead_block_fwd(const void* hidden_bf16, const void* weight_bf16, const void* labels,

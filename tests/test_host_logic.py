@@ -294,6 +294,8 @@ def test_fused_step_block_plans():
     assert token_blocks(1500, 512) == [(0, 512), (512, 1024), (1024, 1500)]
     assert token_blocks(1500, 4096) == [(0, 1500)]
     assert token_blocks(33000, 8192) == [(0, 6656), (6656, 13312), (13312, 19968), (19968, 26624), (26624, 33000)]
+    assert token_blocks(32768, 12288) == [(0, 12288), (12288, 24576), (24576, 32768)]
+    assert token_blocks(1000, 300) == [(0, 512), (512, 1000)]
     cu = [0, 400, 433, 933, 997, 1297, 1500]
     assert sequence_blocks(cu, 512) == [(0, 2), (2, 3), (3, 5), (5, 6)]
     assert sequence_blocks(cu, 499) is None
