@@ -47,8 +47,9 @@ SIGNATURES: dict[str, tuple] = {
                                        _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_scatter_rows": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr]),
     "axon_gemm_nt_bf16": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _ptr]),
+    "axon_row_stats_workspace_bytes": (_i64, [_i64]),
     "axon_row_stats": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
-                              _ptr, _ptr, _ptr, _ptr]),
+                              _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_group_stats": (_i32, [_ptr, _ptr, _i64, _i64, _f32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_row_broadcast_mask": (_i32, [_ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _f32, _ptr, _ptr]),
     "axon_fill_zero": (_i32, [_ptr, _i64, _ptr]),
@@ -92,7 +93,7 @@ SIGNATURES: dict[str, tuple] = {
                                         _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
 }
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -27,6 +27,10 @@ class Rows:
 
     @property
     def cu_ptr(self):
+        # the kernels dereference this pointer: offsets that live in host memory would fault the GPU
+        if self.cu is not None and not self.cu.is_cuda:
+            raise _lib.AxonAmdError(f"cu_seqlens is on {self.cu.device}: the row offsets must live on the GPU "
+                                    "(rows_of puts them on the device of the tensor it is given)")
         return ptr(self.cu)
 
 
@@ -82,8 +86,13 @@ def _zeros(n, device, dtype=torch.float32):
 
 
 def _acc8(n_slots, device):
-    """The eight scalar sums a kernel returns; the library writes all of them unless there are no tokens."""
-    return _zeros(8, device) if n_slots == 0 else torch.empty(8, device=device, dtype=torch.float32)
+    """The eight scalar sums a kernel returns; the library writes all of them unless there are no tokens.  Under
+    stream capture they start as NaN: a replay whose reduction never finished would then show."""
+    if n_slots == 0:
+        return _zeros(8, device)
+    if torch.cuda.is_current_stream_capturing():
+        return torch.full((8,), float("nan"), device=device, dtype=torch.float32)
+    return torch.empty(8, device=device, dtype=torch.float32)
 
 
 _PARTIALS: dict = {}
@@ -92,11 +101,18 @@ _PARTIALS: dict = {}
 def _partials(n_slots, device):
     """Workspace of the per-workgroup partial sums (and the ticket counter behind them) of the elementwise
     kernels.  The counter has to be zero before the first launch and every launch leaves it zero, so one
-    zero-filled buffer per (device, stream) is kept and reused: launches on one stream are ordered."""
+    zero-filled buffer per (device, stream) is kept and reused: launches on one stream are ordered.
+
+    Under stream capture nothing is kept: the fill of a buffer created there is recorded, not executed, and the
+    buffer lives in the graph's own pool, so every captured call gets a workspace of its own whose fill is a node
+    of the same graph (graphs then do not depend on each other's replays, and eager calls never share a buffer
+    that a replay re-zeroes)."""
+    nbytes = _lib.load().axon_reduce_partials_bytes(int(n_slots))
+    if torch.cuda.is_current_stream_capturing():
+        return torch.zeros(nbytes // 4, device=device, dtype=torch.float32)
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr())
     ws = _PARTIALS.get(key)
     if ws is None:
-        nbytes = _lib.load().axon_reduce_partials_bytes(int(n_slots))
         ws = torch.zeros(nbytes // 4, device=device, dtype=torch.float32)
         _PARTIALS[key] = ws
     return ws
@@ -111,16 +127,21 @@ def row_stats(a, b, mask, rows: Rows, *, flag_mode=0, threshold=0.0, want_cnt=Tr
     a = f32(a)
     b = f32(b) if b is not None else None
     mk = (None, MASK_F32) if mask is None else mask_arg(mask)
-    # one zero-filled buffer (one fill launch) carries the up to three per-row outputs
+    # one zero-filled buffer (one fill launch) carries the up to three per-row outputs and, in front of them, the
+    # workspace of the sums (an int64 and a float per row: 8-byte aligned at the start of the allocation)
     parts = [want_cnt, want_sum, bool(flag_mode)]
-    buf = _zeros(sum(parts) * max(rows.n_rows, 1), dev).view(sum(parts), -1) if any(parts) else None
+    r = max(rows.n_rows, 1)
+    ws_floats = 3 * r if want_sum else 0
+    buf = _zeros(ws_floats + sum(parts) * r, dev) if any(parts) else None
+    ws = buf[:ws_floats] if want_sum else None
+    outs = buf[ws_floats:].view(sum(parts), -1) if any(parts) else None
     slots = iter(range(sum(parts)))
-    cnt = buf[next(slots)][: rows.n_rows] if want_cnt else None
-    ssum = buf[next(slots)][: rows.n_rows] if want_sum else None
-    flag = buf[next(slots)][: rows.n_rows].view(torch.int32) if flag_mode else None
+    cnt = outs[next(slots)][: rows.n_rows] if want_cnt else None
+    ssum = outs[next(slots)][: rows.n_rows] if want_sum else None
+    flag = outs[next(slots)][: rows.n_rows].view(torch.int32) if flag_mode else None
     check(
         lib.axon_row_stats(ptr(a), ptr(b), ptr(mk[0]), mk[1], rows.cu_ptr, rows.n_rows, rows.n_slots,
-                           rows.uniform_len, flag_mode, float(threshold), ptr(cnt), ptr(ssum), ptr(flag),
+                           rows.uniform_len, flag_mode, float(threshold), ptr(cnt), ptr(ssum), ptr(flag), ptr(ws),
                            stream_ptr()),
         "axon_row_stats",
     )
@@ -241,12 +262,18 @@ def group_scalar(mode, scores, lens, members, offsets, n_groups, *, eps=1e-6, no
 # beyond ``OWNED_ROWS_MAX_SLOTS`` tokens, a token-parallel row pass followed by a token pass (two reads, float
 # atomics per row).  At 2^26 tokens 0.31-0.34 ms against 0.40-0.43; at the sizes of real micro-batches one launch
 # instead of four or five.
+# A workgroup walks a row it owns 2048 slots at a time, alone: rows of more than ``OWNED_ROWS_MAX_MEAN_LEN`` slots
+# (known for a padded layout; for a packed one only the mean is known on the host) take the two passes, which
+# spread any row over the whole GPU.
 OWNED_ROWS_MAX_SLOTS = 1 << 40
 OWNED_ROWS_MIN_MEAN_LEN = 64
+OWNED_ROWS_MAX_MEAN_LEN = 16384
 
 
 def _own_rows(rows: "Rows") -> bool:
-    return 4 <= rows.n_slots <= OWNED_ROWS_MAX_SLOTS and rows.n_slots >= OWNED_ROWS_MIN_MEAN_LEN * max(rows.n_rows, 1)
+    n_rows = max(rows.n_rows, 1)
+    return (4 <= rows.n_slots <= OWNED_ROWS_MAX_SLOTS and rows.n_slots >= OWNED_ROWS_MIN_MEAN_LEN * n_rows
+            and rows.n_slots <= OWNED_ROWS_MAX_MEAN_LEN * n_rows)
 
 
 IS_MODES = {None: 0, "token": 1, "sequence": 2}

@@ -132,13 +132,19 @@ __device__ __forceinline__ void store_block_partials(float (&v)[NV], float* lds 
 // the last of `n` tickets.  The row goes out with agent-scope stores, which write through; waiting
 // for their acknowledgement orders them before the ticket.  (A release fence would also write back
 // every dirty line of this XCD's L2, the kernel's own output stream included, once per workgroup:
-// +35 % kernel time at 2^26 tokens.)
+// +35 % kernel time at 2^26 tokens.)  What this relies on in the hardware: a store at agent scope is
+// acknowledged (vmcnt) only once it has reached the memory level that all XCDs of the device share, so a
+// reader on another XCD that sees the ticket afterwards and drops its own cached copies (the acquire fence
+// in grid_finish) reads the new values.  For the compiler the relaxed atomics carry no order of their own:
+// the two signal fences pin the row's stores before the wait and the ticket after it.
 __device__ __forceinline__ bool publish_row_take_ticket(float* row, const float (&v)[kPartialStride],
                                                         unsigned* ticket, unsigned n) {
 #pragma unroll
   for (int k = 0; k < kPartialStride; ++k)
     __hip_atomic_store(row + k, v[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0)
+  __atomic_signal_fence(__ATOMIC_SEQ_CST);
   const unsigned t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (t != n - 1) return false;
   __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch

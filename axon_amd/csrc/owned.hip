@@ -594,6 +594,10 @@ extern "C" int axon_policy_loss_rows(int kind, const float* logp, const float* o
   if (n_slots == 0) return AXON_OK;
   if (kind < 0 || kind > 4) return AXON_ERR_ARG;
   if (!logp || !oldp || !adv || !mask || !grad || !acc || !partials) return AXON_ERR_ARG;
+  // 16-byte vector accesses at every multiple of four slots: the token arrays must start on 16-byte boundaries
+  if ((reinterpret_cast<uintptr_t>(logp) | reinterpret_cast<uintptr_t>(oldp) | reinterpret_cast<uintptr_t>(adv) |
+       reinterpret_cast<uintptr_t>(mask) | reinterpret_cast<uintptr_t>(isw) | reinterpret_cast<uintptr_t>(grad)) & 15)
+    return AXON_ERR_ARG;
   if (token_reduce < 0 || token_reduce > 3 || batch_reduce < 0 || batch_reduce > 2) return AXON_ERR_ARG;
   if (token_reduce == 3 && !npt) return AXON_ERR_ARG;
   if (token_reduce == 2 && uniform_len <= 0) return AXON_ERR_ARG;
@@ -644,6 +648,9 @@ extern "C" int axon_sampler_correction_rows(const float* oldp, const float* samp
   if (rc != AXON_OK) return rc;
   if (n_slots == 0) return AXON_OK;
   if (!oldp || !samp || !mask || !new_mask || !acc || !partials) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(oldp) | reinterpret_cast<uintptr_t>(samp) | reinterpret_cast<uintptr_t>(mask) |
+       reinterpret_cast<uintptr_t>(isw) | reinterpret_cast<uintptr_t>(new_mask)) & 15)
+    return AXON_ERR_ARG;
   if (is_mode < 0 || is_mode > 2 || rs_mode < 0 || rs_mode > 3) return AXON_ERR_ARG;
   if (is_mode != 0 && isw == nullptr) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;

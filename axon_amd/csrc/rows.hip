@@ -6,6 +6,15 @@
 // of each run adds the run total to the per-row output with one atomic.  A row
 // that spans several waves costs one atomic per wave, so load balance does not
 // depend on the row-length distribution.
+//
+// The partial sums of a long row arrive in whatever order its wavefronts finish, and float addition
+// is not associative.  The counts are sums of small integers (exact in any order) and the flags are
+// ORs; the sums are added as 64-bit fixed-point integers in units of 2^-32, whose addition is
+// associative, so a row's sum comes out the same bits on every run however many wavefronts it
+// spans.  A partial of 2^20 or more in magnitude, an infinity or a NaN goes to a float slot beside
+// it (whether that slot ends up finite, infinite or NaN does not depend on the order either).  A
+// finishing pass turns the two into the fp32 sum.  Rounding a partial to 2^-32 is finer than the
+// fp32 rounding of any row sum of 2^-8 or more in magnitude.
 #include "common.h"
 
 namespace axon {
@@ -16,15 +25,37 @@ struct Seg {
   int flag;
 };
 
-__device__ __forceinline__ void seg_flush(const Seg& s, float* cnt, float* sum, int32_t* flag) {
+struct RowSumAcc {
+  unsigned long long* fixed;  // [n_rows] two's-complement sums in units of 2^-32
+  float* big;                 // [n_rows] what does not fit the fixed-point range
+};
+constexpr float kRowSumUnit = 4294967296.f;  // 2^32
+constexpr float kRowSumLimit = 1048576.f;    // 2^20 per partial: 2^52 units, 2^11 such partials fit 63 bits
+
+__device__ __forceinline__ void row_sum_add(const RowSumAcc& acc, int row, float v) {
+  if (fabsf(v) < kRowSumLimit)
+    atomicAdd(acc.fixed + row, (unsigned long long)__float2ll_rn(v * kRowSumUnit));
+  else
+    atomicAdd(acc.big + row, v);
+}
+
+__global__ __launch_bounds__(256) void row_sum_finish_kernel(RowSumAcc acc, int64_t n_rows,
+                                                             float* __restrict__ sum) {
+  const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= n_rows) return;
+  const double fixed = (double)(long long)acc.fixed[r] * (1.0 / 4294967296.0);
+  sum[r] = (float)((double)acc.big[r] + fixed);
+}
+
+__device__ __forceinline__ void seg_flush(const Seg& s, float* cnt, const RowSumAcc& sum, int32_t* flag) {
   if (s.row < 0) return;
   if (cnt != nullptr && s.cnt != 0.f) atomicAdd(cnt + s.row, s.cnt);
-  if (sum != nullptr && s.sum != 0.f) atomicAdd(sum + s.row, s.sum);
+  if (sum.fixed != nullptr && s.sum != 0.f) row_sum_add(sum, s.row, s.sum);
   if (flag != nullptr && s.flag) atomicOr(flag + s.row, 1);
 }
 
 // Segmented reduction across the wave; lanes hold (row, values) with rows sorted.
-__device__ __forceinline__ void seg_wave_reduce_flush(Seg s, float* cnt, float* sum,
+__device__ __forceinline__ void seg_wave_reduce_flush(Seg s, float* cnt, const RowSumAcc& sum,
                                                       int32_t* flag) {
   const int lane = threadIdx.x & (kWave - 1);
   // the common case: the whole wavefront sits in one row (rows are mostly longer than 256 slots)
@@ -58,7 +89,7 @@ template <int MK>
 __global__ __launch_bounds__(kBlock) void row_stats_kernel(
     const float* __restrict__ a, const float* __restrict__ b, const void* __restrict__ mask,
     const int32_t* __restrict__ cu, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
-    int flag_mode, float thr, float* cnt, float* sum, int32_t* flag) {
+    int flag_mode, float thr, float* cnt, RowSumAcc sum, int32_t* flag) {
   __shared__ int32_t lds_cu[kLdsRows];
   const int64_t c0 = (int64_t)blockIdx.x * kChunk;
   const int64_t c1 = min(c0 + (int64_t)kChunk, n_slots);
@@ -294,10 +325,14 @@ static int check_rows(const int32_t* cu, int64_t n_rows, int64_t n_slots, int64_
   return AXON_OK;
 }
 
+extern "C" int64_t axon_row_stats_workspace_bytes(int64_t n_rows) {
+  return n_rows < 0 ? -1 : n_rows * 12;
+}
+
 extern "C" int axon_row_stats(const float* a, const float* b, const void* mask, int mask_kind,
                               const int32_t* cu, int64_t n_rows, int64_t n_slots,
                               int64_t uniform_len, int flag_mode, float thr, float* cnt,
-                              float* sum, int32_t* flag, void* stream) {
+                              float* sum, int32_t* flag, void* sum_workspace, void* stream) {
   int rc = check_rows(cu, n_rows, n_slots, uniform_len);
   if (rc != AXON_OK) return rc;
   if (n_slots == 0 || n_rows == 0) return AXON_OK;
@@ -305,14 +340,26 @@ extern "C" int axon_row_stats(const float* a, const float* b, const void* mask, 
   if (flag_mode < 0 || flag_mode > 2) return AXON_ERR_ARG;
   if (flag_mode != 0 && flag == nullptr) return AXON_ERR_ARG;
   if (mask_kind != AXON_MASK_F32 && mask_kind != AXON_MASK_I64) return AXON_ERR_ARG;
+  if (sum != nullptr && (sum_workspace == nullptr || (reinterpret_cast<uintptr_t>(sum_workspace) & 7)))
+    return AXON_ERR_WORKSPACE;
+  RowSumAcc acc{nullptr, nullptr};
+  if (sum != nullptr) {
+    acc.fixed = static_cast<unsigned long long*>(sum_workspace);
+    acc.big = reinterpret_cast<float*>(acc.fixed + n_rows);
+  }
   const dim3 g(grid_for(n_slots)), blk(kBlock);
   if (mask_kind == AXON_MASK_F32)
     hipLaunchKernelGGL(row_stats_kernel<AXON_MASK_F32>, g, blk, 0, (hipStream_t)stream, a, b, mask,
-                       cu, n_rows, n_slots, uniform_len, flag_mode, thr, cnt, sum, flag);
+                       cu, n_rows, n_slots, uniform_len, flag_mode, thr, cnt, acc, flag);
   else
     hipLaunchKernelGGL(row_stats_kernel<AXON_MASK_I64>, g, blk, 0, (hipStream_t)stream, a, b, mask,
-                       cu, n_rows, n_slots, uniform_len, flag_mode, thr, cnt, sum, flag);
+                       cu, n_rows, n_slots, uniform_len, flag_mode, thr, cnt, acc, flag);
   AXON_CHECK_LAUNCH();
+  if (sum != nullptr) {
+    hipLaunchKernelGGL(row_sum_finish_kernel, dim3((unsigned)((n_rows + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, acc, n_rows, sum);
+    AXON_CHECK_LAUNCH();
+  }
   return AXON_OK;
 }
 

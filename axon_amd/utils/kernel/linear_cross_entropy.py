@@ -9,7 +9,10 @@ Drop-in for axon/utils/kernel/linear_cross_entropy.py:50-131 (``LinearCrossEntro
 * ``hidden`` ``[N, H]`` or ``[1, N, H]``, ``weight`` ``[V, H]``, ``labels`` int32/int64.  The kernels compute in
   bf16 with fp32 accumulation (the trainer runs under bf16 autocast, forward_utils.py:216); fp16 or fp32
   operands are accepted like the reference accepts any float dtype (kernels.py:517-522 asserts layout only),
-  are rounded to bf16 first, and receive their gradients in their own dtype;
+  are rounded to bf16 first, and receive their gradients in their own dtype.  That is narrower arithmetic than
+  the reference's op, which computes in the operands' own dtype, and it costs a bf16 copy of each such operand
+  per forward (kept for the backward: 1.2 GB for a 151936 x 4096 fp32 weight) plus the cast of its gradient
+  back; a warning says so once per process;
 * outputs are flat fp32 ``[N]`` (never reshaped back, like the reference);
 * differentiable w.r.t. ``hidden`` and ``weight``; gradients come back in the input dtype;
 * ``reduction`` "sum"/"mean" reduce the log-probs as the reference's epilogue does
@@ -38,6 +41,19 @@ import torch
 from axon_amd import _lib, _ops
 
 _REDUCTIONS = ("none", "sum", "mean")
+_warned_rounding = False
+
+
+def _warn_rounded_to_bf16(hidden_dtype, weight_dtype) -> None:
+    global _warned_rounding
+    if _warned_rounding:
+        return
+    _warned_rounding = True
+    import warnings
+
+    warnings.warn(f"linear_cross_entropy: hidden ({hidden_dtype}) / weight ({weight_dtype}) are rounded to bfloat16 "
+                  "before the head (the kernels compute in bf16 with fp32 accumulation); each call makes a bf16 copy "
+                  "of such an operand and casts its gradient back", stacklevel=3)
 
 
 class LinearCrossEntropy(torch.autograd.Function):
@@ -64,6 +80,8 @@ class LinearCrossEntropy(torch.autograd.Function):
         assert hidden2.shape[0] == labels1.shape[0]
         assert hidden2.is_contiguous() and weight.is_contiguous() and labels1.is_contiguous()
         ctx.in_dtypes = (hidden.dtype, weight.dtype)
+        if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+            _warn_rounded_to_bf16(hidden.dtype, weight.dtype)
         hidden2, weight = hidden2.to(torch.bfloat16), weight.to(torch.bfloat16)  # no copy when already bf16
 
         inv_t = 1.0 / temperature

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 18
+#define AXON_AMD_ABI_VERSION 19
 
 enum {
   AXON_OK = 0,
@@ -255,17 +255,23 @@ int axon_gemm_nt_bf16(const void* a_bf16, int64_t lda, const void* b_bf16, int64
  *   flag[r] = any_t  mask != 0 && cond(a-b)   cond: flag_mode 1: (a-b) <  flag_threshold
  *                                                   flag_mode 2: |a-b| > flag_threshold
  *                                                   flag_mode 0: no flag (flag may be NULL)
- * Any of cnt/sum/flag may be NULL.  Outputs must be zero-filled by the caller
- * (axon_fill_zero).  Serves masked row sums in
+ * Any of cnt/sum/flag may be NULL.  cnt and flag must be zero-filled by the caller
+ * (axon_fill_zero); sum needs no initialisation but a zero-filled, 8-byte aligned sum_workspace of
+ * axon_row_stats_workspace_bytes(n_rows) bytes: the partial sums of a row that spans several
+ * wavefronts are added there as 64-bit fixed-point integers (units of 2^-32; partials of 2^20 or more
+ * in magnitude and non-finite ones in a float beside), so sum[r] repeats bit for bit from run to run
+ * whatever the row lengths, like the reference's CPU sums (axon/utils/rl/sampler.py:70-83), and a
+ * second small launch writes sum[].  Serves masked row sums in
  * compute_sampler_rejection_mask (axon/utils/rl/sampler.py:70-79), the veto
  * any() (sampler.py:418-420), GSPO's sequence mean (axon/trainer/algos/loss/loss.py:143-145),
  * agg_loss row counts (axon/trainer/algos/loss/utils.py:236-251), GRPO's score sum
  * (axon/trainer/algos/advantages/advantage.py:98) and the zero-advantage row test
  * (axon/utils/rl/utils.py:35-36). */
+int64_t axon_row_stats_workspace_bytes(int64_t n_rows);
 int axon_row_stats(const float* a, const float* b, const void* mask, int mask_kind,
                    const int32_t* cu_seqlens, int64_t n_rows, int64_t n_slots, int64_t uniform_len,
                    int flag_mode, float flag_threshold, float* cnt, float* sum, int32_t* flag,
-                   void* stream);
+                   void* sum_workspace, void* stream);
 
 /* group_mean_std (axon/utils/rl/advantage.py:106-150) + the GRPO scalar
  * (axon/trainer/algos/advantages/advantage.py:98-107):
@@ -437,6 +443,11 @@ int axon_policy_loss(int kind, const float* logp, const float* old_logp, const f
  *   Slots that belong to no row (before cu_seqlens[0], after cu_seqlens[n_rows]) receive grad 0.
  *   n_slots of 1, 2 or 3 is refused (AXON_ERR_SHAPE): the kernel reads 16-byte vectors; such inputs are
  *   for the calls it replaces.  The same holds for axon_sampler_correction_rows.
+ *   The per-token arrays (logp, old_logp, adv, mask, is_weights, grad; in axon_sampler_correction_rows
+ *   old_logp, sampler_logp, mask, is_weights, new_mask) must start on 16-byte boundaries (AXON_ERR_ARG
+ *   otherwise): every multiple of four slots is then a 16-byte vector.  cu_seqlens must be non-decreasing
+ *   with 0 <= cu_seqlens[r] <= n_slots (not checked on the device: a row that runs backwards or past the
+ *   arrays would be read out of bounds).
  * partials: workspace of axon_reduce_partials_bytes, ticket counters zero (see there). */
 int axon_policy_loss_rows(int kind, const float* logp, const float* old_logp, const float* adv,
                           const void* mask, int mask_kind, const float* is_weights,

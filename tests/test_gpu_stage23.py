@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from axon_amd import _ops, workloads as W
+from axon_amd import _lib, _ops, workloads as W
 from axon_amd.protocol import DataProto
 from axon_amd.trainer.algos.advantages import compute_advantage
 from axon_amd.trainer.algos.loss import agg_loss, compute_loss_fn, masked_mean
@@ -900,6 +900,45 @@ def test_loss_and_correction_in_a_hip_graph():
         assert torch.equal(g_acc[:6], e_acc[:6]) and torch.equal(g_grad, e_grad) and torch.equal(g_cacc[:6], e_cacc[:6])
 
 
+def test_two_hip_graphs_replayed_in_the_other_order():
+    """Two graphs captured one after the other on the same capture stream, the second replayed before the first has
+    ever run, eager calls in between: each graph must carry the fill of its own reduction workspace (a workspace
+    cached at capture time would reach the second graph unfilled), and eager calls must not share a buffer that a
+    replay re-zeroes."""
+    g = torch.Generator(device=DEV).manual_seed(2)
+    b, t = 24, 1500
+    old = -torch.empty(b, t, device=DEV).exponential_(1.0, generator=g)
+    new = old + 0.05 * torch.randn(b, t, device=DEV, generator=g)
+    adv = torch.randn(b, t, device=DEV, generator=g)
+    mask = (torch.rand(b, t, device=DEV, generator=g) > 0.3).float()
+    rows = _ops.rows_of(new)
+    kw_a = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
+    kw_b = dict(token_reduce="mean", batch_reduce="step-mean", ratio_lo=0.8, ratio_hi=1.28, clip_c=3.0)
+    keep = dict(_ops._PARTIALS)
+    _ops._PARTIALS.clear()  # as in a process whose first call on the capture stream happens under capture
+    try:
+        graph_a, graph_b = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph_a):
+            a_acc, a_grad = _ops.policy_loss(0, new, old, adv, mask, None, rows, **kw_a)
+        with torch.cuda.graph(graph_b):
+            b_acc, b_grad = _ops.policy_loss(0, new, old, adv, mask, None, rows, **kw_b)
+        assert not _ops._PARTIALS, "a workspace created under capture must not be kept"
+        for first, second in ((graph_b, graph_a), (graph_a, graph_b), (graph_b, graph_a)):
+            new.copy_(old + 0.05 * torch.randn(b, t, device=DEV, generator=g))
+            ea_acc, ea_grad = _ops.policy_loss(0, new, old, adv, mask, None, rows, **kw_a)
+            eb_acc, eb_grad = _ops.policy_loss(0, new, old, adv, mask, None, rows, **kw_b)
+            torch.cuda.synchronize()
+            first.replay()
+            ea2_acc, _ = _ops.policy_loss(0, new, old, adv, mask, None, rows, **kw_a)  # eager work between replays
+            second.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(a_acc[:6], ea_acc[:6]) and torch.equal(a_grad, ea_grad)
+            assert torch.equal(b_acc[:6], eb_acc[:6]) and torch.equal(b_grad, eb_grad)
+            assert torch.equal(ea2_acc[:6], ea_acc[:6])
+    finally:
+        _ops._PARTIALS.update(keep)
+
+
 # ---- kernels in which a workgroup owns whole rows (GSPO, per-row aggregation, veto, sequence level) --------
 def _awkward_packed(lens, seed):
     """Packed inputs over rows of the given lengths (zeros allowed), padded twins for the oracle."""
@@ -1005,7 +1044,7 @@ def test_packed_layout_without_rows_is_refused():
     ws = torch.zeros(lib.axon_reduce_partials_bytes(64) // 4, device=DEV)
     st = torch.cuda.current_stream().cuda_stream
     p = lambda x: x.data_ptr()  # noqa: E731
-    assert lib.axon_row_stats(p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 0, 0.0, p(t), p(t), None, st) == -2
+    assert lib.axon_row_stats(p(t), p(t), p(t), 0, p(cu), 0, 64, 0, 0, 0.0, p(t), p(t), None, None, st) == -2
     assert lib.axon_row_broadcast_mask(p(t), p(t), 0, p(cu), 0, 64, 0, 0.0, p(t), st) == -2
     assert lib.axon_policy_loss(1, p(t), p(t), p(t), p(t), 0, None, p(cu), 0, 64, 0, p(t), p(t), 1.0, 0, None, 0.8,
                                 1.2, 3.0, p(t), p(t), p(ws), st) == -2
@@ -1045,6 +1084,52 @@ def test_row_owned_kernels_on_random_layouts(seed, owned_rows_forced):
     w_ref, new_ref, _ = OS.correction(pad["old_log_probs"], pad["sampler_log_probs"], pad["response_mask"], **kw)
     assert torch.equal(new.cpu(), pad_to_packed(new_ref, lens))
     assert torch.allclose(proto.batch["sampler_is_weights"].cpu(), pad_to_packed(w_ref, lens), rtol=1e-5, atol=1e-7)
+
+
+def test_sequence_level_decisions_repeat_on_the_short_row_path():
+    """A batch whose rows average eleven tokens takes the row pass + token pass (the row-owning kernels want
+    longer rows), and one of its rows has 6000 tokens: 24 wavefronts each add a partial sum to that row, in
+    whatever order they finish.  Its log-ratio sum is placed on the upper rejection bound to within an fp32
+    ulp, so a sum that depended on the order would flip the row's keep / reject bit from call to call: the
+    masks and weights of twenty calls must be identical (the sums are added in fixed point, rows.hip)."""
+    g = torch.Generator().manual_seed(77)
+    lens = [8] * 1000 + [6000] + [8] * 1000
+    n = sum(lens)
+    cu = W.cu_from_lengths(lens)
+    rows = _ops.rows_of(torch.empty(n, device=DEV), cu)
+    assert not _ops._own_rows(rows) and rows.cu.is_cuda
+    with pytest.raises(_lib.AxonAmdError, match="must live on the GPU"):  # host offsets are refused, not dereferenced
+        _ops.row_stats(torch.zeros(n, device=DEV), None, None, _ops.rows_of(torch.empty(n), cu))
+    old = -torch.empty(n).exponential_(1.0, generator=g)
+    lr = 0.01 * torch.randn(n, generator=g)
+    a, e = int(cu[1000]), int(cu[1001])
+    hi = math.log(2.0)
+    lr[a] += hi - lr[a:e].double().sum().item()  # the long row's sum is ln 2 up to rounding
+    assert abs(lr[a:e].double().sum().item() - hi) < 1e-6
+    samp = (old.double() - lr.double()).float()
+    mask = torch.ones(n)
+    od, sd, md = old.to(DEV), samp.to(DEV), mask.to(DEV)
+    kw = dict(is_mode=2, is_threshold=2.0, rs_mode=2, rs_lr_lo=-hi, rs_lr_hi=hi, log_veto=None)
+    first = None
+    sums = set()
+    for _ in range(20):
+        _, ssum, _ = _ops.row_stats(od, sd, md, rows)
+        isw, new_mask, acc = _ops.sampler_correction(od, sd, md, rows, **kw)
+        sums.add(ssum[1000].item())
+        if first is None:
+            first = (isw.clone(), new_mask.clone(), ssum.clone())
+        assert torch.equal(new_mask, first[1]) and torch.equal(isw, first[0]) and torch.equal(ssum, first[2])
+    assert len(sums) == 1 and abs(sums.pop() - hi) < 1e-5
+    # a partial beyond the fixed-point range, an infinity and a NaN reach the sum as fp32 would have them
+    big = torch.zeros(n)
+    big[a] = 3.0e7
+    big[a + 300] = 5.0
+    big[0] = float("inf")
+    big[8] = float("nan")
+    _, ssum, _ = _ops.row_stats(big.to(DEV), None, md, rows)
+    assert ssum[1000].item() == torch.tensor(3.0e7 + 5.0, dtype=torch.float32).item()  # the double sum, rounded once
+    assert ssum[0].item() == float("inf") and math.isnan(ssum[1].item())
+    assert float(ssum[2:1000].abs().max()) == 0.0
 
 
 def test_row_owned_entry_points_refuse_fewer_than_four_slots():

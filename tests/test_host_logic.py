@@ -49,7 +49,7 @@ def test_workspace_queries_and_argument_errors_without_gpu():
     assert lib.axon_lmhead_stash_bytes(513, 96, 1501) == 3 * 6 * 131072 + 256 * ((6 * 2 * 513 * 4 + 255) // 256)
     assert lib.axon_lmhead_stash_bytes(16, 100, 50) == -1 and lib.axon_lmhead_stash_bytes(0, 128, 1000) == 0
     # null pointers are rejected before any launch
-    assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None) == -1
+    assert lib.axon_row_stats(None, None, None, 0, None, 4, 16, 4, 0, 0.0, None, None, None, None, None) == -1
     assert lib.axon_policy_loss(7, None, None, None, None, 0, None, None, 1, 4, 4, None, None, 0.0, 0, None, 0.8, 1.2,
                                 3.0, None, None, None, None) == -1
     assert lib.axon_reduce_partials_bytes(4097) == lib.axon_reduce_partials_bytes(1 << 30) == 16384 * 32 + 256 * 32 + 2048 and lib.axon_reduce_partials_bytes(-1) == -1
@@ -264,13 +264,16 @@ def test_kl_controllers_known_answers():
 
 def test_row_owning_dispatch_rule():
     """Operators with a per-row quantity take the one-launch kernel (a workgroup works on one row at a time)
-    when the rows average at least OWNED_ROWS_MIN_MEAN_LEN tokens, the row pass + token pass otherwise."""
+    when the rows average at least OWNED_ROWS_MIN_MEAN_LEN and at most OWNED_ROWS_MAX_MEAN_LEN tokens (a single
+    workgroup walks a row alone), the row pass + token pass otherwise."""
     import torch
 
     from axon_amd import _ops
 
     assert _ops._own_rows(_ops.rows_of(torch.zeros(128, 1024)))           # padded 128 x 1024
-    assert _ops._own_rows(_ops.rows_of(torch.zeros(65536), torch.tensor([0, 30000, 65536], dtype=torch.int32)))
+    assert _ops._own_rows(_ops.rows_of(torch.zeros(65536), torch.tensor([0, 30000, 40000, 50000, 65536], dtype=torch.int32)))
+    assert not _ops._own_rows(_ops.rows_of(torch.zeros(65536), torch.tensor([0, 30000, 65536], dtype=torch.int32)))
+    assert not _ops._own_rows(_ops.rows_of(torch.zeros(1, 1 << 20)))      # one row of a million slots
     assert not _ops._own_rows(_ops.rows_of(torch.zeros(4096, 8)))         # rows of 8 tokens
     assert not _ops._own_rows(_ops.rows_of(torch.zeros(12), torch.arange(0, 13, 3, dtype=torch.int32)))
     keep = _ops.OWNED_ROWS_MAX_SLOTS
