@@ -53,6 +53,7 @@ SIGNATURES: dict[str, tuple] = {
     "axon_group_stats": (_i32, [_ptr, _ptr, _i64, _i64, _f32, _i32, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_row_broadcast_mask": (_i32, [_ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _f32, _ptr, _ptr]),
     "axon_fill_zero": (_i32, [_ptr, _i64, _ptr]),
+    "axon_scale_f32": (_i32, [_ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "axon_logits_fwd": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i32, _ptr, _ptr, _ptr, _ptr]),
     "axon_logits_bwd": (_i32, [_ptr, _i32, _i64, _i64, _i64, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr]),
     "axon_reverse_scan": (_i32, [_i32, _ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _f32, _f32, _ptr, _ptr, _ptr,

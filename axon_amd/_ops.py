@@ -934,6 +934,26 @@ class HeadBlocks:
             "axon_lmhead_block_bwd")
 
 
+def scale_f32(x, s1, s2=None):
+    """``x * s1 * s2`` for an fp32 array and one or two device scalars (0-d or 1-element fp32 tensors), in one
+    launch; a new tensor shaped like ``x``."""
+    lib = _lib.load()
+    require_device(x, "scale_f32")
+    xf = f32(x)
+
+    def scalar(t):
+        t = t.detach()
+        if t.dtype != torch.float32 or t.device != xf.device:
+            t = t.to(device=xf.device, dtype=torch.float32)
+        return t
+
+    a = scalar(s1)
+    b = scalar(s2) if s2 is not None else None
+    out = torch.empty_like(xf)
+    check(lib.axon_scale_f32(ptr(xf), ptr(a), ptr(b), ptr(out), int(xf.numel()), stream_ptr()), "axon_scale_f32")
+    return out.view(x.shape)
+
+
 def scale_bf16_unless_one(x, scale):
     """``x *= scale`` in place (bf16 ``x``, ``scale`` a device scalar); no memory traffic when it is exactly 1."""
     lib = _lib.load()

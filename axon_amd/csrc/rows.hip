@@ -303,6 +303,36 @@ using namespace axon;
 
 static inline int grid_for(int64_t n_slots) { return (int)((n_slots + kChunk - 1) / kChunk); }
 
+// out[i] = x[i] * s1[0] * (s2 ? s2[0] : 1): the chain rule of a scalar loss whose per-token gradient the
+// forward left unscaled (the factors live on the device).
+__global__ __launch_bounds__(kBlock) void scale_by_scalars_kernel(const float* __restrict__ x,
+                                                                  const float* __restrict__ s1,
+                                                                  const float* __restrict__ s2,
+                                                                  float* __restrict__ out, int64_t n) {
+  const float f = s1[0] * (s2 != nullptr ? s2[0] : 1.f);
+  const int64_t n4 = n / 4;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    const float4 v = reinterpret_cast<const float4*>(x)[i];
+    reinterpret_cast<float4*>(out)[i] = make_float4(v.x * f, v.y * f, v.z * f, v.w * f);
+  }
+  const int64_t t = n4 * 4 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (t < n) out[t] = x[t] * f;
+}
+
+extern "C" int axon_scale_f32(const float* x, const float* s1, const float* s2, float* out, int64_t n,
+                              void* stream) {
+  if (n < 0) return AXON_ERR_SHAPE;
+  if (n == 0) return AXON_OK;
+  if (!x || !s1 || !out) return AXON_ERR_ARG;
+  if ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) return AXON_ERR_ARG;
+  const int64_t blocks = (n / 4 + kBlock - 1) / kBlock;
+  const unsigned grid = (unsigned)(blocks < 1 ? 1 : blocks < 4096 ? blocks : 4096);
+  hipLaunchKernelGGL(scale_by_scalars_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream, x, s1, s2,
+                     out, n);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+
 extern "C" int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream) {
   if (n_bytes < 0 || (n_bytes & 3) != 0) return AXON_ERR_ARG;
   if (n_bytes == 0) return AXON_OK;

@@ -36,8 +36,11 @@ class _SideTerms(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_ent, g_kl, _g_acc):
         agg_w, grad_kl, acc = ctx.saved_tensors
-        d_ent = (agg_w * (g_ent * acc[5])).to(ctx.dtypes[0]) if agg_w is not None and ctx.needs_input_grad[0] else None
-        d_lp = (grad_kl * (g_kl * acc[5])).to(ctx.dtypes[1]) if grad_kl is not None and ctx.needs_input_grad[1] else None
+        d_ent = d_lp = None
+        if agg_w is not None and ctx.needs_input_grad[0]:
+            d_ent = _ops.scale_f32(agg_w, g_ent, acc[5]).to(ctx.dtypes[0])
+        if grad_kl is not None and ctx.needs_input_grad[1]:
+            d_lp = _ops.scale_f32(grad_kl, g_kl, acc[5]).to(ctx.dtypes[1])
         return d_ent, d_lp, None, None, None, None, None, None
 
 

@@ -11,6 +11,9 @@ here waits for the GPU.
 
 from __future__ import annotations
 
+import collections
+
+import numpy as np
 import torch
 
 from axon_amd import _ops
@@ -27,15 +30,48 @@ def _home(t, home):
     return t if home is None else t.to(home)
 
 
+# Ranking the group labels (strings: a sort on the host) costs more than the kernels of a small batch, and a
+# trainer asks for the same labels again on every pass over a batch: the ranking is kept per label sequence.
+_RANKED: "collections.OrderedDict" = collections.OrderedDict()
+_RANKED_MAX = 16
+
+
+def _ranked_groups(uid, device=None):
+    """``(gidx on the host, n_groups, gidx on `device` or None)`` for the group labels ``uid``; remembered for
+    label arrays (the key is the label sequence itself, so equal labels always give the same answer)."""
+    key = None
+    if isinstance(uid, np.ndarray) and uid.ndim == 1:
+        key = (uid.dtype.str, tuple(uid.tolist()) if uid.dtype == object else uid.tobytes())
+        hit = _RANKED.get(key)
+        if hit is not None:
+            _RANKED.move_to_end(key)
+    else:
+        hit = None
+    if hit is None:
+        gidx = as_torch_index(uid, device="cpu")
+        n_groups = int(gidx.max()) + 1 if gidx.numel() else 0
+        hit = [gidx, n_groups, {}]
+        if key is not None:
+            _RANKED[key] = hit
+            while len(_RANKED) > _RANKED_MAX:
+                _RANKED.popitem(last=False)
+    on_dev = None
+    if device is not None:
+        on_dev = hit[2].get(device)
+        if on_dev is None:
+            on_dev = hit[0].to(device)
+            hit[2][device] = on_dev
+    return hit[0], hit[1], on_dev
+
+
 def _host_groups(data, n_rows: int):
     """``(gidx on the host, n_groups, members, offsets)``: members lists the rows group by group (row order
     kept inside a group), offsets[g] .. offsets[g+1] is group g's range in it."""
-    gidx = as_torch_index(data.non_tensor_batch["uid"], device="cpu")
+    gidx, n_groups, _ = _ranked_groups(data.non_tensor_batch["uid"])
     if gidx.numel() != n_rows:
         raise ValueError(f"uid has {gidx.numel()} entries, batch has {n_rows} rows")
     if gidx.numel() and int(gidx.min()) < 0:
         raise ValueError("group labels must be non-negative")
-    n_groups = int(gidx.max()) + 1 if gidx.numel() else 0
     members = torch.argsort(gidx, stable=True)
     offsets = torch.zeros(n_groups + 1, dtype=torch.int64)
     if n_groups:
@@ -64,11 +100,9 @@ def _group_advantage(data, mode: int, eps: float, clamp_abs: float):
     rows = _ops.rows_of(rewards, cu)
     # group ids are ranked on the host (labels are strings); the group count is read there as well, so
     # that nothing here waits for the GPU
-    gidx_host = as_torch_index(uid, device="cpu")
+    gidx_host, n_groups, gidx = _ranked_groups(uid, rewards.device)
     if gidx_host.numel() != rows.n_rows:
         raise ValueError(f"uid has {gidx_host.numel()} entries, batch has {rows.n_rows} rows")
-    n_groups = int(gidx_host.max()) + 1 if gidx_host.numel() else 0
-    gidx = gidx_host.to(rewards.device, non_blocking=True)
     _, scores, _ = _ops.row_stats(rewards, None, None, rows, want_cnt=False)
     _, _, _, scalar = _ops.group_stats(scores, gidx, n_groups, eps, norm)
     adv = _ops.row_broadcast_mask(scalar, mask, rows, clamp_abs=clamp_abs)

@@ -40,7 +40,7 @@ class _ClippedPolicyLoss(torch.autograd.Function):
     def backward(ctx, g_loss, _g_acc):
         grad, acc = ctx.saved_tensors
         # acc[5]: the 1/denominator a one-pass token-mean leaves to this multiply
-        return (grad * (g_loss * acc[5])).to(ctx.in_dtype), None, None, None, None
+        return _ops.scale_f32(grad, g_loss, acc[5]).to(ctx.in_dtype), None, None, None, None
 
 
 def _aggregation(b, config, default_token_reduce: str) -> dict:
@@ -169,7 +169,7 @@ class _GmpoLoss(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_loss, _g_acc):
         (grad,) = ctx.saved_tensors
-        return (grad * g_loss).to(ctx.in_dtype), None, None, None, None
+        return _ops.scale_f32(grad, g_loss).to(ctx.in_dtype), None, None, None, None
 
 
 @register_loss(LossFn.GEO_MEAN)
@@ -228,7 +228,7 @@ class _CovPolicyLoss(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_loss, _g_acc):
         grad, acc = ctx.saved_tensors
-        return (grad * (g_loss * acc[5])).to(ctx.in_dtype), None, None, None, None
+        return _ops.scale_f32(grad, g_loss, acc[5]).to(ctx.in_dtype), None, None, None, None
 
 
 def _run_cov(kind: int, data, config, hp: dict, default_token_reduce: str):

@@ -36,7 +36,7 @@ class _WeightedRowSum(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         agg_w, acc = ctx.saved_tensors
-        return (agg_w * (g * acc[5])).to(ctx.in_dtype), None, None, None, None, None
+        return _ops.scale_f32(agg_w, g, acc[5]).to(ctx.in_dtype), None, None, None, None, None
 
 
 def agg_loss(

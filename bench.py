@@ -121,6 +121,31 @@ def cpu_baseline(hid, w, lab, budget_s, check=None):
     return out
 
 
+def graph_replay_ms(chain, reps=200):
+    """The launches of `chain` captured once into a HIP graph and replayed: milliseconds per replay (the GPU's
+    time for the chain without the host's eager-call cost) and the captured outputs of the last replay."""
+    import torch
+
+    side = torch.cuda.Stream()  # warm-up off the capture stream
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = chain()
+    for _ in range(5):
+        graph.replay()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(reps):
+        graph.replay()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) / reps, outs
+
+
 def config1_cpu_vs_gpu():
     """The small published configuration (padded 128 x 1024, 16 groups of 8; GRPO advantage, PPO loss and its
     gradient): the CPU port beside the GPU path on the same inputs, with the errors between the two."""
@@ -173,11 +198,31 @@ def config1_cpu_vs_gpu():
         return (time.perf_counter() - t0) / reps, r
 
     t_cpu, (l_cpu, g_cpu) = timed(cpu, 20, False)
-    t_gpu, (l_gpu, g_gpu) = timed(gpu, 50, True)
+    t_gpu, (l_gpu, g_gpu) = timed(gpu, 200, True)
+
+    # the same kernels (row sums, group statistics, broadcast, loss + gradient, gradient scaling) as one HIP graph
+    from axon_amd import _ops
+    rows = _ops.rows_of(gpu_in["token_level_rewards"])
+    gidx_d, one = gidx.to(dev), torch.ones((), device=dev)
+    hp = dict(token_reduce="sum", batch_reduce="token-mean", ratio_lo=1 - 0.2, ratio_hi=1 + 0.28, clip_c=3.0)
+
+    def chain():
+        _, scores, _ = _ops.row_stats(gpu_in["token_level_rewards"], None, None, rows, want_cnt=False)
+        scalar = _ops.group_stats(scores, gidx_d, int(gidx.max()) + 1, 1e-6, 1)[3]
+        adv = _ops.row_broadcast_mask(scalar, gpu_in["response_mask"], rows)
+        acc, grad = _ops.policy_loss(0, gpu_in["log_probs"], gpu_in["old_log_probs"], adv, gpu_in["response_mask"],
+                                     None, rows, **hp)
+        return acc, _ops.scale_f32(grad, one, acc[5])
+
+    t_graph, (acc_g, grad_g) = graph_replay_ms(chain)
+    assert torch.equal(grad_g, g_gpu) and acc_g[0].item() == l_gpu.item(), "graph replay differs from the eager chain"
     g_gpu = g_gpu.cpu().double()
     return {
         "workload": "128 x 1024 padded, GRPO advantage + PPO loss (0.2 / 0.28 / 3.0, sum / token-mean) + gradient",
         "cpu_ms": 1e3 * t_cpu, "cpu_cores": torch.get_num_threads(), "gpu_ms": 1e3 * t_gpu,
+        "gpu_graph_ms": t_graph,
+        "gpu_graph": "the chain's launches captured once into a HIP graph and replayed: GPU time without the host's "
+                     "eager calls (registry lookups, DataProto, autograd, the metrics readback)",
         "loss_rel_err": abs(l_gpu.item() - l_cpu.item()) / abs(l_cpu.item()),
         "grad_rel_l2": ((g_gpu - g_cpu.double()).norm() / g_cpu.double().norm()).item(),
     }
@@ -250,13 +295,33 @@ def config4_cpu_vs_gpu():
         return (time.perf_counter() - t0) / reps, r
 
     t_cpu, (l_cpu, g_cpu, m_cpu, w_cpu) = timed(cpu, 10, False)
-    t_gpu, (l_gpu, g_gpu, m_gpu, w_gpu) = timed(gpu, 50, True)
+    t_gpu, (l_gpu, g_gpu, m_gpu, w_gpu) = timed(gpu, 200, True)
+
+    # the same two operators (correction with veto, GSPO loss + gradient) and the gradient scaling as one HIP graph
+    import math
+
+    from axon_amd import _ops
+    rows = _ops.rows_of(g_in["log_probs"], cu_d)
+    lr_lo, lr_hi = S.log_interval_for_ratio_bounds(0.5, 2.0)
+    one = torch.ones((), device=dev)
+
+    def chain():
+        isw, new_mask, _ = _ops.sampler_correction(g_in["old_log_probs"], g_in["sampler_log_probs"],
+                                                   g_in["response_mask"], rows, is_mode=1, is_threshold=2.0, rs_mode=1,
+                                                   rs_lr_lo=lr_lo, rs_lr_hi=lr_hi, log_veto=math.log(1e-4))
+        acc, grad = _ops.policy_loss(1, g_in["log_probs"], g_in["old_log_probs"], g_in["advantages"], new_mask, isw,
+                                     rows, token_reduce="mean", batch_reduce="step-mean", ratio_lo=1 - 3e-4,
+                                     ratio_hi=1 + 4e-4, clip_c=3.0)
+        return acc, _ops.scale_f32(grad, one, acc[5]), new_mask
+
+    t_graph, (acc_g, grad_g, mask_g) = graph_replay_ms(chain)
+    assert torch.equal(mask_g, m_gpu) and torch.equal(grad_g, g_gpu), "graph replay differs from the eager chain"
     g_gpu = g_gpu.cpu().double()
     return {
         "workload": "65536 packed tokens: token IS (cap 2) + token rejection [0.5, 2] + veto 1e-4, then GSPO "
                     "(3e-4 / 4e-4, mean / step-mean) + gradient",
         "cpu_ms": 1e3 * t_cpu, "cpu_cores": torch.get_num_threads(), "gpu_ms": 1e3 * t_gpu,
-        "sequences": s_, "cpu_layout": f"padded {s_} x {tmax}", "gpu_layout": "packed",
+        "gpu_graph_ms": t_graph, "sequences": s_, "cpu_layout": f"padded {s_} x {tmax}", "gpu_layout": "packed",
         "masks_equal": bool(torch.equal(m_gpu.cpu(), m_cpu)),
         "weights_max_abs_err": (w_gpu.cpu() - w_cpu).abs().max().item(),
         "loss_rel_err": abs(l_gpu.item() - l_cpu.item()) / abs(l_cpu.item()),

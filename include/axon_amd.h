@@ -299,6 +299,12 @@ int axon_row_broadcast_mask(const float* row_scalar, const void* mask, int mask_
  * ------------------------------------------------------------------------- */
 
 int axon_fill_zero(void* ptr, int64_t n_bytes, void* stream); /* n_bytes % 4 == 0 */
+/* out[i] = x[i] * s1[0] * s2[0] (s2 may be NULL: 1), the scalars read on the device: the backward of the loss
+ * operators, whose forward leaves the per-token gradient without the upstream factor and, for a token-mean whose
+ * denominator is known only at the end of the pass, without acc[5] (torch.autograd's multiply in the reference,
+ * e.g. the backward of agg_loss, axon/trainer/algos/loss/utils.py:120-187).  x and out on 16-byte boundaries
+ * (out may be x). */
+int axon_scale_f32(const float* x, const float* s1, const float* s2, float* out, int64_t n, void* stream);
 
 /* Bytes of the `partials` workspace of axon_sampler_correction / axon_policy_loss /
  * axon_side_terms / axon_cov_policy_loss / axon_gmpo_loss (the same for every n_slots: 8 floats for
