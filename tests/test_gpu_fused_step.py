@@ -117,9 +117,10 @@ GSPO = {"clip_ratio_low": 3e-4, "clip_ratio_high": 4e-4, "token_reduce": "mean",
 GSPO_SIDE = dict(GSPO, entropy_coef=0.01, kl_coef=0.05, kl_type="k2")
 RAGGED = [400, 33, 500, 64, 300, 203]          # 1500 tokens; no sequence ends on a multiple of 256
 ON_BORDERS = [256, 256, 512, 128, 128, 256]     # 1536 tokens; every sequence ends on a block border
+ODD_TOTAL = [400, 33, 500, 64, 300, 205]        # 1502 tokens: a last block of 478 or 222 rows cannot be stashed
 
 
-@pytest.mark.parametrize("lens", [RAGGED, ON_BORDERS], ids=["ragged", "on-borders"])
+@pytest.mark.parametrize("lens", [RAGGED, ON_BORDERS, ODD_TOTAL], ids=["ragged", "on-borders", "odd-total"])
 @pytest.mark.parametrize("block_tokens", [256, 512, 4096], ids=["b256", "b512", "one-block"])
 @pytest.mark.parametrize("case", ["ppo", "dapo-entropy-kl", "gspo", "gspo-entropy-kl"])
 def test_fused_step_vs_oracle(case, block_tokens, lens):
@@ -221,6 +222,46 @@ def test_fused_step_with_sampler_correction_and_global_counts():
     assert set(got[1]) == set(metrics)
     for k, val in metrics.items():
         assert got[1][k] == pytest.approx(val, rel=1e-4, abs=1e-6), k
+
+
+@pytest.mark.parametrize("case", ["ppo", "gspo"])
+def test_fused_step_odd_shapes_softcap_temperature_and_integer_operands(case):
+    """A token count that is no multiple of four (the last block then has no stash and recomputes its logits), a
+    vocabulary that is no multiple of the tile, blocks smaller than a tile, soft-capped logits, a temperature,
+    int64 token ids and an int64 response mask (the production dtypes): the node against the unfused path."""
+    from axon_amd.models.fsdp_models import loss_from_outputs
+    from axon_amd.models.fused_head_loss import fused_head_loss
+    from axon_amd.utils.fsdp.forward_utils import packed_logprobs
+    name, args = {"ppo": ("ppo", DAPO_SIDE), "gspo": ("gspo", GSPO)}[case]
+    lens = [130, 7, 251, 64, 301, 90]  # 843 tokens
+    n, h, v = sum(lens), 96, 1001
+    hid, w, ids, labels, rl, old, ref = _inputs(n, h, v, lens, seed=95)
+    cu = rl["cu_seqlens"].to(DEV)
+    mask_i64 = rl["response_mask"].to(DEV).long()
+    adv = (torch.randn(n, generator=torch.Generator().manual_seed(3)) + (GSPO_ADV_SHIFT if case == "gspo" else 0.0))
+    meta = {"loss_fn": name, "loss_fn_args": args, "temperature": 0.7, "dp_replicas": 1}
+
+    def tensors():
+        return {"old_log_probs": old.to(DEV), "advantages": adv.to(DEV) * mask_i64, "response_mask": mask_i64.clone(),
+                "ref_log_prob": ref.to(DEV)}
+
+    hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    data = DataProto.from_dict(tensors=tensors())
+    loss, metrics = fused_head_loss(hd, wd, ids.to(DEV).long(), cu, data, meta, block_tokens=384 if case == "gspo" else 200,
+                                    logit_softcapping=5.0)
+    loss.backward()
+    assert data.meta_info["head_backward"] == "blocked-stash" and data.meta_info["n_blocks"] >= 3
+
+    h2, w2 = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
+    lp, ent = packed_logprobs(h2, w2, ids.to(DEV).long(), cu, 0.7, 5.0)
+    data2 = DataProto.from_dict(tensors=tensors(), meta_info={"cu_seqlens": cu})
+    loss2, metrics2 = loss_from_outputs(data2, lp, ent, meta)
+    loss2.backward()
+    assert loss.item() == pytest.approx(loss2.item(), rel=2e-6, abs=1e-9)
+    assert torch.equal(data.batch["log_probs"], lp.detach()) and torch.equal(data.batch["entropys"], ent.detach())
+    assert rel_l2(hd.grad, h2.grad) < 5e-3 and rel_l2(wd.grad, w2.grad) < 5e-3
+    for k, val in metrics2.items():
+        assert metrics[k] == pytest.approx(val, rel=1e-4, abs=1e-6), k
 
 
 def test_fused_step_falls_back_where_blocks_do_not_apply():
