@@ -39,14 +39,16 @@ SIGNATURES: dict[str, tuple] = {
     "axon_lmhead_block_fwd": (_i32, [_ptr, _ptr, _ptr, _i32, _i64, _i64, _i64, _f32, _f32, _ptr, _i64,
                                      _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_block_bwd": (_i32, [_ptr, _ptr, _ptr, _ptr, _ptr, _i32, _ptr, _ptr, _i64, _i64, _i64,
-                                     _f32, _f32, _ptr, _i64, _ptr, _ptr, _ptr, _i32, _i32, _i64, _ptr, _i64,
-                                     _ptr, _i64, _ptr, _ptr]),
+                                     _f32, _f32, _ptr, _i64, _ptr, _ptr, _ptr, _i32, _i32, _i64, _i32, _i64,
+                                     _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
+    "axon_lmhead_block_can_group": (_i32, [_i64, _i64, _i64]),
     "axon_scale_bf16_unless_one": (_i32, [_ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_active_rows": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_gather_rows": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64,
                                        _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_scatter_rows": (_i32, [_ptr, _ptr, _i64, _i64, _ptr, _ptr]),
     "axon_gemm_nt_bf16": (_i32, [_ptr, _i64, _ptr, _i64, _ptr, _i64, _i64, _i64, _i64, _ptr]),
+    "axon_gemm_bf16": (_i32, [_ptr, _i64, _i32, _ptr, _i64, _i32, _ptr, _i64, _i64, _i64, _i64, _ptr]),
     "axon_row_stats_workspace_bytes": (_i64, [_i64]),
     "axon_row_stats": (_i32, [_ptr, _ptr, _ptr, _i32, _ptr, _i64, _i64, _i64, _i32, _f32,
                               _ptr, _ptr, _ptr, _ptr, _ptr]),
@@ -94,7 +96,7 @@ SIGNATURES: dict[str, tuple] = {
                                         _ptr, _ptr, _f32, _i32, _ptr, _f32, _f32, _f32, _ptr, _ptr, _ptr]),
 }
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 MASK_F32, MASK_I64 = 0, 1
 
 _lock = threading.Lock()

@@ -836,10 +836,13 @@ class HeadBlocks:
     the previous one ends: the shared rows must reach the earlier block with a zero gradient (it then adds
     nothing for them), the later block writes their outputs and their ``d_hidden`` again.  ``vocab_chunk``: 0 =
     the backward of a block takes the whole vocabulary in one piece (no fp32 read-modify-write of the block's
-    d_hidden; bf16 dlogits of 2 x block x vocab x 2 bytes), else a multiple of 256."""
+    d_hidden; bf16 dlogits of block x vocab x 2 bytes), else a multiple of 256.  ``dw_group``: how many
+    consecutive blocks share one weight-gradient GEMM (their dlogits stay in the workspace until the group's
+    last block: a longer reduction and fewer passes over the fp32 partial sums for ``dw_group`` x the dlogit
+    memory); 1 where the shape does not allow it (``axon_lmhead_block_can_group``)."""
 
     def __init__(self, hidden, weight, labels, inv_temperature, ranges, *, softcap=0.0, seq_start=None,
-                 vocab_chunk=0, stash=True, timing: "Timer | None" = None):
+                 vocab_chunk=0, stash=True, dw_group=2, timing: "Timer | None" = None):
         self.lib = _lib.load()
         require_device(hidden, "HeadBlocks")
         self.n, self.h, self.v = _head_operands("HeadBlocks", hidden, weight, labels, seq_start)
@@ -854,8 +857,20 @@ class HeadBlocks:
         dev = hidden.device
         n_max = max(b - a for a, b in self.ranges)
         self.chunk = int(vocab_chunk) if vocab_chunk else (self.v + 255) // 256 * 256
+        # groups of consecutive blocks that share a weight-gradient GEMM: (group, position in the workspace, last?)
+        g = max(int(dw_group), 1)
+        if g > 1 and not self.lib.axon_lmhead_block_can_group(self.h, self.v, self.chunk):
+            g = 1
+        self.dw_group = g
+        self.place = []
+        for k, (a, b) in enumerate(self.ranges):
+            first = k % g == 0
+            pos = 0 if first else self.place[-1][1] + (self.ranges[k - 1][1] - self.ranges[k - 1][0] + 255) // 256 * 256
+            self.place.append((k // g, pos, k % g == g - 1 or k == len(self.ranges) - 1))
+        self.n_groups = self.place[-1][0] + 1
+        self.ws_tokens = max(pos + (b - a + 255) // 256 * 256 for (_, pos, _), (a, b) in zip(self.place, self.ranges))
         self.fwd_ws_bytes = self.lib.axon_lmhead_fwd_workspace_bytes(n_max, self.h, self.v)
-        self.bwd_ws_bytes = self.lib.axon_lmhead_bwd_workspace_bytes(n_max, self.h, self.v, self.chunk)
+        self.bwd_ws_bytes = self.lib.axon_lmhead_bwd_workspace_bytes(self.ws_tokens, self.h, self.v, self.chunk)
         if self.fwd_ws_bytes < 0 or self.bwd_ws_bytes < 0:
             raise _lib.AxonAmdError(f"HeadBlocks: unsupported shape tokens={n_max} hidden={self.h} vocab={self.v}")
         self.fwd_ws = torch.empty(self.fwd_ws_bytes, device=dev, dtype=torch.uint8)
@@ -867,7 +882,7 @@ class HeadBlocks:
         self.out = torch.zeros(2, max(self.n, 1), device=dev, dtype=torch.float32)
         self.d_hidden = torch.empty_like(hidden)
         self.d_weight = torch.empty_like(weight)
-        self.one_block = len(self.ranges) == 1
+        self.one_block = self.n_groups == 1  # one weight-gradient GEMM: no partial sums to carry
         self.dw_acc_bytes = 0 if self.one_block else int(self.lib.axon_lmhead_block_dw_acc_bytes(self.h, self.v))
         self.dw_acc = torch.empty(self.dw_acc_bytes // 4, device=dev, dtype=torch.float32) if self.dw_acc_bytes else None
         self.wt_ready = False
@@ -922,14 +937,16 @@ class HeadBlocks:
             check(self.lib.axon_lmhead_block_begin(ptr(self.weight), self.h, self.v, self.chunk, ptr(self.bwd_ws),
                                                    self.bwd_ws_bytes, st, th), "axon_lmhead_block_begin")
             self.wt_ready = True
-        last = k == len(self.ranges) - 1
-        mode = DW_STORE if self.one_block else DW_FIRST if k == 0 else DW_LAST if last else DW_ADD
+        group, pos, dw_now = self.place[k]
+        mode = (DW_STORE if self.one_block else DW_FIRST if group == 0
+                else DW_LAST if group == self.n_groups - 1 else DW_ADD)
         check(self.lib.axon_lmhead_block_bwd(
             self._at(dlogprobs, n0), self._at(dentropy, n0), self.hidden.data_ptr() + n0 * self.h * 2,
             ptr(self.weight), self._at(self.labels, n0), int(self.labels.dtype == torch.int64),
             ptr(self.stats[0]), ptr(self.stats[1]), nb, self.h, self.v, self.inv_t, self.softcap,
             self._at(self.seq_start, n0), last_dst, self.d_hidden.data_ptr() + n0 * self.h * 2,
-            ptr(self.d_weight), ptr(self.dw_acc), mode, 1, self.chunk, ptr(self.bwd_ws), self.bwd_ws_bytes,
+            ptr(self.d_weight), ptr(self.dw_acc), mode, 1, pos, int(dw_now), self.ws_tokens, self.chunk,
+            ptr(self.bwd_ws), self.bwd_ws_bytes,
             ptr(self.stash) if self.block_stash_bytes else None, self.block_stash_bytes, st, th),
             "axon_lmhead_block_bwd")
 
@@ -1028,4 +1045,19 @@ def gemm_nt(a, b):
     out = torch.empty(n, m, device=a.device, dtype=torch.float32)
     check(lib.axon_gemm_nt_bf16(ptr(a), a.stride(0), ptr(b), b.stride(0), ptr(out), m, m, n, k, stream_ptr()),
           "axon_gemm_nt_bf16")
+    return out
+
+
+def gemm_layouts(a, b, a_kmajor=False, b_kmajor=False):
+    """out[n][m] = sum_k A[m][k] * B[n][k] with `a` given as [m][k], or as [k][m] when a_kmajor (likewise b):
+    a K-major operand is read as it lies.  bf16 in, fp32 out.  Test/benchmark helper."""
+    lib = _lib.load()
+    require_device(a, "gemm_layouts")
+    k, m = (a.shape if a_kmajor else a.shape[::-1])
+    n = b.shape[1] if b_kmajor else b.shape[0]
+    if (b.shape[0] if b_kmajor else b.shape[1]) != k:
+        raise ValueError("gemm_layouts: reduction lengths differ")
+    out = torch.empty(n, m, device=a.device, dtype=torch.float32)
+    check(lib.axon_gemm_bf16(ptr(a), a.stride(0), int(a_kmajor), ptr(b), b.stride(0), int(b_kmajor), ptr(out), m,
+                             m, n, k, stream_ptr()), "axon_gemm_bf16")
     return out

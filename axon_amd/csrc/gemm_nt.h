@@ -102,19 +102,96 @@ __device__ __forceinline__ void settle_acc() { asm volatile("s_nop 15\n\ts_nop 1
 
 // ---------------------------------------------------------------------------------------
 // DmaLoop: k-tiles of 64 go global -> LDS by buffer_load ... lds (no register staging) into
-// XOR-swizzled [row][128 B] slots.  The 160 KB of LDS hold THREE slots for the A operand and
+// XOR-swizzled 32 KB slots.  The 160 KB of LDS hold THREE slots for the A operand and
 // TWO for B.  A k-tile is two k-steps of 32 (64 MFMAs per wave each).  A of k-tile t+2 is
 // issued under the first k-step of tile t into the slot freed one barrier before; the one
 // barrier of the tile follows; B of k-tile t+2 is issued under the second k-step into the B slot
 // that the barrier has just freed.  Compared with a symmetric double buffer this halves the data
 // that has only one k-tile to arrive.
+//
+// An operand is either K-contiguous (row-major [row][k], the NT form) or K-MAJOR ([k][row], rows
+// contiguous: a matrix that would otherwise need a transposed copy).  A K-major operand's slot holds
+// the k-tile as 64 k-rows of 512 bytes, and its fragments are read with the LDS transpose read
+// (ds_read_b64_tr_b16: the sixteen lanes of a group each name four consecutive 16-bit elements of one
+// k-row; lane i of the group receives element i of each of the group's four k-rows), two reads per
+// fragment instead of one.  kAT / kBT select the form of each side at compile time.
 // ---------------------------------------------------------------------------------------
-struct DmaLoop {
+typedef __attribute__((ext_vector_type(4))) short i16x4;
+typedef __attribute__((ext_vector_type(8))) short i16x8;
+
+// What the loop needs to know of one operand side.  T: the operand is K-major.
+template <bool T>
+struct DmaSide {
+  static constexpr int kVariants = T ? 4 : 2;
+  static constexpr int kFrag = T ? kBlocks : 2;
+  int vo[kVariants];   // per-lane source byte offset of a DMA instruction, by variant(j)
+  int step;            // source bytes from DMA instruction j to j + 1
+  int64_t kt_bytes;    // source bytes from one k-tile to the next
+  const __bf16* base;  // the tile's first element of k-tile 0
+  int frag[kFrag];     // per-lane fragment offsets inside a slot: by k-step (row-major) or by block (K-major)
+
+  __device__ static __forceinline__ int variant(int j) { return T ? (j & 1) + 2 * (j >> 2) : (j & 1); }
+
+  // `row0`: first tile row (m0 or n0); `sub`: which half of the tile the wave computes (wm or wn)
+  __device__ __forceinline__ void init(const __bf16* p, int64_t ld, int row0, int sub, const LanePos& lp) {
+    if (!T) {
+      // One DMA instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns rows [64w, 64w+64) of the
+      // operand (8 instructions).  Lane i lands on row i/8, chunk slot i%8, and therefore fetches
+      // global chunk (i%8) ^ swizzle(row); swizzle(row) = (row/2) % 8.
+      const int lrow = lp.lane >> 3;
+      const int sw_even = (lp.lane >> 4) & 7;
+      const int sw_odd = (4 + (lp.lane >> 4)) & 7;
+      const int row = (lp.wave * 64 + lrow) * (int)ld * 2;
+      vo[0] = row + (((lp.lane & 7) ^ sw_even) << 4);
+      vo[1] = row + (((lp.lane & 7) ^ sw_odd) << 4);
+      step = (int)ld * 16;
+      kt_bytes = 128;
+      base = p + (int64_t)row0 * ld;
+      // fragment addressing: row = 128*sub + 16*i + l16, chunk = 4*kk + lq, swizzle = (l16/2)%8.
+      // Sixteen lanes (one chunk column of sixteen rows) cover all 64 banks once.
+      const int sw = (lp.l16 >> 1) & 7;
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+        frag[kk] = (sub * kWaveTile + lp.l16) * 128 + (((kk * 4 + lp.lq) ^ sw) << 4);
+    } else {
+      // One DMA instruction fills 1 KB of LDS = 2 k-rows x 512 B; wave w owns k-rows [16w, 16w+16) of
+      // the k-tile (8 instructions).  Lane i lands on k-row 2j + i/32, 16-byte granule i%32, and fetches
+      // global granule (i%32) ^ S(k-row), S(r) = 2 * (r%4 + 4 * ((r/8)%4)): the sixteen k-rows that one
+      // transpose read touches (r%4 and (r/8)%4 free) land on sixteen different 32-byte bank groups.
+      const int hi = lp.lane >> 5, p32 = lp.lane & 31;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {  // q = variant(j) = (j & 1) + 2 * (j >> 2)
+        const int s = 4 * (q & 1) + 2 * hi + 8 * ((2 * lp.wave + (q >> 1)) & 3);
+        vo[q] = (16 * lp.wave + hi) * (int)ld * 2 + ((p32 ^ s) << 4);
+      }
+      step = (int)ld * 4;
+      kt_bytes = (int64_t)ld * 128;
+      base = p + row0;
+      // fragment of block i, k-step kk, half h: k-row 32kk + 8lq + 4h + l16/4, elements
+      // 128*sub + 16i + 4*(l16%4) ..+3: granule 16*sub + 2i + (l16%4)/2, second half of it for odd l16.
+      const int s15 = (2 * (lp.l16 >> 2) + 8 * lp.lq) & 15;
+      const int fb = (8 * lp.lq + (lp.l16 >> 2)) * 512 + (((16 * sub) ^ (16 * (lp.lq >> 1))) << 4) +
+                     8 * (lp.l16 & 1) + (((lp.l16 & 3) >> 1) << 4);
+#pragma unroll
+      for (int i = 0; i < kBlocks; ++i) frag[i] = fb + ((i << 5) ^ (s15 << 4));
+    }
+  }
+  // source byte offset of k-tile kt; past the end: refetches the last tile, never consumed
+  __device__ __forceinline__ int64_t k_off(int kt, int kt_n) const { return (int64_t)min(kt, kt_n - 1) * kt_bytes; }
+  __device__ __forceinline__ __amdgpu_buffer_rsrc_t rsrc_at(int64_t ko) const {
+    return __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(base) + ko), 0, 0x7fffffff,
+                                             0x00020000);
+  }
+};
+
+template <bool kAT, bool kBT>
+struct DmaLoopT {
   static constexpr int kBK = 64;
   static constexpr int kRowBytes = 128;
   static constexpr int kOperandBytes = kTile * kRowBytes;  // 32 KB
   static constexpr int kBBase = 3 * kOperandBytes;         // A slots at 0/32/64 KB, B slots at 96/128 KB
   static constexpr bool kShiftsEdgeTiles = true;
+  static constexpr int kReadsA = kAT ? 2 : 1, kReadsB = kBT ? 2 : 1;  // LDS reads per fragment
 
   __device__ static __forceinline__ bool supports(const GemmOperands& g) {
     return g.m_rows >= kTile && g.n_rows >= kTile && (g.k % kBK) == 0;
@@ -140,11 +217,11 @@ struct DmaLoop {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds, 16,
                                              voffset, soffset, IMM, 0);
   }
-  // instruction j of an operand tile (rows 8j .. 8j+7 of the wave's 64): lds = tile base of the wave
-  __device__ static __forceinline__ void dma_row8(__amdgpu_buffer_rsrc_t rsrc, int voffset,
-                                                  int row8_bytes, char* lds, int j) {
+  // instruction j of an operand tile (the wave's j-th kilobyte of the slot): lds = tile base of the wave
+  __device__ static __forceinline__ void dma_kb(__amdgpu_buffer_rsrc_t rsrc, int voffset, int step_bytes,
+                                                char* lds, int j) {
     char* const l = lds + (j >> 2) * 4096;
-    const int so = j * row8_bytes - (j & 3) * 1024;
+    const int so = j * step_bytes - (j & 3) * 1024;
     switch (j & 3) {
       case 0: dma16<0>(rsrc, voffset, so, l); break;
       case 1: dma16<1024>(rsrc, voffset, so, l); break;
@@ -152,69 +229,67 @@ struct DmaLoop {
       default: dma16<3072>(rsrc, voffset, so, l); break;
     }
   }
+  // Written as an instruction: the compiler's builtin for it carries no memory operand, so every such
+  // read would be made to wait for ALL DMA in flight (vmcnt(0)), the next tiles' included.  The compiler
+  // therefore does not count these reads either: the loop waits for them itself (lgkmcnt(0) before the
+  // barrier and before the first MFMA of a k-tile), and the values are used by the MFMAs only.
+  // `imm`: a constant once the loops around the call are unrolled (the instruction's offset field)
+  __device__ static __forceinline__ i16x4 read_tr(const char* lds, int imm) {
+    i16x4 v;
+    const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(a), "i"(imm));
+    return v;
+  }
+  // lgkmcnt(0) alone (vmcnt and expcnt at their maxima)
+  __device__ static __forceinline__ void wait_lds_reads() {
+    if (kAT || kBT) __builtin_amdgcn_s_waitcnt(0xC07F);
+  }
+  __device__ static __forceinline__ bf16x8 join(const i16x4& lo, const i16x4& hi) {
+    return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  }
 
   __device__ static __forceinline__ void run(const GemmOperands& g, const TilePos& t, AccTile& acc,
                                              char* smem) {
     const LanePos lp;
-    // --- DMA addressing.  One wave instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns
-    // rows [64w, 64w+64) of each operand (8 instructions).  Lane i lands on row i/8, chunk slot
-    // i%8, and therefore fetches global chunk (i%8) ^ swizzle(row); swizzle(row) = (row/2) % 8.
-    const int lrow = lp.lane >> 3;
-    const int sw_even = (lp.lane >> 4) & 7;
-    const int sw_odd = (4 + (lp.lane >> 4)) & 7;
-    const int row_a = (lp.wave * 64 + lrow) * (int)g.lda * 2;
-    const int row_b = (lp.wave * 64 + lrow) * (int)g.ldb * 2;
-    const int va_e = row_a + (((lp.lane & 7) ^ sw_even) << 4);
-    const int va_o = row_a + (((lp.lane & 7) ^ sw_odd) << 4);
-    const int vb_e = row_b + (((lp.lane & 7) ^ sw_even) << 4);
-    const int vb_o = row_b + (((lp.lane & 7) ^ sw_odd) << 4);
-    const int step_a = (int)g.lda * 16, step_b = (int)g.ldb * 16;
-    const __bf16* base_a = g.a + (int64_t)t.m0 * g.lda;
-    const __bf16* base_b = g.b + (int64_t)t.n0 * g.ldb;
-    const __amdgpu_buffer_rsrc_t ra =
-        __builtin_amdgcn_make_buffer_rsrc((void*)base_a, 0, 0x7fffffff, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rb =
-        __builtin_amdgcn_make_buffer_rsrc((void*)base_b, 0, 0x7fffffff, 0x00020000);
+    DmaSide<kAT> sa;
+    DmaSide<kBT> sb;
+    sa.init(g.a, g.lda, t.m0, lp.wm, lp);
+    sb.init(g.b, g.ldb, t.n0, lp.wn, lp);
     // wave-uniform, so the LDS destination of every DMA instruction is scalar arithmetic into M0
-    char* const dst = smem + __builtin_amdgcn_readfirstlane(lp.wave) * 64 * kRowBytes;
-
-    // --- fragment addressing: row = 128*wm + 16*i + l16, chunk = 4*kk + lq, swizzle = (l16/2)%8.
-    // Sixteen lanes (one chunk column of sixteen rows) cover all 64 banks once.
-    const int sw = (lp.l16 >> 1) & 7;
-    int fa[2], fb[2];
-#pragma unroll
-    for (int kk = 0; kk < 2; ++kk) {
-      fa[kk] = (lp.wm * kWaveTile + lp.l16) * kRowBytes + (((kk * 4 + lp.lq) ^ sw) << 4);
-      fb[kk] = kBBase + (lp.wn * kWaveTile + lp.l16) * kRowBytes + (((kk * 4 + lp.lq) ^ sw) << 4);
-    }
+    char* const dst = smem + __builtin_amdgcn_readfirstlane(lp.wave) * 8192;
 
     zero_acc(acc);
+    // fragments of two k-steps: whole (one 16-byte read) or as the two halves of a transpose read
     bf16x8 af[2][kBlocks], bf[2][kBlocks];
+    i16x4 aft[2][kBlocks][2], bft[2][kBlocks][2];
     const int kt_n = g.k / kBK;
-    // byte offset of k-tile kt inside a row; past the end: refetches the last tile, never consumed
-    auto k_byte = [&](int kt) { return min(kt, kt_n - 1) * kRowBytes; };
-    // `ko` (the k-tile's byte offset inside a row) rides in the per-lane offsets, added once per tile
     auto dma_a = [&](int slot_off, const __amdgpu_buffer_rsrc_t& r, int j) {
-      dma_row8(r, (j & 1) ? va_o : va_e, step_a, dst + slot_off, j);
+      dma_kb(r, sa.vo[DmaSide<kAT>::variant(j)], sa.step, dst + slot_off, j);
     };
     auto dma_b = [&](int slot_off, const __amdgpu_buffer_rsrc_t& r, int j) {
-      dma_row8(r, (j & 1) ? vb_o : vb_e, step_b, dst + kBBase + slot_off, j);
+      dma_kb(r, sb.vo[DmaSide<kBT>::variant(j)], sb.step, dst + kBBase + slot_off, j);
     };
-    // the k-tile's byte offset inside a row rides in the buffer descriptor's base: scalar arithmetic
-    auto rsrc_at = [&](const __bf16* base, int ko) {
-      return __builtin_amdgcn_make_buffer_rsrc((void*)(reinterpret_cast<const char*>(base) + ko), 0, 0x7fffffff,
-                                               0x00020000);
+    // read `half` of fragment `blk` of k-step kk from the slot at byte offset `slot` into set `set`
+    auto read_a = [&](int slot, int kk, int set, int blk, int half) {
+      if (kAT) aft[set][blk][half] = read_tr(smem + slot + sa.frag[blk], kk * 16384 + half * 2048);
+      else af[set][blk] = *reinterpret_cast<const bf16x8*>(smem + slot + sa.frag[kk] + blk * kBlk * kRowBytes);
+    };
+    auto read_b = [&](int slot, int kk, int set, int blk, int half) {
+      if (kBT) bft[set][blk][half] = read_tr(smem + kBBase + slot + sb.frag[blk], kk * 16384 + half * 2048);
+      else bf[set][blk] = *reinterpret_cast<const bf16x8*>(smem + kBBase + slot + sb.frag[kk] + blk * kBlk * kRowBytes);
     };
     // One k-step of 32: 64 MFMAs on fragment set mm_set.  The sixteen fragments of the next k-step
-    // (k-step rd_kk of the slots rd_a / rd_b) are read under the first half of the step, one per two
-    // MFMAs, into the other set, so that they have landed long before the barrier's wait; NA
-    // A-operand or NB B-operand DMA instructions are issued one per eight MFMAs, in slots that carry
-    // no fragment read.  The scheduling fence after every MFMA keeps the source order: the compiler
-    // treats an LDS DMA and an LDS read as aliasing accesses and would otherwise bunch them.
+    // (k-step rd_kk of the slots rd_a / rd_b) are read under the first part of the step, one read per two
+    // MFMAs (A block 0, then the eight B blocks, then A blocks 1..7), into the other set, so that they
+    // have landed long before the barrier's wait; NA A-operand or NB B-operand DMA instructions are
+    // issued one per eight MFMAs, in slots that carry no fragment read.  The scheduling fence after
+    // every MFMA keeps the source order: the compiler treats an LDS DMA and an LDS read as aliasing
+    // accesses and would otherwise bunch them.
     auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, auto na_c, int b_slot,
                     auto nb_c, const __amdgpu_buffer_rsrc_t& rsrc, auto&& mid) {
       constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
       static_assert((NA == 0 || NA == 8) && (NB == 0 || NB == 8) && NA + NB <= 8, "");
+      constexpr int RA = kReadsA, RB = kReadsB;
       const int rd_set = mm_set ^ 1;
 #pragma unroll
       for (int i = 0; i < kBlocks; ++i) {
@@ -226,16 +301,15 @@ struct DmaLoop {
             if (NB) dma_b(b_slot, rsrc, m >> 3);
             if (NA) dma_a(a_slot, rsrc, m >> 3);
           }
-          const bool rd = (m & 1) == 0 && m < 32;
-          const int r = m >> 1;  // A block 0, then the eight B blocks, then A blocks 1..7
-          if (rd && r == 0) af[rd_set][0] = *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk]);
-          if (rd && r >= 1 && r <= 8)
-            bf[rd_set][r - 1] =
-                *reinterpret_cast<const bf16x8*>(smem + rd_b + fb[rd_kk] + (r - 1) * kBlk * kRowBytes);
-          if (rd && r >= 9)
-            af[rd_set][r - 8] =
-                *reinterpret_cast<const bf16x8*>(smem + rd_a + fa[rd_kk] + (r - 8) * kBlk * kRowBytes);
-          mfma_16x16x32(acc[i][j], af[mm_set][i], bf[mm_set][j]);
+          if ((m & 1) == 0) {
+            const int s = m >> 1;
+            if (s < RA) read_a(rd_a, rd_kk, rd_set, 0, s);
+            else if (s < RA + kBlocks * RB) read_b(rd_b, rd_kk, rd_set, (s - RA) / RB, (s - RA) % RB);
+            else if (s < kBlocks * (RA + RB))
+              read_a(rd_a, rd_kk, rd_set, 1 + (s - RA - kBlocks * RB) / RA, (s - RA - kBlocks * RB) % RA);
+          }
+          mfma_16x16x32(acc[i][j], kAT ? join(aft[mm_set][i][0], aft[mm_set][i][1]) : af[mm_set][i],
+                        kBT ? join(bft[mm_set][j][0], bft[mm_set][j][1]) : bf[mm_set][j]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
@@ -244,12 +318,13 @@ struct DmaLoop {
     using I8 = std::integral_constant<int, 8>;
 
     // prologue: tiles 0 and 1 whole (A slots 0, 1; B slots 0, 1)
-#pragma unroll
-    for (int j = 0; j < 8; ++j) dma_a(0, ra, j);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) dma_b(0, rb, j);
     {
-      const __amdgpu_buffer_rsrc_t ra1 = rsrc_at(base_a, k_byte(1)), rb1 = rsrc_at(base_b, k_byte(1));
+      const __amdgpu_buffer_rsrc_t ra = sa.rsrc_at(0), rb = sb.rsrc_at(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dma_a(0, ra, j);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dma_b(0, rb, j);
+      const __amdgpu_buffer_rsrc_t ra1 = sa.rsrc_at(sa.k_off(1, kt_n)), rb1 = sb.rsrc_at(sb.k_off(1, kt_n));
 #pragma unroll
       for (int j = 0; j < 8; ++j) dma_a(kOperandBytes, ra1, j);
 #pragma unroll
@@ -259,13 +334,16 @@ struct DmaLoop {
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
-      af[0][i] = *reinterpret_cast<const bf16x8*>(smem + fa[0] + i * kBlk * kRowBytes);
-      bf[0][i] = *reinterpret_cast<const bf16x8*>(smem + fb[0] + i * kBlk * kRowBytes);
+#pragma unroll
+      for (int h = 0; h < kReadsA; ++h) read_a(0, 0, 0, i, h);
+#pragma unroll
+      for (int h = 0; h < kReadsB; ++h) read_b(0, 0, 0, i, h);
     }
     __builtin_amdgcn_sched_barrier(0);
+    wait_lds_reads();
 
     // per-tile scalars: slots of the tile being consumed (cur), of the next one (nxt), the A slot
-    // being filled, and the per-lane source offsets of k-tile kt+2; those of the following tile are
+    // being filled, and the buffer descriptors of k-tile kt+2; those of the following tile are
     // computed under the second k-step so that the loop's back edge carries no arithmetic
     struct Tile {
       int a_cur, a_nxt, a_fill, b_cur, b_nxt;
@@ -278,9 +356,8 @@ struct DmaLoop {
       v.a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
       v.a_fill = (v.a_nxt == 2 * kOperandBytes) ? 0 : v.a_nxt + kOperandBytes;  // freed one barrier ago
       v.b_nxt = b_cur ^ kOperandBytes;
-      const int ko2 = k_byte(kt + 2);
-      v.ra = rsrc_at(base_a, ko2);
-      v.rb = rsrc_at(base_b, ko2);
+      v.ra = sa.rsrc_at(sa.k_off(kt + 2, kt_n));
+      v.rb = sb.rsrc_at(sb.k_off(kt + 2, kt_n));
       return v;
     };
     Tile tv = tile_vars(0, 0, 0);
@@ -295,12 +372,14 @@ struct DmaLoop {
       step(tv.a_nxt, tv.b_nxt, 0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb,
            [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); });
       tv = nx;
+      wait_lds_reads();  // the next tile's first fragments, read under the second k-step
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
     __builtin_amdgcn_s_barrier();
     settle_acc();
   }
 };
+using DmaLoop = DmaLoopT<false, false>;
 
 // ---------------------------------------------------------------------------------------
 // RegLoop: loads through registers with per-row clamping; any k % BK == 0

@@ -335,7 +335,7 @@ struct DlogitParams {
   const void* labels;
   int labels_i64;
   __bf16* dl;    // [n_pad][chunk_cols]   token-major
-  __bf16* dlT;   // [chunk_cols][n_pad]   vocab-major
+  __bf16* dlT;   // [chunk_cols][n_pad]   vocab-major; null: not wanted (the dWeight GEMM reads dl as a K-major operand)
   int64_t ld_dl, ld_dlT;
   int n_tokens, vocab, v_begin;  // v_begin: first vocab row of this chunk
   float inv_temp;
@@ -512,7 +512,7 @@ __device__ __forceinline__ void dlogit_copy_out_half(const char* stage, int j0, 
       }
     }
   }
-  {
+  if (p.dlT) {
     const int nq = lp.lane & 15, grp = lp.lane >> 4;
     const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
     char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + grp * 32) * p.ld_dlT + n_base + nq * 4);
@@ -561,7 +561,7 @@ __device__ __forceinline__ void dlogit_copy_out(const char* stage, const DlogitP
     }
   }
   // vocab-major copy: 4x4 blocks transposed in registers; 32 lanes cover 128 tokens of one vocab row
-  {
+  if (p.dlT) {
     const int nq = l32;  // token quad
     const int64_t rstep = p.ld_dlT * 2;  // one row of bf16
     char* d = reinterpret_cast<char*>(p.dlT + (int64_t)(m_base + lhi * 4) * p.ld_dlT + n_base + nq * 4);
@@ -1007,11 +1007,16 @@ struct BwdWs {
   int64_t v_pad, n_pad, chunk, bytes;
   int64_t ld_v, ld_n, ld_c;  // leading dimensions of wT, hT/dlT, dl: padded by kLdPad elements
   int chunks;
+  // The dWeight GEMM reads dl [token][vocab] as it lies, as its K-major operand: no vocab-major copy
+  // (dlT is null).  Needs the DMA loop for every chunk's GEMM and 16-byte vectors along the vocabulary.
+  bool dl_kmajor;
 };
 // Rows a power of two apart land on the same L2 sets and memory channels; 128 bytes of padding
 // per row moves consecutive rows to consecutive cache lines (+5..13 % on a stand-alone GEMM with
 // power-of-two leading dimensions, within noise on the whole backward).
 constexpr int64_t kLdPad = 64;
+// `n`: the tokens the workspace holds (one call's, or the span of a group of blocks whose weight
+// gradient is formed by one GEMM)
 BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
   BwdWs w;
   w.v_pad = round_up(vocab, kTile);
@@ -1022,12 +1027,18 @@ BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
   w.ld_v = w.v_pad + kLdPad;
   w.ld_n = w.n_pad + kLdPad;
   w.ld_c = w.chunk + kLdPad;
+  const int64_t last_rows = vocab - (int64_t)(w.chunks - 1) * w.chunk;
+  w.dl_kmajor = h >= kTile && last_rows >= kTile && vocab % 8 == 0 && w.ld_n < (1 << 21) && w.ld_c < (1 << 21);
   char* p = static_cast<char*>(base);
   int64_t off = 0;
   w.wT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.ld_v * 2, kAlign);
   w.hT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.ld_n * 2, kAlign);
   w.dl = reinterpret_cast<__bf16*>(p + off);  off += round_up(w.n_pad * w.ld_c * 2, kAlign);
-  w.dlT = reinterpret_cast<__bf16*>(p + off); off += round_up(w.chunk * w.ld_n * 2, kAlign);
+  w.dlT = nullptr;
+  if (!w.dl_kmajor) {
+    w.dlT = reinterpret_cast<__bf16*>(p + off);
+    off += round_up(w.chunk * w.ld_n * 2, kAlign);
+  }
   w.dh_acc = reinterpret_cast<float*>(p + off);
   if (w.chunks > 1) off += round_up(n * h * 4, kAlign);
   w.bytes = off;
@@ -1090,6 +1101,33 @@ int check_head_shape(int64_t n, int64_t h, int64_t v) {
 int launch_store(const GemmOperands& g, const StoreParams& sp, hipStream_t st) {
   AXON_LAUNCH_GEMM(gemm_store_kernel, g, sp, st);
   return AXON_OK;
+}
+
+// The same with operands that are K-major ([k][rows], see DmaLoopT): the rows are fetched as 16-byte
+// vectors, so the row count (edge tiles are shifted back by it), the leading dimension and the base are
+// multiples of 8 elements.  The DMA loop only: the caller keeps a K-contiguous copy for other shapes.
+inline bool kmajor_ok(const void* p, int64_t ld, int rows) {
+  return rows % 8 == 0 && ld % 8 == 0 && (reinterpret_cast<uintptr_t>(p) & 15) == 0;
+}
+template <class Loop>
+int launch_store_loop(const GemmOperands& g, const StoreParams& sp, hipStream_t st) {
+  const int tiles_m = (g.m_rows + kTile - 1) / kTile, tiles_n = (g.n_rows + kTile - 1) / kTile;
+  if (set_lds(gemm_store_kernel<Loop>) != AXON_OK) return AXON_ERR_LAUNCH;
+  hipLaunchKernelGGL(gemm_store_kernel<Loop>, dim3(tiles_m * tiles_n), dim3(kGemmThreads), kGemmLdsBytes, st, g,
+                     sp, tiles_m, tiles_n);
+  AXON_CHECK_LAUNCH();
+  return AXON_OK;
+}
+bool store_kmajor_ok(const GemmOperands& g, bool a_kmajor, bool b_kmajor) {
+  return dma_ok(g) && (!a_kmajor || kmajor_ok(g.a, g.lda, g.m_rows)) && (!b_kmajor || kmajor_ok(g.b, g.ldb, g.n_rows));
+}
+int launch_store_kmajor(const GemmOperands& g, const StoreParams& sp, bool a_kmajor, bool b_kmajor,
+                        hipStream_t st) {
+  if (!a_kmajor && !b_kmajor) return launch_store(g, sp, st);
+  if (!store_kmajor_ok(g, a_kmajor, b_kmajor)) return AXON_ERR_SHAPE;
+  if (a_kmajor && b_kmajor) return launch_store_loop<DmaLoopT<true, true>>(g, sp, st);
+  if (a_kmajor) return launch_store_loop<DmaLoopT<true, false>>(g, sp, st);
+  return launch_store_loop<DmaLoopT<false, true>>(g, sp, st);
 }
 
 int launch_transpose(const void* in, int64_t ld_in, int rows, int cols, void* out, int64_t ld_out,
@@ -1195,6 +1233,14 @@ struct BlockArgs {
   int wt_ready = 0;
   int dw_mode = kDwStore;
   float* dw_acc = nullptr;  // axon_lmhead_block_dw_acc_bytes of fp32 partial sums, tile order (modes other than kDwStore)
+  // Several consecutive blocks may share ONE weight-gradient GEMM (a longer reduction, fewer passes over
+  // the fp32 partial sums): each keeps its dlogits and its transposed hidden rows in the workspace, at
+  // `group_pos` tokens from the start (a multiple of 256, the blocks before it rounded up to that), and
+  // the GEMM runs with the block that says `dw_now` over everything up to its end.  `ws_tokens`: the
+  // tokens the workspace was sized for (0: this call's), the same for every call that shares it.
+  int64_t group_pos = 0;
+  int dw_now = 1;
+  int64_t ws_tokens = 0;
 };
 
 int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, const void* weight,
@@ -1210,7 +1256,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   if (blk.dw_mode < kDwStore || blk.dw_mode > kDwLast) return AXON_ERR_ARG;
   if (blk.dw_mode != kDwStore && (!blk.dw_acc || (reinterpret_cast<uintptr_t>(blk.dw_acc) & 15) || n == 0))
     return AXON_ERR_ARG;
-  const bool dw_bf16 = blk.dw_mode == kDwStore || blk.dw_mode == kDwLast;
+  const bool dw_bf16 = blk.dw_now && (blk.dw_mode == kDwStore || blk.dw_mode == kDwLast);
   if (dw_bf16 && !d_weight) return AXON_ERR_ARG;
   const hipStream_t st = (hipStream_t)stream;
   if (n == 0) return axon_fill_zero(d_weight, v * h * 2, stream);
@@ -1220,9 +1266,14 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   if ((reinterpret_cast<uintptr_t>(hidden) | reinterpret_cast<uintptr_t>(weight) |
        reinterpret_cast<uintptr_t>(d_hidden) | (dw_bf16 ? reinterpret_cast<uintptr_t>(d_weight) : 0)) & 15)
     return AXON_ERR_ARG;
+  const int64_t pos = blk.group_pos, n_tile = round_up(n, kTile);
+  const int64_t ws_tokens = blk.ws_tokens > 0 ? blk.ws_tokens : n;
+  if (pos < 0 || pos % kTile != 0 || pos + n_tile > round_up(ws_tokens, kTile)) return AXON_ERR_ARG;
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
-  const BwdWs w = bwd_ws(n, h, v, chunk, base);
+  const BwdWs w = bwd_ws(ws_tokens, h, v, chunk, base);
   if ((base - static_cast<char*>(workspace)) + w.bytes > ws_bytes) return AXON_ERR_WORKSPACE;
+  // blocks that share a weight-gradient GEMM keep their dlogits of the whole vocabulary side by side
+  if ((pos > 0 || !blk.dw_now) && !(w.dl_kmajor && w.chunks == 1)) return AXON_ERR_ARG;
   StashWs sw{};
   if (stash) {
     if (reinterpret_cast<uintptr_t>(stash) & 15) return AXON_ERR_ARG;
@@ -1238,11 +1289,12 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.ld_v, (int)w.v_pad, st);
       if (rc != AXON_OK) return rc;
     }
-    rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT, w.ld_n, (int)w.n_pad, st);
+    rc = launch_transpose(hidden, h, (int)n, (int)h, w.hT + pos, w.ld_n, (int)n_tile, st);
     if (rc != AXON_OK) return rc;
   }
-  const int64_t n_red = round_up(n, 64);  // reduction length of B3
+  const int64_t n_red = round_up(n, 64);  // reduction length of B3 (from this block's first token)
   const int64_t tiles_h = round_up(h, kTile) / kTile;
+  __bf16* const dl = w.dl + pos * w.ld_c;  // this block's rows
 
   for (int ci = 0; ci < w.chunks; ++ci) {
     const int64_t v0 = (int64_t)ci * w.chunk;
@@ -1258,7 +1310,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       DlogitParams p;
       p.lse = lse; p.entropy_b = entropy_b; p.dlogprobs = dlogprobs; p.dentropy = dentropy;
       p.labels = labels; p.labels_i64 = labels_i64;
-      p.dl = w.dl; p.dlT = w.dlT; p.ld_dl = w.ld_c; p.ld_dlT = w.ld_n;
+      p.dl = dl; p.dlT = w.dlT; p.ld_dl = w.ld_c; p.ld_dlT = w.ld_n;
       p.n_tokens = (int)n; p.vocab = (int)v; p.v_begin = (int)v0; p.inv_temp = inv_temp;
       p.cap = softcap; p.inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
       p.is_start = is_start;
@@ -1278,9 +1330,12 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       }
       // reduction padding the tiles did not cover (the shifted-tile path writes no padding; the
       // clamped path writes zeros there already, the extra fill is then redundant but harmless)
-      rc = launch_zero_cols(w.dl, w.ld_c, (int)n, (int)vc, (int)(vc_red - vc), st);
+      rc = launch_zero_cols(dl, w.ld_c, (int)n, (int)vc, (int)(vc_red - vc), st);
       if (rc != AXON_OK) return rc;
-      rc = launch_zero_cols(w.dlT, w.ld_n, (int)vc, (int)n, (int)(n_red - n), st);
+      if (w.dl_kmajor)  // the token rows up to the next tile boundary: reduction padding of B3
+        rc = launch_zero_cols(dl + n * w.ld_c, w.ld_c, (int)(n_tile - n), 0, (int)vc_red, st);
+      else
+        rc = launch_zero_cols(w.dlT, w.ld_n, (int)vc, (int)n, (int)(n_red - n), st);
       if (rc != AXON_OK) return rc;
     }
     // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
@@ -1288,7 +1343,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       Span span(timer, 2);
       GemmOperands g;
       g.a = w.wT + v0;  g.lda = w.ld_v;  g.m_rows = (int)h;
-      g.b = w.dl;       g.ldb = w.ld_c;  g.n_rows = (int)n;
+      g.b = dl;         g.ldb = w.ld_c;  g.n_rows = (int)n;
       g.k = (int)vc_red;
       StoreParams sp;
       const bool last = (ci == w.chunks - 1);
@@ -1299,13 +1354,16 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       rc = launch_store(g, sp, st);
       if (rc != AXON_OK) return rc;
     }
-    // B3: dWeight[v0 + v][h] = sum_t dlT[v][t] * hT[h][t]
-    {
+    // B3: dWeight[v0 + v][h] = sum_t dl[t][v] * hT[h][t] over the tokens the workspace holds up to this
+    // block's end (dl read as the K-major operand, or its vocab-major copy dlT[v][t])
+    if (blk.dw_now) {
       Span span(timer, 3);
       GemmOperands g;
-      g.a = w.hT;   g.lda = w.ld_n;  g.m_rows = (int)h;
-      g.b = w.dlT;  g.ldb = w.ld_n;  g.n_rows = (int)vc;
-      g.k = (int)n_red;
+      g.a = w.hT;  g.lda = w.ld_n;  g.m_rows = (int)h;
+      if (w.dl_kmajor) { g.b = w.dl;   g.ldb = w.ld_c; }
+      else             { g.b = w.dlT;  g.ldb = w.ld_n; }
+      g.n_rows = (int)vc;
+      g.k = (int)(pos + n_red);
       StoreParams sp;
       sp.out_f32 = nullptr;  sp.ld_f32 = 0;
       sp.tile_acc = blk.dw_mode == kDwStore
@@ -1315,7 +1373,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       sp.m_valid = (int)h; sp.n_valid = (int)vc;
       sp.accumulate = blk.dw_mode == kDwAdd || blk.dw_mode == kDwLast;
       sp.keep_f32 = blk.dw_mode != kDwLast;
-      rc = launch_store(g, sp, st);
+      rc = launch_store_kmajor(g, sp, false, w.dl_kmajor, st);
       if (rc != AXON_OK) return rc;
     }
   }
@@ -1502,6 +1560,23 @@ extern "C" int axon_gemm_nt_bf16(const void* a, int64_t lda, const void* b, int6
   return launch_store(g, sp, (hipStream_t)stream);
 }
 
+extern "C" int axon_gemm_bf16(const void* a, int64_t lda, int a_kmajor, const void* b, int64_t ldb,
+                              int b_kmajor, float* out, int64_t ldo, int64_t m, int64_t n, int64_t k,
+                              void* stream) {
+  if (!a || !b || !out) return AXON_ERR_ARG;
+  if (m <= 0 || n <= 0 || k <= 0) return AXON_ERR_ARG;
+  if (k % 32 != 0 || lda % 8 != 0 || ldb % 8 != 0 || m % 4 != 0 || ldo % 4 != 0) return AXON_ERR_SHAPE;
+  if (m >= (1 << 30) || n >= (1 << 30)) return AXON_ERR_SHAPE;
+  GemmOperands g;
+  g.a = static_cast<const __bf16*>(a);  g.lda = lda;  g.m_rows = (int)m;
+  g.b = static_cast<const __bf16*>(b);  g.ldb = ldb;  g.n_rows = (int)n;
+  g.k = (int)k;
+  StoreParams sp;
+  sp.out_f32 = out; sp.ld_f32 = ldo; sp.out_bf16 = nullptr; sp.ld_bf16 = 0;
+  sp.m_valid = (int)m; sp.n_valid = (int)n; sp.accumulate = 0; sp.keep_f32 = 1; sp.tile_acc = nullptr;
+  return launch_store_kmajor(g, sp, a_kmajor != 0, b_kmajor != 0, (hipStream_t)stream);
+}
+
 // ----------------------------------------------------------------------------
 // One step as token blocks: forward (with stash), loss and backward of one block of consecutive
 // tokens before the next block's forward, so that what is kept from a forward to its backward is
@@ -1522,6 +1597,12 @@ bool last_dst_ok(int64_t last_dst, int64_t n) { return last_dst <= n && last_dst
 extern "C" int64_t axon_lmhead_block_dw_acc_bytes(int64_t h, int64_t v) {
   if (check_head_shape(0, h, v) != AXON_OK) return -1;
   return (round_up(h, kTile) / kTile) * (round_up(v, kTile) / kTile) * kTileAccVecs * 16;
+}
+
+extern "C" int axon_lmhead_block_can_group(int64_t h, int64_t v, int64_t chunk) {
+  if (check_head_shape(0, h, v) != AXON_OK || chunk < 0 || chunk % kTile != 0) return 0;
+  const BwdWs w = bwd_ws(kTile, h, v, chunk, nullptr);
+  return (w.dl_kmajor && w.chunks == 1) ? 1 : 0;
 }
 
 extern "C" int axon_lmhead_block_begin(const void* weight, int64_t h, int64_t v, int64_t chunk,
@@ -1560,6 +1641,7 @@ extern "C" int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentro
                                      int64_t v, float inv_temp, float softcap,
                                      const uint8_t* seq_start, int64_t last_dst, void* d_hidden,
                                      void* d_weight, float* dw_acc, int dw_mode, int wt_ready,
+                                     int64_t group_pos, int dw_now, int64_t ws_tokens,
                                      int64_t chunk, void* workspace, int64_t ws_bytes,
                                      const void* stash, int64_t stash_bytes, void* stream,
                                      void* timer) {
@@ -1572,6 +1654,9 @@ extern "C" int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentro
   blk.wt_ready = wt_ready != 0;
   blk.dw_mode = dw_mode;
   blk.dw_acc = dw_acc;
+  blk.group_pos = group_pos;
+  blk.dw_now = dw_now != 0;
+  blk.ws_tokens = ws_tokens;
   return bwd_impl(dlogprobs, dentropy, hidden, weight, labels, labels_i64, lse, entropy_b, n, h, v,
                   inv_temp, softcap, seq_start, d_hidden, d_weight, chunk, workspace, ws_bytes, stash,
                   stash_bytes, stream, t, blk);

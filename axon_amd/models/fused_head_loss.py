@@ -28,9 +28,12 @@ import torch
 from axon_amd import _lib, _ops
 from axon_amd.trainer.algos.loss.loss import POLICY_LOSS_KINDS, policy_loss_metrics, policy_loss_spec
 
-# Tokens per block.  One block's stash is 2 bytes x block x vocab (2.5 GB at 8192 x 151936); the weight gradient
-# is carried across blocks in fp32, one read-modify-write of vocab x hidden x 4 bytes per block.
+# Tokens per block.  One block's stash is 2 bytes x block x vocab (2.5 GB at 8192 x 151936).  The weight
+# gradient is formed once per group of DEFAULT_DW_GROUP blocks (their bf16 dlogits, 2 bytes x block x vocab
+# each, wait in the workspace) and carried from group to group in fp32, one read-modify-write of
+# vocab x hidden x 4 bytes per group.
 DEFAULT_BLOCK_TOKENS = 8192
+DEFAULT_DW_GROUP = 2
 _TILE = 256
 
 
@@ -124,7 +127,8 @@ class _BlockedHeadLoss(torch.autograd.Function):
             slots = [(0 if k == 0 else a + 1, n if k == len(ranges) - 1 else b + 1) for k, (a, b) in enumerate(ranges)]
 
         hb = _ops.HeadBlocks(hidden, weight, spec["ids"], spec["inv_t"], ranges, softcap=spec["softcap"],
-                             seq_start=spec["seq_start"], vocab_chunk=spec["vocab_chunk"], timing=_ops.TIMING)
+                             seq_start=spec["seq_start"], vocab_chunk=spec["vocab_chunk"], dw_group=spec["dw_group"],
+                             timing=_ops.TIMING)
         g_lp = torch.zeros(n + 4, device=dev, dtype=torch.float32)
         want_ent_grad = side is not None and side["entropy_coef"] != 0
         g_en = torch.zeros(n + 4, device=dev, dtype=torch.float32) if want_ent_grad else None
@@ -187,6 +191,7 @@ class _BlockedHeadLoss(torch.autograd.Function):
         ctx.grads = (hb.d_hidden, hb.d_weight)
         ctx.head_workspace_bytes = hb.workspace_bytes
         spec["stash_bytes"], spec["workspace_bytes"], spec["n_blocks"] = hb.stash_bytes, hb.workspace_bytes, len(ranges)
+        spec["dw_group_used"] = hb.dw_group
         log_probs, entropy = hb.logprobs, hb.entropy
         hb.d_hidden = hb.d_weight = None
         ctx.mark_non_differentiable(log_probs, entropy, sums, side_sums)
@@ -205,8 +210,8 @@ class _BlockedHeadLoss(torch.autograd.Function):
 
 
 def blocked_spec(hidden, weight, packed_ids, cu_seqlens, data, loss_fn, loss_fn_args, temperature, *,
-                 block_tokens=DEFAULT_BLOCK_TOKENS, vocab_chunk=0, logit_softcapping=None, side_mask=None,
-                 cu_host=None):
+                 block_tokens=DEFAULT_BLOCK_TOKENS, vocab_chunk=0, dw_group=DEFAULT_DW_GROUP, logit_softcapping=None,
+                 side_mask=None, cu_host=None):
     """What ``_BlockedHeadLoss`` needs, or None when this batch has to take the unfused path.  ``data.batch`` holds
     the packed per-token tensors (after the sampler correction); ``side_mask`` the mask of the entropy / KL
     terms (the one from before the correction, fsdp_models.py:197-211) or None for no side terms."""
@@ -225,7 +230,8 @@ def blocked_spec(hidden, weight, packed_ids, cu_seqlens, data, loss_fn, loss_fn_
     rows_all = _ops.Rows(int(cu.numel()) - 1, n, 0, cu, (n,))
     seq_mode = kind == 1 or hp["token_reduce"] != "sum" or hp["batch_reduce"] != "token-mean"
     spec = dict(kind=kind, tensors=tensors, hp=dict(hp), cu=cu, cu_host=None, seq_mode=seq_mode,
-                block_tokens=int(block_tokens), vocab_chunk=int(vocab_chunk), ids=packed_ids.reshape(-1),
+                block_tokens=int(block_tokens), vocab_chunk=int(vocab_chunk), dw_group=int(dw_group),
+                ids=packed_ids.reshape(-1),
                 inv_t=1.0 / float(temperature), softcap=0.0 if logit_softcapping is None else float(logit_softcapping),
                 seq_start=_ops.seq_start_flags(cu, n), side=None)
     if seq_mode:
@@ -263,7 +269,8 @@ def blocked_head_loss(hidden, weight, spec):
 
 
 def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
-                    block_tokens=DEFAULT_BLOCK_TOKENS, vocab_chunk=0, logit_softcapping=None, cu_host=None):
+                    block_tokens=DEFAULT_BLOCK_TOKENS, vocab_chunk=0, dw_group=DEFAULT_DW_GROUP,
+                    logit_softcapping=None, cu_host=None):
     """Everything of ``forward_backward_fn`` from the final hidden states on (fsdp_models.py:203-278): head, sampler
     correction hook, registry loss, sampler-gap metrics, entropy bonus, KL penalty, ``dp_replicas`` scaling.
 
@@ -274,7 +281,7 @@ def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
     ``n_micro_batches``).  Returns ``(scaled_loss, metrics)`` with the reference's metric names;
     ``data.batch["log_probs"]`` / ``["entropys"]`` are set to the (detached) head outputs and ``meta_info`` of
     ``data`` gets ``head_backward`` ("blocked-stash" or "recompute"), and for the blocked path ``stash_bytes``,
-    ``head_workspace_bytes`` and ``n_blocks``.
+    ``head_workspace_bytes``, ``n_blocks`` and ``dw_group`` (blocks per weight-gradient GEMM).
 
     ``cu_host``: the same offsets as a Python list, for a caller that has them (saves the one readback that the
     sequence-cut blocks need)."""
@@ -304,8 +311,8 @@ def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
             data, corr_metrics = compute_sampler_correction_and_add_to_batch(data, loss_fn_args)
             b = data.batch
         spec = blocked_spec(hidden2, weight, packed_ids, cu_seqlens, data, loss_fn, loss_fn_args, temperature,
-                            block_tokens=block_tokens, vocab_chunk=vocab_chunk, logit_softcapping=logit_softcapping,
-                            side_mask=side_mask, cu_host=cu_host)
+                            block_tokens=block_tokens, vocab_chunk=vocab_chunk, dw_group=dw_group,
+                            logit_softcapping=logit_softcapping, side_mask=side_mask, cu_host=cu_host)
         if spec is None and wanted and "sampler_log_probs" in b:
             # the unfused path applies the correction itself: hand it the batch as it was
             b["response_mask"] = side_mask
@@ -321,7 +328,8 @@ def fused_head_loss(hidden, weight, packed_ids, cu_seqlens, data, meta_info, *,
     loss, log_prob, entropy, _sums, _side_sums = blocked_head_loss(hidden2, weight, spec)
     b["log_probs"], b["entropys"] = log_prob, entropy
     data.meta_info.update(head_backward="blocked-stash", stash_bytes=spec["stash_bytes"],
-                          head_workspace_bytes=spec["workspace_bytes"], n_blocks=spec["n_blocks"])
+                          head_workspace_bytes=spec["workspace_bytes"], n_blocks=spec["n_blocks"],
+                          dw_group=spec["dw_group_used"])
     host, event = spec["readback"]  # the one readback of the step's scalars, started before the last block's backward
     event.synchronize()
     vals = host.tolist()

@@ -52,6 +52,8 @@ def parse_args():
                          "separate autograd functions, nothing of size tokens x vocab in memory), or a stash of "
                          "ALL tokens kept from the forward to the backward (opt-in)")
     ap.add_argument("--block-tokens", type=int, default=8192, help="tokens per block of the blocked-stash step")
+    ap.add_argument("--dw-group", type=int, default=0,
+                    help="blocks that share one weight-gradient GEMM in the blocked-stash step (0: the library's default)")
     ap.add_argument("--no-variants", dest="variants", action="store_false",
                     help="skip the short measurements of the same step on the other head-backward paths")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget; 0 disables it")
@@ -773,7 +775,7 @@ def main():
     loss_args = {"clip_ratio_low": 0.2, "clip_ratio_high": 0.28, "token_reduce": "sum", "batch_reduce": "token-mean"}
     adv_cfg = {"advantage": "grpo", "advantage_args": {"epsilon": 1e-6}}
     meta = {"loss_fn": "ppo", "loss_fn_args": loss_args, "temperature": 1.0, "dp_replicas": 1}
-    from axon_amd.models.fused_head_loss import fused_head_loss
+    from axon_amd.models.fused_head_loss import DEFAULT_DW_GROUP, fused_head_loss
 
     def advantages(mask):
         adv_in = DataProto.from_dict(tensors={"token_level_rewards": tlr, "response_mask": mask},
@@ -798,7 +800,7 @@ def main():
         hg, wg = hd.detach().requires_grad_(True), wd.detach().requires_grad_(True)
         data = DataProto.from_dict(tensors={"old_log_probs": old, "advantages": advantages(mask), "response_mask": mask})
         loss, _ = fused_head_loss(hg, wg, ld, cu, data, meta, block_tokens=args.block_tokens,
-                                  vocab_chunk=args.vocab_chunk)
+                                  vocab_chunk=args.vocab_chunk, dw_group=args.dw_group or DEFAULT_DW_GROUP)
         loss.backward()
         block_info.update(data.meta_info)
         return loss, hg.grad, wg.grad
@@ -908,7 +910,7 @@ def main():
         "frac": (dom["algorithmic_tflops"] or dom["executed_tflops"]) / MFMA_BF16_PEAK_TFLOPS,
         "avg_launch_ms": dom["avg_launch_ms"], "launches_per_step": dom["launches_per_step"],
         "traffic": traffic_from_profile(args.workload, head_path) if not args.tokens and not args.vocab_chunk
-        and args.block_tokens == 8192 and "gemm_store" in dom["kernel"] else None,
+        and args.block_tokens == 8192 and not args.dw_group and "gemm_store" in dom["kernel"] else None,
         "kernels": kernels,
         "path_algorithmic_tflops": 6 * nhv / (ms_per_step * 1e-3) / 1e12,
         "path_frac_of_peak": 6 * nhv / (ms_per_step * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
@@ -942,6 +944,7 @@ def main():
     }
     if head_path == "blocked-stash":
         out["config"].update(block_tokens=args.block_tokens, n_blocks=int(block_info["n_blocks"]),
+                             dw_group=int(block_info["dw_group"]),
                              head_workspace_bytes=int(block_info["head_workspace_bytes"]))
     if args.calibrate:
         cal = gemm_calibration(dev, n, h)

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define AXON_AMD_ABI_VERSION 19
+#define AXON_AMD_ABI_VERSION 20
 
 enum {
   AXON_OK = 0,
@@ -234,8 +234,10 @@ int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentropy, const v
                           int64_t vocab, float inv_temperature, float softcap,
                           const uint8_t* seq_start, int64_t last_dst, void* d_hidden_bf16,
                           void* d_weight_bf16, float* dw_acc, int dw_mode, int wt_ready,
+                          int64_t group_pos, int dw_now, int64_t ws_tokens,
                           int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
                           const void* stash, int64_t stash_bytes, void* stream, void* timer);
+int axon_lmhead_block_can_group(int64_t hidden, int64_t vocab, int64_t vocab_chunk);
 int axon_scale_bf16_unless_one(void* x_bf16, int64_t n, const float* scale, void* stream);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
@@ -244,6 +246,15 @@ int axon_scale_bf16_unless_one(void* x_bf16, int64_t n, const float* scale, void
  * Constraints: k % 32 == 0, lda/ldb multiples of 8 elements. */
 int axon_gemm_nt_bf16(const void* a_bf16, int64_t lda, const void* b_bf16, int64_t ldb,
                       float* out, int64_t ldo, int64_t m, int64_t n, int64_t k, void* stream);
+
+/* The same GEMM with either operand given K-MAJOR instead of K-contiguous: a_kmajor != 0 means `a` is
+ * [k][lda] with the m rows contiguous (out[n][m] = sum_k a[k][m] * b[n][k]), likewise b_kmajor for `b`.
+ * A K-major operand is read as it lies (no transposed copy) through the LDS transpose read of gfx950.
+ * No reference counterpart (test and benchmark helper, like the above).  K-major operands only on the
+ * DMA main loop: m, n >= 256, k % 64 == 0, and for a K-major operand a 16-byte aligned base and a row
+ * count and leading dimension that are multiples of 8; AXON_ERR_SHAPE otherwise. */
+int axon_gemm_bf16(const void* a_bf16, int64_t lda, int a_kmajor, const void* b_bf16, int64_t ldb,
+                   int b_kmajor, float* out, int64_t ldo, int64_t m, int64_t n, int64_t k, void* stream);
 
 /* ------------------------------------------------------------------------- *
  * (b) ragged segmented reductions over cu_seqlens

@@ -89,8 +89,9 @@ def oracle_step(hid, w, labels, rl, old, ref, loss_name, args, dp_replicas=1, n_
 
 
 def fused_step(hid, w, ids, rl, old, ref, loss_name, args, block_tokens, dp_replicas=1, n_micro_batches=1,
-               vocab_chunk=0, extra=None, adv_shift=0.0):
-    from axon_amd.models.fused_head_loss import fused_head_loss
+               vocab_chunk=0, extra=None, adv_shift=0.0, dw_group=None):
+    from axon_amd.models.fused_head_loss import DEFAULT_DW_GROUP, fused_head_loss
+    dw_group = DEFAULT_DW_GROUP if dw_group is None else dw_group
     hd, wd = hid.to(DEV).requires_grad_(True), w.to(DEV).requires_grad_(True)
     cu = rl["cu_seqlens"].to(DEV)
     a_in = DataProto.from_dict(tensors={"token_level_rewards": rl["token_level_rewards"].to(DEV),
@@ -105,7 +106,7 @@ def fused_step(hid, w, ids, rl, old, ref, loss_name, args, block_tokens, dp_repl
     meta = {"loss_fn": loss_name, "loss_fn_args": args, "temperature": 1.0, "dp_replicas": dp_replicas,
             "n_micro_batches": n_micro_batches}
     loss, metrics = fused_head_loss(hd, wd, ids.to(DEV), cu, data, meta, block_tokens=block_tokens,
-                                    vocab_chunk=vocab_chunk)
+                                    vocab_chunk=vocab_chunk, dw_group=dw_group)
     loss.backward()
     return loss.detach(), metrics, data, hd.grad, wd.grad
 
@@ -149,6 +150,27 @@ def test_fused_step_vs_oracle(case, block_tokens, lens):
     keys += ["kl_loss", "kl_coef"] if "kl_coef" in args else []
     for k in keys:
         assert got[1][k] == pytest.approx(want[1][k], rel=1e-4, abs=1e-6), k
+
+
+@pytest.mark.parametrize("lens", [RAGGED, ODD_TOTAL], ids=["ragged", "odd-total"])
+@pytest.mark.parametrize("dw_group", [1, 2, 3, 8])
+@pytest.mark.parametrize("case", ["dapo-entropy-kl", "gspo-entropy-kl"])
+def test_fused_step_with_grouped_weight_gradient_vs_oracle(case, dw_group, lens):
+    """Hidden size 256 and a vocabulary that is a multiple of 8: the weight gradient reads the token-major
+    dlogits as a K-major GEMM operand (no vocab-major copy), and `dw_group` consecutive blocks share one such
+    GEMM (1: every block its own; 8: one GEMM for the step; 2 and 3: groups with a shorter last one, and with
+    blocks that are no multiple of 256 rows inside a group)."""
+    name, args = {"dapo-entropy-kl": ("ppo", DAPO_SIDE), "gspo-entropy-kl": ("gspo", GSPO_SIDE)}[case]
+    n, h, v = sum(lens), 256, 2000
+    hid, w, ids, labels, rl, old, ref = _inputs(n, h, v, lens, seed=73)
+    shift = GSPO_ADV_SHIFT if name == "gspo" else 0.0
+    want = oracle_step(hid, w, labels, rl, old, ref, name, args, adv_shift=shift)
+    got = fused_step(hid, w, ids, rl, old, ref, name, args, 256 if name == "ppo" else 512, adv_shift=shift,
+                     dw_group=dw_group)
+    data = got[2]
+    assert data.meta_info["head_backward"] == "blocked-stash" and data.meta_info["n_blocks"] >= 3
+    assert got[0].item() == pytest.approx(want[0].item(), rel=1e-4, abs=1e-8)
+    assert rel_l2(got[3], want[4]) < 2e-2 and rel_l2(got[4], want[5]) < 2e-2
 
 
 @pytest.mark.parametrize("vocab_chunk", [0, 1024])

@@ -49,6 +49,39 @@ def test_gemm_nt_vs_fp32_matmul(m, n, k):
     assert out.shape == (n, m) and rel_l2(out, ref) < 1e-5
 
 
+def _stored(x, kmajor, pad):
+    """The logical [rows][k] matrix `x` as the GEMM takes it: row-major, or K-major ([k][rows]), either with
+    `pad` unused elements at the end of every stored row."""
+    src = x.t() if kmajor else x
+    buf = torch.full((src.shape[0], src.shape[1] + pad), float("nan"), dtype=torch.bfloat16, device=DEV)
+    buf[:, : src.shape[1]] = src.to(DEV)
+    return buf[:, : src.shape[1]]
+
+
+@pytest.mark.parametrize("a_kmajor,b_kmajor", [(False, True), (True, False), (True, True)])
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (512, 768, 256), (520, 776, 320), (264, 1024, 128),
+                                   (4096, 1000, 192)])
+def test_gemm_with_k_major_operands_vs_fp32_matmul(m, n, k, a_kmajor, b_kmajor):
+    """Operands stored [k][rows] are read as they lie (LDS transpose reads): same result as the NT form, on whole
+    tiles, on edge tiles shifted back by a multiple of 8 rows, with padded leading dimensions."""
+    g = torch.Generator().manual_seed(3 * m + 5 * n + k)
+    a = torch.randn(m, k, generator=g).bfloat16()
+    b = torch.randn(n, k, generator=g).bfloat16()
+    out = _ops.gemm_layouts(_stored(a, a_kmajor, 72), _stored(b, b_kmajor, 8), a_kmajor, b_kmajor)
+    ref = b.float() @ a.float().t()
+    assert out.shape == (n, m) and rel_l2(out, ref) < 1e-5
+    assert torch.equal(out, _ops.gemm_nt(a.to(DEV), b.to(DEV)))  # the same products in the same order
+
+
+def test_gemm_with_k_major_operands_refuses_what_the_dma_loop_cannot_take():
+    a = torch.zeros(64, 260, dtype=torch.bfloat16, device=DEV)   # [k][m], m % 8 != 0
+    b = torch.zeros(256, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="axon_gemm_bf16"):
+        _ops.gemm_layouts(a[:, :260], b, True, False)
+    with pytest.raises(Exception, match="axon_gemm_bf16"):      # fewer than 256 rows: no DMA loop
+        _ops.gemm_layouts(torch.zeros(64, 128, dtype=torch.bfloat16, device=DEV), b, True, False)
+
+
 CASES = [  # n_tokens, hidden, vocab, temperature, label dtype
     (64, 128, 1000, 1.0, torch.int64),
     (300, 96, 777, 0.7, torch.int32),      # hidden % 64 != 0, ragged tiles everywhere
