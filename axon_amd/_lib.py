@@ -42,6 +42,7 @@ SIGNATURES: dict[str, tuple] = {
                                      _f32, _f32, _ptr, _i64, _ptr, _ptr, _ptr, _i32, _i32, _i64, _i32, _i64,
                                      _i64, _ptr, _i64, _ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_block_can_group": (_i32, [_i64, _i64, _i64]),
+    "axon_lmhead_bwd_dlogit_copies": (_i32, [_i64, _i64, _i64]),
     "axon_scale_bf16_unless_one": (_i32, [_ptr, _i64, _ptr, _ptr]),
     "axon_lmhead_active_rows": (_i32, [_ptr, _ptr, _ptr, _i64, _ptr, _ptr, _ptr, _ptr]),
     "axon_lmhead_gather_rows": (_i32, [_ptr, _ptr, _i32, _ptr, _ptr, _ptr, _ptr, _ptr, _i64, _i64, _ptr, _i64,

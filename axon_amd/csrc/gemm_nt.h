@@ -1,10 +1,14 @@
 // bf16 "NT" GEMM main loops for gfx950:  D[m][n] = sum_k A[m][k] * B[n][k]
 //
-// Both operands are K-contiguous, which is the layout the 16x16x32 bf16 MFMA
-// wants on both sides: every lane feeds eight consecutive k of one row.  The
-// LM-head forward, its logit recompute, dHidden and dWeight are all brought to
-// this one form (by pre-transposed copies where needed), so one main loop
-// serves the whole path; they differ only in the epilogue.
+// The 16x16x32 bf16 MFMA wants eight consecutive k of one row in every lane on
+// both sides.  K-contiguous operands ([row][k]) give that with one 16-byte LDS
+// read per fragment; the LM-head forward, its logit recompute and dHidden are
+// brought to this form (by pre-transposed copies of the weight and the hidden
+// states where needed).  An operand stored the other way round ([k][row],
+// "K-major": the dlogits in the dWeight product) is read as it lies with the LDS
+// transpose read of gfx950, two 8-byte reads per fragment, at the same speed
+// within a per cent.  One main loop serves the whole path; the kernels differ
+// only in the epilogue.
 //
 // Workgroup: 256 threads = 4 waves in a 2x2 grid, tile 256(m) x 256(n), each
 // wave 128 x 128 = 8x8 MFMA blocks of 16x16 (256 fp32 accumulators per lane,
@@ -14,7 +18,8 @@
 // TFLOP/s), which is worth more than the larger block's operand reuse.
 //
 // Two main loops:
-//  * DmaLoop  (the fast path; needs m_rows >= 256, n_rows >= 256, k % 64 == 0)
+//  * DmaLoopT<kAT, kBT>, DmaLoop = DmaLoopT<false, false>  (the fast path; needs
+//      m_rows >= 256, n_rows >= 256, k % 64 == 0; kAT / kBT: that side is K-major)
 //      global -> LDS by `buffer_load_dwordx4 ... lds` (no VGPR staging), 32 KB
 //      slots of 256 x 64 bf16 (three for A, two for B), 16-byte chunks
 //      XOR-swizzled by row; fragment reads for k-step kk+1 are issued under the

@@ -5,12 +5,15 @@
 //            epilogue folds each tile into per-token (max, sum exp, sum logit*exp)
 //            partials; a small kernel merges partials and adds the label logit.
 // Backward   per vocab chunk:
-//   B1  recompute the logits tile, form dlogit in registers, write it as bf16
-//       twice: dl[token][vocab] and dlT[vocab][token];
+//   B1  recompute the logits tile (or decode the forward's stash), form dlogit in
+//       registers, write it as bf16 dl[token][vocab];
 //   B2  dHidden[token][h] (+)= sum_v dl[token][v]  * WT[h][v]
-//   B3  dWeight[v][h]      =  sum_t dlT[v][t]      * hiddenT[h][t]
-// WT and hiddenT are bf16 transposes made once per call, so that all four GEMMs
-// run on the same K-contiguous main loops (gemm_nt.h).
+//   B3  dWeight[v][h]      =  sum_t dl[t][v]       * hiddenT[h][t]
+// WT and hiddenT are bf16 transposes made once per call: B2 runs on the
+// K-contiguous main loop of gemm_nt.h, B3 on its variant that reads dl, K-major
+// for this product, as it lies.  Shapes that variant does not take (hidden < 256,
+// a vocabulary that is no multiple of 8) get a second, vocab-major copy
+// dlT[vocab][token] from B1 and the K-contiguous loop.
 #include "common.h"
 #include "gemm_nt.h"
 #include <vector>
@@ -1597,6 +1600,11 @@ bool last_dst_ok(int64_t last_dst, int64_t n) { return last_dst <= n && last_dst
 extern "C" int64_t axon_lmhead_block_dw_acc_bytes(int64_t h, int64_t v) {
   if (check_head_shape(0, h, v) != AXON_OK) return -1;
   return (round_up(h, kTile) / kTile) * (round_up(v, kTile) / kTile) * kTileAccVecs * 16;
+}
+
+extern "C" int axon_lmhead_bwd_dlogit_copies(int64_t h, int64_t v, int64_t chunk) {
+  if (check_head_shape(0, h, v) != AXON_OK || chunk < 0 || chunk % kTile != 0) return -1;
+  return bwd_ws(kTile, h, v, chunk, nullptr).dl_kmajor ? 1 : 2;
 }
 
 extern "C" int axon_lmhead_block_can_group(int64_t h, int64_t v, int64_t chunk) {

@@ -619,19 +619,22 @@ def baseline_sizes_cold(dev):
     return out
 
 
-def kernel_table(timing, steps, n, h, v, stash_bytes):
+def kernel_table(timing, steps, n, h, v, stash_bytes, vocab_chunk=0):
     """Per kernel class of the head: launches and milliseconds per step (HIP events on the launch stream),
     algorithmic and executed TFLOP/s.  With the forward's stash the backward's first kernel is a streaming one:
-    per logit it reads 2 bytes of stash and writes the bf16 dlogit twice (token-major and vocab-major), and no
-    flop of the path is executed twice; without it that kernel recomputes the logits (2 N H V executed flop that
-    do not count as algorithmic)."""
+    per logit it reads 2 bytes of stash and writes the bf16 dlogit (once, token-major, where the weight-gradient
+    GEMM can read that K-major; else a vocab-major copy as well), and no flop of the path is executed twice;
+    without it that kernel recomputes the logits (2 N H V executed flop that do not count as algorithmic)."""
+    from axon_amd import _lib
+
     nhv = float(n) * h * v
+    copies = max(int(_lib.load().axon_lmhead_bwd_dlogit_copies(h, v, vocab_chunk)), 1)
     classes = [
         ("gemm_store_kernel (dHidden + dWeight GEMMs)", ("bwd/dhidden", "bwd/dweight"), 4 * nhv, 4 * nhv, 0.0),
         ("lmhead_fwd_stash_kernel (logits + online softmax statistics + stash)" if stash_bytes else
          "lmhead_fwd_kernel (logits + online softmax statistics)", ("fwd/logits_stats",), 2 * nhv, 2 * nhv, 0.0),
-        ("lmhead_dlogit_stash_kernel (stash -> dlogit in both orientations; HBM-bound)", ("bwd/dlogit",), 0.0, 0.0,
-         6.0 * n * v) if stash_bytes else
+        (f"lmhead_dlogit_stash_kernel (stash -> bf16 dlogit, {copies} cop{'y' if copies == 1 else 'ies'}; HBM-bound)",
+         ("bwd/dlogit",), 0.0, 0.0, (2.0 + 2.0 * copies) * n * v) if stash_bytes else
         ("lmhead_dlogit_kernel (logit recompute + dlogit)", ("bwd/dlogit",), 0.0, 2 * nhv, 0.0),
     ]
     kernels = []
@@ -832,6 +835,11 @@ def main():
 
     _ops.DEFAULT_VOCAB_CHUNK = args.vocab_chunk
     head_path = args.head_backward
+
+    def chunk_of(path):
+        """Vocabulary columns per backward chunk on a path: the blocks take the whole vocabulary unless told otherwise."""
+        return args.vocab_chunk or ((v + 255) // 256 * 256 if path == "blocked-stash" else 0)
+
     elapsed, timing, (loss, dh, dw) = run_path(head_path, args.steps, args.warmup)
     assert torch.isfinite(loss).item() and torch.isfinite(dh.float()).all().item()
     if head_path == "blocked-stash":
@@ -868,7 +876,7 @@ def main():
                 "path_frac_of_peak": 6 * nhv / (el / 3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                 "loss": loss_v.item(), "headline_loss": loss.item(),
                 "dhidden_rel_l2_vs_headline": rel(dh_v, dh), "dweight_rel_l2_vs_headline": rel(dw_v, dw),
-                "kernels": kernel_table(timing_v, 3, n, h, v, sb),
+                "kernels": kernel_table(timing_v, 3, n, h, v, sb, chunk_of(path)),
             }
             del loss_v, dh_v, dw_v
             torch.cuda.empty_cache()
@@ -902,7 +910,7 @@ def main():
 
     # kernel classes: (label, timing keys, algorithmic flops per step, executed flops per step)
     executed = 8 if head_path == "recompute" else 6
-    kernels = kernel_table(timing, args.steps, n, h, v, stash_bytes)
+    kernels = kernel_table(timing, args.steps, n, h, v, stash_bytes, chunk_of(head_path))
     dom = max(kernels, key=lambda k: k["ms_per_step"])
     roofline = {
         "bound": "mfma", "kernel": dom["kernel"], "achieved": dom["algorithmic_tflops"] or dom["executed_tflops"],

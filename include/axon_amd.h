@@ -238,6 +238,11 @@ int axon_lmhead_block_bwd(const float* dlogprobs, const float* dentropy, const v
                           int64_t vocab_chunk, void* workspace, int64_t workspace_bytes,
                           const void* stash, int64_t stash_bytes, void* stream, void* timer);
 int axon_lmhead_block_can_group(int64_t hidden, int64_t vocab, int64_t vocab_chunk);
+/* How many bf16 copies of a chunk's dlogits the backward (axon_lmhead_bwd, axon_lmhead_block_bwd) writes for
+ * this shape: 1 = token-major only (the weight-gradient GEMM reads it K-major), 2 = token-major and
+ * vocab-major (hidden < 256, vocab % 8 != 0, or a last vocabulary chunk of fewer than 256 rows).  For
+ * byte accounting; negative for an unsupported shape.  No reference counterpart. */
+int axon_lmhead_bwd_dlogit_copies(int64_t hidden, int64_t vocab, int64_t vocab_chunk);
 int axon_scale_bf16_unless_one(void* x_bf16, int64_t n, const float* scale, void* stream);
 
 /* Plain bf16 NT GEMM on the same MFMA main loop, out[n][m] = sum_k A[m][k]*B[n][k]
