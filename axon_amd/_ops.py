@@ -823,6 +823,22 @@ def lmhead_backward(dlogprobs, dentropy, hidden, weight, labels, lse, entropy_b,
 DW_STORE, DW_FIRST, DW_ADD, DW_LAST = 0, 1, 2, 3
 
 
+def head_block_groups(ranges, group):
+    """Where the blocks of a step keep their dlogits when ``group`` consecutive blocks share one weight-gradient
+    GEMM: per block ``(group index, first token of the block inside the group's workspace, is the group's last
+    block)``, then the number of groups and the tokens the workspace must hold.  Inside a group every block
+    begins on a multiple of 256 tokens (the blocks before it rounded up)."""
+    place = []
+    for k, (a, b) in enumerate(ranges):
+        pos = 0
+        if k % group:
+            pa, pb = ranges[k - 1]
+            pos = place[-1][1] + (pb - pa + 255) // 256 * 256
+        place.append((k // group, pos, k % group == group - 1 or k == len(ranges) - 1))
+    ws_tokens = max(pos + (b - a + 255) // 256 * 256 for (_, pos, _), (a, b) in zip(place, ranges))
+    return place, place[-1][0] + 1, ws_tokens
+
+
 class HeadBlocks:
     """One step of the head as blocks of consecutive tokens (``axon_lmhead_block_*``): forward of a block over
     the whole vocabulary with a stash, then (by the caller) the loss on the block's positions, then the block's
@@ -862,13 +878,7 @@ class HeadBlocks:
         if g > 1 and not self.lib.axon_lmhead_block_can_group(self.h, self.v, self.chunk):
             g = 1
         self.dw_group = g
-        self.place = []
-        for k, (a, b) in enumerate(self.ranges):
-            first = k % g == 0
-            pos = 0 if first else self.place[-1][1] + (self.ranges[k - 1][1] - self.ranges[k - 1][0] + 255) // 256 * 256
-            self.place.append((k // g, pos, k % g == g - 1 or k == len(self.ranges) - 1))
-        self.n_groups = self.place[-1][0] + 1
-        self.ws_tokens = max(pos + (b - a + 255) // 256 * 256 for (_, pos, _), (a, b) in zip(self.place, self.ranges))
+        self.place, self.n_groups, self.ws_tokens = head_block_groups(self.ranges, g)
         self.fwd_ws_bytes = self.lib.axon_lmhead_fwd_workspace_bytes(n_max, self.h, self.v)
         self.bwd_ws_bytes = self.lib.axon_lmhead_bwd_workspace_bytes(self.ws_tokens, self.h, self.v, self.chunk)
         if self.fwd_ws_bytes < 0 or self.bwd_ws_bytes < 0:

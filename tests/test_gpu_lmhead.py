@@ -88,6 +88,7 @@ CASES = [  # n_tokens, hidden, vocab, temperature, label dtype
     (257, 256, 2049, 1.3, torch.int64),
     (1, 32, 5, 1.0, torch.int32),
     (513, 2880, 1500, 1.0, torch.int32),   # GPT-OSS hidden size
+    (516, 256, 1504, 0.8, torch.int32),    # hidden >= 256, vocab % 8 == 0: the weight gradient reads the dlogits K-major
 ]
 
 
@@ -391,6 +392,13 @@ STASH_CASES = [
     (301, 96, 777, 512, 4.0, True),
     (64, 128, 1000, 0, 0.0, False),
     (1, 32, 5, 0, 0.0, False),
+    # hidden >= 256 and vocab % 8 == 0: the dlogits are written once and the weight gradient reads them K-major;
+    # chunks of 512 + 512 + 480 and 512 + 512 + 264 rows (edge tiles shifted back by 32 and 248 rows), one chunk,
+    # and a last chunk of 136 rows, which sends the whole call back to the two-copy path
+    (516, 256, 1504, 512, 0.0, False),
+    (772, 320, 1288, 512, 3.0, True),
+    (1100, 256, 2048, 0, 0.0, False),
+    (516, 256, 1160, 512, 0.0, False),
 ]
 
 

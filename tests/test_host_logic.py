@@ -291,6 +291,37 @@ def test_row_owning_dispatch_rule():
         _ops.OWNED_ROWS_MIN_MEAN_LEN = keep
 
 
+def test_which_shapes_write_the_dlogits_once_and_may_group_blocks():
+    """Host-side shape rules of the head's backward (no GPU call): the dlogits are written once when the
+    weight-gradient GEMM can read them K-major (hidden >= 256, vocab % 8 == 0, every chunk at least 256 rows),
+    twice otherwise; blocks may share a weight-gradient GEMM when, in addition, a block takes the whole vocabulary
+    in one chunk."""
+    from axon_amd import _lib
+    lib = _lib.load()
+    copies, group = lib.axon_lmhead_bwd_dlogit_copies, lib.axon_lmhead_block_can_group
+    assert copies(4096, 151936, 0) == 1 and copies(4096, 151936, 152064) == 1      # Qwen3-8B, chunks of 32768 / one
+    assert copies(2880, 201088, 0) == 1 and copies(896, 151936, 0) == 1            # GPT-OSS, Qwen2.5-0.5B
+    assert copies(256, 1504, 512) == 1 and copies(256, 1160, 512) == 2             # last chunk of 480 / 136 rows
+    assert copies(256, 1500, 512) == 2 and copies(192, 2048, 512) == 2             # vocab % 8, hidden < 256
+    assert copies(4096, 151936, 100) < 0 and copies(4097, 151936, 0) < 0           # chunk % 256, hidden % 32
+    assert group(4096, 151936, 152064) == 1 and group(4096, 151936, 0) == 0        # one chunk only
+    assert group(256, 2048, 0) == 1 and group(128, 2048, 0) == 0 and group(256, 2044, 0) == 0
+
+
+def test_blocks_that_share_a_weight_gradient_gemm_are_placed_on_tile_borders():
+    from axon_amd._ops import head_block_groups
+    four = [(0, 8192), (8192, 16384), (16384, 24576), (24576, 32768)]
+    assert head_block_groups(four, 1) == ([(0, 0, True), (1, 0, True), (2, 0, True), (3, 0, True)], 4, 8192)
+    assert head_block_groups(four, 2) == ([(0, 0, False), (0, 8192, True), (1, 0, False), (1, 8192, True)], 2, 16384)
+    assert head_block_groups(four, 8) == ([(0, 0, False), (0, 8192, False), (0, 16384, False), (0, 24576, True)], 1,
+                                          32768)
+    # ragged blocks (sequence cuts, lengthened to a multiple of four rows): rounded up to 256 inside a group
+    ragged = [(0, 436), (433, 936), (933, 1500)]
+    assert head_block_groups(ragged, 2) == ([(0, 0, False), (0, 512, True), (1, 0, True)], 2, 1024)
+    assert head_block_groups(ragged, 3) == ([(0, 0, False), (0, 512, False), (0, 1024, True)], 1, 1792)
+    assert head_block_groups([(0, 100)], 2) == ([(0, 0, True)], 1, 256)
+
+
 def test_fused_step_block_plans():
     from axon_amd.models.fused_head_loss import sequence_blocks, token_blocks
     assert token_blocks(32768, 8192) == [(0, 8192), (8192, 16384), (16384, 24576), (24576, 32768)]
