@@ -137,8 +137,13 @@ struct DmaSide {
 
   __device__ static __forceinline__ int variant(int j) { return T ? (j & 1) + 2 * (j >> 2) : (j & 1); }
 
-  // `row0`: first tile row (m0 or n0); `sub`: which half of the tile the wave computes (wm or wn)
-  __device__ __forceinline__ void init(const __bf16* p, int64_t ld, int row0, int sub, const LanePos& lp) {
+  // `row0`: first tile row (m0 or n0); `sub`: which half of the tile the wave computes (wm or wn);
+  // `lds_base`: where the operand's first slot begins.  It is part of the per-lane fragment offsets so that
+  // what is left to add per read (the slot: a scalar; block, k-step, half: constants) fits the 16-bit offset
+  // field of the LDS instructions: a constant beyond it costs a vector addition right before the read that
+  // needs its result, and every such pair delays the MFMA behind it.
+  __device__ __forceinline__ void init(const __bf16* p, int64_t ld, int row0, int sub, const LanePos& lp,
+                                       int lds_base) {
     if (!T) {
       // One DMA instruction fills 1 KB of LDS = 8 rows x 128 B; wave w owns rows [64w, 64w+64) of the
       // operand (8 instructions).  Lane i lands on row i/8, chunk slot i%8, and therefore fetches
@@ -157,7 +162,7 @@ struct DmaSide {
       const int sw = (lp.l16 >> 1) & 7;
 #pragma unroll
       for (int kk = 0; kk < 2; ++kk)
-        frag[kk] = (sub * kWaveTile + lp.l16) * 128 + (((kk * 4 + lp.lq) ^ sw) << 4);
+        frag[kk] = lds_base + (sub * kWaveTile + lp.l16) * 128 + (((kk * 4 + lp.lq) ^ sw) << 4);
     } else {
       // One DMA instruction fills 1 KB of LDS = 2 k-rows x 512 B; wave w owns k-rows [16w, 16w+16) of
       // the k-tile (8 instructions).  Lane i lands on k-row 2j + i/32, 16-byte granule i%32, and fetches
@@ -178,7 +183,7 @@ struct DmaSide {
       const int fb = (8 * lp.lq + (lp.l16 >> 2)) * 512 + (((16 * sub) ^ (16 * (lp.lq >> 1))) << 4) +
                      8 * (lp.l16 & 1) + (((lp.l16 & 3) >> 1) << 4);
 #pragma unroll
-      for (int i = 0; i < kBlocks; ++i) frag[i] = fb + ((i << 5) ^ (s15 << 4));
+      for (int i = 0; i < kBlocks; ++i) frag[i] = lds_base + fb + ((i << 5) ^ (s15 << 4));
     }
   }
   // source byte offset of k-tile kt; past the end: refetches the last tile, never consumed
@@ -239,9 +244,9 @@ struct DmaLoopT {
   // therefore does not count these reads either: the loop waits for them itself (lgkmcnt(0) before the
   // barrier and before the first MFMA of a k-tile), and the values are used by the MFMAs only.
   // `imm`: a constant once the loops around the call are unrolled (the instruction's offset field)
-  __device__ static __forceinline__ i16x4 read_tr(const char* lds, int imm) {
+  // `a`: LDS byte address
+  __device__ static __forceinline__ i16x4 read_tr(uint32_t a, int imm) {
     i16x4 v;
-    const uint32_t a = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)lds;
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(a), "i"(imm));
     return v;
   }
@@ -258,8 +263,8 @@ struct DmaLoopT {
     const LanePos lp;
     DmaSide<kAT> sa;
     DmaSide<kBT> sb;
-    sa.init(g.a, g.lda, t.m0, lp.wm, lp);
-    sb.init(g.b, g.ldb, t.n0, lp.wn, lp);
+    sa.init(g.a, g.lda, t.m0, lp.wm, lp, 0);
+    sb.init(g.b, g.ldb, t.n0, lp.wn, lp, kBBase);
     // wave-uniform, so the LDS destination of every DMA instruction is scalar arithmetic into M0
     char* const dst = smem + __builtin_amdgcn_readfirstlane(lp.wave) * 8192;
 
@@ -274,27 +279,45 @@ struct DmaLoopT {
     auto dma_b = [&](int slot_off, const __amdgpu_buffer_rsrc_t& r, int j) {
       dma_kb(r, sb.vo[DmaSide<kBT>::variant(j)], sb.step, dst + kBBase + slot_off, j);
     };
-    // read `half` of fragment `blk` of k-step kk from the slot at byte offset `slot` into set `set`
-    auto read_a = [&](int slot, int kk, int set, int blk, int half) {
-      if (kAT) aft[set][blk][half] = read_tr(smem + slot + sa.frag[blk], kk * 16384 + half * 2048);
-      else af[set][blk] = *reinterpret_cast<const bf16x8*>(smem + slot + sa.frag[kk] + blk * kBlk * kRowBytes);
+    // LDS addresses of the fragments in the slots being read: slot + per-lane offset, formed well before the
+    // reads that use them (a vector addition right before the read that needs its result delays the MFMA
+    // behind the pair; sixteen such pairs per k-tile cost 3-4 % of the loop).  The reads under a tile's second
+    // k-step (k-step 0 of the next tile) and under the next tile's first k-step (its k-step 1) go to the same
+    // slots, so the addresses change once per k-tile: after the last read of a tile's first k-step.
+    constexpr int kAddrA = DmaSide<kAT>::kFrag, kAddrB = DmaSide<kBT>::kFrag;
+    // room for the additions behind the reads of a k-step (not with both operands K-major, whose reads fill it:
+    // that form, which no kernel of the library uses, forms them in one piece after the barrier)
+    constexpr bool kLateAdr = 2 * kBlocks * (kReadsA + kReadsB) + kAddrA + kAddrB <= kBlocks * kBlocks;
+    typedef __attribute__((address_space(3))) const char* LdsPtr;
+    const uint32_t smem_lds = (uint32_t)(uintptr_t)(LdsPtr)smem;
+    uint32_t adr_a[kAddrA], adr_b[kAddrB];
+    auto set_adr_a = [&](int q, int slot) { adr_a[q] = smem_lds + slot + sa.frag[q]; };
+    auto set_adr_b = [&](int q, int slot) { adr_b[q] = smem_lds + slot + sb.frag[q]; };
+    // read `half` of fragment `blk` of k-step kk from the slots the addresses were formed for into set `set`
+    auto read_a = [&](int kk, int set, int blk, int half) {
+      if (kAT) aft[set][blk][half] = read_tr(adr_a[blk], kk * 16384 + half * 2048);
+      else af[set][blk] = *(const __attribute__((address_space(3))) bf16x8*)(LdsPtr)(uintptr_t)(adr_a[kk] + blk * kBlk * kRowBytes);
     };
-    auto read_b = [&](int slot, int kk, int set, int blk, int half) {
-      if (kBT) bft[set][blk][half] = read_tr(smem + kBBase + slot + sb.frag[blk], kk * 16384 + half * 2048);
-      else bf[set][blk] = *reinterpret_cast<const bf16x8*>(smem + kBBase + slot + sb.frag[kk] + blk * kBlk * kRowBytes);
+    auto read_b = [&](int kk, int set, int blk, int half) {
+      if (kBT) bft[set][blk][half] = read_tr(adr_b[blk], kk * 16384 + half * 2048);
+      else bf[set][blk] = *(const __attribute__((address_space(3))) bf16x8*)(LdsPtr)(uintptr_t)(adr_b[kk] + blk * kBlk * kRowBytes);
     };
     // One k-step of 32: 64 MFMAs on fragment set mm_set.  The sixteen fragments of the next k-step
-    // (k-step rd_kk of the slots rd_a / rd_b) are read under the first part of the step, one read per two
-    // MFMAs (A block 0, then the eight B blocks, then A blocks 1..7), into the other set, so that they
+    // (k-step rd_kk of the slots the addresses stand for) are read under the first part of the step, one read
+    // per two MFMAs (A block 0, then the eight B blocks, then A blocks 1..7), into the other set, so that they
     // have landed long before the barrier's wait; NA A-operand or NB B-operand DMA instructions are
-    // issued one per eight MFMAs, in slots that carry no fragment read.  The scheduling fence after
+    // issued one per eight MFMAs, in slots that carry no fragment read.  With `adr_c` the addresses for the
+    // slots nxt_a / nxt_b are formed after the step's last read, one per MFMA.  The scheduling fence after
     // every MFMA keeps the source order: the compiler treats an LDS DMA and an LDS read as aliasing
     // accesses and would otherwise bunch them.
-    auto step = [&](int rd_a, int rd_b, int rd_kk, int mm_set, int a_slot, auto na_c, int b_slot,
-                    auto nb_c, const __amdgpu_buffer_rsrc_t& rsrc, auto&& mid) {
+    auto step = [&](int rd_kk, int mm_set, int a_slot, auto na_c, int b_slot, auto nb_c,
+                    const __amdgpu_buffer_rsrc_t& rsrc, auto&& mid, auto adr_c, int nxt_a, int nxt_b) {
       constexpr int NA = decltype(na_c)::value, NB = decltype(nb_c)::value;
+      constexpr bool kAdr = decltype(adr_c)::value != 0;
       static_assert((NA == 0 || NA == 8) && (NB == 0 || NB == 8) && NA + NB <= 8, "");
       constexpr int RA = kReadsA, RB = kReadsB;
+      constexpr int kFirstAdr = 2 * kBlocks * (RA + RB);  // the MFMA after the last read
+      static_assert(!kAdr || kLateAdr, "");
       const int rd_set = mm_set ^ 1;
 #pragma unroll
       for (int i = 0; i < kBlocks; ++i) {
@@ -308,11 +331,14 @@ struct DmaLoopT {
           }
           if ((m & 1) == 0) {
             const int s = m >> 1;
-            if (s < RA) read_a(rd_a, rd_kk, rd_set, 0, s);
-            else if (s < RA + kBlocks * RB) read_b(rd_b, rd_kk, rd_set, (s - RA) / RB, (s - RA) % RB);
+            if (s < RA) read_a(rd_kk, rd_set, 0, s);
+            else if (s < RA + kBlocks * RB) read_b(rd_kk, rd_set, (s - RA) / RB, (s - RA) % RB);
             else if (s < kBlocks * (RA + RB))
-              read_a(rd_a, rd_kk, rd_set, 1 + (s - RA - kBlocks * RB) / RA, (s - RA - kBlocks * RB) % RA);
+              read_a(rd_kk, rd_set, 1 + (s - RA - kBlocks * RB) / RA, (s - RA - kBlocks * RB) % RA);
           }
+          if (kAdr && m >= kFirstAdr && m < kFirstAdr + kAddrA) set_adr_a(m - kFirstAdr, nxt_a);
+          if (kAdr && m >= kFirstAdr + kAddrA && m < kFirstAdr + kAddrA + kAddrB)
+            set_adr_b(m - kFirstAdr - kAddrA, nxt_b);
           mfma_16x16x32(acc[i][j], kAT ? join(aft[mm_set][i][0], aft[mm_set][i][1]) : af[mm_set][i],
                         kBT ? join(bft[mm_set][j][0], bft[mm_set][j][1]) : bf[mm_set][j]);
           __builtin_amdgcn_sched_barrier(0);
@@ -338,11 +364,15 @@ struct DmaLoopT {
     __builtin_amdgcn_s_waitcnt(0x4F70);  // vmcnt(16): tile 0 has landed
     __builtin_amdgcn_s_barrier();
 #pragma unroll
+    for (int q = 0; q < kAddrA; ++q) set_adr_a(q, 0);
+#pragma unroll
+    for (int q = 0; q < kAddrB; ++q) set_adr_b(q, 0);
+#pragma unroll
     for (int i = 0; i < kBlocks; ++i) {
 #pragma unroll
-      for (int h = 0; h < kReadsA; ++h) read_a(0, 0, 0, i, h);
+      for (int h = 0; h < kReadsA; ++h) read_a(0, 0, i, h);
 #pragma unroll
-      for (int h = 0; h < kReadsB; ++h) read_b(0, 0, 0, i, h);
+      for (int h = 0; h < kReadsB; ++h) read_b(0, 0, i, h);
     }
     __builtin_amdgcn_sched_barrier(0);
     wait_lds_reads();
@@ -368,14 +398,21 @@ struct DmaLoopT {
     Tile tv = tile_vars(0, 0, 0);
     for (int kt = 0; kt < kt_n; ++kt) {
       Tile nx;
-      // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read
-      step(tv.a_cur, tv.b_cur, 1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [] {});
+      // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read (the addresses stand
+      // for this tile's slots), then the addresses move on to the next tile's slots
+      step(1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [] {}, std::integral_constant<int, kLateAdr ? 1 : 0>{}, tv.a_nxt,
+           tv.b_nxt);
       // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
-      step(tv.a_nxt, tv.b_nxt, 0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb,
-           [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); });
+      if (!kLateAdr) {
+#pragma unroll
+        for (int q = 0; q < kAddrA; ++q) set_adr_a(q, tv.a_nxt);
+#pragma unroll
+        for (int q = 0; q < kAddrB; ++q) set_adr_b(q, tv.b_nxt);
+      }
+      step(0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb, [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); }, I0{}, 0, 0);
       tv = nx;
       wait_lds_reads();  // the next tile's first fragments, read under the second k-step
     }
