@@ -250,10 +250,10 @@ struct DmaLoopT {
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(a), "i"(imm));
     return v;
   }
-  // lgkmcnt(0) alone (vmcnt and expcnt at their maxima)
-  __device__ static __forceinline__ void wait_lds_reads() {
-    if (kAT || kBT) __builtin_amdgcn_s_waitcnt(0xC07F);
-  }
+  // lgkmcnt(0) alone (vmcnt and expcnt at their maxima).  For every form of the loop: left to the compiler,
+  // the wait for the fragments read under a tile's second k-step comes out BEHIND the next tile's first read
+  // and waits for that one as well, a full LDS latency per k-tile.
+  __device__ static __forceinline__ void wait_lds_reads() { __builtin_amdgcn_s_waitcnt(0xC07F); }
   __device__ static __forceinline__ bf16x8 join(const i16x4& lo, const i16x4& hi) {
     return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
   }
@@ -324,7 +324,10 @@ struct DmaLoopT {
 #pragma unroll
         for (int j = 0; j < kBlocks; ++j) {
           const int m = i * kBlocks + j;
-          if (m == 37) mid();  // index arithmetic for the coming k-tile, in a slot without other work
+          // index arithmetic for the coming k-tile in three pieces, in slots without other work
+          if (m == 37) mid(std::integral_constant<int, 0>{});
+          if (m == 45) mid(std::integral_constant<int, 1>{});
+          if (m == 53) mid(std::integral_constant<int, 2>{});
           if ((m & 7) == 3) {
             if (NB) dma_b(b_slot, rsrc, m >> 3);
             if (NA) dma_a(a_slot, rsrc, m >> 3);
@@ -384,24 +387,23 @@ struct DmaLoopT {
       int a_cur, a_nxt, a_fill, b_cur, b_nxt;
       __amdgpu_buffer_rsrc_t ra, rb;
     };
-    auto tile_vars = [&](int a_cur, int b_cur, int kt) {
-      Tile v;
+    auto tile_slots = [&](Tile& v, int a_cur, int b_cur) {
       v.a_cur = a_cur;
       v.b_cur = b_cur;
       v.a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
       v.a_fill = (v.a_nxt == 2 * kOperandBytes) ? 0 : v.a_nxt + kOperandBytes;  // freed one barrier ago
       v.b_nxt = b_cur ^ kOperandBytes;
-      v.ra = sa.rsrc_at(sa.k_off(kt + 2, kt_n));
-      v.rb = sb.rsrc_at(sb.k_off(kt + 2, kt_n));
-      return v;
     };
-    Tile tv = tile_vars(0, 0, 0);
+    Tile tv;
+    tile_slots(tv, 0, 0);
+    tv.ra = sa.rsrc_at(sa.k_off(2, kt_n));
+    tv.rb = sb.rsrc_at(sb.k_off(2, kt_n));
     for (int kt = 0; kt < kt_n; ++kt) {
       Tile nx;
       // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read (the addresses stand
       // for this tile's slots), then the addresses move on to the next tile's slots
-      step(1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [] {}, std::integral_constant<int, kLateAdr ? 1 : 0>{}, tv.a_nxt,
-           tv.b_nxt);
+      step(1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [](auto) {}, std::integral_constant<int, kLateAdr ? 1 : 0>{},
+           tv.a_nxt, tv.b_nxt);
       // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
@@ -412,7 +414,13 @@ struct DmaLoopT {
 #pragma unroll
         for (int q = 0; q < kAddrB; ++q) set_adr_b(q, tv.b_nxt);
       }
-      step(0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb, [&] { nx = tile_vars(tv.a_nxt, tv.b_nxt, kt + 1); }, I0{}, 0, 0);
+      step(0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb,
+           [&](auto part) {
+             if (decltype(part)::value == 0) tile_slots(nx, tv.a_nxt, tv.b_nxt);
+             if (decltype(part)::value == 1) nx.ra = sa.rsrc_at(sa.k_off(kt + 3, kt_n));
+             if (decltype(part)::value == 2) nx.rb = sb.rsrc_at(sb.k_off(kt + 3, kt_n));
+           },
+           I0{}, 0, 0);
       tv = nx;
       wait_lds_reads();  // the next tile's first fragments, read under the second k-step
     }

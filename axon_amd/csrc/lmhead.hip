@@ -1013,6 +1013,10 @@ struct BwdWs {
   // The dWeight GEMM reads dl [token][vocab] as it lies, as its K-major operand: no vocab-major copy
   // (dlT is null).  Needs the DMA loop for every chunk's GEMM and 16-byte vectors along the vocabulary.
   bool dl_kmajor;
+  // The dHidden GEMM reads the weight [vocab][hidden] as it lies, as its K-major operand: no transposed
+  // copy (wT is null).  Needs the DMA loop (fewer than 256 tokens are padded to 256 with zero dlogit rows)
+  // and a reduction that ends with the weight's last row (vocab % 64 == 0).
+  bool w_kmajor;
 };
 // Rows a power of two apart land on the same L2 sets and memory channels; 128 bytes of padding
 // per row moves consecutive rows to consecutive cache lines (+5..13 % on a stand-alone GEMM with
@@ -1032,9 +1036,14 @@ BwdWs bwd_ws(int64_t n, int64_t h, int64_t vocab, int64_t chunk, void* base) {
   w.ld_c = w.chunk + kLdPad;
   const int64_t last_rows = vocab - (int64_t)(w.chunks - 1) * w.chunk;
   w.dl_kmajor = h >= kTile && last_rows >= kTile && vocab % 8 == 0 && w.ld_n < (1 << 21) && w.ld_c < (1 << 21);
+  w.w_kmajor = h >= kTile && vocab % 64 == 0 && h < (1 << 21) && w.ld_c < (1 << 21);
   char* p = static_cast<char*>(base);
   int64_t off = 0;
-  w.wT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.ld_v * 2, kAlign);
+  w.wT = nullptr;
+  if (!w.w_kmajor) {
+    w.wT = reinterpret_cast<__bf16*>(p + off);
+    off += round_up(h * w.ld_v * 2, kAlign);
+  }
   w.hT = reinterpret_cast<__bf16*>(p + off);  off += round_up(h * w.ld_n * 2, kAlign);
   w.dl = reinterpret_cast<__bf16*>(p + off);  off += round_up(w.n_pad * w.ld_c * 2, kAlign);
   w.dlT = nullptr;
@@ -1288,7 +1297,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
   // K-contiguous copies for the two output GEMMs
   {
     Span span(timer, 0);
-    if (!blk.wt_ready) {
+    if (!blk.wt_ready && !w.w_kmajor) {
       rc = launch_transpose(weight, h, (int)v, (int)h, w.wT, w.ld_v, (int)w.v_pad, st);
       if (rc != AXON_OK) return rc;
     }
@@ -1335,18 +1344,24 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       // clamped path writes zeros there already, the extra fill is then redundant but harmless)
       rc = launch_zero_cols(dl, w.ld_c, (int)n, (int)vc, (int)(vc_red - vc), st);
       if (rc != AXON_OK) return rc;
-      if (w.dl_kmajor)  // the token rows up to the next tile boundary: reduction padding of B3
+      // the token rows up to the next tile boundary: reduction padding of B3 when it reads dl K-major, and
+      // rows of B2's operand when fewer than 256 tokens run on the DMA loop
+      if (w.dl_kmajor || (w.w_kmajor && n < kTile))
         rc = launch_zero_cols(dl + n * w.ld_c, w.ld_c, (int)(n_tile - n), 0, (int)vc_red, st);
-      else
+      if (rc == AXON_OK && !w.dl_kmajor)
         rc = launch_zero_cols(w.dlT, w.ld_n, (int)vc, (int)n, (int)(n_red - n), st);
       if (rc != AXON_OK) return rc;
     }
-    // B2: dHidden[n][h] (+)= sum_v dl[n][v] * wT[h][v0 + v]
+    // B2: dHidden[n][h] (+)= sum_v dl[n][v] * W[v0 + v][h]  (the weight read K-major where it lies, or its
+    // transposed copy wT[h][v0 + v])
     {
       Span span(timer, 2);
       GemmOperands g;
-      g.a = w.wT + v0;  g.lda = w.ld_v;  g.m_rows = (int)h;
-      g.b = dl;         g.ldb = w.ld_c;  g.n_rows = (int)n;
+      if (w.w_kmajor) { g.a = static_cast<const __bf16*>(weight) + v0 * h;  g.lda = h; }
+      else            { g.a = w.wT + v0;                                     g.lda = w.ld_v; }
+      g.m_rows = (int)h;
+      // fewer than 256 tokens: the zero rows up to 256 are part of the operand, the stores stop at n
+      g.b = dl;  g.ldb = w.ld_c;  g.n_rows = (int)((w.w_kmajor && n < kTile) ? kTile : n);
       g.k = (int)vc_red;
       StoreParams sp;
       const bool last = (ci == w.chunks - 1);
@@ -1354,7 +1369,7 @@ int bwd_impl(const float* dlogprobs, const float* dentropy, const void* hidden, 
       sp.out_bf16 = last ? static_cast<__bf16*>(d_hidden) : nullptr;  sp.ld_bf16 = h;
       sp.m_valid = (int)h; sp.n_valid = (int)n; sp.accumulate = (ci > 0); sp.keep_f32 = 1;
       sp.tile_acc = nullptr;
-      rc = launch_store(g, sp, st);
+      rc = launch_store_kmajor(g, sp, w.w_kmajor, false, st);
       if (rc != AXON_OK) return rc;
     }
     // B3: dWeight[v0 + v][h] = sum_t dl[t][v] * hT[h][t] over the tokens the workspace holds up to this
@@ -1623,6 +1638,7 @@ extern "C" int axon_lmhead_block_begin(const void* weight, int64_t h, int64_t v,
   if (rc != AXON_OK) return rc;
   char* base = reinterpret_cast<char*>(round_up(reinterpret_cast<int64_t>(workspace), kAlign));
   const BwdWs w = bwd_ws(0, h, v, chunk, base);
+  if (w.w_kmajor) return AXON_OK;  // the dHidden GEMM reads the weight where it lies
   if ((base - static_cast<char*>(workspace)) + round_up(h * w.ld_v * 2, kAlign) > ws_bytes)
     return AXON_ERR_WORKSPACE;
   Span span(t, 0);

@@ -89,6 +89,8 @@ CASES = [  # n_tokens, hidden, vocab, temperature, label dtype
     (1, 32, 5, 1.0, torch.int32),
     (513, 2880, 1500, 1.0, torch.int32),   # GPT-OSS hidden size
     (516, 256, 1504, 0.8, torch.int32),    # hidden >= 256, vocab % 8 == 0: the weight gradient reads the dlogits K-major
+    (130, 256, 1024, 1.2, torch.int64),    # vocab % 64 == 0: dHidden reads the weight K-major; fewer than 256 tokens
+    (700, 320, 1280, 1.0, torch.int32),    # both, ragged token tiles
 ]
 
 
@@ -399,6 +401,11 @@ STASH_CASES = [
     (772, 320, 1288, 512, 3.0, True),
     (1100, 256, 2048, 0, 0.0, False),
     (516, 256, 1160, 512, 0.0, False),
+    # vocab % 64 == 0 as well: no transposed copy of the weight either (dHidden reads it K-major); fewer than 256
+    # tokens run that GEMM on 256 rows of which the last are zero
+    (100, 256, 1024, 512, 0.0, False),
+    (200, 512, 1280, 0, 2.0, True),
+    (772, 256, 1536, 512, 0.0, True),
 ]
 
 

@@ -305,6 +305,9 @@ def test_which_shapes_write_the_dlogits_once_and_may_group_blocks():
     assert copies(256, 1500, 512) == 2 and copies(192, 2048, 512) == 2             # vocab % 8, hidden < 256
     assert copies(4096, 151936, 100) < 0 and copies(4097, 151936, 0) < 0           # chunk % 256, hidden % 32
     assert group(4096, 151936, 152064) == 1 and group(4096, 151936, 0) == 0        # one chunk only
+    # with vocab % 64 == 0 the workspace holds no transposed weight either: hidden x (vocab + 64) x 2 bytes less
+    ws = lib.axon_lmhead_bwd_workspace_bytes
+    assert ws(8192, 256, 2048 + 8, 2304) - ws(8192, 256, 2048, 2048) > 256 * 2048 * 2
     assert group(256, 2048, 0) == 1 and group(128, 2048, 0) == 0 and group(256, 2044, 0) == 0
 
 
