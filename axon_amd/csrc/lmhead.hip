@@ -92,6 +92,23 @@ __device__ __forceinline__ void merge_stats(float M, float& s, float& e, float M
   s = s * f1 + s2 * f2;
 }
 
+// All-reduce over the four 16-lane rows of the wavefront (lanes l, l^16, l^32, l^48: the four lanes that hold
+// the same token), the result in every lane: v_permlane16_swap / v_permlane32_swap hand a lane its
+// neighbour row's value and its own in one vector instruction each, where a shuffle would take two trips
+// through the LDS crossbar with a wait behind each.  The same pairs in the same order as the xor-16, xor-32
+// butterfly, so sums come out bit for bit the same.
+// Written as instructions: through the builtins the compiler takes the two results of a swap for one
+// value and folds op(a, b) to op(a, a).  The s_nop covers the wait states the swaps need after a
+// vector instruction has written their operands.
+template <class Op>
+__device__ __forceinline__ float rows_all_reduce(float v, Op op) {
+  float a = v, b = v;
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));  // a: rows 0 0 2 2, b: rows 1 1 3 3
+  float c = op(a, b), d = c;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(c), "+v"(d));  // c: rows 01 01 01 01, d: 23 23 23 23
+  return op(c, d);
+}
+
 // Fold one 256x256 logits tile into per-token partials.  MASKED: some rows of the tile
 // do not count (beyond the vocabulary, or duplicates of the neighbouring tile); they are
 // excluded by predicate — their accumulators hold finite values.  STASH: also store every
@@ -112,8 +129,7 @@ __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, c
         mx = ok ? fmaxf(mx, acc[i][j][r]) : mx;
       }
     // the four lanes that hold the same token (lane ^ 16, lane ^ 32) share one reference
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = rows_all_reduce(mx, [](float a, float b) { return fmaxf(a, b); });
     const float M = (MASKED && mx == -INFINITY) ? kEmptyMax : mx * p.c;
     float s = 0.f, e = 0.f;
     uint32_t hw[kBlocks][2];
@@ -143,11 +159,8 @@ __device__ __forceinline__ void fwd_epilogue(AccTile& acc, const FwdParams& p, c
         __builtin_nontemporal_store(x, reinterpret_cast<u32x4*>(stash_wave + (j * 4 + ip) * 64));
       }
     }
-#pragma unroll
-    for (int off = 16; off <= 32; off <<= 1) {
-      s += __shfl_xor(s, off, 64);
-      e += __shfl_xor(e, off, 64);
-    }
+    s = rows_all_reduce(s, [](float a, float b) { return a + b; });
+    e = rows_all_reduce(e, [](float a, float b) { return a + b; });
     const int nr = lp.n(j);
     const int n = t.n0 + nr;
     if (lp.lq == 0 && nr >= t.n_lo && n < p.n_tokens) {
