@@ -206,7 +206,9 @@ int axon_lmhead_bwd_timed(const float* dlogprobs, const float* dentropy, const v
  *        of the whole arrays, a sequence start).  0 is the whole-stream call, as axon_lmhead_fwd.
  *   axon_lmhead_block_begin: once per step, before the first backward: the transposed weight into
  *        `workspace` (the same workspace, of axon_lmhead_bwd_workspace_bytes(largest block, ...) bytes,
- *        must then be handed to every axon_lmhead_block_bwd of the step, with wt_ready = 1).
+ *        must then be handed to every axon_lmhead_block_bwd of the step, with wt_ready = 1).  For
+ *        hidden >= 256 and vocab % 64 == 0 the backward reads the weight where it lies: the call then
+ *        launches nothing and the workspace holds no transposed weight.
  *   axon_lmhead_block_bwd: d_hidden rows of the block (bf16, complete: a row sums over the vocabulary
  *        only).  The weight gradient sums over all blocks: dw_mode 0 = this block is the whole step,
  *        d_weight (bf16) is written; 1 = first block, dw_acc (fp32 partial sums,
