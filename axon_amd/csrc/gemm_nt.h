@@ -324,10 +324,14 @@ struct DmaLoopT {
 #pragma unroll
         for (int j = 0; j < kBlocks; ++j) {
           const int m = i * kBlocks + j;
-          // index arithmetic for the coming k-tile in three pieces, in slots without other work
+          // scalar bookkeeping for the coming k-tile, in pieces of at most four instructions, in slots without
+          // other work (a wavefront issues in order: a dozen scalar instructions in one MFMA gap hold up the
+          // MFMA behind them); pieces 3 and 4 come behind the step's last DMA instruction
           if (m == 37) mid(std::integral_constant<int, 0>{});
-          if (m == 45) mid(std::integral_constant<int, 1>{});
-          if (m == 53) mid(std::integral_constant<int, 2>{});
+          if (m == 39) mid(std::integral_constant<int, 1>{});
+          if (m == 41) mid(std::integral_constant<int, 2>{});
+          if (m == 61) mid(std::integral_constant<int, 3>{});
+          if (m == 63) mid(std::integral_constant<int, 4>{});
           if ((m & 7) == 3) {
             if (NB) dma_b(b_slot, rsrc, m >> 3);
             if (NA) dma_a(a_slot, rsrc, m >> 3);
@@ -380,48 +384,45 @@ struct DmaLoopT {
     __builtin_amdgcn_sched_barrier(0);
     wait_lds_reads();
 
-    // per-tile scalars: slots of the tile being consumed (cur), of the next one (nxt), the A slot
-    // being filled, and the buffer descriptors of k-tile kt+2; those of the following tile are
-    // computed under the second k-step so that the loop's back edge carries no arithmetic
-    struct Tile {
-      int a_cur, a_nxt, a_fill, b_cur, b_nxt;
-      __amdgpu_buffer_rsrc_t ra, rb;
+    // per-tile scalars: the slots of the tile being consumed (cur; the next tile's B slot is the other one),
+    // of the next one (nxt), the A slot being filled, and where k-tile kt+2 of either operand begins in
+    // memory.  Each is moved on to the next k-tile in place, under the second k-step, as soon as its value for
+    // this tile has been used for the last time (`pin` keeps the compiler from gathering the arithmetic at the
+    // loop's back edge), so that the back edge carries the counter and the branch only.
+    auto next_a_slot = [](int slot) { return (slot == 2 * kOperandBytes) ? 0 : slot + kOperandBytes; };
+    auto pin = [](auto& x) { asm volatile("" : "+s"(x)); };
+    int a_nxt = kOperandBytes, a_fill = 2 * kOperandBytes, b_cur = 0;
+    const char* pa = reinterpret_cast<const char*>(sa.base) + sa.k_off(2, kt_n);
+    const char* pb = reinterpret_cast<const char*>(sb.base) + sb.k_off(2, kt_n);
+    auto rsrc_of = [](const char* p) {
+      return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
     };
-    auto tile_slots = [&](Tile& v, int a_cur, int b_cur) {
-      v.a_cur = a_cur;
-      v.b_cur = b_cur;
-      v.a_nxt = (a_cur == 2 * kOperandBytes) ? 0 : a_cur + kOperandBytes;
-      v.a_fill = (v.a_nxt == 2 * kOperandBytes) ? 0 : v.a_nxt + kOperandBytes;  // freed one barrier ago
-      v.b_nxt = b_cur ^ kOperandBytes;
-    };
-    Tile tv;
-    tile_slots(tv, 0, 0);
-    tv.ra = sa.rsrc_at(sa.k_off(2, kt_n));
-    tv.rb = sb.rsrc_at(sb.k_off(2, kt_n));
     for (int kt = 0; kt < kt_n; ++kt) {
-      Tile nx;
       // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read (the addresses stand
       // for this tile's slots), then the addresses move on to the next tile's slots
-      step(1, 0, tv.a_fill, I8{}, 0, I0{}, tv.ra, [](auto) {}, std::integral_constant<int, kLateAdr ? 1 : 0>{},
-           tv.a_nxt, tv.b_nxt);
+      step(1, 0, a_fill, I8{}, 0, I0{}, rsrc_of(pa), [](auto) {}, std::integral_constant<int, kLateAdr ? 1 : 0>{},
+           a_nxt, b_cur ^ kOperandBytes);
       // second k-step: tile kt+1 must have landed for every wave (the eight younger instructions are
       // A of tile kt+2) and every wave must be done reading this tile's B slot before it is refilled
       __builtin_amdgcn_s_waitcnt(0x0078);  // vmcnt(8) lgkmcnt(0)
       __builtin_amdgcn_s_barrier();
       if (!kLateAdr) {
 #pragma unroll
-        for (int q = 0; q < kAddrA; ++q) set_adr_a(q, tv.a_nxt);
+        for (int q = 0; q < kAddrA; ++q) set_adr_a(q, a_nxt);
 #pragma unroll
-        for (int q = 0; q < kAddrB; ++q) set_adr_b(q, tv.b_nxt);
+        for (int q = 0; q < kAddrB; ++q) set_adr_b(q, b_cur ^ kOperandBytes);
       }
-      step(0, 1, 0, I0{}, tv.b_cur, I8{}, tv.rb,
+      const bool more = kt + 3 < kt_n;  // else: past the end, the last tile is fetched again and never consumed
+      step(0, 1, 0, I0{}, b_cur, I8{}, rsrc_of(pb),
            [&](auto part) {
-             if (decltype(part)::value == 0) tile_slots(nx, tv.a_nxt, tv.b_nxt);
-             if (decltype(part)::value == 1) nx.ra = sa.rsrc_at(sa.k_off(kt + 3, kt_n));
-             if (decltype(part)::value == 2) nx.rb = sb.rsrc_at(sb.k_off(kt + 3, kt_n));
+             constexpr int kPart = decltype(part)::value;
+             if (kPart == 0) { a_nxt = next_a_slot(a_nxt); pin(a_nxt); }
+             if (kPart == 1) { a_fill = next_a_slot(a_nxt); pin(a_fill); }
+             if (kPart == 2) { pa += more ? sa.kt_bytes : 0; pin(pa); }
+             if (kPart == 3) { pb += more ? sb.kt_bytes : 0; pin(pb); }
+             if (kPart == 4) { b_cur ^= kOperandBytes; pin(b_cur); }
            },
            I0{}, 0, 0);
-      tv = nx;
       wait_lds_reads();  // the next tile's first fragments, read under the second k-step
     }
     __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
