@@ -397,7 +397,7 @@ struct DmaLoopT {
     auto rsrc_of = [](const char* p) {
       return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, 0x7fffffff, 0x00020000);
     };
-    for (int kt = 0; kt < kt_n; ++kt) {
+    auto k_tile = [&](int kt) {
       // first k-step: A of tile kt+2; the fragments of this tile's second k-step are read (the addresses stand
       // for this tile's slots), then the addresses move on to the next tile's slots
       step(1, 0, a_fill, I8{}, 0, I0{}, rsrc_of(pa), [](auto) {}, std::integral_constant<int, kLateAdr ? 1 : 0>{},
@@ -424,7 +424,14 @@ struct DmaLoopT {
            },
            I0{}, 0, 0);
       wait_lds_reads();  // the next tile's first fragments, read under the second k-step
+    };
+    // two k-tiles per trip: half as many back edges
+    int kt = 0;
+    for (; kt + 1 < kt_n; kt += 2) {
+      k_tile(kt);
+      k_tile(kt + 1);
     }
+    if (kt < kt_n) k_tile(kt);
     __builtin_amdgcn_s_waitcnt(0x0070);  // drain the DMA issued for tiles past the end
     __builtin_amdgcn_s_barrier();
     settle_acc();
